@@ -1,0 +1,87 @@
+"""ctypes binding of ``libdeepshift_hip.so`` (the C ABI declared in ``include/deepshift_hip.h``).
+
+The library is the only compute path of this package: if it is missing, loading fails loudly --
+there is no CPU or eager-PyTorch fallback.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libdeepshift_hip.so")
+
+DS_Q_ROUND_TO_FIXED = 0
+DS_Q_CAST = 1
+
+_c_int = ctypes.c_int
+_c_i64 = ctypes.c_int64
+_ptr = ctypes.c_void_p
+_size = ctypes.c_size_t
+
+# name -> (restype, argtypes); mirrors include/deepshift_hip.h one to one
+SIGNATURES = {
+    "ds_version": (_c_int, []),
+    "ds_status_string": (ctypes.c_char_p, [_c_int]),
+    "ds_pack_i32": (_c_int, [_ptr, _ptr, _ptr, _c_int, _c_int, _c_int, _c_int, _ptr]),
+    "ds_tiled_bytes": (_size, [_c_int, _c_int, _c_int]),
+    "ds_tile_weights_i32": (_c_int, [_ptr, _ptr, _c_int, _c_int, _c_int, _c_int, _ptr]),
+    "ds_linear_workspace_bytes": (_size, [_c_int] * 4),
+    "ds_linear_i32": (_c_int, [_ptr] * 4 + [_c_int] * 5 + [_ptr, _size, _ptr]),
+    "ds_linear_tiled_workspace_bytes": (_size, [_c_int] * 4),
+    "ds_linear_tiled_i32": (_c_int, [_ptr, _c_int, _ptr, _ptr, _ptr] + [_c_int] * 5 + [_ptr, _size, _ptr]),
+    "ds_conv2d_workspace_bytes": (_size, [_c_int] * 10),
+    "ds_conv2d_i32": (_c_int, [_ptr] * 4 + [_c_int] * 11 + [_ptr, _size, _ptr]),
+    "ds_conv2d_tiled_workspace_bytes": (_size, [_c_int] * 10),
+    "ds_conv2d_tiled_i32": (_c_int, [_ptr] * 4 + [_c_int] * 11 + [_ptr, _size, _ptr]),
+    "ds_quantize_f32_i32": (_c_int, [_ptr, _ptr, _c_i64, _c_int, _c_int, _c_int, _ptr]),
+    "ds_quantize_pad_f32_i32": (_c_int, [_ptr, _ptr] + [_c_int] * 9 + [_ptr]),
+    "ds_quantize_transpose_f32_i32": (_c_int, [_ptr, _ptr] + [_c_int] * 6 + [_ptr]),
+    "ds_pad_i32": (_c_int, [_ptr, _ptr] + [_c_int] * 6 + [_ptr]),
+    "ds_transpose_i32": (_c_int, [_ptr, _ptr, _c_int, _c_int, _c_int, _ptr]),
+    "ds_dequantize_i32_f32": (_c_int, [_ptr, _ptr, _c_i64, _c_int, _ptr]),
+    "ds_valu_calibrate": (_c_int, [_ptr, _c_int, _c_int, _ptr]),
+    "ds_copy_i32": (_c_int, [_ptr, _ptr, _c_i64, _ptr]),
+}
+
+_LIB = None
+
+
+class DeepShiftError(RuntimeError):
+    """A libdeepshift_hip entry point returned a non-zero status."""
+
+    def __init__(self, fn, status, message):
+        super().__init__("%s failed: %s (status %d)" % (fn, message, status))
+        self.status = status
+
+
+def lib():
+    """The loaded library; raises if it has not been built (``python -m deepshift_amd.build``)."""
+    global _LIB
+    if _LIB is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "%s is missing: build it with `python -m deepshift_amd.build` "
+                "(there is no fallback path)" % LIB_PATH)
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _LIB = handle
+    return _LIB
+
+
+def call(name, *args):
+    """Invoke a status-returning entry point and raise :class:`DeepShiftError` on failure."""
+    handle = lib()
+    status = getattr(handle, name)(*args)
+    if status != 0:
+        raise DeepShiftError(name, status, handle.ds_status_string(status).decode())
+
+
+def current_stream(device):
+    import torch
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def ptr(tensor):
+    return None if tensor is None else ctypes.c_void_p(tensor.data_ptr())

@@ -1,0 +1,66 @@
+// Version / status strings and the VALU calibration kernel.
+#include "ds_common.h"
+
+namespace ds {
+
+// A dependency-free stream of the two instructions one shift-add term costs (v_ashrrev_i32 then
+// v_xad_u32) with wave-uniform shift amounts and sign masks, i.e. the instruction mix of
+// shift_kernel with nothing else in the way.  16 accumulators x 4 activations = 64 pairs per
+// iteration and lane.
+__global__ __launch_bounds__(256) void valu_calibrate_kernel(int32_t *sink, int iters, uint32_t seed)
+{
+    int32_t acc[16][4];
+    int32_t xv[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) xv[r] = (int32_t)(threadIdx.x * 2654435761u + r * 40503u + blockIdx.x);
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[j][r] = j + r;
+    uint32_t w = seed;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const uint32_t s = (w >> j) & 31u;
+            const int32_t mask = -(int32_t)((w >> (j + 8)) & 1u);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[j][r] = ((xv[r] >> s) ^ mask) + acc[j][r];
+        }
+        w = w * 1664525u + 1013904223u;
+    }
+    int32_t total = 0;
+#pragma unroll
+    for (int j = 0; j < 16; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) total += acc[j][r];
+    sink[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = total;
+}
+
+}  // namespace ds
+
+using namespace ds;
+
+DS_EXPORT int ds_version(void) { return 100; }
+
+DS_EXPORT const char *ds_status_string(int status)
+{
+    switch (status) {
+    case DS_OK: return "ok";
+    case DS_EINVAL: return "invalid argument (null pointer, negative or inconsistent size)";
+    case DS_EBITS: return "unsupported bits (1..6 supported)";
+    case DS_EBASE: return "unsupported base (must be in -31..0)";
+    case DS_EWORKSPACE: return "workspace missing or too small";
+    case DS_ETOOLARGE: return "tensor too large for 32-bit offsets";
+    default: break;
+    }
+    if (status <= DS_EHIP) return hipGetErrorString((hipError_t)(DS_EHIP - status));
+    return "unknown status";
+}
+
+DS_EXPORT int ds_valu_calibrate(int32_t *sink, int blocks, int iters, ds_stream_t stream)
+{
+    if (!sink || blocks < 1 || iters < 0) return DS_EINVAL;
+    hipLaunchKernelGGL(valu_calibrate_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, sink,
+                       iters, 0x9E3779B9u);
+    return launch_status();
+}

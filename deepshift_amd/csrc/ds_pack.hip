@@ -1,0 +1,149 @@
+// Weight packing (sign + shift codes -> 32-bit words) and re-tiling for the compute kernels.
+#include "ds_common.h"
+
+namespace ds {
+
+// One thread per output word of the reference format (kernels/cuda/shift.cu:27-55), whole tensor
+// in one launch.  Consecutive threads read consecutive runs of `num` codes -> coalesced enough for
+// a conversion-time kernel.
+__global__ void pack_kernel(const int32_t *__restrict__ s, const int32_t *__restrict__ sign,
+                            int32_t *__restrict__ out, long words, int K, int comm, int bits, int num,
+                            int base)
+{
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= words) return;
+    const long o = idx / comm;
+    const int j = (int)(idx - o * comm);
+    const int k0 = j * num;
+    int len = K - k0;
+    if (len > num) len = num;
+    const int32_t *sp = s + o * K + k0;
+    const int32_t *gp = sign + o * K + k0;
+    const uint32_t fmask = (1u << bits) - 1u;
+    uint32_t value = 0;
+    int pos = 0;
+    for (int i = 0; i < len; ++i) {
+        value |= ((uint32_t)(sp[i] - base) & fmask) << pos;
+        pos += bits;
+        value |= (uint32_t)(gp[i] > 0 ? 1 : 0) << pos;
+        pos += 1;
+    }
+    out[idx] = (int32_t)value;
+}
+
+int launch_pack(const int32_t *s, const int32_t *sign, int32_t *out, int O, int K, int bits,
+                int base, hipStream_t st)
+{
+    const int num = codes_per_word(bits);
+    const int comm = ceil_div(K, num);
+    const long words = (long)O * comm;
+    if (words == 0) return DS_OK;
+    const long blocks = (words + 255) / 256;
+    hipLaunchKernelGGL(pack_kernel, dim3((unsigned)blocks), dim3(256), 0, st, s, sign, out, words, K,
+                       comm, bits, num, base);
+    return launch_status();
+}
+
+// Reference-format words [N][comm] -> tiled words [ntiles16][comm][16].
+//   * code sign bit inverted: 1 = negative (the compute kernel sign-extends it into an xor mask);
+//   * codes past K, and every code of a padding channel, become (field 0, positive): with the
+//     activation read as 0 they add nothing;
+//   * zero-weight codes (field >= 32, bits == 6 only) are made positive so that they neither add
+//     nor need the negative-count correction.
+__global__ void tile_kernel(const int32_t *__restrict__ w_ref, uint32_t *__restrict__ wt, int N, int K,
+                            int comm, int bits, int num, long words)
+{
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= words) return;
+    const int j = (int)(idx % kTileWords);
+    const long rest = idx / kTileWords;
+    const int g = (int)(rest % comm);
+    const int t = (int)(rest / comm);
+    const int n = t * kTileWords + j;
+    uint32_t out = 0;
+    const int cb = bits + 1;
+    const uint32_t fmask = (1u << bits) - 1u;
+    if (n < N) {
+        const uint32_t in = (uint32_t)w_ref[(long)n * comm + g];
+        for (int i = 0; i < num; ++i) {
+            const int k = g * num + i;
+            if (k >= K) break;
+            const uint32_t code = in >> (i * cb);
+            const uint32_t field = code & fmask;
+            uint32_t neg = ((code >> bits) & 1u) ^ 1u;
+            if (field >= 32u) neg = 0;
+            out |= (field | (neg << bits)) << (i * cb);
+        }
+    }
+    wt[idx] = out;
+}
+
+// negcount[n] = number of real, non-zero, negative codes of channel n (0 for padding channels)
+__global__ void negcount_kernel(const int32_t *__restrict__ w_ref, int32_t *__restrict__ negcount,
+                                int N, int Npad, int K, int comm, int bits, int num)
+{
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= Npad) return;
+    int count = 0;
+    if (n < N) {
+        const int cb = bits + 1;
+        const uint32_t fmask = (1u << bits) - 1u;
+        for (int g = 0; g < comm; ++g) {
+            const uint32_t in = (uint32_t)w_ref[(long)n * comm + g];
+            for (int i = 0; i < num; ++i) {
+                if (g * num + i >= K) break;
+                const uint32_t code = in >> (i * cb);
+                if ((code & fmask) < 32u && ((code >> bits) & 1u) == 0u) ++count;
+            }
+        }
+    }
+    negcount[n] = count;
+}
+
+int launch_tile(const int32_t *w_ref, void *tiled, int N, int K, int bits, hipStream_t st)
+{
+    const TiledGeom g = tiled_geom(N, K, bits);
+    if (g.word_count) {
+        const long blocks = ((long)g.word_count + 255) / 256;
+        hipLaunchKernelGGL(tile_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w_ref,
+                           (uint32_t *)tiled, N, K, g.comm, bits, g.num, (long)g.word_count);
+    }
+    const int Npad = g.ntiles16 * kTileWords;
+    if (Npad) {
+        hipLaunchKernelGGL(negcount_kernel, dim3(ceil_div(Npad, 64)), dim3(64), 0, st, w_ref,
+                           (int32_t *)tiled_negcount(tiled, g), N, Npad, K, g.comm, bits, g.num);
+    }
+    return launch_status();
+}
+
+}  // namespace ds
+
+using namespace ds;
+
+DS_EXPORT int ds_pack_i32(const int32_t *s, const int32_t *sign, int32_t *out, int O, int K, int bits,
+                          int base, ds_stream_t stream)
+{
+    if (bits < 1 || bits > 6) return DS_EBITS;
+    if (base > 0) return DS_EBASE;
+    if (O < 0 || K < 0) return DS_EINVAL;
+    if (O == 0 || K == 0) return DS_OK;
+    if (!s || !sign || !out) return DS_EINVAL;
+    return launch_pack(s, sign, out, O, K, bits, base, (hipStream_t)stream);
+}
+
+DS_EXPORT size_t ds_tiled_bytes(int N, int K, int bits)
+{
+    if (bits < 1 || bits > 6 || N < 0 || K < 0) return 0;
+    return tiled_geom(N, K, bits).bytes;
+}
+
+DS_EXPORT int ds_tile_weights_i32(const int32_t *w_ref, void *tiled, int N, int K, int bits, int base,
+                                  ds_stream_t stream)
+{
+    if (bits < 1 || bits > 6) return DS_EBITS;
+    if (base > 0 || base < -31) return DS_EBASE;
+    if (N < 0 || K < 0) return DS_EINVAL;
+    if (N == 0) return DS_OK;
+    if (!tiled || (!w_ref && K > 0)) return DS_EINVAL;
+    return launch_tile(w_ref, tiled, N, K, bits, (hipStream_t)stream);
+}

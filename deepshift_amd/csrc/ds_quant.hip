@@ -1,0 +1,284 @@
+// Fixed-point conversion passes around the shift kernels (HBM-bound, one read + one write each).
+#include "ds_common.h"
+
+namespace ds {
+
+// float -> int32 on the 2^-F grid.
+//   ROUND_TO_FIXED: utils.round_to_fixed (utils.py:7-21) followed by (x * 2**F).int()
+//   (modules.py:153).  floor(x / 2^-F) * 2^-F is clamped to [-2^(I-1), 2^(I-1) - 1] and scaled back
+//   by 2^F; all three scalings are by powers of two, hence exact, so the clamp can be applied to
+//   floor(x * 2^F) directly with bounds scaled by 2^F.  I == 1 is the reference's special case
+//   sign(x) - 1.
+//   CAST: (x * 2**F).int() alone (modules.py:25): truncation toward zero; the hardware conversion
+//   saturates and maps NaN to 0.
+struct QuantSpec {
+    float scale, lo, hi;
+    int mode, I;
+};
+
+// float -> int32 toward zero, saturating, NaN -> 0 (what v_cvt_i32_f32 returns; spelled out because
+// an out-of-range C++ conversion is undefined).
+__device__ __forceinline__ int32_t f2i_sat(float v)
+{
+    if (v != v) return 0;
+    if (v >= 2147483648.0f) return 2147483647;
+    if (v <= -2147483648.0f) return (int32_t)0x80000000;
+    return (int32_t)v;
+}
+
+__device__ __forceinline__ int32_t quantize_one(float v, const QuantSpec &q)
+{
+    if (q.mode == DS_Q_CAST) return f2i_sat(v * q.scale);
+    float r;
+    if (q.I == 1) {
+        r = ((v > 0.0f) ? 1.0f : ((v < 0.0f) ? -1.0f : 0.0f)) - 1.0f;
+        if (v != v) r = v;
+        r *= q.scale;
+    } else {
+        r = floorf(v * q.scale);
+        // torch.clamp semantics: NaN propagates
+        r = (r < q.lo) ? q.lo : r;
+        r = (r > q.hi) ? q.hi : r;
+    }
+    return f2i_sat(r);
+}
+
+static QuantSpec make_spec(int I, int F, int mode)
+{
+    QuantSpec q;
+    q.scale = ldexpf(1.0f, F);
+    q.lo = -ldexpf(1.0f, I - 1 + F);
+    q.hi = (ldexpf(1.0f, I - 1) - 1.0f) * q.scale;
+    q.mode = mode;
+    q.I = I;
+    return q;
+}
+
+__global__ void quantize_kernel(const float *__restrict__ x, int32_t *__restrict__ q, long n,
+                                QuantSpec spec)
+{
+    const long stride = (long)gridDim.x * blockDim.x;
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long n4 = n >> 2;
+    const bool aligned = (((uintptr_t)x | (uintptr_t)q) & 15) == 0;
+    if (aligned) {
+        const float4 *x4 = (const float4 *)x;
+        int4 *q4 = (int4 *)q;
+        for (; i < n4; i += stride) {
+            const float4 v = x4[i];
+            int4 o;
+            o.x = quantize_one(v.x, spec);
+            o.y = quantize_one(v.y, spec);
+            o.z = quantize_one(v.z, spec);
+            o.w = quantize_one(v.w, spec);
+            q4[i] = o;
+        }
+        for (long t = (n4 << 2) + (long)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += stride)
+            q[t] = quantize_one(x[t], spec);
+    } else {
+        for (; i < n; i += stride) q[i] = quantize_one(x[i], spec);
+    }
+}
+
+// One thread per padded output element; rows of the padded image are written contiguously.
+template <bool FROM_FLOAT>
+__global__ void pad_kernel(const void *__restrict__ xin, int32_t *__restrict__ q, long planes, int H,
+                           int W, int ph, int pw, QuantSpec spec)
+{
+    const int Hp = H + 2 * ph, Wp = W + 2 * pw;
+    const long total = planes * Hp * Wp;
+    const long stride = (long)gridDim.x * blockDim.x;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+        const long plane = idx / ((long)Hp * Wp);
+        const int rem = (int)(idx - plane * Hp * Wp);
+        const int hp = rem / Wp;
+        const int wp = rem - hp * Wp;
+        const int h = hp - ph, w = wp - pw;
+        int32_t v = 0;
+        if ((unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W) {
+            const long src = (plane * H + h) * W + w;
+            if (FROM_FLOAT) v = quantize_one(((const float *)xin)[src], spec);
+            else v = ((const int32_t *)xin)[src];
+        }
+        q[idx] = v;
+    }
+}
+
+// x[M][K] float -> qT[K][ldx] int32 through a 64x64 LDS tile (both sides coalesced).
+__global__ __launch_bounds__(256) void quantize_transpose_kernel(const float *__restrict__ x,
+                                                                 int32_t *__restrict__ qT, int M, int K,
+                                                                 int ldx, QuantSpec spec)
+{
+    __shared__ int32_t tile[64][65];
+    const int k0 = blockIdx.x * 64, m0 = blockIdx.y * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int r = ty; r < 64; r += 4) {
+        const int m = m0 + r, k = k0 + tx;
+        int32_t v = 0;
+        if (m < M && k < K) v = quantize_one(x[(long)m * K + k], spec);
+        tile[r][tx] = v;
+    }
+    __syncthreads();
+    for (int r = ty; r < 64; r += 4) {
+        const int k = k0 + r, m = m0 + tx;
+        if (k < K && m < ldx) qT[(long)k * ldx + m] = tile[tx][r];
+    }
+}
+
+__global__ __launch_bounds__(256) void transpose_i32_kernel(const int32_t *__restrict__ x,
+                                                            int32_t *__restrict__ xT, int M, int K,
+                                                            int ldx)
+{
+    __shared__ int32_t tile[64][65];
+    const int k0 = blockIdx.x * 64, m0 = blockIdx.y * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int r = ty; r < 64; r += 4) {
+        const int m = m0 + r, k = k0 + tx;
+        tile[r][tx] = (m < M && k < K) ? x[(long)m * K + k] : 0;
+    }
+    __syncthreads();
+    for (int r = ty; r < 64; r += 4) {
+        const int k = k0 + r, m = m0 + tx;
+        if (k < K && m < ldx) xT[(long)k * ldx + m] = tile[tx][r];
+    }
+}
+
+int launch_transpose(const int32_t *x, int32_t *xT, int M, int K, int ldx, hipStream_t st)
+{
+    dim3 grid(ceil_div(K, 64), ceil_div(ldx, 64));
+    hipLaunchKernelGGL(transpose_i32_kernel, grid, dim3(256), 0, st, x, xT, M, K, ldx);
+    return launch_status();
+}
+
+__global__ void dequantize_kernel(const int32_t *__restrict__ y, float *__restrict__ out, long n,
+                                  float scale)
+{
+    const long stride = (long)gridDim.x * blockDim.x;
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const bool aligned = (((uintptr_t)y | (uintptr_t)out) & 15) == 0;
+    if (aligned) {
+        const long n4 = n >> 2;
+        const int4 *y4 = (const int4 *)y;
+        float4 *o4 = (float4 *)out;
+        for (; i < n4; i += stride) {
+            const int4 v = y4[i];
+            float4 o;
+            // out.float() / 2**F: int32 -> fp32 rounds to nearest even, the division is exact
+            o.x = (float)v.x / scale;
+            o.y = (float)v.y / scale;
+            o.z = (float)v.z / scale;
+            o.w = (float)v.w / scale;
+            o4[i] = o;
+        }
+        for (long t = (n4 << 2) + (long)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += stride)
+            out[t] = (float)y[t] / scale;
+    } else {
+        for (; i < n; i += stride) out[i] = (float)y[i] / scale;
+    }
+}
+
+__global__ void copy_kernel(const int4 *__restrict__ src, int4 *__restrict__ dst, long n4)
+{
+    const long stride = (long)gridDim.x * blockDim.x;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) dst[i] = src[i];
+}
+
+static int grid_for(long work_items)
+{
+    long blocks = (work_items + 255) / 256;
+    if (blocks > 256 * 32) blocks = 256 * 32;
+    if (blocks < 1) blocks = 1;
+    return (int)blocks;
+}
+
+}  // namespace ds
+
+using namespace ds;
+
+static int check_fixed(int I, int F, int mode)
+{
+    if (mode != DS_Q_ROUND_TO_FIXED && mode != DS_Q_CAST) return DS_EINVAL;
+    if (I < 1 || F < 0 || I + F > 32) return DS_EINVAL;
+    return DS_OK;
+}
+
+DS_EXPORT int ds_quantize_f32_i32(const float *x, int32_t *q, int64_t n, int I, int F, int mode,
+                                  ds_stream_t stream)
+{
+    int rc = check_fixed(I, F, mode);
+    if (rc) return rc;
+    if (n < 0) return DS_EINVAL;
+    if (n == 0) return DS_OK;
+    if (!x || !q) return DS_EINVAL;
+    hipLaunchKernelGGL(quantize_kernel, dim3(grid_for((n + 3) / 4)), dim3(256), 0, (hipStream_t)stream,
+                       x, q, (long)n, make_spec(I, F, mode));
+    return launch_status();
+}
+
+DS_EXPORT int ds_quantize_pad_f32_i32(const float *x, int32_t *q, int Nb, int C, int H, int W, int ph,
+                                      int pw, int I, int F, int mode, ds_stream_t stream)
+{
+    int rc = check_fixed(I, F, mode);
+    if (rc) return rc;
+    if (Nb < 0 || C < 0 || H < 0 || W < 0 || ph < 0 || pw < 0) return DS_EINVAL;
+    const long total = (long)Nb * C * (H + 2 * ph) * (W + 2 * pw);
+    if (total == 0) return DS_OK;
+    if (!x || !q) return DS_EINVAL;
+    hipLaunchKernelGGL((pad_kernel<true>), dim3(grid_for(total)), dim3(256), 0, (hipStream_t)stream,
+                       (const void *)x, q, (long)Nb * C, H, W, ph, pw, make_spec(I, F, mode));
+    return launch_status();
+}
+
+DS_EXPORT int ds_pad_i32(const int32_t *x, int32_t *xp, int Nb, int C, int H, int W, int ph, int pw,
+                         ds_stream_t stream)
+{
+    if (Nb < 0 || C < 0 || H < 0 || W < 0 || ph < 0 || pw < 0) return DS_EINVAL;
+    const long total = (long)Nb * C * (H + 2 * ph) * (W + 2 * pw);
+    if (total == 0) return DS_OK;
+    if (!x || !xp) return DS_EINVAL;
+    hipLaunchKernelGGL((pad_kernel<false>), dim3(grid_for(total)), dim3(256), 0, (hipStream_t)stream,
+                       (const void *)x, xp, (long)Nb * C, H, W, ph, pw, make_spec(16, 16, 0));
+    return launch_status();
+}
+
+DS_EXPORT int ds_quantize_transpose_f32_i32(const float *x, int32_t *qT, int M, int K, int ldx, int I,
+                                            int F, int mode, ds_stream_t stream)
+{
+    int rc = check_fixed(I, F, mode);
+    if (rc) return rc;
+    if (M < 0 || K < 0 || ldx < M) return DS_EINVAL;
+    if (K == 0 || ldx == 0) return DS_OK;
+    if (!qT || (!x && M > 0)) return DS_EINVAL;
+    dim3 grid(ceil_div(K, 64), ceil_div(ldx, 64));
+    hipLaunchKernelGGL(quantize_transpose_kernel, grid, dim3(256), 0, (hipStream_t)stream, x, qT, M, K,
+                       ldx, make_spec(I, F, mode));
+    return launch_status();
+}
+
+DS_EXPORT int ds_transpose_i32(const int32_t *x, int32_t *xT, int M, int K, int ldx, ds_stream_t stream)
+{
+    if (M < 0 || K < 0 || ldx < M) return DS_EINVAL;
+    if (K == 0 || ldx == 0) return DS_OK;
+    if (!xT || (!x && M > 0)) return DS_EINVAL;
+    return launch_transpose(x, xT, M, K, ldx, (hipStream_t)stream);
+}
+
+DS_EXPORT int ds_dequantize_i32_f32(const int32_t *y, float *out, int64_t n, int F, ds_stream_t stream)
+{
+    if (n < 0 || F < 0 || F > 31) return DS_EINVAL;
+    if (n == 0) return DS_OK;
+    if (!y || !out) return DS_EINVAL;
+    hipLaunchKernelGGL(dequantize_kernel, dim3(grid_for((n + 3) / 4)), dim3(256), 0,
+                       (hipStream_t)stream, y, out, (long)n, ldexpf(1.0f, F));
+    return launch_status();
+}
+
+DS_EXPORT int ds_copy_i32(const int32_t *src, int32_t *dst, int64_t n, ds_stream_t stream)
+{
+    if (n < 0 || (n & 3)) return DS_EINVAL;
+    if (n == 0) return DS_OK;
+    if (!src || !dst || (((uintptr_t)src | (uintptr_t)dst) & 15)) return DS_EINVAL;
+    hipLaunchKernelGGL(copy_kernel, dim3(grid_for(n / 4)), dim3(256), 0, (hipStream_t)stream,
+                       (const int4 *)src, (int4 *)dst, (long)(n / 4));
+    return launch_status();
+}

@@ -1,0 +1,457 @@
+// Shift-add convolution / GEMM for gfx950.
+//
+// One kernel serves Conv2dShift and LinearShift.  The work is y[m][n] = bias[n] +
+// sum_k sgn(n,k) * (x[m,k] >> s(n,k)) with m running over output pixels (or batch rows)
+// and n over output channels.
+//
+// Mapping onto CDNA4:
+//   * the 64 lanes of a wavefront are 64 consecutive output pixels m, so activation loads are
+//     coalesced along the image row and every lane owns whole accumulators;
+//   * the weight codes of a (channel, k) pair are the same for every lane, so the packed words are
+//     fetched with scalar loads and decoded on the scalar ALU (one bit-field extract for the shift
+//     amount, one for the sign mask) -- the vector ALU only executes the two instructions a
+//     shift-add term really needs:  t = x >> s  (v_ashrrev_i32)  and  acc = (t ^ mask) + acc
+//     (v_xad_u32).  -t = (t ^ -1) + 1, and the "+ 1" of every negative code of a channel is a
+//     constant that is added once in the epilogue (the tiled weight blob carries the count);
+//   * each lane keeps R pixels x J channels of int32 accumulators in registers, so one activation
+//     load feeds 2*J vector instructions and one decoded code feeds 2*R of them;
+//   * no LDS, no barriers: waves are independent, occupancy is bounded by registers only;
+//   * layers with few pixels split K over gridDim.y and combine with integer atomics (wrap-around
+//     addition commutes, so the result stays bit-exact).
+#include "ds_common.h"
+
+namespace ds {
+
+struct ShiftArgs {
+    const int32_t *x;       // activations: element (m, k) lives at x[xoff(m) + ktab[k]]
+    const uint32_t *wt;     // tiled words [ntiles16][comm][16]
+    const int32_t *negcnt;  // per channel: number of negative codes
+    const int32_t *bias;    // per channel or nullptr
+    const int32_t *ktab;    // [comm*num] activation offset of reduction index k
+    int32_t *y;
+    int M, N, K, comm;
+    int pix_per_img, OW;                  // m -> (img, oh, ow)
+    int x_img_stride, x_row_stride, x_col_stride;
+    int y_img_stride, y_pix_stride, y_ch_stride;
+    int groups_per_split;                 // k-groups (words) per gridDim.y slice
+    int nbase;                            // -base (left shift applied after the right shift)
+    int tiles_m4;                         // number of 4-wave pixel tiles
+    int tiles_n;                          // number of channel tiles
+    int blocks_per_xcd;                   // ceil(tiles / 8)
+    int atomic_out;                       // 1: y pre-filled with bias, accumulate atomically
+};
+
+// (t ^ mask) + acc in ONE vector instruction with the wave-uniform mask read from a scalar
+// register.  Spelled as v_xad_u32 because the compiler otherwise re-associates pairs of terms into
+// v_xor + v_xor + v_add3 (2.5 instructions per term instead of 2).
+__device__ __forceinline__ int32_t xor_add(int32_t t, int32_t mask, int32_t acc)
+{
+    int32_t out;
+    asm("v_xad_u32 %0, %1, %2, %3" : "=v"(out) : "v"(t), "s"(mask), "v"(acc));
+    return out;
+}
+
+__device__ __forceinline__ int32_t *at_lane(int32_t *uniform_base, uint32_t lane_bytes)
+{
+    return (int32_t *)((char *)uniform_base + lane_bytes);
+}
+__device__ __forceinline__ int32_t ld_lane(const int32_t *uniform_base, uint32_t lane_bytes)
+{
+    return *(const int32_t *)((const char *)uniform_base + lane_bytes);
+}
+
+template <int BITS, bool GENERAL, int R, int J>
+__device__ __forceinline__ void accumulate_code(int32_t (&acc)[R][J], const int32_t (&xv)[R],
+                                                const uint32_t (&w)[J], const int i, const int nbase)
+{
+    constexpr int CB = BITS + 1;
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        const uint32_t code = w[j] >> (i * CB);
+        // tiled format: bit BITS of a code is 1 for a NEGATIVE weight
+        const int32_t mask = -(int32_t)((code >> BITS) & 1u);
+        const uint32_t field = code & ((1u << BITS) - 1u);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            int32_t t = xv[r] >> (field & 31u);
+            if (GENERAL) {
+                t = (int32_t)((uint32_t)t << nbase);
+                if (BITS == 6) t &= -(int32_t)(((field >> 5) & 1u) ^ 1u);  // field >= 32: zero weight
+            }
+            acc[r][j] = xor_add(t, mask, acc[r][j]);
+        }
+    }
+}
+
+template <int BITS, bool GENERAL, int R, int J>
+__global__ __launch_bounds__(256) void shift_kernel(const ShiftArgs p)
+{
+    constexpr int NUM = 32 / (BITS + 1);
+    static_assert(J % kTileWords == 0, "J must be a multiple of the layout tile");
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+
+    // XCD-aware tile order: consecutive workgroup ids land on different XCDs, so give each XCD a
+    // contiguous range of tiles (neighbouring pixel tiles and all channel tiles of a pixel range
+    // then share one L2).
+    const int bid = blockIdx.x;
+    const int tile = (bid & 7) * p.blocks_per_xcd + (bid >> 3);
+    if (tile >= p.tiles_m4 * p.tiles_n) return;
+    const int ntile = tile % p.tiles_n;
+    const int mtile = (tile / p.tiles_n) * 4 + wave;
+    const int m0 = mtile * (R * kWave);
+    if (m0 >= p.M) return;
+
+    // per-lane pixel coordinates
+    uint32_t xoff[R], yoff[R];
+    bool live[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        int m = m0 + r * kWave + lane;
+        live[r] = m < p.M;
+        if (!live[r]) m = p.M - 1;
+        const int img = m / p.pix_per_img;
+        const int rem = m - img * p.pix_per_img;
+        const int oh = rem / p.OW;
+        const int ow = rem - oh * p.OW;
+        // byte offsets (every tensor is < 2^31 bytes): a uniform 64-bit base plus a 32-bit lane
+        // offset is the addressing mode global loads and stores take directly
+        xoff[r] = 4u * (uint32_t)(img * p.x_img_stride + oh * p.x_row_stride + ow * p.x_col_stride);
+        yoff[r] = 4u * (uint32_t)(img * p.y_img_stride + rem * p.y_pix_stride);
+    }
+
+    int32_t acc[R][J];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int j = 0; j < J; ++j) acc[r][j] = 0;
+
+    const int g_begin = blockIdx.y * p.groups_per_split;
+    int g_end = g_begin + p.groups_per_split;
+    if (g_end > p.comm) g_end = p.comm;
+    const int full_groups = p.K / NUM;  // groups whose NUM codes are all real
+    const int g_full_end = g_end < full_groups ? g_end : full_groups;
+
+    const uint32_t *wrow = p.wt + (size_t)(ntile * (J / kTileWords)) * p.comm * kTileWords;
+    const size_t tile_stride = (size_t)p.comm * kTileWords;
+
+    for (int g = g_begin; g < g_full_end; ++g) {
+        uint32_t w[J];
+#pragma unroll
+        for (int j = 0; j < J; ++j)
+            w[j] = wrow[(j / kTileWords) * tile_stride + (size_t)g * kTileWords + (j % kTileWords)];
+        int32_t xv[NUM][R];
+#pragma unroll
+        for (int i = 0; i < NUM; ++i) {
+            const int32_t *xk = p.x + p.ktab[g * NUM + i];
+#pragma unroll
+            for (int r = 0; r < R; ++r) xv[i][r] = ld_lane(xk, xoff[r]);
+        }
+#pragma unroll
+        for (int i = 0; i < NUM; ++i) accumulate_code<BITS, GENERAL, R, J>(acc, xv[i], w, i, p.nbase);
+    }
+    // tail group: codes with k >= K read as x = 0 (the tiled blob holds neutral codes there)
+    for (int g = g_full_end; g < g_end; ++g) {
+        uint32_t w[J];
+#pragma unroll
+        for (int j = 0; j < J; ++j)
+            w[j] = wrow[(j / kTileWords) * tile_stride + (size_t)g * kTileWords + (j % kTileWords)];
+#pragma unroll
+        for (int i = 0; i < NUM; ++i) {
+            int32_t xv[R];
+            const bool real = g * NUM + i < p.K;
+            const int32_t *xk = p.x + (real ? p.ktab[g * NUM + i] : 0);
+#pragma unroll
+            for (int r = 0; r < R; ++r) xv[r] = real ? ld_lane(xk, xoff[r]) : 0;
+            accumulate_code<BITS, GENERAL, R, J>(acc, xv, w, i, p.nbase);
+        }
+    }
+
+    // epilogue
+    const int n0 = ntile * J;
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        const int n = n0 + j;
+        if (n >= p.N) break;
+        int32_t *yc = p.y + (size_t)n * p.y_ch_stride;
+        if (p.atomic_out) {
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                if (live[r]) atomicAdd(at_lane(yc, yoff[r]), acc[r][j]);
+        } else {
+            const int32_t add = p.negcnt[n] + (p.bias ? p.bias[n] : 0);
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                if (live[r]) *at_lane(yc, yoff[r]) = acc[r][j] + add;
+        }
+    }
+}
+
+// y = bias[n] + negcnt[n] for the split-K path.  Both output layouts ([img][n][pix] and [m][n])
+// are dense, so the flat index is the address and n = (idx / y_ch_stride) % N.
+__global__ void fill_bias_kernel(const ShiftArgs p)
+{
+    const long total = (long)p.M * p.N;
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long)gridDim.x * blockDim.x) {
+        const int n = (int)((idx / p.y_ch_stride) % p.N);
+        p.y[idx] = p.negcnt[n] + (p.bias ? p.bias[n] : 0);
+    }
+}
+
+// ktab[k] = ic*plane + fh*row + fw for k = (ic, fh, fw); entries past K are 0
+__global__ void ktab_kernel(int32_t *ktab, int K, int Kpad, int FH, int FW, int plane, int row)
+{
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= Kpad) return;
+    int v = 0;
+    if (k < K) {
+        const int ic = k / (FH * FW);
+        const int rem = k - ic * FH * FW;
+        const int fh = rem / FW;
+        const int fw = rem - fh * FW;
+        v = ic * plane + fh * row + fw;
+    }
+    ktab[k] = v;
+}
+
+template <int BITS, bool GENERAL, int R, int J>
+static int launch_shift(ShiftArgs a, int nsplit, hipStream_t st)
+{
+    a.tiles_m4 = ceil_div(ceil_div(a.M, R * kWave), 4);
+    a.tiles_n = ceil_div(a.N, J);
+    const int tiles = a.tiles_m4 * a.tiles_n;
+    a.blocks_per_xcd = ceil_div(tiles, 8);
+    a.groups_per_split = ceil_div(a.comm, nsplit);
+    nsplit = ceil_div(a.comm, a.groups_per_split);
+    a.atomic_out = nsplit > 1;
+    if (a.atomic_out) {
+        const long total = (long)a.M * a.N;
+        int blocks = (int)((total + 255) / 256);
+        if (blocks > 65536) blocks = 65536;
+        hipLaunchKernelGGL(fill_bias_kernel, dim3(blocks), dim3(256), 0, st, a);
+    }
+    dim3 grid(a.blocks_per_xcd * 8, nsplit);
+    hipLaunchKernelGGL((shift_kernel<BITS, GENERAL, R, J>), grid, dim3(256), 0, st, a);
+    return launch_status();
+}
+
+// Tile shape / split-K choice.  256 CUs x 4 SIMDs want a few thousand waves in flight.
+template <int BITS, bool GENERAL>
+static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
+{
+    const long waves_2x32 = (long)ceil_div(a.M, 128) * ceil_div(a.N, 32);
+    const int target_waves = 3072;
+    int nsplit = 1;
+    if (waves_2x32 < target_waves) {
+        nsplit = (int)((target_waves + waves_2x32 - 1) / waves_2x32);
+        const int max_split = a.comm / 8 > 0 ? a.comm / 8 : 1;  // keep >= 8 words per slice
+        if (nsplit > max_split) nsplit = max_split;
+        if (nsplit > 64) nsplit = 64;
+    }
+    if (a.N <= 16) return launch_shift<BITS, GENERAL, 4, 16>(a, nsplit, st);
+    return launch_shift<BITS, GENERAL, 2, 32>(a, nsplit, st);
+}
+
+static int dispatch_bits(const ShiftArgs &a, int bits, bool general, hipStream_t st)
+{
+    switch (bits) {
+    case 1: return general ? dispatch_shape<1, true>(a, st) : dispatch_shape<1, false>(a, st);
+    case 2: return general ? dispatch_shape<2, true>(a, st) : dispatch_shape<2, false>(a, st);
+    case 3: return general ? dispatch_shape<3, true>(a, st) : dispatch_shape<3, false>(a, st);
+    case 4: return general ? dispatch_shape<4, true>(a, st) : dispatch_shape<4, false>(a, st);
+    case 5: return general ? dispatch_shape<5, true>(a, st) : dispatch_shape<5, false>(a, st);
+    case 6: return dispatch_shape<6, true>(a, st);
+    default: return DS_EBITS;
+    }
+}
+
+static int check_common(int bits, int base)
+{
+    if (bits < 1 || bits > 6) return DS_EBITS;
+    if (base > 0) return DS_EBASE;
+    if (base < -31) return DS_EBASE;
+    return DS_OK;
+}
+
+constexpr size_t kMaxBytes = (size_t)1 << 31;
+
+}  // namespace ds
+
+using namespace ds;
+
+// ---------------------------------------------------------------------------------------------
+// Conv2dShift
+// ---------------------------------------------------------------------------------------------
+
+DS_EXPORT size_t ds_conv2d_tiled_workspace_bytes(int Nb, int C, int Hp, int Wp, int O, int FH,
+                                                 int FW, int sh, int sw, int bits)
+{
+    (void)Nb; (void)Hp; (void)Wp; (void)O; (void)sh; (void)sw;
+    if (bits < 1 || bits > 6 || C < 0 || FH < 1 || FW < 1) return 0;
+    const int num = codes_per_word(bits);
+    const size_t K = (size_t)C * FH * FW;
+    return align_up((K + num - 1) / num * num * 4, 256);
+}
+
+DS_EXPORT size_t ds_conv2d_workspace_bytes(int Nb, int C, int Hp, int Wp, int O, int FH, int FW,
+                                           int sh, int sw, int bits)
+{
+    if (bits < 1 || bits > 6 || C < 0 || O < 0 || FH < 1 || FW < 1) return 0;
+    return ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits) +
+           align_up(tiled_geom(O, C * FH * FW, bits).bytes, 256);
+}
+
+DS_EXPORT int ds_conv2d_tiled_i32(const int32_t *x, const void *tiled, const int32_t *bias,
+                                  int32_t *y, int Nb, int C, int Hp, int Wp, int O, int FH, int FW,
+                                  int sh, int sw, int bits, int base, void *workspace,
+                                  size_t workspace_bytes, ds_stream_t stream)
+{
+    int rc = check_common(bits, base);
+    if (rc) return rc;
+    if (Nb < 0 || C < 0 || O < 0 || FH < 1 || FW < 1 || sh < 1 || sw < 1 || Hp < FH || Wp < FW)
+        return DS_EINVAL;
+    const int OH = (Hp - FH) / sh + 1, OW = (Wp - FW) / sw + 1;
+    const size_t M = (size_t)Nb * OH * OW;
+    if (M == 0 || O == 0) return DS_OK;
+    if (!x || !tiled || !y) return DS_EINVAL;
+    const size_t K = (size_t)C * FH * FW;
+    if ((size_t)Nb * C * Hp * Wp * 4 >= kMaxBytes || M * O * 4 >= kMaxBytes || K >= (1u << 24))
+        return DS_ETOOLARGE;
+    const size_t need = ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits);
+    if (need && (!workspace || workspace_bytes < need)) return DS_EWORKSPACE;
+    hipStream_t st = (hipStream_t)stream;
+    const TiledGeom g = tiled_geom(O, (int)K, bits);
+
+    ShiftArgs a{};
+    a.x = x;
+    a.wt = (const uint32_t *)tiled;
+    a.negcnt = tiled_negcount(tiled, g);
+    a.bias = bias;
+    a.y = y;
+    a.M = (int)M; a.N = O; a.K = (int)K; a.comm = g.comm;
+    a.pix_per_img = OH * OW; a.OW = OW;
+    a.x_img_stride = C * Hp * Wp; a.x_row_stride = sh * Wp; a.x_col_stride = sw;
+    a.y_img_stride = O * OH * OW; a.y_pix_stride = 1; a.y_ch_stride = OH * OW;
+    a.nbase = -base;
+    int32_t *ktab = (int32_t *)workspace;
+    a.ktab = ktab;
+    const int Kpad = g.comm * g.num;
+    if (Kpad > 0) {
+        hipLaunchKernelGGL(ktab_kernel, dim3(ceil_div(Kpad, 256)), dim3(256), 0, st, ktab, (int)K,
+                           Kpad, FH, FW, Hp * Wp, Wp);
+    }
+    return dispatch_bits(a, bits, base != 0 || bits == 6, st);
+}
+
+DS_EXPORT int ds_conv2d_i32(const int32_t *x, const int32_t *w_ref, const int32_t *bias, int32_t *y,
+                            int Nb, int C, int Hp, int Wp, int O, int FH, int FW, int sh, int sw,
+                            int bits, int base, void *workspace, size_t workspace_bytes,
+                            ds_stream_t stream)
+{
+    int rc = check_common(bits, base);
+    if (rc) return rc;
+    if (Nb < 0 || C < 0 || O < 0 || FH < 1 || FW < 1 || sh < 1 || sw < 1 || Hp < FH || Wp < FW)
+        return DS_EINVAL;
+    if ((size_t)C * FH * FW >= (1u << 24)) return DS_ETOOLARGE;
+    const size_t inner = ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits);
+    const size_t need = ds_conv2d_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits);
+    if (!workspace || workspace_bytes < need) return DS_EWORKSPACE;
+    if (O == 0) return DS_OK;
+    if (!w_ref) return DS_EINVAL;
+    void *tiled = (char *)workspace + inner;
+    rc = launch_tile(w_ref, tiled, O, C * FH * FW, bits, (hipStream_t)stream);
+    if (rc) return rc;
+    return ds_conv2d_tiled_i32(x, tiled, bias, y, Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits, base,
+                               workspace, inner, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// LinearShift
+// ---------------------------------------------------------------------------------------------
+
+namespace ds {
+int launch_transpose(const int32_t *x, int32_t *xT, int M, int K, int ldx, hipStream_t st);
+}
+
+DS_EXPORT size_t ds_linear_tiled_workspace_bytes(int M, int K, int N, int bits)
+{
+    (void)M; (void)N;
+    if (bits < 1 || bits > 6 || K < 0) return 0;
+    const int num = codes_per_word(bits);
+    return align_up((size_t)ceil_div(K, num) * num * 4, 256);
+}
+
+DS_EXPORT size_t ds_linear_workspace_bytes(int M, int K, int N, int bits)
+{
+    if (bits < 1 || bits > 6 || M < 0 || K < 0 || N < 0) return 0;
+    const size_t ldx = align_up((size_t)M, 64);
+    return ds_linear_tiled_workspace_bytes(M, K, N, bits) + align_up(tiled_geom(N, K, bits).bytes, 256) +
+           align_up(ldx * K * 4, 256);
+}
+
+DS_EXPORT int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled, const int32_t *bias,
+                                  int32_t *y, int M, int K, int N, int bits, int base,
+                                  void *workspace, size_t workspace_bytes, ds_stream_t stream)
+{
+    int rc = check_common(bits, base);
+    if (rc) return rc;
+    if (M < 0 || K < 0 || N < 0 || ldx < M) return DS_EINVAL;
+    if (M == 0 || N == 0) return DS_OK;
+    if (!xT || !tiled || !y) return DS_EINVAL;
+    if ((size_t)ldx * K * 4 >= kMaxBytes || (size_t)M * N * 4 >= kMaxBytes || K >= (1 << 24))
+        return DS_ETOOLARGE;
+    const size_t need = ds_linear_tiled_workspace_bytes(M, K, N, bits);
+    if (need && (!workspace || workspace_bytes < need)) return DS_EWORKSPACE;
+    hipStream_t st = (hipStream_t)stream;
+    const TiledGeom g = tiled_geom(N, K, bits);
+
+    ShiftArgs a{};
+    a.x = xT;
+    a.wt = (const uint32_t *)tiled;
+    a.negcnt = tiled_negcount(tiled, g);
+    a.bias = bias;
+    a.y = y;
+    a.M = M; a.N = N; a.K = K; a.comm = g.comm;
+    a.pix_per_img = M; a.OW = M;
+    a.x_img_stride = 0; a.x_row_stride = 0; a.x_col_stride = 1;
+    a.y_img_stride = 0; a.y_pix_stride = N; a.y_ch_stride = 1;
+    a.nbase = -base;
+    int32_t *ktab = (int32_t *)workspace;
+    a.ktab = ktab;
+    const int Kpad = g.comm * g.num;
+    if (Kpad > 0) {
+        // a 1x1 "filter" over K planes of ldx elements: ktab[k] = k * ldx
+        hipLaunchKernelGGL(ktab_kernel, dim3(ceil_div(Kpad, 256)), dim3(256), 0, st, ktab, K, Kpad, 1,
+                           1, ldx, 0);
+    }
+    return dispatch_bits(a, bits, base != 0 || bits == 6, st);
+}
+
+DS_EXPORT int ds_linear_i32(const int32_t *x, const int32_t *w_ref, const int32_t *bias, int32_t *y,
+                            int M, int K, int N, int bits, int base, void *workspace,
+                            size_t workspace_bytes, ds_stream_t stream)
+{
+    int rc = check_common(bits, base);
+    if (rc) return rc;
+    if (M < 0 || K < 0 || N < 0) return DS_EINVAL;
+    if (K >= (1 << 24)) return DS_ETOOLARGE;
+    const size_t need = ds_linear_workspace_bytes(M, K, N, bits);
+    if (!workspace || workspace_bytes < need) return DS_EWORKSPACE;
+    if (M == 0 || N == 0) return DS_OK;
+    if (!x && K > 0) return DS_EINVAL;
+    if (!w_ref && K > 0) return DS_EINVAL;
+    const int ldx = (int)align_up((size_t)M, 64);
+    if ((size_t)ldx * K * 4 >= kMaxBytes) return DS_ETOOLARGE;
+    const size_t inner = ds_linear_tiled_workspace_bytes(M, K, N, bits);
+    void *tiled = (char *)workspace + inner;
+    int32_t *xT = (int32_t *)((char *)tiled + align_up(tiled_geom(N, K, bits).bytes, 256));
+    hipStream_t st = (hipStream_t)stream;
+    rc = launch_tile(w_ref, tiled, N, K, bits, st);
+    if (rc) return rc;
+    if (K > 0) {
+        rc = launch_transpose(x, xT, M, K, ldx, st);
+        if (rc) return rc;
+    }
+    return ds_linear_tiled_i32(xT, ldx, tiled, bias, y, M, K, N, bits, base, workspace, inner, stream);
+}

@@ -1,0 +1,281 @@
+"""Kernel dispatch: the counterpart of the reference's ``deepshift/kernels/kernels.py``.
+
+``linear`` (kernels.py:10-26), ``conv2d`` (kernels.py:28-67) and ``compress_sign_and_shift``
+(kernels.py:69-73) keep the reference's names, argument order and meaning, and call the gfx950
+library through its C ABI instead of the ``deepshift_cuda`` pybind module.  Everything runs on
+the current HIP stream of the input's device; outputs are new int32 tensors.
+
+Differences from the reference, all deliberate:
+
+* ``use_cuda=False`` (the reference's CPU kernel) is not offered here: it raises.
+* ``dilation != 1`` / ``groups != 1`` raise instead of being silently ignored (kernels.py:28).
+* padding ``(ph, pw)`` pads H by ph and W by pw (the reference's tuple order,
+  kernels.py:32-33, swaps them; identical for square padding).
+* weights that have to stay zero contribute exactly 0 (see ``utils.compress_bits``).
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+
+__all__ = ["linear", "conv2d", "compress_sign_and_shift", "quantize", "quantize_pad",
+           "quantize_transpose", "dequantize", "tile_weights", "linear_tiled", "conv2d_tiled"]
+
+
+def _pair(v):
+    if isinstance(v, (tuple, list)):
+        if len(v) == 1:
+            return int(v[0]), int(v[0])
+        return int(v[0]), int(v[1])
+    return int(v), int(v)
+
+
+def _require_device_i32(name, t):
+    if not t.is_cuda:
+        raise ValueError("%s must be a GPU tensor" % name)
+    if t.dtype != torch.int32:
+        raise TypeError("%s must be int32, got %s" % (name, t.dtype))
+    return t.contiguous()
+
+
+def _workspace(nbytes, device):
+    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+
+
+_TIMING_SINK = None
+
+
+def set_timing_sink(sink):
+    """Measurement hook: when ``sink`` is a list, every shift-kernel launch is bracketed by HIP
+    events on the launch stream and ``(kind, M, K, N, start_event, end_event)`` is appended to it;
+    ``None`` switches the hook off (the default: no events are recorded)."""
+    global _TIMING_SINK
+    _TIMING_SINK = sink
+
+
+class _Timed:
+    def __init__(self, kind, M, K, N, device):
+        self.meta = (kind, M, K, N)
+        self.device = device
+
+    def __enter__(self):
+        if _TIMING_SINK is not None:
+            self.start = torch.cuda.Event(enable_timing=True)
+            self.end = torch.cuda.Event(enable_timing=True)
+            self.start.record(torch.cuda.current_stream(self.device))
+        return self
+
+    def __exit__(self, *exc):
+        if _TIMING_SINK is not None:
+            self.end.record(torch.cuda.current_stream(self.device))
+            _TIMING_SINK.append(self.meta + (self.start, self.end))
+        return False
+
+
+def _no_cpu_kernel():
+    raise NotImplementedError(
+        "use_cuda=False selects the reference's CPU shift kernel, which this GPU library does "
+        "not provide; run the layer with use_cuda=True on a ROCm device")
+
+
+# ---------------------------------------------------------------------------------------------
+# weight packing
+# ---------------------------------------------------------------------------------------------
+
+def compress_sign_and_shift(shift, sign, comp_size, base, bits, row_length, num):
+    """Pack codes into 32-bit words (reference layout): kernels.py:69-73.
+
+    ``shift`` holds the negated shifts ``s`` (what ``utils.compress_bits`` passes, utils.py:74) as
+    an int32 GPU tensor of shape [O, C, FH, FW] (or [O, K]); ``sign`` likewise.  Returns int32
+    [comp_size] = [O * row_length]; word j of row o packs codes ``j*num .. j*num+num-1``, code i
+    as ``(s - base) << i*(bits+1) | (sign > 0) << (i*(bits+1) + bits)``.
+    """
+    shift = _require_device_i32("shift", shift)
+    sign = _require_device_i32("sign", sign)
+    O = shift.shape[0]
+    K = shift[0].numel() if O else 0
+    if num != 32 // (bits + 1) or row_length != (K + num - 1) // num or comp_size != O * row_length:
+        raise ValueError("comp_size/row_length/num are inconsistent with the tensor shape and bits")
+    out = torch.empty([comp_size], dtype=torch.int32, device=shift.device)
+    _lib.call("ds_pack_i32", _lib.ptr(shift), _lib.ptr(sign), _lib.ptr(out), O, K, int(bits),
+              int(base), _lib.current_stream(shift.device))
+    return out
+
+
+def tile_weights(packed, N, K, bits, base=0):
+    """Reference-layout words [N*comm] -> the library's tiled blob (uint8 tensor)."""
+    packed = _require_device_i32("packed", packed)
+    num = 32 // (bits + 1)
+    if packed.numel() != N * ((K + num - 1) // num):
+        raise ValueError("packed weight has %d words, expected %d" %
+                         (packed.numel(), N * ((K + num - 1) // num)))
+    nbytes = _lib.lib().ds_tiled_bytes(N, K, bits)
+    blob = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=packed.device)
+    _lib.call("ds_tile_weights_i32", _lib.ptr(packed), _lib.ptr(blob), N, K, int(bits), int(base),
+              _lib.current_stream(packed.device))
+    return blob
+
+
+def _tiled_of(conc_weight, N, K):
+    """The tiled blob of a ConcWeight, built once and cached on the object."""
+    data = conc_weight.data
+    key = (data.data_ptr(), data._version, N, K, conc_weight.bits, conc_weight.base)
+    cached = getattr(conc_weight, "_tiled", None)
+    if cached is None or cached[0] != key:
+        cached = (key, tile_weights(data, N, K, conc_weight.bits, conc_weight.base))
+        conc_weight._tiled = cached
+    return cached[1]
+
+
+# ---------------------------------------------------------------------------------------------
+# fixed-point conversion
+# ---------------------------------------------------------------------------------------------
+
+def quantize(x, integer_bits=16, fraction_bits=16, round_to_fixed=True):
+    """float32 -> int32: ``(round_to_fixed(x) * 2**F).int()`` or, with ``round_to_fixed=False``,
+    ``(x * 2**F).int()`` (utils.py:7-21, modules.py:25,153) in one pass."""
+    x = x.contiguous()
+    if x.dtype != torch.float32 or not x.is_cuda:
+        raise TypeError("quantize expects a float32 GPU tensor")
+    q = torch.empty(x.shape, dtype=torch.int32, device=x.device)
+    _lib.call("ds_quantize_f32_i32", _lib.ptr(x), _lib.ptr(q), x.numel(), integer_bits,
+              fraction_bits, _lib.DS_Q_ROUND_TO_FIXED if round_to_fixed else _lib.DS_Q_CAST,
+              _lib.current_stream(x.device))
+    return q
+
+
+def quantize_pad(x, padding, integer_bits=16, fraction_bits=16, round_to_fixed=True):
+    """float32 NCHW -> zero padded int32 NCHW (conversion fused with kernels.py:32-36)."""
+    x = x.contiguous()
+    if x.dtype != torch.float32 or not x.is_cuda or x.dim() != 4:
+        raise TypeError("quantize_pad expects a 4-D float32 GPU tensor")
+    ph, pw = _pair(padding)
+    Nb, C, H, W = x.shape
+    q = torch.empty([Nb, C, H + 2 * ph, W + 2 * pw], dtype=torch.int32, device=x.device)
+    _lib.call("ds_quantize_pad_f32_i32", _lib.ptr(x), _lib.ptr(q), Nb, C, H, W, ph, pw,
+              integer_bits, fraction_bits,
+              _lib.DS_Q_ROUND_TO_FIXED if round_to_fixed else _lib.DS_Q_CAST,
+              _lib.current_stream(x.device))
+    return q
+
+
+def quantize_transpose(x, integer_bits=16, fraction_bits=16, round_to_fixed=True):
+    """float32 [M, K] -> int32 [K, ldx] (ldx = M rounded up to 64): the LinearShift input layout."""
+    x = x.contiguous()
+    if x.dtype != torch.float32 or not x.is_cuda or x.dim() != 2:
+        raise TypeError("quantize_transpose expects a 2-D float32 GPU tensor")
+    M, K = x.shape
+    ldx = (M + 63) // 64 * 64
+    qT = torch.empty([K, ldx], dtype=torch.int32, device=x.device)
+    _lib.call("ds_quantize_transpose_f32_i32", _lib.ptr(x), _lib.ptr(qT), M, K, ldx, integer_bits,
+              fraction_bits, _lib.DS_Q_ROUND_TO_FIXED if round_to_fixed else _lib.DS_Q_CAST,
+              _lib.current_stream(x.device))
+    return qT
+
+
+def dequantize(y, fraction_bits=16):
+    """int32 -> float32 ``y.float() / 2**F`` (modules.py:30-31,161-162)."""
+    y = _require_device_i32("y", y)
+    out = torch.empty(y.shape, dtype=torch.float32, device=y.device)
+    _lib.call("ds_dequantize_i32_f32", _lib.ptr(y), _lib.ptr(out), y.numel(), fraction_bits,
+              _lib.current_stream(y.device))
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# LinearShift / Conv2dShift kernels
+# ---------------------------------------------------------------------------------------------
+
+def linear_tiled(xT, M, tiled, bias, N, bits, base=0):
+    """Shift GEMM on transposed int32 activations ``xT[K, ldx]`` and a tiled weight blob."""
+    xT = _require_device_i32("xT", xT)
+    K, ldx = xT.shape
+    out = torch.empty([M, N], dtype=torch.int32, device=xT.device)
+    L = _lib.lib()
+    ws_bytes = L.ds_linear_tiled_workspace_bytes(M, K, N, bits)
+    ws = _workspace(ws_bytes, xT.device)
+    with _Timed("linear", M, K, N, xT.device):
+        _lib.call("ds_linear_tiled_i32", _lib.ptr(xT), ldx, _lib.ptr(tiled), _lib.ptr(bias),
+                  _lib.ptr(out), M, K, N, int(bits), int(base), _lib.ptr(ws), ws_bytes,
+                  _lib.current_stream(xT.device))
+    return out
+
+
+def linear(input, shift, sign, bias=None, conc_weight=None, use_cuda=True):
+    """``out[m, n] = bias[n] + sum_k sign[n,k] * (input[m,k] >> -shift[n,k])`` on packed weights.
+
+    Same contract as the reference's ``kernels.linear`` (kernels.py:10-26): ``input`` int32
+    [M, K] fixed-point activations, ``shift``/``sign`` only give the layer shape (the arithmetic
+    reads ``conc_weight``), ``bias`` int32 [N] or None (treated as zeros, kernels.py:18).
+    Returns int32 [M, N].
+    """
+    if not use_cuda:
+        _no_cpu_kernel()
+    assert conc_weight is not None
+    input = _require_device_i32("input", input)
+    if input.dim() != 2:
+        raise ValueError("input must be [M, K]")
+    M, K = input.shape
+    N = shift.size(0)
+    if bias is not None:
+        bias = _require_device_i32("bias", bias)
+    tiled = _tiled_of(conc_weight, N, K)
+    ldx = (M + 63) // 64 * 64
+    xT = torch.empty([K, ldx], dtype=torch.int32, device=input.device)
+    _lib.call("ds_transpose_i32", _lib.ptr(input), _lib.ptr(xT), M, K, ldx,
+              _lib.current_stream(input.device))
+    return linear_tiled(xT, M, tiled, bias, N, conc_weight.bits, conc_weight.base)
+
+
+def conv2d_tiled(x_padded, tiled, bias, O, kernel_size, stride, bits, base=0):
+    """Shift convolution on an already padded int32 NCHW input and a tiled weight blob."""
+    x_padded = _require_device_i32("x_padded", x_padded)
+    Nb, C, Hp, Wp = x_padded.shape
+    FH, FW = _pair(kernel_size)
+    sh, sw = _pair(stride)
+    if Hp < FH or Wp < FW:
+        raise ValueError("padded input %dx%d is smaller than the %dx%d filter" % (Hp, Wp, FH, FW))
+    OH, OW = (Hp - FH) // sh + 1, (Wp - FW) // sw + 1
+    out = torch.empty([Nb, O, OH, OW], dtype=torch.int32, device=x_padded.device)
+    L = _lib.lib()
+    ws_bytes = L.ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits)
+    ws = _workspace(ws_bytes, x_padded.device)
+    with _Timed("conv", Nb * OH * OW, C * FH * FW, O, x_padded.device):
+        _lib.call("ds_conv2d_tiled_i32", _lib.ptr(x_padded), _lib.ptr(tiled), _lib.ptr(bias),
+                  _lib.ptr(out), Nb, C, Hp, Wp, O, FH, FW, sh, sw, int(bits), int(base),
+                  _lib.ptr(ws), ws_bytes, _lib.current_stream(x_padded.device))
+    return out
+
+
+def conv2d(input, shift, sign, bias=None, conc_weight=None, stride=1, padding=0, dilation=1,
+           groups=1, use_cuda=True):
+    """Shift convolution with the contract of the reference's ``kernels.conv2d`` (kernels.py:28-67).
+
+    ``input`` int32 NCHW (unpadded), ``shift`` [O, C, FH, FW] gives the filter shape, weights come
+    from ``conc_weight`` (K ordered (ic, fh, fw)), zero ``padding``, ``stride``; returns int32
+    [Nb, O, OH, OW] with OH = (H + 2*ph - FH) // sh + 1.
+    """
+    if not use_cuda:
+        _no_cpu_kernel()
+    assert conc_weight is not None
+    if _pair(dilation) != (1, 1) or groups != 1:
+        raise NotImplementedError("the shift kernel supports dilation=1 and groups=1 only")
+    input = _require_device_i32("input", input)
+    if input.dim() != 4:
+        raise ValueError("input must be NCHW")
+    ph, pw = _pair(padding)
+    Nb, C, H, W = input.shape
+    O, Cw, FH, FW = shift.shape
+    if Cw != C:
+        raise ValueError("filter has %d input channels, input has %d" % (Cw, C))
+    if bias is not None:
+        bias = _require_device_i32("bias", bias)
+    if ph or pw:
+        xp = torch.empty([Nb, C, H + 2 * ph, W + 2 * pw], dtype=torch.int32, device=input.device)
+        _lib.call("ds_pad_i32", _lib.ptr(input), _lib.ptr(xp), Nb, C, H, W, ph, pw,
+                  _lib.current_stream(input.device))
+    else:
+        xp = input
+    tiled = _tiled_of(conc_weight, O, C * FH * FW)
+    return conv2d_tiled(xp, tiled, bias, O, (FH, FW), stride, conc_weight.bits, conc_weight.base)

@@ -1,0 +1,260 @@
+"""DeepShift-PS layers: the counterpart of the reference's ``deepshift/modules.py``.
+
+``LinearShift`` (modules.py:78-142) and ``Conv2dShift`` (modules.py:292-340) keep the reference's
+constructor arguments, parameters (``shift``, ``sign``, ``bias``) and attributes
+(``conc_weight``, ``use_kernel``, ``use_cuda``, ``shift_range``, ...).  With ``use_kernel=True``
+the forward pass is the fixed-point shift kernel on the GPU:
+
+    float input --quantise--> int32 --shift-add kernel on packed weights--> int32 --/2^F--> float
+
+(LinearShiftFunction.forward modules.py:24-31, Conv2dShiftFunction.forward :152-162), otherwise
+the float path of the reference (``F.linear`` / ``F.conv2d`` with +-2^shift weights, :135,:339).
+"""
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch.nn import init
+from torch.nn.modules.utils import _pair
+
+from . import kernels, ste, utils
+
+__all__ = ["LinearShift", "Conv2dShift"]
+
+
+def _shift_range(weight_bits):
+    # one code point of the sign/shift alphabet is kept for ternary signs (modules.py:88)
+    return (-1 * (2 ** (weight_bits - 1) - 2), 0)
+
+
+def _param_tensor(check_grad, *shape):
+    # double precision when the layer is built for gradient checking (modules.py:98-101)
+    return torch.empty(*shape, dtype=torch.float64 if check_grad else torch.float32)
+
+
+def pack_module_weights(module):
+    """Build ``module.conc_weight`` from its (shift, sign) parameters, clamped to ``shift_range``
+    and rounded the way the float path reads them (modules.py:125-128,313-316)."""
+    shift = module.shift.detach().clamp(*module.shift_range).round()
+    sign = module.sign.detach().round().sign()
+    module.conc_weight = utils.compress_bits(shift, sign)
+    return module.conc_weight
+
+
+class _FixedBias:
+    """int32 fixed-point copy of a float bias, rebuilt only when the parameter changes."""
+
+    def __init__(self):
+        self.key = None
+        self.value = None
+
+    def get(self, bias, integer_bits, fraction_bits, round_to_fixed):
+        if bias is None:
+            return None
+        key = (bias.data_ptr(), bias._version, integer_bits, fraction_bits, round_to_fixed)
+        if key != self.key:
+            self.value = kernels.quantize(bias.detach().float(), integer_bits, fraction_bits,
+                                          round_to_fixed)
+            self.key = key
+        return self.value
+
+
+class LinearShift(nn.Module):
+    def __init__(self, in_features, out_features, bias=True, check_grad=False, freeze_sign=False,
+                 use_kernel=False, use_cuda=True, rounding='deterministic', weight_bits=5,
+                 act_integer_bits=16, act_fraction_bits=16):
+        super(LinearShift, self).__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.use_kernel = use_kernel
+        self.check_grad = check_grad
+        self.use_cuda = use_cuda
+        self.conc_weight = None
+        self.rounding = rounding
+        self.shift_range = _shift_range(weight_bits)
+        self.act_integer_bits, self.act_fraction_bits = act_integer_bits, act_fraction_bits
+
+        self.shift = nn.Parameter(_param_tensor(check_grad, out_features, in_features))
+        self.sign = nn.Parameter(_param_tensor(check_grad, out_features, in_features),
+                                 requires_grad=(freeze_sign == False))  # noqa: E712
+        if bias:
+            self.bias = nn.Parameter(_param_tensor(check_grad, out_features))
+        else:
+            self.register_parameter('bias', None)
+        self._fixed_bias = _FixedBias()
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        self.shift.data.uniform_(*self.shift_range)
+        self.sign.data.uniform_(-1, 1)
+        if self.bias is not None:
+            fan_in, _ = init._calculate_fan_in_and_fan_out(self.shift)
+            bound = 1 / math.sqrt(fan_in)
+            init.uniform_(self.bias, -bound, bound)
+
+    def _kernel_forward(self, input):
+        # modules.py:24-31: the input is cast, NOT rounded/clamped first (truncation toward zero)
+        if not self.use_cuda:
+            kernels._no_cpu_kernel()
+        if self.conc_weight is None:
+            pack_module_weights(self)
+        I, Fb = self.act_integer_bits, self.act_fraction_bits
+        lead = input.shape[:-1]
+        x2d = input.reshape(-1, self.in_features).float()
+        M = x2d.shape[0]
+        xT = kernels.quantize_transpose(x2d, I, Fb, round_to_fixed=False)
+        bias = self._fixed_bias.get(self.bias, I, Fb, round_to_fixed=False)
+        tiled = kernels._tiled_of(self.conc_weight, self.out_features, self.in_features)
+        out = kernels.linear_tiled(xT, M, tiled, bias, self.out_features, self.conc_weight.bits,
+                                   self.conc_weight.base)
+        return kernels.dequantize(out, Fb).reshape(*lead, self.out_features)
+
+    def forward(self, input):
+        self.shift.data = ste.clamp(self.shift.data, *self.shift_range)
+        if self.use_kernel:
+            return self._kernel_forward(input)
+        shift_rounded = ste.round(self.shift, rounding=self.rounding)
+        sign_rounded_signed = ste.sign(ste.round(self.sign, rounding=self.rounding))
+        weight_ps = ste.unsym_grad_mul(2 ** shift_rounded, sign_rounded_signed)
+        return F.linear(input, weight_ps, self.bias)
+
+    def extra_repr(self):
+        return 'in_features={}, out_features={}, bias={}'.format(
+            self.in_features, self.out_features, self.bias is not None)
+
+
+class _ConvNdShift(nn.Module):
+    __constants__ = ['stride', 'padding', 'dilation', 'groups', 'bias', 'padding_mode']
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride, padding, dilation, transposed,
+                 output_padding, groups, bias, padding_mode, check_grad=False, freeze_sign=False,
+                 rounding='deterministic', weight_bits=5, act_integer_bits=16,
+                 act_fraction_bits=16):
+        super(_ConvNdShift, self).__init__()
+        if in_channels % groups != 0:
+            raise ValueError('in_channels must be divisible by groups')
+        if out_channels % groups != 0:
+            raise ValueError('out_channels must be divisible by groups')
+        self.in_channels = in_channels
+        self.out_channels = out_channels
+        self.kernel_size = kernel_size
+        self.stride = stride
+        self.padding = padding
+        self.dilation = dilation
+        self.transposed = transposed
+        self.output_padding = output_padding
+        self.groups = groups
+        self.padding_mode = padding_mode
+        self.rounding = rounding
+        self.shift_range = _shift_range(weight_bits)
+        self.act_integer_bits, self.act_fraction_bits = act_integer_bits, act_fraction_bits
+
+        if transposed:
+            wshape = (in_channels, out_channels // groups) + tuple(kernel_size)
+        else:
+            wshape = (out_channels, in_channels // groups) + tuple(kernel_size)
+        self.shift = nn.Parameter(_param_tensor(check_grad, *wshape))
+        self.sign = nn.Parameter(_param_tensor(check_grad, *wshape),
+                                 requires_grad=(freeze_sign == False))  # noqa: E712
+        if bias:
+            self.bias = nn.Parameter(_param_tensor(check_grad, out_channels))
+        else:
+            self.register_parameter('bias', None)
+        self._fixed_bias = _FixedBias()
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        self.shift.data.uniform_(-10, -1)  # modules.py:268
+        self.sign.data.uniform_(-1, 1)
+        if self.bias is not None:
+            fan_in, _ = init._calculate_fan_in_and_fan_out(self.shift)
+            bound = 1 / math.sqrt(fan_in)
+            init.uniform_(self.bias, -bound, bound)
+
+    def extra_repr(self):
+        s = ('{in_channels}, {out_channels}, kernel_size={kernel_size}'
+             ', stride={stride}')
+        if self.padding != (0,) * len(self.padding):
+            s += ', padding={padding}'
+        if self.dilation != (1,) * len(self.dilation):
+            s += ', dilation={dilation}'
+        if self.output_padding != (0,) * len(self.output_padding):
+            s += ', output_padding={output_padding}'
+        if self.groups != 1:
+            s += ', groups={groups}'
+        if self.bias is None:
+            s += ', bias=False'
+        return s.format(**self.__dict__)
+
+
+def _circular_pad(x, padding):
+    # modules.py:323-328: circular padding is materialised, then the convolution runs unpadded
+    expanded = ((padding[1] + 1) // 2, padding[1] // 2, (padding[0] + 1) // 2, padding[0] // 2)
+    return F.pad(x, expanded, mode='circular')
+
+
+def conv_kernel_forward(module, input, conc_weight, input_is_fixed=False):
+    """Fixed-point shift convolution of a float NCHW input (modules.py:152-162,317-337)."""
+    if not module.use_cuda:
+        kernels._no_cpu_kernel()
+    if module.dilation != (1, 1) or module.groups != 1:
+        raise NotImplementedError("the shift kernel supports dilation=1 and groups=1 only")
+    I, Fb = module.act_integer_bits, module.act_fraction_bits
+    padding = module.padding
+    input = input.float()
+    if module.padding_mode == 'circular':
+        input = _circular_pad(input, padding)
+        padding = (0, 0)
+    # round_to_fixed + cast + zero padding in one pass
+    xq = kernels.quantize_pad(input, padding, I, Fb, round_to_fixed=True)
+    bias = module._fixed_bias.get(module.bias, I, Fb, round_to_fixed=True)
+    K = module.in_channels * module.kernel_size[0] * module.kernel_size[1]
+    tiled = kernels._tiled_of(conc_weight, module.out_channels, K)
+    out = kernels.conv2d_tiled(xq, tiled, bias, module.out_channels, module.kernel_size,
+                               module.stride, conc_weight.bits, conc_weight.base)
+    return kernels.dequantize(out, Fb)
+
+
+class Conv2dShift(_ConvNdShift):
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
+                 groups=1, bias=True, padding_mode='zeros', check_grad=False, freeze_sign=False,
+                 use_kernel=False, use_cuda=True, rounding='deterministic', weight_bits=5,
+                 act_integer_bits=16, act_fraction_bits=16):
+        kernel_size = _pair(kernel_size)
+        stride = _pair(stride)
+        padding = _pair(padding)
+        dilation = _pair(dilation)
+        self.use_kernel = use_kernel
+        self.use_cuda = use_cuda
+        self.conc_weight = None
+        super(Conv2dShift, self).__init__(
+            in_channels, out_channels, kernel_size, stride, padding, dilation, False, _pair(0),
+            groups, bias, padding_mode, check_grad, freeze_sign, rounding, weight_bits,
+            act_integer_bits, act_fraction_bits)
+
+    def forward(self, input):
+        self.shift.data = ste.clamp(self.shift.data, *self.shift_range)
+        if self.use_kernel:
+            if self.conc_weight is None:
+                pack_module_weights(self)
+            return conv_kernel_forward(self, input, self.conc_weight)
+
+        shift_rounded = ste.round(self.shift, self.rounding)
+        sign_rounded_signed = ste.sign(ste.round(self.sign, self.rounding))
+        weight_ps = ste.unsym_grad_mul(2 ** shift_rounded, sign_rounded_signed)
+        input_fixed_point = ste.round_fixed_point(input, self.act_integer_bits,
+                                                  self.act_fraction_bits)
+        if self.bias is not None:
+            bias_fixed_point = ste.round_fixed_point(self.bias, self.act_integer_bits,
+                                                     self.act_fraction_bits)
+        else:
+            bias_fixed_point = None
+        if self.padding_mode == 'circular':
+            input_padded = _circular_pad(input_fixed_point, self.padding)
+            padding = _pair(0)
+        else:
+            input_padded = input_fixed_point
+            padding = self.padding
+        return F.conv2d(input_padded, weight_ps, bias_fixed_point, self.stride, padding,
+                        self.dilation, self.groups)

@@ -1,0 +1,156 @@
+/*
+ * deepshift_hip.h -- C ABI of libdeepshift_hip.so, the gfx950 (MI355X) implementation of
+ * DeepShift's shift-kernel inference path.
+ *
+ * Every entry point takes plain device pointers and sizes, runs asynchronously on the HIP
+ * stream it is given (NULL = the default stream), allocates nothing and returns an int
+ * status: 0 on success, a negative DS_E* code otherwise (ds_status_string() names it).
+ * All tensors are contiguous, row-major, int32 unless stated; images are NCHW.
+ *
+ * Citations name the interface of the reference (paths relative to pytorch/deepshift/) that
+ * each entry point replaces.
+ */
+#ifndef DEEPSHIFT_HIP_H
+#define DEEPSHIFT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *ds_stream_t; /* a hipStream_t */
+
+enum {
+    DS_OK = 0,
+    DS_EINVAL = -1,      /* null pointer / negative or inconsistent size */
+    DS_EBITS = -2,       /* bits outside 1..6 (the reference's bits==7 decode is broken, bits==0 unhandled) */
+    DS_EBASE = -3,       /* base > 0 (base is min(-shift) when that is negative, else 0: utils.py:75-80) */
+    DS_EWORKSPACE = -4,  /* workspace missing or smaller than ds_*_workspace_bytes() */
+    DS_ETOOLARGE = -5,   /* a tensor exceeds the 32-bit offsets the kernels use (>= 2^31 bytes) */
+    DS_EHIP = -100       /* DS_EHIP - hipError_t for a failed launch */
+};
+
+/* Quantisation modes of ds_quantize_*. */
+enum {
+    DS_Q_ROUND_TO_FIXED = 0, /* utils.py:7-21 then modules.py:153: floor to 2^-F grid, clamp, * 2^F */
+    DS_Q_CAST = 1            /* modules.py:25 only: (x * 2^F) truncated toward zero, saturating */
+};
+
+int ds_version(void);
+const char *ds_status_string(int status);
+
+/* ---- weight packing -------------------------------------------------------------------- */
+
+/* Replaces COMPRESS_SIGN_SHIFT (kernels/cuda/shift_cuda.cpp:55-61 -> shift.cu:388-397, kernel
+ * :40-55, word format :27-38), as ONE launch for the whole tensor instead of one per output
+ * channel.  s[O][K] is the negated shift the reference passes (utils.py:74), sign[O][K] in
+ * {-1,0,+1}.  out[O][comm], comm = ceil(K/num), num = 32/(bits+1): code i of a word has
+ * (s - base) in bits [i*(bits+1), i*(bits+1)+bits) and (sign > 0) in bit i*(bits+1)+bits;
+ * tail codes are 0.  The field is masked to `bits` bits. */
+int ds_pack_i32(const int32_t *s, const int32_t *sign, int32_t *out, int O, int K, int bits,
+                int base, ds_stream_t stream);
+
+/* Bytes of the tiled weight blob that ds_tile_weights_i32 writes for an [N][K] layer. */
+size_t ds_tiled_bytes(int N, int K, int bits);
+
+/* Re-lays reference-format words w_ref[N][comm] (the output of ds_pack_i32 / the reference's
+ * ConcWeight.data, utils.py:54-88) into the private, coalesced layout the compute kernels read:
+ * words grouped [ceil(N/32)*2][comm][16] so that the 16 words a wavefront decodes together are
+ * one 64-byte scalar load, sign bit inverted (1 = negative), tail codes neutralised, followed
+ * by a per-channel count of negative codes that the kernels fold into the bias.  No
+ * counterpart in the reference (it consumes the row-major words directly, shift.cu:84). */
+int ds_tile_weights_i32(const int32_t *w_ref, void *tiled, int N, int K, int bits, int base,
+                        ds_stream_t stream);
+
+/* ---- LinearShift ----------------------------------------------------------------------- */
+
+/* Workspace bytes ds_linear_i32 needs (transposed activations, tiled weights, offset table). */
+size_t ds_linear_workspace_bytes(int M, int K, int N, int bits);
+
+/* Replaces DEEP_SHIFT_LINEAR (kernels/cuda/shift_cuda.cpp:26-39 -> shift.cu:174-387, kernel
+ * :57-120), called from kernels.py:10-26:
+ *   y[m][n] = bias[n] + sum_k sgn(n,k) * ((x[m][k] >> field(n,k)) << -base)
+ * x[M][K], w_ref[N][comm] reference-format words, bias[N] or NULL (the reference substitutes
+ * zeros, kernels.py:18), y[M][N] fully overwritten (no pre-zeroing needed).  Accumulation wraps
+ * modulo 2^32.  A field >= 32 (only possible with bits == 6, the reference's encoding of a
+ * zero weight, utils.py:68-70) contributes exactly 0. */
+int ds_linear_i32(const int32_t *x, const int32_t *w_ref, const int32_t *bias, int32_t *y, int M,
+                  int K, int N, int bits, int base, void *workspace, size_t workspace_bytes,
+                  ds_stream_t stream);
+
+/* Same computation on pre-tiled weights and pre-transposed activations xT[K][ldx]
+ * (ldx >= M, a multiple of 64 -- what ds_quantize_transpose_f32_i32 writes).  Workspace:
+ * ds_linear_tiled_workspace_bytes(). */
+size_t ds_linear_tiled_workspace_bytes(int M, int K, int N, int bits);
+int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled, const int32_t *bias,
+                        int32_t *y, int M, int K, int N, int bits, int base, void *workspace,
+                        size_t workspace_bytes, ds_stream_t stream);
+
+/* ---- Conv2dShift ----------------------------------------------------------------------- */
+
+size_t ds_conv2d_workspace_bytes(int Nb, int C, int Hp, int Wp, int O, int FH, int FW, int sh,
+                                 int sw, int bits);
+
+/* Replaces DEEP_SHIFT_CONV (kernels/cuda/shift_cuda.cpp:41-53 -> shift.cu:399-669: IM2COL
+ * :122-153 + GEMM :57-120 + COL2IM :155-172) as one direct convolution with no im2col buffer.
+ * As in the reference the input is ALREADY zero padded by the caller (kernels.py:32-36):
+ * x[Nb][C][Hp][Wp]; w_ref[O][comm] packs K = C*FH*FW codes per output channel in (ic, fh, fw)
+ * order (shift.cu:144-146); y[Nb][O][OH][OW], OH = (Hp-FH)/sh + 1 (kernels.py:43-44), fully
+ * overwritten.  Same arithmetic as ds_linear_i32. */
+int ds_conv2d_i32(const int32_t *x_padded, const int32_t *w_ref, const int32_t *bias, int32_t *y,
+                  int Nb, int C, int Hp, int Wp, int O, int FH, int FW, int sh, int sw, int bits,
+                  int base, void *workspace, size_t workspace_bytes, ds_stream_t stream);
+
+/* Same computation on pre-tiled weights. */
+size_t ds_conv2d_tiled_workspace_bytes(int Nb, int C, int Hp, int Wp, int O, int FH, int FW,
+                                       int sh, int sw, int bits);
+int ds_conv2d_tiled_i32(const int32_t *x_padded, const void *tiled, const int32_t *bias,
+                        int32_t *y, int Nb, int C, int Hp, int Wp, int O, int FH, int FW, int sh,
+                        int sw, int bits, int base, void *workspace, size_t workspace_bytes,
+                        ds_stream_t stream);
+
+/* ---- fixed-point conversion ------------------------------------------------------------ */
+
+/* Replaces utils.round_to_fixed (utils.py:7-21) + the (x * 2**F).int() cast (modules.py:25,153)
+ * [mode DS_Q_ROUND_TO_FIXED], or the cast alone [mode DS_Q_CAST], as one pass; n elements. */
+int ds_quantize_f32_i32(const float *x, int32_t *q, int64_t n, int I, int F, int mode,
+                        ds_stream_t stream);
+
+/* The same conversion fused with the zero padding of kernels.py:32-36:
+ * x[Nb][C][H][W] float -> q[Nb][C][H+2ph][W+2pw] int32 (border = 0). */
+int ds_quantize_pad_f32_i32(const float *x, int32_t *q, int Nb, int C, int H, int W, int ph,
+                            int pw, int I, int F, int mode, ds_stream_t stream);
+
+/* The same conversion fused with a transpose: x[M][K] float -> qT[K][ldx] int32, ldx >= M
+ * (columns M..ldx-1 are zero filled). */
+int ds_quantize_transpose_f32_i32(const float *x, int32_t *qT, int M, int K, int ldx, int I,
+                                  int F, int mode, ds_stream_t stream);
+
+/* Zero padding of an int32 image (kernels.py:32-36, F.pad): x[Nb][C][H][W] -> [..][H+2ph][W+2pw]. */
+int ds_pad_i32(const int32_t *x, int32_t *xp, int Nb, int C, int H, int W, int ph, int pw,
+               ds_stream_t stream);
+
+/* x[M][K] -> xT[K][ldx] (ldx >= M, columns M..ldx-1 zero filled): the activation layout
+ * ds_linear_tiled_i32 reads.  No counterpart in the reference. */
+int ds_transpose_i32(const int32_t *x, int32_t *xT, int M, int K, int ldx, ds_stream_t stream);
+
+/* Replaces out.float() / 2**F (modules.py:30-31,161-162); n elements. */
+int ds_dequantize_i32_f32(const int32_t *y, float *out, int64_t n, int F, ds_stream_t stream);
+
+/* ---- measurement ----------------------------------------------------------------------- */
+
+/* VALU calibration: every lane of `blocks` x 256 threads runs `iters` x 64 independent
+ * (arithmetic-shift, xor-add) pairs -- the two instructions one shift-add term costs -- so that
+ * pairs/s = blocks*256*iters*64 / elapsed is the sustained ceiling the roofline is priced
+ * against.  sink[blocks*256] receives the accumulators.  No counterpart in the reference. */
+int ds_valu_calibrate(int32_t *sink, int blocks, int iters, ds_stream_t stream);
+
+/* Plain copy kernel of n int32 (used to scale HBM byte counters). */
+int ds_copy_i32(const int32_t *src, int32_t *dst, int64_t n, ds_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DEEPSHIFT_HIP_H */

@@ -1,0 +1,114 @@
+"""GPU: BASELINE.json's full-size cases.  The oracle is too slow for a whole tensor here, so parity
+is checked on slices the oracle finishes in seconds plus size-independent properties."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from deepshift_amd import kernels, utils
+from oracle import shift_oracle as so
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+NTHREADS = min(16, os.cpu_count() or 1)
+
+
+def _codes(g, shape, lo=-15):
+    shift = torch.randint(lo, 1, shape, generator=g).float()
+    sign = (torch.randint(0, 2, shape, generator=g) * 2 - 1).float()
+    return shift, sign
+
+
+def test_config2_conv_full_size(oracle):
+    """3x3 s1 p1, 64 -> 64, input 32x64x56x56, 16.16, shifts in [-15, 0]."""
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(32, 64, 56, 56, generator=g).clamp_min(0)
+    shift, sign = _codes(g, (64, 64, 3, 3))
+    bias = torch.randint(-2 ** 20, 2 ** 20, (64,), generator=g, dtype=torch.int32)
+    cw = utils.compress_bits(shift, sign)
+    assert cw.bits == 4
+    xq = kernels.quantize(x.to(DEV))
+    y = kernels.conv2d(xq, shift, sign, bias.to(DEV), cw, (1, 1), (1, 1))
+    assert y.shape == (32, 64, 56, 56)
+    # oracle on the first and last image
+    s_np, sg_np = shift.numpy().astype(np.int32), sign.numpy().astype(np.int32)
+    for img in (0, 31):
+        xp = np.pad(xq[img:img + 1].cpu().numpy(), ((0, 0), (0, 0), (1, 1), (1, 1)))
+        want = oracle.conv2d(xp, s_np, sg_np, bias.numpy(), (1, 1), nthreads=NTHREADS)
+        np.testing.assert_array_equal(y[img:img + 1].cpu().numpy(), want)
+    # flipping every sign negates y - bias (mod 2^32)
+    y_flip = kernels.conv2d(xq, shift, -sign, bias.to(DEV), utils.compress_bits(shift, -sign), (1, 1), (1, 1))
+    assert torch.equal((y - bias.to(DEV).view(1, -1, 1, 1)), -(y_flip - bias.to(DEV).view(1, -1, 1, 1)))
+    # a batch permutation permutes the output
+    perm = torch.randperm(32, generator=g).to(DEV)
+    assert torch.equal(kernels.conv2d(xq[perm].contiguous(), shift, sign, bias.to(DEV), cw, (1, 1), (1, 1)), y[perm])
+
+
+def test_config2_gemm_full_size(oracle):
+    """LinearShift GEMM M = K = N = 4096."""
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(4096, 4096, generator=g).clamp_min(0)
+    shift, sign = _codes(g, (4096, 4096))
+    bias = torch.randint(-2 ** 20, 2 ** 20, (4096,), generator=g, dtype=torch.int32)
+    cw = utils.compress_bits(shift, sign)
+    assert cw.bits == 4 and cw.data.numel() == 4096 * 683
+    xq = kernels.quantize(x.to(DEV))
+    y = kernels.linear(xq, shift, sign, bias.to(DEV), cw)
+    rows = [0, 1, 63, 64, 2047, 4095]
+    want = oracle.linear(xq[rows].cpu().numpy(), shift.numpy().astype(np.int32), sign.numpy().astype(np.int32),
+                         bias.numpy(), NTHREADS)
+    np.testing.assert_array_equal(y[rows].cpu().numpy(), want)
+    # a row permutation of x permutes the rows of y; zero input gives the bias
+    perm = torch.randperm(4096, generator=g).to(DEV)
+    assert torch.equal(kernels.linear(xq[perm].contiguous(), shift, sign, bias.to(DEV), cw), y[perm])
+    y0 = kernels.linear(torch.zeros_like(xq), shift, sign, bias.to(DEV), cw)
+    assert torch.equal(y0, bias.to(DEV).view(1, -1).expand(4096, -1))
+
+
+def test_resnet18_layer_shapes_small_batch(oracle):
+    """Every distinct shift-layer shape of ResNet-18 (config 4) at batch 2, bit-exact."""
+    from deepshift_amd import workloads
+    g = torch.Generator().manual_seed(2)
+    seen = set()
+    for L in workloads.shift_layer_shapes(workloads.ResNet18(), (3, 224, 224), 2):
+        key = tuple(sorted((k, v) for k, v in L.items() if k != "name"))
+        if key in seen:
+            continue
+        seen.add(key)
+        if L["kind"] == "linear":
+            x = torch.randint(0, 2 ** 20, (L["M"], L["K"]), generator=g, dtype=torch.int32)
+            shift, sign = _codes(g, (L["N"], L["K"]))
+            cw = utils.compress_bits(shift, sign)
+            y = kernels.linear(x.to(DEV), shift, sign, None, cw)
+            want = oracle.linear(x.numpy(), shift.numpy().astype(np.int32), sign.numpy().astype(np.int32), None, NTHREADS)
+        else:
+            x = torch.randint(-2 ** 18, 2 ** 20, (L["Nb"], L["C"], L["H"], L["W"]), generator=g, dtype=torch.int32)
+            shift, sign = _codes(g, (L["O"], L["C"], L["FH"], L["FW"]))
+            cw = utils.compress_bits(shift, sign)
+            y = kernels.conv2d(x.to(DEV), shift, sign, None, cw, L["stride"], L["padding"])
+            ph, pw = L["padding"]
+            xp = np.pad(x.numpy(), ((0, 0), (0, 0), (ph, ph), (pw, pw)))
+            want = oracle.conv2d(xp, shift.numpy().astype(np.int32), sign.numpy().astype(np.int32), None,
+                                 L["stride"], nthreads=NTHREADS)
+        np.testing.assert_array_equal(y.cpu().numpy(), want, err_msg=L["name"])
+    assert len(seen) == 12
+
+
+def test_config5_bottleneck_shapes_wb3_act35(oracle):
+    """ResNet-50 style layers with weight_bits 3 (shift in [-3, 0], 10 codes per word) and 3.5
+    activations: a 1x1, a 3x3/2 and a 1x1 expansion at batch 2."""
+    g = torch.Generator().manual_seed(5)
+    for (C, H, O, F, stride, pad) in [(256, 56, 64, 1, 1, 0), (128, 56, 128, 3, 2, 1), (512, 7, 2048, 1, 1, 0),
+                                      (1024, 14, 512, 1, 2, 0)]:
+        x = utils.round_to_fixed(torch.randn(2, C, H, H, generator=g), 3, 5)
+        xq = (x * 32).int()
+        assert int(xq.min()) >= -128 and int(xq.max()) <= 96
+        shift, sign = _codes(g, (O, C, F, F), lo=-3)
+        cw = utils.compress_bits(shift, sign)
+        assert cw.bits == 2
+        y = kernels.conv2d(xq.to(DEV), shift, sign, None, cw, (stride, stride), (pad, pad))
+        xp = np.pad(xq.numpy(), ((0, 0), (0, 0), (pad, pad), (pad, pad)))
+        want = oracle.conv2d(xp, shift.numpy().astype(np.int32), sign.numpy().astype(np.int32), None,
+                             (stride, stride), nthreads=NTHREADS)
+        np.testing.assert_array_equal(y.cpu().numpy(), want)

@@ -1,0 +1,205 @@
+"""GPU: the Python-level API (kernels.*, utils.compress_bits, the shift modules, convert_to_shift)
+against the oracle (bit-exact on the int32 results) and against the float path (stated bound)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+from deepshift_amd import convert, kernels, modules, modules_q, utils, workloads
+from oracle import shift_oracle as so
+from tests.conftest import random_activations, random_codes
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+NTHREADS = min(16, os.cpu_count() or 1)
+
+
+def float_bound(K, F, scale):
+    """|kernel - float path| < K * 2^-F (one floor per term) + fp32 accumulation slack."""
+    return K * 2.0 ** -F + 4 * K * 2.0 ** -24 * scale + 1e-6
+
+
+def test_compress_bits_matches_reference_format(oracle, rng):
+    for max_s, want_bits in [(1, 1), (3, 2), (7, 3), (15, 4), (14, 4), (31, 5)]:
+        s, sign = random_codes(rng, (9, 4, 3, 3), max_s=max_s)
+        s.reshape(-1)[0] = max_s
+        cw = utils.compress_bits(torch.from_numpy(-s).float(), torch.from_numpy(sign).float())
+        assert (cw.bits, cw.base) == (want_bits, 0)
+        want, _ = oracle.pack_words(s.reshape(9, -1), sign.reshape(9, -1), want_bits)
+        np.testing.assert_array_equal(cw.data.cpu().numpy().reshape(9, -1), want)
+    # ternary: zeros become the s = 32 code element-wise, bits = 6, inputs untouched
+    s, sign = random_codes(rng, (6, 20), max_s=15, zero_frac=0.3)
+    shift_t, sign_t = torch.from_numpy(-s).float(), torch.from_numpy(sign).float()
+    cw = utils.compress_bits(shift_t, sign_t)
+    assert (cw.bits, cw.base) == (6, 0)
+    assert torch.equal(sign_t, torch.from_numpy(sign).float())
+    f, sg = so.np_unpack_words(cw.data.cpu().numpy().reshape(6, -1), 20, 6)
+    np.testing.assert_array_equal(f, np.where(sign == 0, 32, s))
+    np.testing.assert_array_equal(sg, np.where(sign == 0, 1, sign))
+    # left shifts: base < 0, subtracted once
+    shift = torch.tensor([[2.0, -3.0, 0.0, -1.0]])
+    cw = utils.compress_bits(shift, torch.ones_like(shift))
+    assert (cw.bits, cw.base) == (3, -2)
+    f, _ = so.np_unpack_words(cw.data.cpu().numpy().reshape(1, -1), 4, 3, base=-2)
+    np.testing.assert_array_equal(f, [[-2, 3, 0, 1]])
+
+
+def test_kernels_linear_and_conv2d_api(oracle, rng):
+    M, K, N = 100, 300, 40
+    x = random_activations(rng, (M, K))
+    s, sign = random_codes(rng, (N, K), max_s=15, zero_frac=0.1)
+    bias = rng.integers(-2 ** 20, 2 ** 20, size=N).astype(np.int32)
+    shift_t, sign_t = torch.from_numpy(-s).float().to(DEV), torch.from_numpy(sign).float().to(DEV)
+    cw = utils.compress_bits(shift_t, sign_t)
+    want = oracle.linear(x, -s, sign, bias)
+    got = kernels.linear(torch.from_numpy(x).to(DEV), shift_t, sign_t, torch.from_numpy(bias).to(DEV), cw)
+    assert got.dtype == torch.int32 and got.shape == (M, N)
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+    got = kernels.linear(torch.from_numpy(x).to(DEV), shift_t, sign_t, None, cw)
+    np.testing.assert_array_equal(got.cpu().numpy(), oracle.linear(x, -s, sign, None))
+
+    Nb, C, H, W, O = 3, 6, 11, 13, 10
+    xi = random_activations(rng, (Nb, C, H, W))
+    s, sign = random_codes(rng, (O, C, 3, 3), max_s=15)
+    bias = rng.integers(-2 ** 20, 2 ** 20, size=O).astype(np.int32)
+    shift_t, sign_t = torch.from_numpy(-s).float().to(DEV), torch.from_numpy(sign).float().to(DEV)
+    cw = utils.compress_bits(shift_t, sign_t)
+    for stride, padding in [((1, 1), (1, 1)), ((2, 2), (1, 1)), ((1, 1), (0, 0)), ((2, 1), (2, 1))]:
+        ph, pw = padding
+        xp = np.pad(xi, ((0, 0), (0, 0), (ph, ph), (pw, pw)))
+        want = oracle.conv2d(xp, -s, sign, bias, stride)
+        got = kernels.conv2d(torch.from_numpy(xi).to(DEV), shift_t, sign_t, torch.from_numpy(bias).to(DEV),
+                             cw, stride, padding)
+        np.testing.assert_array_equal(got.cpu().numpy(), want)
+    with pytest.raises(NotImplementedError):
+        kernels.conv2d(torch.from_numpy(xi).to(DEV), shift_t, sign_t, None, cw, 1, 1, dilation=2)
+    with pytest.raises(TypeError):
+        kernels.linear(torch.zeros(2, 300, device=DEV), shift_t, sign_t, None, cw)
+
+
+def _oracle_linear_module(oracle, x, layer, round_input):
+    F_ = layer.act_fraction_bits
+    I = layer.act_integer_bits
+    xq = oracle.quantize(x, I, F_) if round_input else oracle.cast(x, F_)
+    shift = layer.shift.detach().cpu().clamp(*layer.shift_range).round().numpy().astype(np.int32)
+    sign = layer.sign.detach().cpu().round().sign().numpy().astype(np.int32)
+    b = layer.bias.detach().cpu().numpy()
+    bq = oracle.cast(b, F_)
+    y = oracle.linear(xq, shift, sign, bq)
+    return y.astype(np.float32) / np.float32(2.0 ** F_)
+
+
+def test_linear_shift_module(oracle):
+    torch.manual_seed(0)
+    layer = modules.LinearShift(784, 512, use_kernel=True).to(DEV)
+    x = torch.rand(64, 784)
+    got = layer(x.to(DEV))
+    assert layer.conc_weight is not None and layer.conc_weight.bits == 6  # ternary signs
+    want = _oracle_linear_module(oracle, x.numpy(), layer, round_input=False)
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+    # float path of the same layer, fed with the value the kernel really sees
+    layer.use_kernel = False
+    ref = layer((x.to(DEV) * 65536).int().float() / 65536)
+    scale = float(x.abs().sum(1).max())
+    assert (got - ref).abs().max().item() < float_bound(784, 16, scale)
+    # 3-D input and no bias
+    layer2 = modules.LinearShift(33, 17, bias=False, use_kernel=True).to(DEV)
+    x3 = torch.randn(4, 5, 33, device=DEV)
+    out = layer2(x3)
+    assert out.shape == (4, 5, 17)
+    layer2.use_kernel = False
+    assert (out - layer2((x3 * 65536).int().float() / 65536)).abs().max().item() < float_bound(33, 16, 40.0)
+
+
+@pytest.mark.parametrize("I,F", [(16, 16), (3, 5)])
+def test_conv2d_shift_module(oracle, I, F):
+    torch.manual_seed(1)
+    layer = modules.Conv2dShift(16, 24, 3, stride=1, padding=1, use_kernel=True, weight_bits=5 if F == 16 else 3,
+                                act_integer_bits=I, act_fraction_bits=F).to(DEV)
+    layer.sign.data = torch.where(layer.sign.data >= 0, torch.ones_like(layer.sign), -torch.ones_like(layer.sign))
+    x = torch.randn(4, 16, 14, 14)
+    got = layer(x.to(DEV))
+    xq = oracle.quantize(np.pad(x.numpy(), ((0, 0), (0, 0), (1, 1), (1, 1))), I, F)
+    shift = layer.shift.detach().cpu().clamp(*layer.shift_range).round().numpy().astype(np.int32)
+    sign = layer.sign.detach().cpu().numpy().astype(np.int32)
+    bq = oracle.quantize(layer.bias.detach().cpu().numpy(), I, F)
+    want = oracle.conv2d(xq, shift, sign, bq, (1, 1)).astype(np.float32) / np.float32(2.0 ** F)
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+    layer.use_kernel = False
+    ref = layer(x.to(DEV))
+    scale = float(utils.round_to_fixed(x, I, F).abs().max()) * 144
+    assert (got - ref).abs().max().item() < float_bound(144, F, scale)
+
+
+def test_q_modules_and_circular_padding():
+    torch.manual_seed(2)
+    lq = modules_q.LinearShiftQ(64, 32, use_kernel=True).to(DEV)
+    x = torch.randn(16, 64, device=DEV)
+    got = lq(x)
+    lq.use_kernel = False
+    ref = utils.round_to_fixed(x).mm(utils.round_power_of_2(lq.weight.data).t()) + utils.round_to_fixed(lq.bias.data)
+    assert (got - ref).abs().max().item() < float_bound(64, 16, 300.0)
+    cq = modules_q.Conv2dShiftQ(8, 8, 3, padding=1, padding_mode='circular', use_kernel=True).to(DEV)
+    xi = torch.randn(2, 8, 9, 9, device=DEV)
+    got = cq(xi)
+    cq.use_kernel = False
+    assert (got - cq(xi)).abs().max().item() < float_bound(72, 16, 300.0)
+    with pytest.raises(NotImplementedError):
+        modules.Conv2dShift(4, 4, 3, dilation=2, use_kernel=True).to(DEV)(torch.randn(1, 4, 9, 9, device=DEV))
+
+
+def test_mlp_config1_end_to_end(oracle):
+    """BASELINE config 1: 784-512-512-10, batch 64, ternary sign, shift in [-15, 0], 16.16."""
+    g = torch.Generator().manual_seed(0)
+    x = torch.rand(64, 784, generator=g)
+    model = workloads.MLP()
+    model, _ = convert.convert_to_shift(model, 0, 'PS', convert_weights=False, use_kernel=True, weight_bits=6)
+    model = model.to(DEV)
+    for layer in model.layers:
+        layer.sign.data = torch.randint(-1, 2, layer.sign.shape, generator=g).float().to(DEV)
+        layer.shift.data = torch.randint(-15, 1, layer.shift.shape, generator=g).float().to(DEV)
+        layer.bias.data = (torch.randn(layer.bias.shape, generator=g) * 0.01).to(DEV)
+        layer.conc_weight = None  # repacked lazily from the new codes
+    with torch.no_grad():
+        got = model(x.to(DEV)).cpu().numpy()
+    h = x.numpy()
+    for i, layer in enumerate(model.layers):
+        h = _oracle_linear_module(oracle, h, layer, round_input=False)
+        if i < 2:
+            h = np.maximum(h, 0)
+    np.testing.assert_array_equal(got, h)
+
+
+def test_resnet20_config3_kernel_vs_float_path():
+    """BASELINE config 3 at a reduced batch: every conv + FC shift-kernelised; the kernel model and
+    the float model agree layer by layer within the fixed-point bound on the same inputs."""
+    g = torch.Generator().manual_seed(3)
+    model = workloads.randomize_batchnorm(workloads.ResNet20(), g).eval()
+    model, n = convert.convert_to_shift(model, 1000, 'PS', convert_weights=True, use_kernel=True)
+    assert n == 19
+    model = model.to(DEV)
+    convert.round_shift_weights(model)
+    x = torch.randn(8, 3, 32, 32, generator=g).to(DEV)
+    layers = [m for m in model.modules() if isinstance(m, (modules.Conv2dShift, modules.LinearShift))]
+    captured = {}
+    hooks = [m.register_forward_hook(lambda mod, inp, out, k=i: captured.__setitem__(k, (inp[0], out)))
+             for i, m in enumerate(layers)]
+    with torch.no_grad():
+        model(x)
+    for h in hooks:
+        h.remove()
+    assert len(captured) == 20
+    for i, m in enumerate(layers):
+        inp, out = captured[i]
+        m.use_kernel = False
+        with torch.no_grad():
+            if isinstance(m, modules.LinearShift):
+                ref = m((inp * 65536).int().float() / 65536)
+            else:
+                ref = m(inp)
+        m.use_kernel = True
+        K = m.shift[0].numel()
+        scale = float(inp.abs().max()) * K
+        assert (out - ref).abs().max().item() < float_bound(K, 16, scale), (i, K)

@@ -1,0 +1,313 @@
+"""GPU parity: the HIP library, called through its C ABI, against the CPU oracle -- bit-exact."""
+import ctypes
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from deepshift_amd import _lib
+from oracle import shift_oracle as so
+from tests.conftest import random_activations, random_codes
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+KAT = json.load(open(os.path.join(HERE, "golden", "kat.json")))
+DEV = "cuda:0"
+NTHREADS = min(16, os.cpu_count() or 1)
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def stream():
+    return _lib.current_stream(torch.device(DEV))
+
+
+def abi_pack(s, sign, bits, base=0):
+    O, K = s.shape
+    num = 32 // (bits + 1)
+    comm = (K + num - 1) // num
+    out = torch.full((O, comm), -1, dtype=torch.int32, device=DEV)
+    _lib.call("ds_pack_i32", _lib.ptr(dev(s)), _lib.ptr(dev(sign)), _lib.ptr(out), O, K, bits, base,
+              stream())
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+def abi_linear(x, w_ref, bias, N, bits, base=0):
+    """ds_linear_i32 with canaries around the output and an exactly sized workspace."""
+    M, K = x.shape
+    L = _lib.lib()
+    ws_bytes = L.ds_linear_workspace_bytes(M, K, N, bits)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=DEV)
+    guard = 64
+    ybuf = torch.full((M * N + 2 * guard,), 0x5A5A5A5A, dtype=torch.int32, device=DEV)
+    y = ybuf[guard:guard + M * N]
+    xd, wd = dev(x), dev(w_ref)
+    bd = None if bias is None else dev(bias)
+    _lib.call("ds_linear_i32", _lib.ptr(xd), _lib.ptr(wd), _lib.ptr(bd), ctypes.c_void_p(y.data_ptr()),
+              M, K, N, bits, base, _lib.ptr(ws), ws_bytes, stream())
+    torch.cuda.synchronize()
+    host = ybuf.cpu().numpy()
+    assert (host[:guard] == 0x5A5A5A5A).all() and (host[guard + M * N:] == 0x5A5A5A5A).all(), \
+        "write outside the output"
+    return host[guard:guard + M * N].reshape(M, N)
+
+
+def abi_conv(xp, w_ref, bias, O, FH, FW, stride, bits, base=0):
+    Nb, C, Hp, Wp = xp.shape
+    sh, sw = stride
+    OH, OW = (Hp - FH) // sh + 1, (Wp - FW) // sw + 1
+    L = _lib.lib()
+    ws_bytes = L.ds_conv2d_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=DEV)
+    total = Nb * O * OH * OW
+    guard = 64
+    ybuf = torch.full((total + 2 * guard,), 0x5A5A5A5A, dtype=torch.int32, device=DEV)
+    y = ybuf[guard:guard + total]
+    xd, wd = dev(xp), dev(w_ref)
+    bd = None if bias is None else dev(bias)
+    _lib.call("ds_conv2d_i32", _lib.ptr(xd), _lib.ptr(wd), _lib.ptr(bd), ctypes.c_void_p(y.data_ptr()),
+              Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits, base, _lib.ptr(ws), ws_bytes, stream())
+    torch.cuda.synchronize()
+    host = ybuf.cpu().numpy()
+    assert (host[:guard] == 0x5A5A5A5A).all() and (host[guard + total:] == 0x5A5A5A5A).all(), \
+        "write outside the output"
+    return host[guard:guard + total].reshape(Nb, O, OH, OW)
+
+
+# ----------------------------------------------------------------------------- packing
+
+@pytest.mark.parametrize("case", KAT["pack"], ids=lambda c: "bits%d" % c["bits"])
+def test_pack_known_answers(case):
+    s = np.array([case["s"]], np.int32)
+    sign = np.array([case["sign"]], np.int32)
+    want = np.array([int(h, 16) for h in case["words_hex"]], np.uint32).view(np.int32)[None, :]
+    np.testing.assert_array_equal(abi_pack(s, sign, case["bits"]), want)
+
+
+@pytest.mark.parametrize("bits", [1, 2, 3, 4, 5, 6])
+def test_pack_matches_oracle(oracle, rng, bits):
+    for (O, K) in [(1, 1), (3, 7), (64, 576), (10, 4099), (1000, 512)]:
+        s = rng.integers(0, 2 ** bits, size=(O, K)).astype(np.int32)
+        sign = rng.choice(np.array([-1, 0, 1], np.int32), size=(O, K))
+        want, ovf = oracle.pack_words(s, sign, bits)
+        assert ovf == 0
+        np.testing.assert_array_equal(abi_pack(s, sign, bits), want)
+    # non-zero base: field = s - base
+    s = rng.integers(-3, 2 ** bits - 3, size=(5, 29)).astype(np.int32)
+    sign = rng.choice(np.array([-1, 1], np.int32), size=(5, 29))
+    want, ovf = oracle.pack_words(s, sign, bits, -3)
+    assert ovf == 0
+    np.testing.assert_array_equal(abi_pack(s, sign, bits, -3), want)
+
+
+# ----------------------------------------------------------------------------- LinearShift GEMM
+
+def test_gemm_known_answer(oracle):
+    g = KAT["gemm"]
+    x, s, sign = np.array(g["x"], np.int32), np.array(g["s"], np.int32), np.array(g["sign"], np.int32)
+    bias, want = np.array(g["bias"], np.int32), np.array(g["y"], np.int32)
+    w, _ = oracle.pack_words(s, sign, 5)
+    np.testing.assert_array_equal(abi_linear(x, w, bias, 3, 5), want)
+    w6, _ = oracle.pack_words(s, sign, 6)
+    np.testing.assert_array_equal(abi_linear(x, w6, bias, 3, 6), want)
+
+
+LINEAR_SHAPES = [(1, 1, 1), (2, 5, 3), (5, 17, 7), (64, 784, 512), (64, 512, 10), (130, 100, 33),
+                 (257, 6, 16), (63, 36, 17), (1000, 13, 65), (129, 577, 48)]
+
+
+@pytest.mark.parametrize("bits", [1, 2, 3, 4, 5])
+@pytest.mark.parametrize("shape", LINEAR_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_linear_matches_oracle(oracle, rng, bits, shape):
+    M, K, N = shape
+    x = random_activations(rng, (M, K))
+    s, sign = random_codes(rng, (N, K), max_s=2 ** bits - 1)
+    bias = rng.integers(-2 ** 31, 2 ** 31 - 1, size=N, dtype=np.int64).astype(np.int32)
+    w, ovf = oracle.pack_words(s, sign, bits)
+    assert ovf == 0
+    want = oracle.linear(x, -s, sign, bias, NTHREADS)
+    np.testing.assert_array_equal(oracle.gemm_packed(x, w, bias, N, bits, nthreads=NTHREADS), want)
+    np.testing.assert_array_equal(abi_linear(x, w, bias, N, bits), want)
+
+
+@pytest.mark.parametrize("shape", LINEAR_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_linear_ternary_zero_codes(oracle, rng, shape):
+    """sign == 0 is packed as the zero code (s = 32, bits = 6) and must add exactly 0 even for
+    negative activations (shift_cpu.cpp:190-201)."""
+    M, K, N = shape
+    x = random_activations(rng, (M, K))
+    s, sign = random_codes(rng, (N, K), max_s=31, zero_frac=0.3)
+    bias = rng.integers(-2 ** 20, 2 ** 20, size=N).astype(np.int32)
+    want = oracle.linear(x, -s, sign, bias, NTHREADS)
+    s_z = np.where(sign == 0, 32, s).astype(np.int32)
+    sign_z = np.where(sign == 0, 1, sign).astype(np.int32)
+    w, _ = oracle.pack_words(s_z, sign_z, 6)
+    np.testing.assert_array_equal(abi_linear(x, w, bias, N, 6), want)
+
+
+def test_linear_without_bias_and_nonzero_base(oracle, rng):
+    M, K, N = 70, 45, 20
+    x = random_activations(rng, (M, K))
+    s, sign = random_codes(rng, (N, K), max_s=15)
+    w, _ = oracle.pack_words(s, sign, 4)
+    np.testing.assert_array_equal(abi_linear(x, w, None, N, 4), oracle.linear(x, -s, sign, None))
+    for bits, base in [(4, -3), (5, -7), (6, -2)]:
+        s2 = rng.integers(base, base + 2 ** min(bits, 5), size=(N, K)).astype(np.int32)
+        w2, ovf = oracle.pack_words(s2, sign, bits, base)
+        assert ovf == 0
+        want = so.np_linear_planes(x, s2, sign, None, base)
+        np.testing.assert_array_equal(oracle.gemm_packed(x, w2, None, N, bits, base), want)
+        np.testing.assert_array_equal(abi_linear(x, w2, None, N, bits, base), want)
+
+
+def test_linear_split_k_path(oracle, rng):
+    """Few rows and a long reduction: K is split over workgroups and combined with integer atomics."""
+    for (M, K, N, bits) in [(64, 4608, 64, 4), (10, 9000, 33, 2), (200, 2304, 256, 4)]:
+        x = random_activations(rng, (M, K))
+        s, sign = random_codes(rng, (N, K), max_s=2 ** bits - 1)
+        bias = rng.integers(-2 ** 31, 2 ** 31 - 1, size=N, dtype=np.int64).astype(np.int32)
+        w, _ = oracle.pack_words(s, sign, bits)
+        np.testing.assert_array_equal(abi_linear(x, w, bias, N, bits), oracle.linear(x, -s, sign, bias, NTHREADS))
+
+
+def test_linear_against_reference_vectors():
+    """Outputs of the reference's own CPU kernel (tests/golden/ref_cpu_vectors.npz)."""
+    z = np.load(os.path.join(HERE, "golden", "ref_cpu_vectors.npz"))
+    s = (-z["lin_shift"].astype(np.int32))
+    sign = z["lin_sign"]
+    s_z = np.where(sign == 0, 32, s).astype(np.int32)
+    sign_z = np.where(sign == 0, 1, sign).astype(np.int32)
+    w = so.np_pack_words(s_z, sign_z, 6)
+    np.testing.assert_array_equal(abi_linear(z["lin_x"], w, z["lin_bias"], s.shape[0], 6), z["lin_y"])
+
+
+# ----------------------------------------------------------------------------- Conv2dShift
+
+CONV_CASES = [
+    # Nb, C, Hp, Wp, O, FH, FW, stride
+    (1, 1, 3, 3, 1, 3, 3, (1, 1)),
+    (2, 3, 9, 11, 5, 3, 3, (1, 1)),
+    (2, 3, 9, 11, 5, 3, 3, (2, 2)),
+    (3, 16, 18, 18, 32, 3, 3, (1, 1)),
+    (2, 64, 16, 16, 64, 3, 3, (1, 1)),
+    (2, 64, 15, 15, 128, 1, 1, (2, 2)),
+    (1, 3, 38, 38, 64, 7, 7, (2, 2)),
+    (2, 5, 12, 9, 7, 5, 2, (1, 2)),
+    (4, 32, 9, 9, 33, 3, 3, (1, 1)),
+    (70, 8, 5, 5, 16, 3, 3, (1, 1)),
+]
+
+
+@pytest.mark.parametrize("bits", [2, 4])
+@pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: "n%d_c%d_%dx%d_o%d_f%dx%d_s%d%d" % (c[:7] + c[7]))
+def test_conv_matches_oracle(oracle, rng, bits, case):
+    Nb, C, Hp, Wp, O, FH, FW, stride = case
+    xp = random_activations(rng, (Nb, C, Hp, Wp))
+    s, sign = random_codes(rng, (O, C, FH, FW), max_s=2 ** bits - 1)
+    bias = rng.integers(-2 ** 31, 2 ** 31 - 1, size=O, dtype=np.int64).astype(np.int32)
+    w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)
+    want = oracle.conv2d(xp, -s, sign, bias, stride, nthreads=NTHREADS)
+    np.testing.assert_array_equal(abi_conv(xp, w, bias, O, FH, FW, stride, bits), want)
+
+
+def test_conv_ternary_and_reference_vectors(oracle, rng):
+    Nb, C, Hp, Wp, O, FH, FW = 2, 6, 10, 10, 9, 3, 3
+    xp = random_activations(rng, (Nb, C, Hp, Wp))
+    s, sign = random_codes(rng, (O, C, FH, FW), max_s=31, zero_frac=0.3)
+    want = oracle.conv2d(xp, -s, sign, None, (1, 1))
+    s_z = np.where(sign == 0, 32, s).astype(np.int32)
+    sign_z = np.where(sign == 0, 1, sign).astype(np.int32)
+    w = so.np_pack_words(s_z.reshape(O, -1), sign_z.reshape(O, -1), 6)
+    np.testing.assert_array_equal(abi_conv(xp, w, None, O, FH, FW, (1, 1), 6), want)
+
+    z = np.load(os.path.join(HERE, "golden", "ref_cpu_vectors.npz"))
+    s = -z["conv_shift"].astype(np.int32)
+    O2 = s.shape[0]
+    w = so.np_pack_words(s.reshape(O2, -1), z["conv_sign"].reshape(O2, -1), 4)
+    got = abi_conv(z["conv_x"], w, z["conv_bias"], O2, s.shape[2], s.shape[3],
+                   tuple(int(v) for v in z["conv_stride"]), 4)
+    np.testing.assert_array_equal(got, z["conv_y"])
+
+
+def test_conv_split_k_path(oracle, rng):
+    # 7x7 output, 512 channels: few pixels, K = 4608
+    Nb, C, Hp, Wp, O = 2, 512, 9, 9, 64
+    xp = random_activations(rng, (Nb, C, Hp, Wp))
+    s, sign = random_codes(rng, (O, C, 3, 3), max_s=15)
+    bias = rng.integers(-2 ** 20, 2 ** 20, size=O).astype(np.int32)
+    w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), 4)
+    want = oracle.conv2d(xp, -s, sign, bias, (1, 1), nthreads=NTHREADS)
+    np.testing.assert_array_equal(abi_conv(xp, w, bias, O, 3, 3, (1, 1), 4), want)
+
+
+# ----------------------------------------------------------------------------- fixed point
+
+def _float_samples(rng, n):
+    x = (rng.standard_normal(n) * rng.choice([1e-6, 1e-3, 1.0, 100.0, 1e5, 1e12], size=n)).astype(np.float32)
+    special = np.array([0.0, -0.0, 1.99999, -7.62939453125e-06, 40000.0, -40000.0, 32767.0, 32767.99999,
+                        -32768.0, -32768.5, 3.99, -5.0, 0.03, 0.04, np.inf, -np.inf, 1e-40, -1e-40],
+                       np.float32)
+    x[:special.size] = special
+    return x
+
+
+@pytest.mark.parametrize("I,F", [(16, 16), (3, 5), (8, 8), (1, 7), (4, 0), (20, 12)])
+def test_quantize_matches_oracle(oracle, rng, I, F):
+    x = _float_samples(rng, 10007)
+    q = torch.empty(x.size, dtype=torch.int32, device=DEV)
+    for mode, want in [(0, oracle.quantize(x, I, F)), (1, oracle.cast(x, F))]:
+        _lib.call("ds_quantize_f32_i32", _lib.ptr(dev(x)), _lib.ptr(q), x.size, I, F, mode, stream())
+        np.testing.assert_array_equal(q.cpu().numpy(), want)
+    # an independent statement of the rounding: torch's own ops on the CPU (utils.py:7-21)
+    from deepshift_amd import utils
+    finite = np.isfinite(x)
+    ref = (utils.round_to_fixed(torch.from_numpy(x[finite]), I, F) * 2 ** F).double().numpy()
+    _lib.call("ds_quantize_f32_i32", _lib.ptr(dev(x)), _lib.ptr(q), x.size, I, F, 0, stream())
+    np.testing.assert_array_equal(q.cpu().numpy()[finite], ref.astype(np.int64))
+
+
+def test_quantize_known_answers():
+    for case in KAT["round_to_fixed"]:
+        x = np.array(case["x"], np.float32)
+        q = torch.empty(x.size, dtype=torch.int32, device=DEV)
+        _lib.call("ds_quantize_f32_i32", _lib.ptr(dev(x)), _lib.ptr(q), x.size, case["I"], case["F"], 0, stream())
+        want = (np.array(case["y"], np.float64) * 2 ** case["F"]).astype(np.int64)
+        np.testing.assert_array_equal(q.cpu().numpy(), want)
+
+
+def test_quantize_pad_transpose_dequantize(oracle, rng):
+    Nb, C, H, W, ph, pw = 3, 5, 13, 9, 2, 1
+    x = (rng.standard_normal((Nb, C, H, W)) * 50).astype(np.float32)
+    q = torch.full((Nb, C, H + 2 * ph, W + 2 * pw), 77, dtype=torch.int32, device=DEV)
+    _lib.call("ds_quantize_pad_f32_i32", _lib.ptr(dev(x)), _lib.ptr(q), Nb, C, H, W, ph, pw, 16, 16, 0, stream())
+    want = np.zeros((Nb, C, H + 2 * ph, W + 2 * pw), np.int32)
+    want[:, :, ph:ph + H, pw:pw + W] = oracle.quantize(x, 16, 16)
+    np.testing.assert_array_equal(q.cpu().numpy(), want)
+
+    xi = oracle.quantize(x, 16, 16)
+    p = torch.full_like(q, 77)
+    _lib.call("ds_pad_i32", _lib.ptr(dev(xi)), _lib.ptr(p), Nb, C, H, W, ph, pw, stream())
+    np.testing.assert_array_equal(p.cpu().numpy(), want)
+
+    M, K = 70, 133
+    x2 = (rng.standard_normal((M, K)) * 3).astype(np.float32)
+    ldx = 128
+    qT = torch.full((K, ldx), 77, dtype=torch.int32, device=DEV)
+    _lib.call("ds_quantize_transpose_f32_i32", _lib.ptr(dev(x2)), _lib.ptr(qT), M, K, ldx, 16, 16, 1, stream())
+    wantT = np.zeros((K, ldx), np.int32)
+    wantT[:, :M] = oracle.cast(x2, 16).T
+    np.testing.assert_array_equal(qT.cpu().numpy(), wantT)
+    xT = torch.full((K, ldx), 77, dtype=torch.int32, device=DEV)
+    _lib.call("ds_transpose_i32", _lib.ptr(dev(oracle.cast(x2, 16))), _lib.ptr(xT), M, K, ldx, stream())
+    np.testing.assert_array_equal(xT.cpu().numpy(), wantT)
+
+    y = rng.integers(-2 ** 31, 2 ** 31 - 1, size=10001, dtype=np.int64).astype(np.int32)
+    out = torch.empty(y.size, dtype=torch.float32, device=DEV)
+    _lib.call("ds_dequantize_i32_f32", _lib.ptr(dev(y)), _lib.ptr(out), y.size, 16, stream())
+    np.testing.assert_array_equal(out.cpu().numpy(), y.astype(np.float32) / np.float32(65536.0))

@@ -1,0 +1,142 @@
+"""CPU-only checks of the Python host layer (the mirror of the reference's deepshift package)."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+import deepshift_amd
+from deepshift_amd import convert, kernels, modules, modules_q, utils, workloads
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+KAT = json.load(open(os.path.join(HERE, "golden", "kat.json")))
+
+
+@pytest.mark.parametrize("case", KAT["round_to_fixed"], ids=lambda c: "I%dF%d" % (c["I"], c["F"]))
+def test_round_to_fixed_known_answers(case):
+    got = utils.round_to_fixed(torch.tensor(case["x"], dtype=torch.float32), case["I"], case["F"])
+    np.testing.assert_array_equal(got.numpy(), np.array(case["y"], np.float32))
+
+
+def test_round_to_fixed_matches_oracle(oracle, rng):
+    x = (rng.standard_normal(5000) * rng.choice([1e-4, 1.0, 1e3, 1e6], size=5000)).astype(np.float32)
+    for I, F in [(16, 16), (3, 5), (8, 8), (1, 4)]:
+        np.testing.assert_array_equal(utils.round_to_fixed(torch.from_numpy(x), I, F).numpy(),
+                                      oracle.round_to_fixed(x, I, F))
+
+
+def test_get_shift_and_sign_known_answers():
+    k = KAT["shift_and_sign"]
+    shift, sign = utils.get_shift_and_sign(torch.tensor(k["w"], dtype=torch.float32))
+    np.testing.assert_array_equal(shift.numpy(), np.array(k["shift"], np.float32))
+    np.testing.assert_array_equal(sign.numpy(), np.array(k["sign"], np.float32))
+    shift, sign = utils.get_shift_and_sign(torch.zeros(1))
+    assert shift.item() == -np.inf and sign.item() == 0
+    np.testing.assert_array_equal(utils.round_power_of_2(torch.tensor([0.7, -0.1, 3.0])).numpy(),
+                                  np.array([0.5, -0.125, 4.0], np.float32))
+
+
+def test_bits_table():
+    for k, v in KAT["bits_from_min_shift"]["table"].items():
+        assert utils.shift_field_bits(int(k)) == v, k
+
+
+def test_clampabs_and_round():
+    x = torch.tensor([-3.0, -0.001, 0.0, 0.002, 0.5, 7.0])
+    np.testing.assert_allclose(utils.clampabs(x.clone(), 0.01, 1.0).numpy(), [-1, -0.01, 0, 0.01, 0.5, 1])
+    np.testing.assert_array_equal(utils.round(torch.tensor([0.5, 1.5, 2.5, -0.5])).numpy(), [0, 2, 2, -0])
+    r = utils.round(torch.full((1000,), 0.25), 'stochastic')
+    assert set(r.unique().tolist()) <= {0.0, 1.0} and 100 < r.sum() < 400
+
+
+def test_module_constructors_mirror_reference_defaults():
+    lin = modules.LinearShift(7, 5)
+    assert lin.shift.shape == (5, 7) and lin.sign.shape == (5, 7) and lin.bias.shape == (5,)
+    assert lin.shift_range == (-14, 0) and lin.conc_weight is None and lin.use_kernel is False
+    assert modules.LinearShift(7, 5, weight_bits=3).shift_range == (-2, 0)
+    assert modules_q.LinearShiftQ(7, 5, weight_bits=3).shift_range == (-3, 0)
+    conv = modules.Conv2dShift(3, 8, 3, stride=2, padding=1, bias=False)
+    assert conv.shift.shape == (8, 3, 3, 3) and conv.bias is None and conv.stride == (2, 2)
+    assert "kernel_size=(3, 3)" in repr(conv)
+    assert not modules.LinearShift(3, 2, freeze_sign=True).sign.requires_grad
+    assert modules.LinearShift(3, 2, check_grad=True).shift.dtype == torch.float64
+    with pytest.raises(ValueError):
+        modules.Conv2dShift(3, 8, 3, groups=2)
+
+
+def test_float_paths_use_power_of_two_weights():
+    torch.manual_seed(0)
+    lin = modules.LinearShift(6, 4)
+    x = torch.randn(3, 6)
+    w = 2.0 ** lin.shift.data.clamp(-14, 0).round() * lin.sign.data.round().sign()
+    torch.testing.assert_close(lin(x), x @ w.t() + lin.bias)
+    conv = modules.Conv2dShift(2, 3, 3, padding=1)
+    xi = torch.randn(1, 2, 5, 5)
+    w = 2.0 ** conv.shift.data.round() * conv.sign.data.round().sign()
+    want = torch.nn.functional.conv2d(utils.round_to_fixed(xi), w, utils.round_to_fixed(conv.bias.data), padding=1)
+    torch.testing.assert_close(conv(xi), want)
+    q = modules_q.Conv2dShiftQ(2, 3, 3, padding=1)
+    wq = utils.round_power_of_2(utils.clampabs(q.weight.data.clone(), 2.0 ** -15, 1.0))
+    want = torch.nn.functional.conv2d(utils.round_to_fixed(xi), wq, utils.round_to_fixed(q.bias.data), padding=1)
+    torch.testing.assert_close(q(xi), want)
+    # gradients flow straight through the rounding
+    lin(x).sum().backward()
+    assert lin.shift.grad is not None and lin.sign.grad is not None
+
+
+def test_convert_to_shift_walks_backwards_and_counts():
+    model = nn.Sequential(nn.Conv2d(3, 4, 3), nn.ReLU(), nn.Conv2d(4, 4, 3), nn.Flatten(), nn.Linear(16, 2))
+    m, n = convert.convert_to_shift(model, shift_depth=1, shift_type='PS', convert_weights=True)
+    # the LAST conv is converted first; linears are always converted with convert_all_linear
+    assert n == 1
+    assert type(m[0]) is nn.Conv2d and type(m[2]) is modules.Conv2dShift and type(m[4]) is modules.LinearShift
+    assert convert.count_layer_type(m, modules.Conv2dShift) == 1
+    model = workloads.ResNet20()
+    w0 = model.stem[0].weight.detach().clone()
+    m, n = convert.convert_to_shift(model, 1000, 'PS', convert_weights=True)
+    assert n == 19 and convert.count_layer_type(m, modules.Conv2dShift) == 19
+    assert convert.count_layer_type(m, modules.LinearShift) == 1
+    shift, sign = utils.get_shift_and_sign(w0)
+    torch.testing.assert_close(m.stem[0].shift.data, shift)
+    torch.testing.assert_close(m.stem[0].sign.data, sign)
+    mq, n = convert.convert_to_shift(workloads.MLP(), 0, 'Q')
+    assert n == 0 and convert.count_layer_type(mq, modules_q.LinearShiftQ) == 3
+    with pytest.raises(ValueError):
+        convert.convert_to_shift(nn.Sequential(nn.Linear(2, 2)), 1, 'XYZ')
+
+
+def test_round_shift_weights():
+    torch.manual_seed(1)
+    model = nn.Sequential(modules.Conv2dShift(2, 2, 3), modules_q.LinearShiftQ(4, 3))
+    model[0].shift.data += 0.3
+    out = convert.round_shift_weights(model, clone=True)
+    assert torch.equal(out[0].shift.data, out[0].shift.data.round())
+    assert set(out[0].sign.data.unique().tolist()) <= {-1.0, 0.0, 1.0}
+    w = out[1].weight.data
+    assert torch.equal(w.abs().log2(), w.abs().log2().round())
+    assert torch.equal(out[0].bias.data, utils.round_to_fixed(out[0].bias.data))
+    assert not torch.equal(model[0].shift.data, out[0].shift.data)  # clone left the original alone
+
+
+def test_kernel_path_has_no_cpu_fallback():
+    lin = modules.LinearShift(4, 3, use_kernel=True, use_cuda=False)
+    with pytest.raises(NotImplementedError):
+        lin(torch.randn(2, 4))
+    with pytest.raises(NotImplementedError):
+        kernels.linear(torch.zeros(1, 1, dtype=torch.int32), torch.zeros(1, 1), torch.zeros(1, 1),
+                       conc_weight=utils.ConcWeight(), use_cuda=False)
+    with pytest.raises((ValueError, RuntimeError, AssertionError)):
+        kernels.linear(torch.zeros(1, 1, dtype=torch.int32), torch.zeros(1, 1), torch.zeros(1, 1),
+                       conc_weight=utils.ConcWeight(torch.zeros(1, dtype=torch.int32), 0, 4))
+
+
+def test_workload_pair_counts():
+    for cls, chw, batch, want in [(workloads.ResNet18, (3, 224, 224), 64, 116.1e9),
+                                  (workloads.ResNet20, (3, 32, 32), 256, 10.38e9),
+                                  (workloads.MLP, (784,), 64, 42.8e6)]:
+        shapes = workloads.shift_layer_shapes(cls(), chw, batch)
+        pairs = sum(l["M"] * l["K"] * l["N"] for l in shapes)
+        assert abs(pairs - want) / want < 2e-3
+    assert deepshift_amd.__version__
