@@ -222,8 +222,9 @@ static int launch_shift(ShiftArgs a, int nsplit, hipStream_t st)
     a.tiles_n = ceil_div(a.N, J);
     const int tiles = a.tiles_m4 * a.tiles_n;
     a.blocks_per_xcd = ceil_div(tiles, 8);
-    a.groups_per_split = ceil_div(a.comm, nsplit);
-    nsplit = ceil_div(a.comm, a.groups_per_split);
+    if (nsplit < 1 || a.comm == 0) nsplit = 1;
+    a.groups_per_split = a.comm == 0 ? 1 : ceil_div(a.comm, nsplit);
+    nsplit = a.comm == 0 ? 1 : ceil_div(a.comm, a.groups_per_split);
     a.atomic_out = nsplit > 1;
     if (a.atomic_out) {
         const long total = (long)a.M * a.N;

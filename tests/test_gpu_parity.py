@@ -32,8 +32,8 @@ def abi_pack(s, sign, bits, base=0):
     num = 32 // (bits + 1)
     comm = (K + num - 1) // num
     out = torch.full((O, comm), -1, dtype=torch.int32, device=DEV)
-    _lib.call("ds_pack_i32", _lib.ptr(dev(s)), _lib.ptr(dev(sign)), _lib.ptr(out), O, K, bits, base,
-              stream())
+    sd, gd = dev(s), dev(sign)  # keep the device copies alive across the asynchronous launch
+    _lib.call("ds_pack_i32", _lib.ptr(sd), _lib.ptr(gd), _lib.ptr(out), O, K, bits, base, stream())
     torch.cuda.synchronize()
     return out.cpu().numpy()
 
@@ -261,14 +261,15 @@ def _float_samples(rng, n):
 def test_quantize_matches_oracle(oracle, rng, I, F):
     x = _float_samples(rng, 10007)
     q = torch.empty(x.size, dtype=torch.int32, device=DEV)
+    xd = dev(x)
     for mode, want in [(0, oracle.quantize(x, I, F)), (1, oracle.cast(x, F))]:
-        _lib.call("ds_quantize_f32_i32", _lib.ptr(dev(x)), _lib.ptr(q), x.size, I, F, mode, stream())
+        _lib.call("ds_quantize_f32_i32", _lib.ptr(xd), _lib.ptr(q), x.size, I, F, mode, stream())
         np.testing.assert_array_equal(q.cpu().numpy(), want)
     # an independent statement of the rounding: torch's own ops on the CPU (utils.py:7-21)
     from deepshift_amd import utils
     finite = np.isfinite(x)
     ref = (utils.round_to_fixed(torch.from_numpy(x[finite]), I, F) * 2 ** F).double().numpy()
-    _lib.call("ds_quantize_f32_i32", _lib.ptr(dev(x)), _lib.ptr(q), x.size, I, F, 0, stream())
+    _lib.call("ds_quantize_f32_i32", _lib.ptr(xd), _lib.ptr(q), x.size, I, F, 0, stream())
     np.testing.assert_array_equal(q.cpu().numpy()[finite], ref.astype(np.int64))
 
 
@@ -276,7 +277,8 @@ def test_quantize_known_answers():
     for case in KAT["round_to_fixed"]:
         x = np.array(case["x"], np.float32)
         q = torch.empty(x.size, dtype=torch.int32, device=DEV)
-        _lib.call("ds_quantize_f32_i32", _lib.ptr(dev(x)), _lib.ptr(q), x.size, case["I"], case["F"], 0, stream())
+        xd = dev(x)
+        _lib.call("ds_quantize_f32_i32", _lib.ptr(xd), _lib.ptr(q), x.size, case["I"], case["F"], 0, stream())
         want = (np.array(case["y"], np.float64) * 2 ** case["F"]).astype(np.int64)
         np.testing.assert_array_equal(q.cpu().numpy(), want)
 
@@ -285,29 +287,34 @@ def test_quantize_pad_transpose_dequantize(oracle, rng):
     Nb, C, H, W, ph, pw = 3, 5, 13, 9, 2, 1
     x = (rng.standard_normal((Nb, C, H, W)) * 50).astype(np.float32)
     q = torch.full((Nb, C, H + 2 * ph, W + 2 * pw), 77, dtype=torch.int32, device=DEV)
-    _lib.call("ds_quantize_pad_f32_i32", _lib.ptr(dev(x)), _lib.ptr(q), Nb, C, H, W, ph, pw, 16, 16, 0, stream())
+    xd = dev(x)
+    _lib.call("ds_quantize_pad_f32_i32", _lib.ptr(xd), _lib.ptr(q), Nb, C, H, W, ph, pw, 16, 16, 0, stream())
     want = np.zeros((Nb, C, H + 2 * ph, W + 2 * pw), np.int32)
     want[:, :, ph:ph + H, pw:pw + W] = oracle.quantize(x, 16, 16)
     np.testing.assert_array_equal(q.cpu().numpy(), want)
 
     xi = oracle.quantize(x, 16, 16)
     p = torch.full_like(q, 77)
-    _lib.call("ds_pad_i32", _lib.ptr(dev(xi)), _lib.ptr(p), Nb, C, H, W, ph, pw, stream())
+    xid = dev(xi)
+    _lib.call("ds_pad_i32", _lib.ptr(xid), _lib.ptr(p), Nb, C, H, W, ph, pw, stream())
     np.testing.assert_array_equal(p.cpu().numpy(), want)
 
     M, K = 70, 133
     x2 = (rng.standard_normal((M, K)) * 3).astype(np.float32)
     ldx = 128
     qT = torch.full((K, ldx), 77, dtype=torch.int32, device=DEV)
-    _lib.call("ds_quantize_transpose_f32_i32", _lib.ptr(dev(x2)), _lib.ptr(qT), M, K, ldx, 16, 16, 1, stream())
+    x2d = dev(x2)
+    _lib.call("ds_quantize_transpose_f32_i32", _lib.ptr(x2d), _lib.ptr(qT), M, K, ldx, 16, 16, 1, stream())
     wantT = np.zeros((K, ldx), np.int32)
     wantT[:, :M] = oracle.cast(x2, 16).T
     np.testing.assert_array_equal(qT.cpu().numpy(), wantT)
     xT = torch.full((K, ldx), 77, dtype=torch.int32, device=DEV)
-    _lib.call("ds_transpose_i32", _lib.ptr(dev(oracle.cast(x2, 16))), _lib.ptr(xT), M, K, ldx, stream())
+    x2q = dev(oracle.cast(x2, 16))
+    _lib.call("ds_transpose_i32", _lib.ptr(x2q), _lib.ptr(xT), M, K, ldx, stream())
     np.testing.assert_array_equal(xT.cpu().numpy(), wantT)
 
     y = rng.integers(-2 ** 31, 2 ** 31 - 1, size=10001, dtype=np.int64).astype(np.int32)
     out = torch.empty(y.size, dtype=torch.float32, device=DEV)
-    _lib.call("ds_dequantize_i32_f32", _lib.ptr(dev(y)), _lib.ptr(out), y.size, 16, stream())
+    yd = dev(y)
+    _lib.call("ds_dequantize_i32_f32", _lib.ptr(yd), _lib.ptr(out), y.size, 16, stream())
     np.testing.assert_array_equal(out.cpu().numpy(), y.astype(np.float32) / np.float32(65536.0))
