@@ -19,6 +19,8 @@
 //   * layers with few pixels split K over gridDim.y and combine with integer atomics (wrap-around
 //     addition commutes, so the result stays bit-exact).
 #include "ds_common.h"
+#include <cstdio>
+#include <cstdlib>
 
 namespace ds {
 
@@ -237,21 +239,49 @@ static int launch_shift(ShiftArgs a, int nsplit, hipStream_t st)
     return launch_status();
 }
 
-// Tile shape / split-K choice.  256 CUs x 4 SIMDs want a few thousand waves in flight.
+// Tile shape / split-K choice.
+//
+// The kernel is VALU-bound and every wave of a launch does the same amount of work, so the launch
+// time is set by the SIMD that holds the most waves: W waves on 1024 SIMDs run at
+// (W/1024) / ceil(W/1024) of the balanced rate.  A ResNet layer at R=2, J=32 has only 400..3136
+// tiles, i.e. 1..3.06 waves per SIMD, which caps it at ~77 %.  Splitting K multiplies the number of
+// (shorter) waves; measured on MI355X the best point is ~24k waves of >= 12 packed words each
+// (the atomic combine is hidden behind the VALU work), e.g. layer1 3x3x64: 60 % -> 80 % of peak.
+// DS_TUNE_TILE=RxJ and DS_TUNE_SPLIT=n (environment) override the choice for experiments.
+struct TileChoice {
+    int R, J, nsplit;
+};
+
+static TileChoice choose_tile(const ShiftArgs &a)
+{
+    TileChoice c{2, 32, 1};
+    if (a.N <= 16) { c.R = 4; c.J = 16; }                   // few channels: more pixels per lane
+    else if (a.M <= 64 || a.OW <= 8) { c.R = 1; c.J = 32; } // few / scattered pixels
+    else if (a.comm <= 32 && a.N >= 64) { c.R = 4; c.J = 16; }  // short reduction (e.g. 7x7x3 stem)
+    const long tiles = (long)ceil_div(a.M, c.R * kWave) * ceil_div(a.N, c.J);
+    const long simds = 1024;
+    const double per_simd = (double)tiles / simds;
+    const double balance = per_simd / (double)((tiles + simds - 1) / simds);
+    if (tiles >= 12 * simds || (tiles >= 4 * simds && balance >= 0.94)) return c;
+    long want = (24 * simds + tiles / 2) / tiles;
+    const long max_by_k = a.comm / 12 > 0 ? a.comm / 12 : 1;
+    if (want > max_by_k) want = max_by_k;
+    if (want > 64) want = 64;
+    if (want < 1) want = 1;
+    c.nsplit = (int)want;
+    return c;
+}
+
 template <int BITS, bool GENERAL>
 static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
 {
-    const long waves_2x32 = (long)ceil_div(a.M, 128) * ceil_div(a.N, 32);
-    const int target_waves = 3072;
-    int nsplit = 1;
-    if (waves_2x32 < target_waves) {
-        nsplit = (int)((target_waves + waves_2x32 - 1) / waves_2x32);
-        const int max_split = a.comm / 8 > 0 ? a.comm / 8 : 1;  // keep >= 8 words per slice
-        if (nsplit > max_split) nsplit = max_split;
-        if (nsplit > 64) nsplit = 64;
-    }
-    if (a.N <= 16) return launch_shift<BITS, GENERAL, 4, 16>(a, nsplit, st);
-    return launch_shift<BITS, GENERAL, 2, 32>(a, nsplit, st);
+    TileChoice c = choose_tile(a);
+    if (const char *t = getenv("DS_TUNE_TILE")) sscanf(t, "%dx%d", &c.R, &c.J);
+    if (const char *t = getenv("DS_TUNE_SPLIT")) c.nsplit = atoi(t);
+    if (c.R == 4 && c.J == 16) return launch_shift<BITS, GENERAL, 4, 16>(a, c.nsplit, st);
+    if (c.R == 3 && c.J == 16) return launch_shift<BITS, GENERAL, 3, 16>(a, c.nsplit, st);
+    if (c.R == 1 && c.J == 32) return launch_shift<BITS, GENERAL, 1, 32>(a, c.nsplit, st);
+    return launch_shift<BITS, GENERAL, 2, 32>(a, c.nsplit, st);
 }
 
 static int dispatch_bits(const ShiftArgs &a, int bits, bool general, hipStream_t st)
