@@ -70,7 +70,7 @@ def parity_gate(model, x):
     h.remove()
     xin = captured["x"][:1].contiguous()
     xq = kernels.quantize_pad(xin, layer.padding, 16, 16)
-    tiled = kernels._tiled_of(layer.conc_weight, layer.out_channels, layer.shift[0].numel())
+    tiled = kernels._tiled_of(layer.conc_weight, layer.out_channels, layer.in_channels, *layer.kernel_size)
     y = kernels.conv2d_tiled(xq, tiled, None, layer.out_channels, layer.kernel_size, layer.stride,
                              layer.conc_weight.bits, layer.conc_weight.base)
     shift = layer.shift.detach().clamp(*layer.shift_range).round().cpu().numpy().astype(np.int32)
@@ -161,7 +161,7 @@ def config2(device, reps=10):
     shift, sign = codes((64, 64, 3, 3))
     cw = utils.compress_bits(shift, sign)
     xq = kernels.quantize_pad(x, (1, 1))
-    tiled = kernels._tiled_of(cw, 64, 576)
+    tiled = kernels._tiled_of(cw, 64, 64, 3, 3)
     t = timeit(lambda: kernels.conv2d_tiled(xq, tiled, None, 64, (3, 3), (1, 1), cw.bits, cw.base))
     pairs = 32 * 56 * 56 * 576 * 64
     out["conv3x3_64x64_32x56x56"] = dict(ms=t * 1e3, gops=2 * pairs / t / 1e9, valu_frac=pairs / t / PEAK_PAIRS)

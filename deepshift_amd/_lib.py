@@ -23,7 +23,7 @@ SIGNATURES = {
     "ds_status_string": (ctypes.c_char_p, [_c_int]),
     "ds_pack_i32": (_c_int, [_ptr, _ptr, _ptr, _c_int, _c_int, _c_int, _c_int, _ptr]),
     "ds_tiled_bytes": (_size, [_c_int, _c_int, _c_int]),
-    "ds_tile_weights_i32": (_c_int, [_ptr, _ptr, _c_int, _c_int, _c_int, _c_int, _ptr]),
+    "ds_tile_weights_i32": (_c_int, [_ptr, _ptr] + [_c_int] * 6 + [_ptr]),
     "ds_linear_workspace_bytes": (_size, [_c_int] * 4),
     "ds_linear_i32": (_c_int, [_ptr] * 4 + [_c_int] * 5 + [_ptr, _size, _ptr]),
     "ds_linear_tiled_workspace_bytes": (_size, [_c_int] * 4),

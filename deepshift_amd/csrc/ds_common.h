@@ -10,8 +10,7 @@
 namespace ds {
 
 constexpr int kWave = 64;           // CDNA wavefront width
-constexpr int kTileWords = 16;      // words per (channel-tile, k-group) row of the tiled layout
-constexpr int kChannelPad = 32;     // tiled layout pads the channel count to a multiple of this
+constexpr int kTileWords = 32;      // words per (channel-tile, k-group) row of the tiled layout
 
 __host__ __device__ constexpr int codes_per_word(int bits) { return 32 / (bits + 1); }
 __host__ __device__ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
@@ -20,29 +19,42 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 inline int hip_status(hipError_t e) { return e == hipSuccess ? DS_OK : DS_EHIP - (int)e; }
 inline int launch_status() { return hip_status(hipGetLastError()); }
 
-// Geometry of the tiled weight blob: words[ntiles16][comm][16] then negcount[ntiles16*16].
+// Geometry of the tiled weight blob:
+//   words   [ntiles][comm][32]        packed codes, 32 consecutive channels per row
+//   negcount[ntiles*32]               negative codes per channel
+//   ktab    [(comm+1)*num]            reduction index k -> (ic << 10 | fh << 5 | fw); zero past K,
+//                                     with one spare group so that a prefetch of group comm is valid
 struct TiledGeom {
-    int num, comm, ntiles16;
-    size_t word_count, bytes;
+    int num, comm, ntiles;
+    size_t word_count, negcount_offset, ktab_offset, ktab_count, bytes;
 };
 inline TiledGeom tiled_geom(int N, int K, int bits)
 {
     TiledGeom g;
     g.num = codes_per_word(bits);
     g.comm = ceil_div(K, g.num);
-    g.ntiles16 = ceil_div(N, kChannelPad) * (kChannelPad / kTileWords);
-    g.word_count = (size_t)g.ntiles16 * g.comm * kTileWords;
-    g.bytes = align_up(g.word_count * 4, 256) + (size_t)g.ntiles16 * kTileWords * 4;
+    g.ntiles = ceil_div(N, kTileWords);
+    g.word_count = (size_t)g.ntiles * g.comm * kTileWords;
+    g.negcount_offset = align_up(g.word_count * 4, 256);
+    g.ktab_offset = g.negcount_offset + align_up((size_t)g.ntiles * kTileWords * 4, 256);
+    g.ktab_count = (size_t)(g.comm + 1) * g.num;
+    g.bytes = g.ktab_offset + align_up(g.ktab_count * 4, 256);
     return g;
 }
 inline const int32_t *tiled_negcount(const void *tiled, const TiledGeom &g)
 {
-    return (const int32_t *)((const char *)tiled + align_up(g.word_count * 4, 256));
+    return (const int32_t *)((const char *)tiled + g.negcount_offset);
+}
+inline const uint32_t *tiled_ktab(const void *tiled, const TiledGeom &g)
+{
+    return (const uint32_t *)((const char *)tiled + g.ktab_offset);
 }
 
 // Launchers implemented across the .hip files.
 int launch_pack(const int32_t *s, const int32_t *sign, int32_t *out, int O, int K, int bits,
                 int base, hipStream_t st);
-int launch_tile(const int32_t *w_ref, void *tiled, int N, int K, int bits, hipStream_t st);
+int launch_tile(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW, int bits,
+                hipStream_t st);
+int launch_transpose(const int32_t *x, int32_t *xT, int M, int K, int ldx, hipStream_t st);
 
 }  // namespace ds

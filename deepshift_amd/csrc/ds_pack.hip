@@ -44,7 +44,7 @@ int launch_pack(const int32_t *s, const int32_t *sign, int32_t *out, int O, int 
     return launch_status();
 }
 
-// Reference-format words [N][comm] -> tiled words [ntiles16][comm][16].
+// Reference-format words [N][comm] -> tiled words [ntiles][comm][32].
 //   * code sign bit inverted: 1 = negative (the compute kernel sign-extends it into an xor mask);
 //   * codes past K, and every code of a padding channel, become (field 0, positive): with the
 //     activation read as 0 they add nothing;
@@ -100,19 +100,39 @@ __global__ void negcount_kernel(const int32_t *__restrict__ w_ref, int32_t *__re
     negcount[n] = count;
 }
 
-int launch_tile(const int32_t *w_ref, void *tiled, int N, int K, int bits, hipStream_t st)
+// ktab[k] = ic << 10 | fh << 5 | fw for k = (ic, fh, fw) < K, 0 beyond: the geometry-independent
+// part of an activation offset (the compute kernel multiplies by the plane and row pitch).
+__global__ void ktab_kernel(uint32_t *ktab, int K, int count, int FH, int FW)
 {
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= count) return;
+    uint32_t v = 0;
+    if (k < K) {
+        const int ic = k / (FH * FW);
+        const int rem = k - ic * FH * FW;
+        const int fh = rem / FW;
+        v = ((uint32_t)ic << 10) | ((uint32_t)fh << 5) | (uint32_t)(rem - fh * FW);
+    }
+    ktab[k] = v;
+}
+
+int launch_tile(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW, int bits,
+                hipStream_t st)
+{
+    const int K = C * FH * FW;
     const TiledGeom g = tiled_geom(N, K, bits);
     if (g.word_count) {
         const long blocks = ((long)g.word_count + 255) / 256;
         hipLaunchKernelGGL(tile_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w_ref,
                            (uint32_t *)tiled, N, K, g.comm, bits, g.num, (long)g.word_count);
     }
-    const int Npad = g.ntiles16 * kTileWords;
+    const int Npad = g.ntiles * kTileWords;
     if (Npad) {
         hipLaunchKernelGGL(negcount_kernel, dim3(ceil_div(Npad, 64)), dim3(64), 0, st, w_ref,
                            (int32_t *)tiled_negcount(tiled, g), N, Npad, K, g.comm, bits, g.num);
     }
+    hipLaunchKernelGGL(ktab_kernel, dim3(ceil_div((int)g.ktab_count, 256)), dim3(256), 0, st,
+                       (uint32_t *)tiled_ktab(tiled, g), K, (int)g.ktab_count, FH, FW);
     return launch_status();
 }
 
@@ -137,13 +157,14 @@ DS_EXPORT size_t ds_tiled_bytes(int N, int K, int bits)
     return tiled_geom(N, K, bits).bytes;
 }
 
-DS_EXPORT int ds_tile_weights_i32(const int32_t *w_ref, void *tiled, int N, int K, int bits, int base,
-                                  ds_stream_t stream)
+DS_EXPORT int ds_tile_weights_i32(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW,
+                                  int bits, int base, ds_stream_t stream)
 {
     if (bits < 1 || bits > 6) return DS_EBITS;
     if (base > 0 || base < -31) return DS_EBASE;
-    if (N < 0 || K < 0) return DS_EINVAL;
+    if (N < 0 || C < 0 || FH < 1 || FW < 1) return DS_EINVAL;
+    if (C >= (1 << 22) || FH > 31 || FW > 31 || (size_t)C * FH * FW >= (1u << 24)) return DS_ETOOLARGE;
     if (N == 0) return DS_OK;
-    if (!tiled || (!w_ref && K > 0)) return DS_EINVAL;
-    return launch_tile(w_ref, tiled, N, K, bits, (hipStream_t)stream);
+    if (!tiled || (!w_ref && C > 0)) return DS_EINVAL;
+    return launch_tile(w_ref, tiled, N, C, FH, FW, bits, (hipStream_t)stream);
 }

@@ -15,6 +15,10 @@
 //     constant that is added once in the epilogue (the tiled weight blob carries the count);
 //   * each lane keeps R pixels x J channels of int32 accumulators in registers, so one activation
 //     load feeds 2*J vector instructions and one decoded code feeds 2*R of them;
+//   * activation (m, k) lives at x[xoff(m) + koff(k)]: xoff is a per-lane byte offset computed once,
+//     koff = ic*Hp*Wp + fh*Wp + fw is wave-uniform and advanced incrementally on the scalar ALU, so a
+//     load is one buffer_load_dword (VGPR offset + SGPR offset) with no vector address arithmetic;
+//     the loads of the next K group are issued before the current group is accumulated;
 //   * no LDS, no barriers: waves are independent, occupancy is bounded by registers only;
 //   * layers with few pixels split K over gridDim.y and combine with integer atomics (wrap-around
 //     addition commutes, so the result stays bit-exact).
@@ -25,16 +29,18 @@
 namespace ds {
 
 struct ShiftArgs {
-    const int32_t *x;       // activations: element (m, k) lives at x[xoff(m) + ktab[k]]
+    const int32_t *x;       // activations
     const uint32_t *wt;     // tiled words [ntiles16][comm][16]
     const int32_t *negcnt;  // per channel: number of negative codes
     const int32_t *bias;    // per channel or nullptr
-    const int32_t *ktab;    // [comm*num] activation offset of reduction index k
+    const uint32_t *ktab;   // [(comm+1)*num] k -> ic << 10 | fh << 5 | fw (0 past K)
     int32_t *y;
+    uint32_t x_bytes;       // size of x (bound of the buffer descriptor)
     int M, N, K, comm;
     int pix_per_img, OW;                  // m -> (img, oh, ow)
     int x_img_stride, x_row_stride, x_col_stride;
     int y_img_stride, y_pix_stride, y_ch_stride;
+    int x_plane, x_row;                   // koff(k) = ic*x_plane + fh*x_row + fw
     int groups_per_split;                 // k-groups (words) per gridDim.y slice
     int nbase;                            // -base (left shift applied after the right shift)
     int tiles_m4;                         // number of 4-wave pixel tiles
@@ -57,9 +63,23 @@ __device__ __forceinline__ int32_t *at_lane(int32_t *uniform_base, uint32_t lane
 {
     return (int32_t *)((char *)uniform_base + lane_bytes);
 }
-__device__ __forceinline__ int32_t ld_lane(const int32_t *uniform_base, uint32_t lane_bytes)
+
+// Issues the R activation loads of each of the NUM reduction indices of K group g.  The element
+// offset of k, ic*x_plane + fh*x_row + fw, is wave-uniform: (ic, fh, fw) come packed from the k
+// table of the weight blob through a scalar load and the offset is formed on the scalar ALU, so a
+// load is one buffer_load_dword (per-lane VGPR offset + SGPR offset) with no vector arithmetic.
+template <int NUM, int R>
+__device__ __forceinline__ void load_group(int32_t (&xv)[NUM][R], __amdgpu_buffer_rsrc_t rsrc,
+                                           const uint32_t (&xoff)[R], const ShiftArgs &p, int g)
 {
-    return *(const int32_t *)((const char *)uniform_base + lane_bytes);
+#pragma unroll
+    for (int i = 0; i < NUM; ++i) {
+        const uint32_t v = p.ktab[g * NUM + i];
+        const int koff = (int)(v >> 10) * p.x_plane + (int)((v >> 5) & 31u) * p.x_row + (int)(v & 31u);
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            xv[i][r] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, xoff[r], koff * 4, 0);
+    }
 }
 
 template <int BITS, bool GENERAL, int R, int J>
@@ -89,7 +109,7 @@ template <int BITS, bool GENERAL, int R, int J>
 __global__ __launch_bounds__(256) void shift_kernel(const ShiftArgs p)
 {
     constexpr int NUM = 32 / (BITS + 1);
-    static_assert(J % kTileWords == 0, "J must be a multiple of the layout tile");
+    static_assert(kTileWords % J == 0, "the layout tile must hold whole channel tiles");
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
 
@@ -104,7 +124,7 @@ __global__ __launch_bounds__(256) void shift_kernel(const ShiftArgs p)
     const int m0 = mtile * (R * kWave);
     if (m0 >= p.M) return;
 
-    // per-lane pixel coordinates
+    // per-lane pixel coordinates, as byte offsets (every tensor is < 2^31 bytes)
     uint32_t xoff[R], yoff[R];
     bool live[R];
 #pragma unroll
@@ -116,8 +136,6 @@ __global__ __launch_bounds__(256) void shift_kernel(const ShiftArgs p)
         const int rem = m - img * p.pix_per_img;
         const int oh = rem / p.OW;
         const int ow = rem - oh * p.OW;
-        // byte offsets (every tensor is < 2^31 bytes): a uniform 64-bit base plus a 32-bit lane
-        // offset is the addressing mode global loads and stores take directly
         xoff[r] = 4u * (uint32_t)(img * p.x_img_stride + oh * p.x_row_stride + ow * p.x_col_stride);
         yoff[r] = 4u * (uint32_t)(img * p.y_img_stride + rem * p.y_pix_stride);
     }
@@ -134,38 +152,45 @@ __global__ __launch_bounds__(256) void shift_kernel(const ShiftArgs p)
     const int full_groups = p.K / NUM;  // groups whose NUM codes are all real
     const int g_full_end = g_end < full_groups ? g_end : full_groups;
 
-    const uint32_t *wrow = p.wt + (size_t)(ntile * (J / kTileWords)) * p.comm * kTileWords;
-    const size_t tile_stride = (size_t)p.comm * kTileWords;
+    // words of this wave's J channels for K group g: wrow[g * 32 + j]
+    const uint32_t *wrow = p.wt + (size_t)((ntile * J) / kTileWords) * p.comm * kTileWords +
+                           (ntile * J) % kTileWords;
+    const __amdgpu_buffer_rsrc_t xrsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, (int)p.x_bytes, 0x00020000);
 
+    int32_t xcur[NUM][R];
+    if (g_begin < g_full_end) load_group<NUM, R>(xcur, xrsrc, xoff, p, g_begin);
+
+#pragma clang loop unroll(disable)
     for (int g = g_begin; g < g_full_end; ++g) {
         uint32_t w[J];
 #pragma unroll
-        for (int j = 0; j < J; ++j)
-            w[j] = wrow[(j / kTileWords) * tile_stride + (size_t)g * kTileWords + (j % kTileWords)];
-        int32_t xv[NUM][R];
+        for (int j = 0; j < J; ++j) w[j] = wrow[(size_t)g * kTileWords + j];
+        // Issue the next group's loads before accumulating this one.  The prefetch is unconditional
+        // (the k table has a spare zero group, so group g + 1 always names valid addresses) so that
+        // the number of loads in flight is the same on every path and the wait counts stay exact.
+        int32_t xnext[NUM][R];
+        load_group<NUM, R>(xnext, xrsrc, xoff, p, g + 1);
 #pragma unroll
-        for (int i = 0; i < NUM; ++i) {
-            const int32_t *xk = p.x + p.ktab[g * NUM + i];
+        for (int i = 0; i < NUM; ++i) accumulate_code<BITS, GENERAL, R, J>(acc, xcur[i], w, i, p.nbase);
 #pragma unroll
-            for (int r = 0; r < R; ++r) xv[i][r] = ld_lane(xk, xoff[r]);
-        }
+        for (int i = 0; i < NUM; ++i)
 #pragma unroll
-        for (int i = 0; i < NUM; ++i) accumulate_code<BITS, GENERAL, R, J>(acc, xv[i], w, i, p.nbase);
+            for (int r = 0; r < R; ++r) xcur[i][r] = xnext[i][r];
     }
     // tail group: codes with k >= K read as x = 0 (the tiled blob holds neutral codes there)
     for (int g = g_full_end; g < g_end; ++g) {
         uint32_t w[J];
 #pragma unroll
-        for (int j = 0; j < J; ++j)
-            w[j] = wrow[(j / kTileWords) * tile_stride + (size_t)g * kTileWords + (j % kTileWords)];
+        for (int j = 0; j < J; ++j) w[j] = wrow[(size_t)g * kTileWords + j];
+        int32_t xt[NUM][R];
+        load_group<NUM, R>(xt, xrsrc, xoff, p, g);
 #pragma unroll
         for (int i = 0; i < NUM; ++i) {
-            int32_t xv[R];
             const bool real = g * NUM + i < p.K;
-            const int32_t *xk = p.x + (real ? p.ktab[g * NUM + i] : 0);
 #pragma unroll
-            for (int r = 0; r < R; ++r) xv[r] = real ? ld_lane(xk, xoff[r]) : 0;
-            accumulate_code<BITS, GENERAL, R, J>(acc, xv, w, i, p.nbase);
+            for (int r = 0; r < R; ++r) xt[i][r] = real ? xt[i][r] : 0;
+            accumulate_code<BITS, GENERAL, R, J>(acc, xt[i], w, i, p.nbase);
         }
     }
 
@@ -199,22 +224,6 @@ __global__ void fill_bias_kernel(const ShiftArgs p)
         const int n = (int)((idx / p.y_ch_stride) % p.N);
         p.y[idx] = p.negcnt[n] + (p.bias ? p.bias[n] : 0);
     }
-}
-
-// ktab[k] = ic*plane + fh*row + fw for k = (ic, fh, fw); entries past K are 0
-__global__ void ktab_kernel(int32_t *ktab, int K, int Kpad, int FH, int FW, int plane, int row)
-{
-    const int k = blockIdx.x * blockDim.x + threadIdx.x;
-    if (k >= Kpad) return;
-    int v = 0;
-    if (k < K) {
-        const int ic = k / (FH * FW);
-        const int rem = k - ic * FH * FW;
-        const int fh = rem / FW;
-        const int fw = rem - fh * FW;
-        v = ic * plane + fh * row + fw;
-    }
-    ktab[k] = v;
 }
 
 template <int BITS, bool GENERAL, int R, int J>
@@ -318,19 +327,17 @@ using namespace ds;
 DS_EXPORT size_t ds_conv2d_tiled_workspace_bytes(int Nb, int C, int Hp, int Wp, int O, int FH,
                                                  int FW, int sh, int sw, int bits)
 {
-    (void)Nb; (void)Hp; (void)Wp; (void)O; (void)sh; (void)sw;
-    if (bits < 1 || bits > 6 || C < 0 || FH < 1 || FW < 1) return 0;
-    const int num = codes_per_word(bits);
-    const size_t K = (size_t)C * FH * FW;
-    return align_up((K + num - 1) / num * num * 4, 256);
+    (void)Nb; (void)C; (void)Hp; (void)Wp; (void)O; (void)FH; (void)FW; (void)sh; (void)sw; (void)bits;
+    return 0;  // the tiled entry point needs no scratch memory
 }
 
 DS_EXPORT size_t ds_conv2d_workspace_bytes(int Nb, int C, int Hp, int Wp, int O, int FH, int FW,
                                            int sh, int sw, int bits)
 {
+    (void)Nb; (void)Hp; (void)Wp; (void)sh; (void)sw;
     if (bits < 1 || bits > 6 || C < 0 || O < 0 || FH < 1 || FW < 1) return 0;
-    return ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits) +
-           align_up(tiled_geom(O, C * FH * FW, bits).bytes, 256);
+    if ((size_t)C * FH * FW >= (1u << 24)) return 0;
+    return align_up(tiled_geom(O, C * FH * FW, bits).bytes, 256);
 }
 
 DS_EXPORT int ds_conv2d_tiled_i32(const int32_t *x, const void *tiled, const int32_t *bias,
@@ -338,6 +345,7 @@ DS_EXPORT int ds_conv2d_tiled_i32(const int32_t *x, const void *tiled, const int
                                   int sh, int sw, int bits, int base, void *workspace,
                                   size_t workspace_bytes, ds_stream_t stream)
 {
+    (void)workspace; (void)workspace_bytes;
     int rc = check_common(bits, base);
     if (rc) return rc;
     if (Nb < 0 || C < 0 || O < 0 || FH < 1 || FW < 1 || sh < 1 || sw < 1 || Hp < FH || Wp < FW)
@@ -345,17 +353,17 @@ DS_EXPORT int ds_conv2d_tiled_i32(const int32_t *x, const void *tiled, const int
     const int OH = (Hp - FH) / sh + 1, OW = (Wp - FW) / sw + 1;
     const size_t M = (size_t)Nb * OH * OW;
     if (M == 0 || O == 0) return DS_OK;
-    if (!x || !tiled || !y) return DS_EINVAL;
+    if (!tiled || !y || (!x && C > 0)) return DS_EINVAL;
     const size_t K = (size_t)C * FH * FW;
-    if ((size_t)Nb * C * Hp * Wp * 4 >= kMaxBytes || M * O * 4 >= kMaxBytes || K >= (1u << 24))
+    const size_t x_bytes = (size_t)Nb * C * Hp * Wp * 4;
+    if (x_bytes >= kMaxBytes || M * O * 4 >= kMaxBytes || K >= (1u << 24) || C >= (1 << 22) ||
+        FH > 31 || FW > 31)
         return DS_ETOOLARGE;
-    const size_t need = ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits);
-    if (need && (!workspace || workspace_bytes < need)) return DS_EWORKSPACE;
-    hipStream_t st = (hipStream_t)stream;
     const TiledGeom g = tiled_geom(O, (int)K, bits);
 
     ShiftArgs a{};
     a.x = x;
+    a.x_bytes = (uint32_t)x_bytes;
     a.wt = (const uint32_t *)tiled;
     a.negcnt = tiled_negcount(tiled, g);
     a.bias = bias;
@@ -364,15 +372,10 @@ DS_EXPORT int ds_conv2d_tiled_i32(const int32_t *x, const void *tiled, const int
     a.pix_per_img = OH * OW; a.OW = OW;
     a.x_img_stride = C * Hp * Wp; a.x_row_stride = sh * Wp; a.x_col_stride = sw;
     a.y_img_stride = O * OH * OW; a.y_pix_stride = 1; a.y_ch_stride = OH * OW;
+    a.ktab = tiled_ktab(tiled, g);
+    a.x_plane = Hp * Wp; a.x_row = Wp;
     a.nbase = -base;
-    int32_t *ktab = (int32_t *)workspace;
-    a.ktab = ktab;
-    const int Kpad = g.comm * g.num;
-    if (Kpad > 0) {
-        hipLaunchKernelGGL(ktab_kernel, dim3(ceil_div(Kpad, 256)), dim3(256), 0, st, ktab, (int)K,
-                           Kpad, FH, FW, Hp * Wp, Wp);
-    }
-    return dispatch_bits(a, bits, base != 0 || bits == 6, st);
+    return dispatch_bits(a, bits, base != 0 || bits == 6, (hipStream_t)stream);
 }
 
 DS_EXPORT int ds_conv2d_i32(const int32_t *x, const int32_t *w_ref, const int32_t *bias, int32_t *y,
@@ -384,61 +387,52 @@ DS_EXPORT int ds_conv2d_i32(const int32_t *x, const int32_t *w_ref, const int32_
     if (rc) return rc;
     if (Nb < 0 || C < 0 || O < 0 || FH < 1 || FW < 1 || sh < 1 || sw < 1 || Hp < FH || Wp < FW)
         return DS_EINVAL;
-    if ((size_t)C * FH * FW >= (1u << 24)) return DS_ETOOLARGE;
-    const size_t inner = ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits);
+    if ((size_t)C * FH * FW >= (1u << 24) || C >= (1 << 22) || FH > 31 || FW > 31) return DS_ETOOLARGE;
     const size_t need = ds_conv2d_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits);
     if (!workspace || workspace_bytes < need) return DS_EWORKSPACE;
     if (O == 0) return DS_OK;
-    if (!w_ref) return DS_EINVAL;
-    void *tiled = (char *)workspace + inner;
-    rc = launch_tile(w_ref, tiled, O, C * FH * FW, bits, (hipStream_t)stream);
+    if (!w_ref && C > 0) return DS_EINVAL;
+    rc = launch_tile(w_ref, workspace, O, C, FH, FW, bits, (hipStream_t)stream);
     if (rc) return rc;
-    return ds_conv2d_tiled_i32(x, tiled, bias, y, Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits, base,
-                               workspace, inner, stream);
+    return ds_conv2d_tiled_i32(x, workspace, bias, y, Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits, base,
+                               nullptr, 0, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
 // LinearShift
 // ---------------------------------------------------------------------------------------------
 
-namespace ds {
-int launch_transpose(const int32_t *x, int32_t *xT, int M, int K, int ldx, hipStream_t st);
-}
-
 DS_EXPORT size_t ds_linear_tiled_workspace_bytes(int M, int K, int N, int bits)
 {
-    (void)M; (void)N;
-    if (bits < 1 || bits > 6 || K < 0) return 0;
-    const int num = codes_per_word(bits);
-    return align_up((size_t)ceil_div(K, num) * num * 4, 256);
+    (void)M; (void)K; (void)N; (void)bits;
+    return 0;  // the tiled entry point needs no scratch memory
 }
 
 DS_EXPORT size_t ds_linear_workspace_bytes(int M, int K, int N, int bits)
 {
     if (bits < 1 || bits > 6 || M < 0 || K < 0 || N < 0) return 0;
     const size_t ldx = align_up((size_t)M, 64);
-    return ds_linear_tiled_workspace_bytes(M, K, N, bits) + align_up(tiled_geom(N, K, bits).bytes, 256) +
-           align_up(ldx * K * 4, 256);
+    return align_up(tiled_geom(N, K, bits).bytes, 256) + align_up(ldx * K * 4, 256);
 }
 
 DS_EXPORT int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled, const int32_t *bias,
                                   int32_t *y, int M, int K, int N, int bits, int base,
                                   void *workspace, size_t workspace_bytes, ds_stream_t stream)
 {
+    (void)workspace; (void)workspace_bytes;
     int rc = check_common(bits, base);
     if (rc) return rc;
     if (M < 0 || K < 0 || N < 0 || ldx < M) return DS_EINVAL;
     if (M == 0 || N == 0) return DS_OK;
-    if (!xT || !tiled || !y) return DS_EINVAL;
-    if ((size_t)ldx * K * 4 >= kMaxBytes || (size_t)M * N * 4 >= kMaxBytes || K >= (1 << 24))
-        return DS_ETOOLARGE;
-    const size_t need = ds_linear_tiled_workspace_bytes(M, K, N, bits);
-    if (need && (!workspace || workspace_bytes < need)) return DS_EWORKSPACE;
-    hipStream_t st = (hipStream_t)stream;
+    if (!tiled || !y || (!xT && K > 0)) return DS_EINVAL;
+    const size_t x_bytes = (size_t)ldx * K * 4;
+    if (x_bytes >= kMaxBytes || (size_t)M * N * 4 >= kMaxBytes || K >= (1 << 22)) return DS_ETOOLARGE;
     const TiledGeom g = tiled_geom(N, K, bits);
 
+    // a 1x1 "convolution" over K planes of ldx pixels each
     ShiftArgs a{};
     a.x = xT;
+    a.x_bytes = (uint32_t)x_bytes;
     a.wt = (const uint32_t *)tiled;
     a.negcnt = tiled_negcount(tiled, g);
     a.bias = bias;
@@ -447,16 +441,10 @@ DS_EXPORT int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled,
     a.pix_per_img = M; a.OW = M;
     a.x_img_stride = 0; a.x_row_stride = 0; a.x_col_stride = 1;
     a.y_img_stride = 0; a.y_pix_stride = N; a.y_ch_stride = 1;
+    a.ktab = tiled_ktab(tiled, g);
+    a.x_plane = ldx; a.x_row = 1;
     a.nbase = -base;
-    int32_t *ktab = (int32_t *)workspace;
-    a.ktab = ktab;
-    const int Kpad = g.comm * g.num;
-    if (Kpad > 0) {
-        // a 1x1 "filter" over K planes of ldx elements: ktab[k] = k * ldx
-        hipLaunchKernelGGL(ktab_kernel, dim3(ceil_div(Kpad, 256)), dim3(256), 0, st, ktab, K, Kpad, 1,
-                           1, ldx, 0);
-    }
-    return dispatch_bits(a, bits, base != 0 || bits == 6, st);
+    return dispatch_bits(a, bits, base != 0 || bits == 6, (hipStream_t)stream);
 }
 
 DS_EXPORT int ds_linear_i32(const int32_t *x, const int32_t *w_ref, const int32_t *bias, int32_t *y,
@@ -466,7 +454,7 @@ DS_EXPORT int ds_linear_i32(const int32_t *x, const int32_t *w_ref, const int32_
     int rc = check_common(bits, base);
     if (rc) return rc;
     if (M < 0 || K < 0 || N < 0) return DS_EINVAL;
-    if (K >= (1 << 24)) return DS_ETOOLARGE;
+    if (K >= (1 << 22)) return DS_ETOOLARGE;
     const size_t need = ds_linear_workspace_bytes(M, K, N, bits);
     if (!workspace || workspace_bytes < need) return DS_EWORKSPACE;
     if (M == 0 || N == 0) return DS_OK;
@@ -474,15 +462,14 @@ DS_EXPORT int ds_linear_i32(const int32_t *x, const int32_t *w_ref, const int32_
     if (!w_ref && K > 0) return DS_EINVAL;
     const int ldx = (int)align_up((size_t)M, 64);
     if ((size_t)ldx * K * 4 >= kMaxBytes) return DS_ETOOLARGE;
-    const size_t inner = ds_linear_tiled_workspace_bytes(M, K, N, bits);
-    void *tiled = (char *)workspace + inner;
+    void *tiled = workspace;
     int32_t *xT = (int32_t *)((char *)tiled + align_up(tiled_geom(N, K, bits).bytes, 256));
     hipStream_t st = (hipStream_t)stream;
-    rc = launch_tile(w_ref, tiled, N, K, bits, st);
+    rc = launch_tile(w_ref, tiled, N, K, 1, 1, bits, st);
     if (rc) return rc;
     if (K > 0) {
         rc = launch_transpose(x, xT, M, K, ldx, st);
         if (rc) return rc;
     }
-    return ds_linear_tiled_i32(xT, ldx, tiled, bias, y, M, K, N, bits, base, workspace, inner, stream);
+    return ds_linear_tiled_i32(xT, ldx, tiled, bias, y, M, K, N, bits, base, nullptr, 0, stream);
 }

@@ -103,27 +103,29 @@ def compress_sign_and_shift(shift, sign, comp_size, base, bits, row_length, num)
     return out
 
 
-def tile_weights(packed, N, K, bits, base=0):
-    """Reference-layout words [N*comm] -> the library's tiled blob (uint8 tensor)."""
+def tile_weights(packed, N, C, FH, FW, bits, base=0):
+    """Reference-layout words [N*comm] of an [N, C, FH, FW] layer (linear: FH = FW = 1) -> the
+    library's tiled blob (uint8 tensor)."""
     packed = _require_device_i32("packed", packed)
+    K = C * FH * FW
     num = 32 // (bits + 1)
     if packed.numel() != N * ((K + num - 1) // num):
         raise ValueError("packed weight has %d words, expected %d" %
                          (packed.numel(), N * ((K + num - 1) // num)))
     nbytes = _lib.lib().ds_tiled_bytes(N, K, bits)
     blob = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=packed.device)
-    _lib.call("ds_tile_weights_i32", _lib.ptr(packed), _lib.ptr(blob), N, K, int(bits), int(base),
-              _lib.current_stream(packed.device))
+    _lib.call("ds_tile_weights_i32", _lib.ptr(packed), _lib.ptr(blob), N, C, FH, FW, int(bits),
+              int(base), _lib.current_stream(packed.device))
     return blob
 
 
-def _tiled_of(conc_weight, N, K):
+def _tiled_of(conc_weight, N, C, FH=1, FW=1):
     """The tiled blob of a ConcWeight, built once and cached on the object."""
     data = conc_weight.data
-    key = (data.data_ptr(), data._version, N, K, conc_weight.bits, conc_weight.base)
+    key = (data.data_ptr(), data._version, N, C, FH, FW, conc_weight.bits, conc_weight.base)
     cached = getattr(conc_weight, "_tiled", None)
     if cached is None or cached[0] != key:
-        cached = (key, tile_weights(data, N, K, conc_weight.bits, conc_weight.base))
+        cached = (key, tile_weights(data, N, C, FH, FW, conc_weight.bits, conc_weight.base))
         conc_weight._tiled = cached
     return cached[1]
 
@@ -194,7 +196,7 @@ def linear_tiled(xT, M, tiled, bias, N, bits, base=0):
     out = torch.empty([M, N], dtype=torch.int32, device=xT.device)
     L = _lib.lib()
     ws_bytes = L.ds_linear_tiled_workspace_bytes(M, K, N, bits)
-    ws = _workspace(ws_bytes, xT.device)
+    ws = _workspace(ws_bytes, xT.device) if ws_bytes else None
     with _Timed("linear", M, K, N, xT.device):
         _lib.call("ds_linear_tiled_i32", _lib.ptr(xT), ldx, _lib.ptr(tiled), _lib.ptr(bias),
                   _lib.ptr(out), M, K, N, int(bits), int(base), _lib.ptr(ws), ws_bytes,
@@ -240,7 +242,7 @@ def conv2d_tiled(x_padded, tiled, bias, O, kernel_size, stride, bits, base=0):
     out = torch.empty([Nb, O, OH, OW], dtype=torch.int32, device=x_padded.device)
     L = _lib.lib()
     ws_bytes = L.ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits)
-    ws = _workspace(ws_bytes, x_padded.device)
+    ws = _workspace(ws_bytes, x_padded.device) if ws_bytes else None
     with _Timed("conv", Nb * OH * OW, C * FH * FW, O, x_padded.device):
         _lib.call("ds_conv2d_tiled_i32", _lib.ptr(x_padded), _lib.ptr(tiled), _lib.ptr(bias),
                   _lib.ptr(out), Nb, C, Hp, Wp, O, FH, FW, sh, sw, int(bits), int(base),
@@ -277,5 +279,5 @@ def conv2d(input, shift, sign, bias=None, conc_weight=None, stride=1, padding=0,
                   _lib.current_stream(input.device))
     else:
         xp = input
-    tiled = _tiled_of(conc_weight, O, C * FH * FW)
+    tiled = _tiled_of(conc_weight, O, C, FH, FW)
     return conv2d_tiled(xp, tiled, bias, O, (FH, FW), stride, conc_weight.bits, conc_weight.base)

@@ -209,8 +209,8 @@ def conv_kernel_forward(module, input, conc_weight, input_is_fixed=False):
     # round_to_fixed + cast + zero padding in one pass
     xq = kernels.quantize_pad(input, padding, I, Fb, round_to_fixed=True)
     bias = module._fixed_bias.get(module.bias, I, Fb, round_to_fixed=True)
-    K = module.in_channels * module.kernel_size[0] * module.kernel_size[1]
-    tiled = kernels._tiled_of(conc_weight, module.out_channels, K)
+    tiled = kernels._tiled_of(conc_weight, module.out_channels, module.in_channels,
+                              module.kernel_size[0], module.kernel_size[1])
     out = kernels.conv2d_tiled(xq, tiled, bias, module.out_channels, module.kernel_size,
                                module.stride, conc_weight.bits, conc_weight.base)
     return kernels.dequantize(out, Fb)

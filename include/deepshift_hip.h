@@ -56,13 +56,15 @@ int ds_pack_i32(const int32_t *s, const int32_t *sign, int32_t *out, int O, int 
 size_t ds_tiled_bytes(int N, int K, int bits);
 
 /* Re-lays reference-format words w_ref[N][comm] (the output of ds_pack_i32 / the reference's
- * ConcWeight.data, utils.py:54-88) into the private, coalesced layout the compute kernels read:
- * words grouped [ceil(N/32)*2][comm][16] so that the 16 words a wavefront decodes together are
- * one 64-byte scalar load, sign bit inverted (1 = negative), tail codes neutralised, followed
- * by a per-channel count of negative codes that the kernels fold into the bias.  No
- * counterpart in the reference (it consumes the row-major words directly, shift.cu:84). */
-int ds_tile_weights_i32(const int32_t *w_ref, void *tiled, int N, int K, int bits, int base,
-                        ds_stream_t stream);
+ * ConcWeight.data, utils.py:54-88) of an [N][C][FH][FW] layer (a linear layer is C = K,
+ * FH = FW = 1) into the private layout the compute kernels read: words grouped
+ * [ceil(N/32)][comm][32] so that the words a wavefront decodes together are consecutive scalar
+ * loads, sign bit inverted (1 = negative), tail codes neutralised; then a per-channel count of
+ * negative codes that the kernels fold into the bias; then a table that maps the reduction index
+ * k to its (ic, fh, fw).  Limits: C < 2^22, FH, FW <= 31.  No counterpart in the reference (it
+ * consumes the row-major words directly, shift.cu:84). */
+int ds_tile_weights_i32(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW, int bits,
+                        int base, ds_stream_t stream);
 
 /* ---- LinearShift ----------------------------------------------------------------------- */
 

@@ -39,11 +39,13 @@ def test_version_and_status_strings():
 def test_size_queries():
     L = _lib.lib()
     # bits 4 -> 6 codes per word; N=64,K=576 -> comm 96; 64 channels = 4 tiles of 16 words
-    assert L.ds_tiled_bytes(64, 576, 4) == 4 * 96 * 16 * 4 + 64 * 4
+    # words [2 tiles][96][32] + negcount[64] + k table [(96+1)*6], each part padded to 256 bytes
+    assert L.ds_tiled_bytes(64, 576, 4) == 2 * 96 * 32 * 4 + 256 + 2560
     # channels are padded to a multiple of 32
-    assert L.ds_tiled_bytes(10, 6, 4) == 256 + 32 * 4
+    assert L.ds_tiled_bytes(10, 6, 4) == 256 + 256 + 256
     assert L.ds_tiled_bytes(64, 576, 7) == 0
-    assert L.ds_conv2d_tiled_workspace_bytes(1, 64, 58, 58, 64, 3, 3, 1, 1, 4) == 576 * 4
+    assert L.ds_conv2d_tiled_workspace_bytes(1, 64, 58, 58, 64, 3, 3, 1, 1, 4) == 0
+    assert L.ds_conv2d_workspace_bytes(1, 64, 58, 58, 64, 3, 3, 1, 1, 4) == L.ds_tiled_bytes(64, 576, 4)
     assert L.ds_linear_workspace_bytes(64, 784, 512, 6) > 64 * 784 * 4
 
 
