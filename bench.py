@@ -177,6 +177,26 @@ def config2(device, reps=10):
     return out
 
 
+def pmc_target(device):
+    """Counter targets for `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`: a plain copy of 64 MiB (reads
+    64 MiB, writes 64 MiB: the scale of the counters) and the dominant shift-kernel launch."""
+    from deepshift_amd import _lib, kernels, utils
+    g = torch.Generator().manual_seed(0)
+    n = 16 * 1024 * 1024
+    src = torch.randint(0, 2 ** 20, (n,), generator=g, dtype=torch.int32).to(device)
+    dst = torch.empty_like(src)
+    x = torch.randint(0, 2 ** 20, (BATCH, 64, 58, 58), generator=g, dtype=torch.int32).to(device)
+    shift = torch.randint(-15, 1, (64, 64, 3, 3), generator=g).float()
+    sign = (torch.randint(0, 2, (64, 64, 3, 3), generator=g) * 2 - 1).float()
+    cw = utils.compress_bits(shift, sign)
+    tiled = kernels._tiled_of(cw, 64, 64, 3, 3)
+    torch.cuda.synchronize()
+    for _ in range(3):
+        _lib.call("ds_copy_i32", _lib.ptr(src), _lib.ptr(dst), n, _lib.current_stream(device))
+        kernels.conv2d_tiled(x, tiled, None, 64, (3, 3), (1, 1), cw.bits, cw.base)
+    torch.cuda.synchronize()
+
+
 def cpu_baseline(shapes):
     """The oracle's restatement of the reference CPU kernel (shift_cpu.cpp loop nests, batch rows /
     images split over threads) on every shift layer of ResNet-18 at a reduced batch."""
@@ -224,6 +244,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--layers", action="store_true", help="per-layer table on stderr")
+    ap.add_argument("--resnet-only", action="store_true",
+                    help="skip config 2 and the VALU calibration (clean kernel-trace profiles)")
+    ap.add_argument("--pmc-target", action="store_true",
+                    help="only launch the counter targets: a 64 MiB copy kernel and the dominant shift "
+                         "kernel (ResNet-18 layer1 3x3 conv, batch 64), 3 times each")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path "
@@ -231,6 +256,10 @@ def main():
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a ROCm GPU")
     device = torch.device("cuda:0")
+
+    if args.pmc_target:
+        pmc_target(device)
+        return
 
     from deepshift_amd import workloads
     model, x, n_conv = build_model(device)
@@ -257,8 +286,8 @@ def main():
                 L["name"], L["M"], L["K"], L["N"], L["seconds"] * 1e6, p / L["seconds"] / 1e12,
                 100 * p / L["seconds"] / PEAK_PAIRS, 100 * L["bytes"] / L["seconds"] / HBM_PEAK))
 
-    peak_cal = calibrate_valu(device)
-    cfg2 = config2(device)
+    peak_cal = None if args.resnet_only else calibrate_valu(device)
+    cfg2 = None if args.resnet_only else config2(device)
     result = {
         "metric": "resnet18_bs64_images_per_s",
         "value": BATCH / sec_per_step,
@@ -288,14 +317,14 @@ def main():
             "frac": pairs / kernel_s / PEAK_PAIRS,
             "traffic": None,
             "avg_launch_us": kernel_s / len(layers) * 1e6,
-            "peak_calibrated": peak_cal / 1e12,
-            "frac_of_calibrated": pairs / kernel_s / peak_cal,
+            "peak_calibrated": peak_cal / 1e12 if peak_cal else None,
+            "frac_of_calibrated": pairs / kernel_s / peak_cal if peak_cal else None,
             "hbm_achieved_GBps": alg_bytes / kernel_s / 1e9,
             "hbm_frac": alg_bytes / kernel_s / HBM_PEAK,
             "algorithmic_bytes_per_step": alg_bytes,
         },
         "config2": cfg2,
-        "shift_gemm_gops": cfg2["gemm_4096"]["gops"],
+        "shift_gemm_gops": cfg2["gemm_4096"]["gops"] if cfg2 else None,
     }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(workloads.shift_layer_shapes(workloads.ResNet18(), CHW, 1))

@@ -265,8 +265,9 @@ static TileChoice choose_tile(const ShiftArgs &a)
 {
     TileChoice c{2, 32, 1};
     if (a.N <= 16) { c.R = 4; c.J = 16; }                   // few channels: more pixels per lane
-    else if (a.M <= 64 || a.OW <= 8) { c.R = 1; c.J = 32; } // few / scattered pixels
+    else if (a.M <= 64) { c.R = 1; c.J = 32; }              // a single wave of rows
     else if (a.comm <= 32 && a.N >= 64) { c.R = 4; c.J = 16; }  // short reduction (e.g. 7x7x3 stem)
+    else if (a.x_col_stride > 1) { c.R = 3; c.J = 16; }     // strided pixels: half-used cache lines
     const long tiles = (long)ceil_div(a.M, c.R * kWave) * ceil_div(a.N, c.J);
     const long simds = 1024;
     const double per_simd = (double)tiles / simds;
@@ -275,7 +276,7 @@ static TileChoice choose_tile(const ShiftArgs &a)
     long want = (24 * simds + tiles / 2) / tiles;
     const long max_by_k = a.comm / 12 > 0 ? a.comm / 12 : 1;
     if (want > max_by_k) want = max_by_k;
-    if (want > 64) want = 64;
+    if (want > 32) want = 32;
     if (want < 1) want = 1;
     c.nsplit = (int)want;
     return c;
