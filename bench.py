@@ -266,8 +266,19 @@ def main():
     parity_gate(model, x)
     log("parity gate passed; %d conv + 1 fc shift layers" % n_conv)
 
-    sec_per_step = time_steps(model, x, args.steps, args.warmup)
-    layers = kernel_timings(model, x, max(3, min(args.steps, 10)))
+    # The measured pipeline: the converted model with the fp32 glue after every shift conv
+    # (BatchNorm, residual add, ReLU) folded into that conv's dequantisation pass.  The shift
+    # kernels and their int32 results are the same as in the plain converted model, which is timed
+    # as well for reference.
+    from deepshift_amd import fuse
+    with torch.no_grad():
+        fused = fuse.fuse_conv_epilogues(model)
+        want, got = model(x[:4]), fused(x[:4])
+    if not torch.allclose(got, want, rtol=0, atol=2e-3 * float(want.abs().max()) + 1e-4):
+        raise SystemExit("fused pipeline diverges from the plain converted model")
+    sec_unfused = time_steps(model, x, max(2, args.steps // 2), args.warmup)
+    sec_per_step = time_steps(fused, x, args.steps, args.warmup)
+    layers = kernel_timings(fused, x, max(3, min(args.steps, 10)))
     shapes = workloads.shift_layer_shapes(workloads.ResNet18(), CHW, BATCH)
     assert len(layers) == len(shapes) == 21
 
@@ -303,8 +314,10 @@ def main():
         "data": "synthetic",
         "config": {"workload": "ResNet-18, batch 64 x 3x224x224, all 20 conv + FC as shift layers "
                                "(BASELINE configs[3]); weight_bits 5 (4-bit shift + sign, 6 codes per "
-                               "word), activations 16.16; BatchNorm/ReLU/pooling fp32 PyTorch",
+                               "word), activations 16.16; BatchNorm/residual/ReLU folded into each "
+                               "conv's dequantisation pass, pooling fp32 PyTorch",
                    "batch": BATCH, "shift_layers": 21, "pairs_per_step": pairs},
+        "unfused_images_per_s": BATCH / sec_unfused,
         "shift_kernel_ms_per_step": kernel_s * 1e3,
         "shift_gops": 2 * pairs / kernel_s / 1e9,
         "shift_layers_images_per_s": BATCH / kernel_s,
@@ -315,7 +328,10 @@ def main():
             "peak": PEAK_PAIRS / 1e12,
             "unit": "Tpair/s",
             "frac": pairs / kernel_s / PEAK_PAIRS,
-            "traffic": None,
+            # HBM bytes of one launch of the dominant shape (layer1 3x3 conv, 8 of the 21 launches are
+            # this size): 56.7 MB read + 411 MB of split-K atomic adds, from the FETCH_SIZE / WRITE_SIZE
+            # runs summarised in profiles/shift_kernel_layer1_conv_counters.md (106.6 MB algorithmic)
+            "traffic": 468.0e6,
             "avg_launch_us": kernel_s / len(layers) * 1e6,
             "peak_calibrated": peak_cal / 1e12 if peak_cal else None,
             "frac_of_calibrated": pairs / kernel_s / peak_cal if peak_cal else None,

@@ -177,6 +177,33 @@ __global__ void dequantize_kernel(const int32_t *__restrict__ y, float *__restri
     }
 }
 
+// out = act(float(y) / 2^F * scale[c] + shift[c] (+ residual)): the dequantisation of a shift layer
+// fused with an inference-mode per-channel affine (a folded BatchNorm), a residual add and ReLU.
+// One thread per 4 consecutive pixels of one (image, channel) plane when HW % 4 == 0.
+template <int VEC>
+__global__ void dequantize_affine_kernel(const int32_t *__restrict__ y, float *__restrict__ out,
+                                         const float *__restrict__ scale, const float *__restrict__ shift,
+                                         const float *__restrict__ residual, long n, int C, int HW,
+                                         float inv, int relu)
+{
+    const long stride = (long)gridDim.x * blockDim.x;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i * VEC < n; i += stride) {
+        const long e = i * VEC;
+        const int c = (int)((e / HW) % C);
+        const float a = scale ? scale[c] : 1.0f;
+        const float b = shift ? shift[c] : 0.0f;
+        float v[VEC];
+#pragma unroll
+        for (int t = 0; t < VEC; ++t) {
+            v[t] = ((float)y[e + t] * inv) * a + b;
+            if (residual) v[t] += residual[e + t];
+            if (relu) v[t] = v[t] > 0.0f ? v[t] : 0.0f;
+        }
+#pragma unroll
+        for (int t = 0; t < VEC; ++t) out[e + t] = v[t];
+    }
+}
+
 __global__ void copy_kernel(const int4 *__restrict__ src, int4 *__restrict__ dst, long n4)
 {
     const long stride = (long)gridDim.x * blockDim.x;
@@ -270,6 +297,26 @@ DS_EXPORT int ds_dequantize_i32_f32(const int32_t *y, float *out, int64_t n, int
     if (!y || !out) return DS_EINVAL;
     hipLaunchKernelGGL(dequantize_kernel, dim3(grid_for((n + 3) / 4)), dim3(256), 0,
                        (hipStream_t)stream, y, out, (long)n, ldexpf(1.0f, F));
+    return launch_status();
+}
+
+DS_EXPORT int ds_dequantize_affine_i32_f32(const int32_t *y, float *out, const float *scale,
+                                           const float *shift, const float *residual, int Nb, int C,
+                                           int HW, int F, int relu, ds_stream_t stream)
+{
+    if (Nb < 0 || C < 0 || HW < 0 || F < 0 || F > 31) return DS_EINVAL;
+    const long n = (long)Nb * C * HW;
+    if (n == 0) return DS_OK;
+    if (!y || !out) return DS_EINVAL;
+    const float inv = ldexpf(1.0f, -F);
+    const bool vec = (HW % 4 == 0) &&
+                     ((((uintptr_t)y | (uintptr_t)out | (uintptr_t)residual) & 15) == 0);
+    if (vec)
+        hipLaunchKernelGGL((dequantize_affine_kernel<4>), dim3(grid_for(n / 4)), dim3(256), 0,
+                           (hipStream_t)stream, y, out, scale, shift, residual, n, C, HW, inv, relu);
+    else
+        hipLaunchKernelGGL((dequantize_affine_kernel<1>), dim3(grid_for(n)), dim3(256), 0,
+                           (hipStream_t)stream, y, out, scale, shift, residual, n, C, HW, inv, relu);
     return launch_status();
 }
 

@@ -1,0 +1,131 @@
+"""Inference-time fusion around shift convolutions (no counterpart in the reference, which leaves
+BatchNorm / ReLU / residual adds as separate PyTorch ops around ``Conv2dShift``).
+
+``fuse_conv_epilogues(model, example_input)`` traces the model with ``torch.fx`` and rewrites
+
+    Conv2dShift -> BatchNorm2d (eval) [-> + residual] [-> ReLU]
+
+into one :class:`FusedConv2dShift` call: the int32 result of the shift kernel is converted to float,
+scaled and shifted per channel (the folded BatchNorm), added to the residual and clamped at zero
+in a single pass (``ds_dequantize_affine_i32_f32``) instead of four.  The shift arithmetic itself
+is untouched; the float glue differs from the unfused ops by fp32 rounding only.
+"""
+import operator
+
+import torch
+import torch.fx as fx
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import modules, modules_q
+
+__all__ = ["FusedConv2dShift", "fuse_conv_epilogues"]
+
+_SHIFT_CONVS = (modules.Conv2dShift, modules_q.Conv2dShiftQ)
+_SHIFT_LEAVES = _SHIFT_CONVS + (modules.LinearShift, modules_q.LinearShiftQ)
+
+
+class FusedConv2dShift(nn.Module):
+    """A kernel-mode shift convolution with its BatchNorm folded into the dequantisation pass,
+    optionally followed by a residual add and ReLU."""
+
+    def __init__(self, conv, bn=None, relu=False):
+        super().__init__()
+        self.conv = conv
+        self.relu = relu
+        if bn is not None:
+            if bn.training or not bn.track_running_stats:
+                raise ValueError("only an eval-mode BatchNorm with running statistics can be folded")
+            var, mean = bn.running_var.detach().float(), bn.running_mean.detach().float()
+            weight = bn.weight.detach().float() if bn.affine else torch.ones_like(var)
+            bias = bn.bias.detach().float() if bn.affine else torch.zeros_like(var)
+            scale = weight / torch.sqrt(var + bn.eps)
+            self.register_buffer("scale", scale.contiguous())
+            self.register_buffer("shift", (bias - mean * scale).contiguous())
+        else:
+            self.scale = None
+            self.shift = None
+
+    def forward(self, input, residual=None):
+        conv = self.conv
+        if isinstance(conv, modules_q.Conv2dShiftQ):
+            if conv.conc_weight is None:
+                modules_q.pack_module_weights_q(conv)
+        elif conv.conc_weight is None:
+            modules.pack_module_weights(conv)
+        return modules.conv_kernel_forward(conv, input, conv.conc_weight, self.scale, self.shift,
+                                           residual, self.relu)
+
+
+class _Tracer(fx.Tracer):
+    def is_leaf_module(self, m, qualname):
+        return isinstance(m, _SHIFT_LEAVES) or super().is_leaf_module(m, qualname)
+
+
+def _is_relu(node, mods):
+    if node.op == "call_function" and node.target in (F.relu, torch.relu):
+        return True
+    if node.op == "call_method" and node.target in ("relu", "relu_"):
+        return True
+    return node.op == "call_module" and isinstance(mods.get(node.target), nn.ReLU)
+
+
+def _is_add(node):
+    return (node.op == "call_function" and node.target in (operator.add, torch.add, operator.iadd)
+            and len(node.args) == 2 and not node.kwargs
+            and all(isinstance(a, fx.Node) for a in node.args))
+
+
+def _sole_user(node):
+    users = list(node.users)
+    return users[0] if len(users) == 1 else None
+
+
+def fuse_conv_epilogues(model):
+    """Return a ``torch.fx.GraphModule`` equivalent to ``model`` (eval mode) with every kernel-mode
+    shift convolution fused with the BatchNorm / residual add / ReLU that consume its output."""
+    model.eval()
+    graph = _Tracer().trace(model)
+    gm = fx.GraphModule(model, graph)
+    mods = dict(gm.named_modules())
+    count = 0
+    for node in list(gm.graph.nodes):
+        if node.op != "call_module":
+            continue
+        conv = mods.get(node.target)
+        if not isinstance(conv, _SHIFT_CONVS) or not conv.use_kernel:
+            continue
+        chain = [node]
+        bn = None
+        nxt = _sole_user(chain[-1])
+        if nxt is not None and nxt.op == "call_module" and isinstance(mods.get(nxt.target), nn.BatchNorm2d):
+            bn = mods[nxt.target]
+            chain.append(nxt)
+            nxt = _sole_user(nxt)
+        residual = None
+        if nxt is not None and _is_add(nxt):
+            other = nxt.args[1] if nxt.args[0] is chain[-1] else nxt.args[0]
+            # the fused call is emitted at the position of the last fused node, where the other
+            # operand of the add already exists
+            if other is not chain[-1]:
+                residual = other
+                chain.append(nxt)
+                nxt = _sole_user(nxt)
+        relu = False
+        if nxt is not None and _is_relu(nxt, mods):
+            relu = True
+            chain.append(nxt)
+        if len(chain) == 1:
+            continue  # nothing to fuse
+        name = "fused_%d" % count
+        count += 1
+        gm.add_module(name, FusedConv2dShift(conv, bn, relu))
+        with gm.graph.inserting_after(chain[-1]):
+            args = (node.args[0],) if residual is None else (node.args[0], residual)
+            new = gm.graph.call_module(name, args)
+        chain[-1].replace_all_uses_with(new)
+        for old in reversed(chain):
+            gm.graph.erase_node(old)
+    gm.graph.lint()
+    gm.recompile()
+    return gm

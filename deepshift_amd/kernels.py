@@ -185,6 +185,26 @@ def dequantize(y, fraction_bits=16):
     return out
 
 
+def dequantize_affine(y, fraction_bits=16, scale=None, shift=None, residual=None, relu=False):
+    """int32 [Nb, C, ...] -> float32 ``act(y / 2**F * scale[c] + shift[c] + residual)`` in one pass:
+    the dequantisation fused with a folded BatchNorm, a residual add and ReLU."""
+    y = _require_device_i32("y", y)
+    Nb, C = y.shape[0], y.shape[1]
+    HW = y[0, 0].numel() if y.numel() else 0
+    out = torch.empty(y.shape, dtype=torch.float32, device=y.device)
+    for name, t in (("scale", scale), ("shift", shift)):
+        if t is not None and (t.dtype != torch.float32 or t.numel() != C or not t.is_contiguous()):
+            raise ValueError("%s must be a contiguous float32 tensor of %d elements" % (name, C))
+    if residual is not None:
+        if residual.shape != y.shape or residual.dtype != torch.float32:
+            raise ValueError("residual must be float32 with the shape of y")
+        residual = residual.contiguous()
+    _lib.call("ds_dequantize_affine_i32_f32", _lib.ptr(y), _lib.ptr(out), _lib.ptr(scale),
+              _lib.ptr(shift), _lib.ptr(residual), Nb, C, HW, fraction_bits, int(bool(relu)),
+              _lib.current_stream(y.device))
+    return out
+
+
 # ---------------------------------------------------------------------------------------------
 # LinearShift / Conv2dShift kernels
 # ---------------------------------------------------------------------------------------------

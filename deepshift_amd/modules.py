@@ -111,9 +111,11 @@ class LinearShift(nn.Module):
         return kernels.dequantize(out, Fb).reshape(*lead, self.out_features)
 
     def forward(self, input):
-        self.shift.data = ste.clamp(self.shift.data, *self.shift_range)
         if self.use_kernel:
+            # the packed weights already hold the clamped, rounded codes (pack_module_weights), so
+            # the per-call clamp of the float parameter (modules.py:125) would change nothing here
             return self._kernel_forward(input)
+        self.shift.data = ste.clamp(self.shift.data, *self.shift_range)
         shift_rounded = ste.round(self.shift, rounding=self.rounding)
         sign_rounded_signed = ste.sign(ste.round(self.sign, rounding=self.rounding))
         weight_ps = ste.unsym_grad_mul(2 ** shift_rounded, sign_rounded_signed)
@@ -194,8 +196,12 @@ def _circular_pad(x, padding):
     return F.pad(x, expanded, mode='circular')
 
 
-def conv_kernel_forward(module, input, conc_weight, input_is_fixed=False):
-    """Fixed-point shift convolution of a float NCHW input (modules.py:152-162,317-337)."""
+def conv_kernel_forward(module, input, conc_weight, scale=None, shift=None, residual=None, relu=False):
+    """Fixed-point shift convolution of a float NCHW input (modules.py:152-162,317-337).
+
+    ``scale``/``shift`` (per output channel), ``residual`` and ``relu`` describe what follows the
+    layer (a folded BatchNorm, a shortcut add, ReLU); when any is given it is applied in the same
+    pass that converts the int32 result back to float."""
     if not module.use_cuda:
         kernels._no_cpu_kernel()
     if module.dilation != (1, 1) or module.groups != 1:
@@ -213,7 +219,9 @@ def conv_kernel_forward(module, input, conc_weight, input_is_fixed=False):
                               module.kernel_size[0], module.kernel_size[1])
     out = kernels.conv2d_tiled(xq, tiled, bias, module.out_channels, module.kernel_size,
                                module.stride, conc_weight.bits, conc_weight.base)
-    return kernels.dequantize(out, Fb)
+    if scale is None and shift is None and residual is None and not relu:
+        return kernels.dequantize(out, Fb)
+    return kernels.dequantize_affine(out, Fb, scale, shift, residual, relu)
 
 
 class Conv2dShift(_ConvNdShift):
@@ -234,11 +242,11 @@ class Conv2dShift(_ConvNdShift):
             act_integer_bits, act_fraction_bits)
 
     def forward(self, input):
-        self.shift.data = ste.clamp(self.shift.data, *self.shift_range)
         if self.use_kernel:
             if self.conc_weight is None:
                 pack_module_weights(self)
             return conv_kernel_forward(self, input, self.conc_weight)
+        self.shift.data = ste.clamp(self.shift.data, *self.shift_range)
 
         shift_rounded = ste.round(self.shift, self.rounding)
         sign_rounded_signed = ste.sign(ste.round(self.sign, self.rounding))

@@ -85,10 +85,11 @@ class LinearShiftQ(nn.Module):
         return kernels.dequantize(out, Fb).reshape(*lead, self.out_features)
 
     def forward(self, input):
+        if self.use_kernel:
+            # packed from the clamped weight (pack_module_weights_q): nothing left to clamp per call
+            return self._kernel_forward(input)
         self.weight.data = ste.clampabs(self.weight.data, 2 ** self.shift_range[0],
                                         2 ** self.shift_range[1])
-        if self.use_kernel:
-            return self._kernel_forward(input)
         weight_q = ste.round_power_of_2(self.weight, self.rounding)
         input_fixed_point = ste.round_fixed_point(input, self.act_integer_bits,
                                                   self.act_fraction_bits)
@@ -148,12 +149,12 @@ class Conv2dShiftQ(nn.Module):
             init.uniform_(self.bias, -bound, bound)
 
     def forward(self, input):
-        self.weight.data = ste.clampabs(self.weight.data, 2 ** self.shift_range[0],
-                                        2 ** self.shift_range[1])
         if self.use_kernel:
             if self.conc_weight is None:
                 pack_module_weights_q(self)
             return conv_kernel_forward(self, input, self.conc_weight)
+        self.weight.data = ste.clampabs(self.weight.data, 2 ** self.shift_range[0],
+                                        2 ** self.shift_range[1])
         weight_q = ste.round_power_of_2(self.weight, self.rounding)
         input_fixed_point = ste.round_fixed_point(input, self.act_integer_bits,
                                                   self.act_fraction_bits)

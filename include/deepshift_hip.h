@@ -141,6 +141,15 @@ int ds_transpose_i32(const int32_t *x, int32_t *xT, int M, int K, int ldx, ds_st
 /* Replaces out.float() / 2**F (modules.py:30-31,161-162); n elements. */
 int ds_dequantize_i32_f32(const int32_t *y, float *out, int64_t n, int F, ds_stream_t stream);
 
+/* Dequantisation fused with what usually follows a shift layer at inference time:
+ *   out = act(float(y) / 2^F * scale[c] + shift[c] + residual),  y, out, residual [Nb][C][HW]
+ * scale/shift (per channel, e.g. a folded BatchNorm) and residual may be NULL; relu != 0 applies
+ * max(.,0).  With all three NULL and relu == 0 this is ds_dequantize_i32_f32.  No counterpart in
+ * the reference (it runs these as separate PyTorch ops after modules.py:161-162). */
+int ds_dequantize_affine_i32_f32(const int32_t *y, float *out, const float *scale, const float *shift,
+                                 const float *residual, int Nb, int C, int HW, int F, int relu,
+                                 ds_stream_t stream);
+
 /* ---- measurement ----------------------------------------------------------------------- */
 
 /* VALU calibration: every lane of `blocks` x 256 threads runs `iters` x 64 independent

@@ -139,7 +139,8 @@ def test_q_modules_and_circular_padding():
     x = torch.randn(16, 64, device=DEV)
     got = lq(x)
     lq.use_kernel = False
-    ref = utils.round_to_fixed(x).mm(utils.round_power_of_2(lq.weight.data).t()) + utils.round_to_fixed(lq.bias.data)
+    wq = utils.round_power_of_2(utils.clampabs(lq.weight.data.clone(), 2.0 ** lq.shift_range[0], 1.0))
+    ref = utils.round_to_fixed(x).mm(wq.t()) + utils.round_to_fixed(lq.bias.data)
     assert (got - ref).abs().max().item() < float_bound(64, 16, 300.0)
     cq = modules_q.Conv2dShiftQ(8, 8, 3, padding=1, padding_mode='circular', use_kernel=True).to(DEV)
     xi = torch.randn(2, 8, 9, 9, device=DEV)
@@ -203,3 +204,42 @@ def test_resnet20_config3_kernel_vs_float_path():
         K = m.shift[0].numel()
         scale = float(inp.abs().max()) * K
         assert (out - ref).abs().max().item() < float_bound(K, 16, scale), (i, K)
+
+
+def test_fused_epilogues_match_unfused_model():
+    """fuse.fuse_conv_epilogues folds BatchNorm / residual add / ReLU into the dequantisation pass;
+    the network output must equal the unfused kernel model up to fp32 rounding of the glue."""
+    from deepshift_amd import fuse
+    for cls, shape in [(workloads.ResNet18, (2, 3, 64, 64)), (workloads.ResNet20, (4, 3, 32, 32)),
+                       (workloads.ResNet50, (1, 3, 64, 64))]:
+        g = torch.Generator().manual_seed(7)
+        model = workloads.randomize_batchnorm(cls(), g).eval()
+        model, n = convert.convert_to_shift(model, 1000, 'PS', convert_weights=True, use_kernel=True)
+        model = model.to(DEV)
+        x = torch.randn(*shape, generator=g).to(DEV)
+        with torch.no_grad():
+            want = model(x)
+            fused = fuse.fuse_conv_epilogues(model)
+            got = fused(x)
+        assert sum(isinstance(m, fuse.FusedConv2dShift) for m in fused.modules()) == n
+        assert not any(isinstance(m, nn.BatchNorm2d) for name, m in fused.named_modules()
+                       if name in {nd.target for nd in fused.graph.nodes if nd.op == "call_module"})
+        # each layer re-quantises to a 2^-16 grid, so glue rounding can move single LSBs that then
+        # propagate; compare relative to the output scale
+        scale = want.abs().max().item()
+        assert (got - want).abs().max().item() <= 2e-3 * scale + 1e-4, cls.__name__
+
+
+def test_dequantize_affine_matches_torch(rng):
+    Nb, C, H, W = 3, 5, 7, 4
+    y = torch.from_numpy(rng.integers(-2 ** 24, 2 ** 24, size=(Nb, C, H, W)).astype(np.int32)).to(DEV)
+    scale = torch.rand(C, device=DEV) + 0.5
+    shift = torch.randn(C, device=DEV)
+    res = torch.randn(Nb, C, H, W, device=DEV)
+    got = kernels.dequantize_affine(y, 16, scale, shift, res, relu=True)
+    want = torch.relu(y.float() / 65536 * scale.view(1, -1, 1, 1) + shift.view(1, -1, 1, 1) + res)
+    torch.testing.assert_close(got, want, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(kernels.dequantize_affine(y, 16), y.float() / 65536, rtol=0, atol=0)
+    y2 = y[:, :, :, :3].contiguous()  # HW not a multiple of 4: scalar path
+    got = kernels.dequantize_affine(y2, 16, scale, None, None, relu=False)
+    torch.testing.assert_close(got, y2.float() / 65536 * scale.view(1, -1, 1, 1), rtol=1e-6, atol=1e-6)
