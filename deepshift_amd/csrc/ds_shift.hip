@@ -214,6 +214,156 @@ __global__ __launch_bounds__(256) void shift_kernel(const ShiftArgs p)
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Shift-plane variant of the kernel (R = 4 pixels x J = 32 channels per lane, fields of <= 4 bits).
+//
+// For one reduction index k and one pixel the 32 channels only ever ask for the 2^BITS values
+// x >> 0 .. x >> (2^BITS - 1).  The kernel computes these "planes" once (2^BITS vector shifts per
+// pixel row), keeps them in consecutive VGPRs, and lets every (k, channel) term pick its plane by
+// VGPR-relative addressing: the scalar ALU writes the code's shift field to M0
+// (s_set_gpr_idx_idx) and the single vector instruction v_xad_u32 acc, plane[M0], mask, acc
+// does the sign flip and the accumulation.  A term costs 1 + 2^BITS/32 vector instructions
+// (1.5 for 4-bit fields, 1.125 for 2-bit fields) instead of 2.  Relative addressing needs a fixed
+// register map, so the main loop is one generated inline-asm block (gen_planes_asm.py ->
+// ds_planes_asm.inc); tile mapping, the partial last K group and the epilogue stay C++.
+#include "ds_planes_asm.inc"
+
+typedef int32_t v16i __attribute__((ext_vector_type(16)));
+typedef int32_t v4i __attribute__((ext_vector_type(4)));
+
+#define DS_PLANES_OPERANDS                                                                        \
+    : "+{v[96:111]}"(a[0]), "+{v[112:127]}"(a[1]), "+{v[128:143]}"(a[2]), "+{v[144:159]}"(a[3]),  \
+      "+{v[160:175]}"(a[4]), "+{v[176:191]}"(a[5]), "+{v[192:207]}"(a[6]), "+{v[208:223]}"(a[7])  \
+    : "v"(xoff[0]), "v"(xoff[1]), "v"(xoff[2]), "v"(xoff[3]), "s"(rsrc), "s"(wptr), "s"(kptr),    \
+      "s"(groups), "s"(x_plane), "s"(x_row)
+
+template <int BITS>
+__device__ __forceinline__ void planes_main_loop(v16i (&a)[8], const uint32_t (&xoff)[4], v4i rsrc,
+                                                 const uint32_t *wptr, const uint32_t *kptr, int groups,
+                                                 int x_plane, int x_row);
+template <>
+__device__ __forceinline__ void planes_main_loop<1>(v16i (&a)[8], const uint32_t (&xoff)[4], v4i rsrc,
+                                                    const uint32_t *wptr, const uint32_t *kptr,
+                                                    int groups, int x_plane, int x_row)
+{
+    asm volatile(DS_PLANES_ASM_B1 DS_PLANES_OPERANDS : DS_PLANES_CLOBBERS_B1);
+}
+template <>
+__device__ __forceinline__ void planes_main_loop<2>(v16i (&a)[8], const uint32_t (&xoff)[4], v4i rsrc,
+                                                    const uint32_t *wptr, const uint32_t *kptr,
+                                                    int groups, int x_plane, int x_row)
+{
+    asm volatile(DS_PLANES_ASM_B2 DS_PLANES_OPERANDS : DS_PLANES_CLOBBERS_B2);
+}
+template <>
+__device__ __forceinline__ void planes_main_loop<3>(v16i (&a)[8], const uint32_t (&xoff)[4], v4i rsrc,
+                                                    const uint32_t *wptr, const uint32_t *kptr,
+                                                    int groups, int x_plane, int x_row)
+{
+    asm volatile(DS_PLANES_ASM_B3 DS_PLANES_OPERANDS : DS_PLANES_CLOBBERS_B3);
+}
+template <>
+__device__ __forceinline__ void planes_main_loop<4>(v16i (&a)[8], const uint32_t (&xoff)[4], v4i rsrc,
+                                                    const uint32_t *wptr, const uint32_t *kptr,
+                                                    int groups, int x_plane, int x_row)
+{
+    asm volatile(DS_PLANES_ASM_B4 DS_PLANES_OPERANDS : DS_PLANES_CLOBBERS_B4);
+}
+
+template <int BITS>
+__global__ __launch_bounds__(256) void shift_planes_kernel(const ShiftArgs p)
+{
+    constexpr int NUM = 32 / (BITS + 1);
+    constexpr int R = 4, J = 32;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int bid = blockIdx.x;
+    const int tile = (bid & 7) * p.blocks_per_xcd + (bid >> 3);
+    if (tile >= p.tiles_m4 * p.tiles_n) return;
+    const int ntile = tile % p.tiles_n;
+    const int mtile = (tile / p.tiles_n) * 4 + wave;
+    const int m0 = mtile * (R * kWave);
+    if (m0 >= p.M) return;
+
+    uint32_t xoff[R], yoff[R];
+    bool live[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        int m = m0 + r * kWave + lane;
+        live[r] = m < p.M;
+        if (!live[r]) m = p.M - 1;
+        const int img = m / p.pix_per_img;
+        const int rem = m - img * p.pix_per_img;
+        const int oh = rem / p.OW;
+        const int ow = rem - oh * p.OW;
+        xoff[r] = 4u * (uint32_t)(img * p.x_img_stride + oh * p.x_row_stride + ow * p.x_col_stride);
+        yoff[r] = 4u * (uint32_t)(img * p.y_img_stride + rem * p.y_pix_stride);
+    }
+
+    const int g_begin = blockIdx.y * p.groups_per_split;
+    int g_end = g_begin + p.groups_per_split;
+    if (g_end > p.comm) g_end = p.comm;
+    const int full_groups = p.K / NUM;
+    const int g_full_end = g_end < full_groups ? g_end : full_groups;
+    const uint32_t *wrow = p.wt + (size_t)ntile * p.comm * kTileWords;
+
+    v16i a[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) a[i] = (v16i)(0);
+    if (g_begin < g_full_end) {
+        const uint64_t xaddr = (uint64_t)p.x;
+        v4i rsrc;
+        rsrc.x = (int32_t)(uint32_t)xaddr;
+        rsrc.y = (int32_t)(uint32_t)(xaddr >> 32);  // stride 0: raw buffer
+        rsrc.z = (int32_t)p.x_bytes;
+        rsrc.w = 0x00020000;
+        planes_main_loop<BITS>(a, xoff, rsrc, wrow + (size_t)g_begin * kTileWords,
+                               p.ktab + (size_t)g_begin * NUM, g_full_end - g_begin, p.x_plane, p.x_row);
+    }
+
+    int32_t acc[R][J];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int j = 0; j < J; ++j) acc[r][j] = a[2 * r + j / 16][j % 16];
+
+    // partial last group (codes with k >= K read as x = 0)
+    const __amdgpu_buffer_rsrc_t xrsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, (int)p.x_bytes, 0x00020000);
+    for (int g = g_full_end; g < g_end; ++g) {
+        uint32_t w[J];
+#pragma unroll
+        for (int j = 0; j < J; ++j) w[j] = wrow[(size_t)g * kTileWords + j];
+        int32_t xt[NUM][R];
+        load_group<NUM, R>(xt, xrsrc, xoff, p, g);
+#pragma unroll
+        for (int i = 0; i < NUM; ++i) {
+            const bool real = g * NUM + i < p.K;
+#pragma unroll
+            for (int r = 0; r < R; ++r) xt[i][r] = real ? xt[i][r] : 0;
+            accumulate_code<BITS, false, R, J>(acc, xt[i], w, i, 0);
+        }
+    }
+
+    const int n0 = ntile * J;
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        const int n = n0 + j;
+        if (n >= p.N) break;
+        int32_t *yc = p.y + (size_t)n * p.y_ch_stride;
+        if (p.atomic_out) {
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                if (live[r]) atomicAdd(at_lane(yc, yoff[r]), acc[r][j]);
+        } else {
+            const int32_t add = p.negcnt[n] + (p.bias ? p.bias[n] : 0);
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                if (live[r]) *at_lane(yc, yoff[r]) = acc[r][j] + add;
+        }
+    }
+}
+
 // y = bias[n] + negcnt[n] for the split-K path.  Both output layouts ([img][n][pix] and [m][n])
 // are dense, so the flat index is the address and n = (idx / y_ch_stride) % N.
 __global__ void fill_bias_kernel(const ShiftArgs p)
@@ -282,9 +432,40 @@ static TileChoice choose_tile(const ShiftArgs &a)
     return c;
 }
 
+template <int BITS>
+static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
+{
+    constexpr int R = 4, J = 32;
+    a.tiles_m4 = ceil_div(ceil_div(a.M, R * kWave), 4);
+    a.tiles_n = ceil_div(a.N, J);
+    const int tiles = a.tiles_m4 * a.tiles_n;
+    a.blocks_per_xcd = ceil_div(tiles, 8);
+    if (nsplit < 1 || a.comm == 0) nsplit = 1;
+    a.groups_per_split = a.comm == 0 ? 1 : ceil_div(a.comm, nsplit);
+    nsplit = a.comm == 0 ? 1 : ceil_div(a.comm, a.groups_per_split);
+    a.atomic_out = nsplit > 1;
+    if (a.atomic_out) {
+        const long total = (long)a.M * a.N;
+        int blocks = (int)((total + 255) / 256);
+        if (blocks > 65536) blocks = 65536;
+        hipLaunchKernelGGL(fill_bias_kernel, dim3(blocks), dim3(256), 0, st, a);
+    }
+    dim3 grid(a.blocks_per_xcd * 8, nsplit);
+    hipLaunchKernelGGL((shift_planes_kernel<BITS>), grid, dim3(256), 0, st, a);
+    return launch_status();
+}
+
 template <int BITS, bool GENERAL>
 static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
 {
+    if constexpr (!GENERAL && BITS <= 4) {
+        const char *t = getenv("DS_TUNE_PLANES");
+        if (t && atoi(t) > 0) {
+            int nsplit = 1;
+            if (const char *sp = getenv("DS_TUNE_SPLIT")) nsplit = atoi(sp);
+            return launch_planes<BITS>(a, nsplit, st);
+        }
+    }
     TileChoice c = choose_tile(a);
     if (const char *t = getenv("DS_TUNE_TILE")) sscanf(t, "%dx%d", &c.R, &c.J);
     if (const char *t = getenv("DS_TUNE_SPLIT")) c.nsplit = atoi(t);
