@@ -285,7 +285,12 @@ def main():
     pairs = sum(L["M"] * L["K"] * L["N"] for L in layers)
     kernel_s = sum(L["seconds"] for L in layers)
     alg_bytes = 0
-    for L, S in zip(layers, shapes):
+    # the fused graph may run the two branches of a block in another order than the module tree:
+    # match the timed launches to the traced shapes by their (M, K, N)
+    pool = list(shapes)
+    for L in layers:
+        S = next(c for c in pool if (c["M"], c["K"], c["N"]) == (L["M"], L["K"], L["N"]))
+        pool.remove(S)
         uniq = S["Nb"] * S["C"] * S["H"] * S["W"] if S["kind"] == "conv" else None
         L["bytes"] = algorithmic_bytes(L, uniq)
         alg_bytes += L["bytes"]

@@ -41,6 +41,7 @@ struct ShiftArgs {
     int x_img_stride, x_row_stride, x_col_stride;
     int y_img_stride, y_pix_stride, y_ch_stride;
     int x_plane, x_row;                   // koff(k) = ic*x_plane + fh*x_row + fw
+    int FH, FW;                           // filter extent (1, 1 for a linear layer)
     int groups_per_split;                 // k-groups (words) per gridDim.y slice
     int nbase;                            // -base (left shift applied after the right shift)
     int tiles_m4;                         // number of 4-wave pixel tiles
@@ -231,59 +232,45 @@ __global__ __launch_bounds__(256) void shift_kernel(const ShiftArgs p)
 typedef int32_t v16i __attribute__((ext_vector_type(16)));
 typedef int32_t v4i __attribute__((ext_vector_type(4)));
 
+// Walk over the reduction index handed to the asm loop: offset / fw / fh of the first k, the filter
+// extent, the offset steps taken when fw and fh wrap, and the largest valid offset.
+struct PlaneWalk {
+    int koff, fw, fh, FW, FH, row_step, plane_step, koff_max;
+};
+
 #define DS_PLANES_OPERANDS                                                                        \
     : "+{v[96:111]}"(a[0]), "+{v[112:127]}"(a[1]), "+{v[128:143]}"(a[2]), "+{v[144:159]}"(a[3]),  \
       "+{v[160:175]}"(a[4]), "+{v[176:191]}"(a[5]), "+{v[192:207]}"(a[6]), "+{v[208:223]}"(a[7])  \
-    : "v"(xoff[0]), "v"(xoff[1]), "v"(xoff[2]), "v"(xoff[3]), "s"(rsrc), "s"(wptr), "s"(kptr),    \
-      "s"(groups), "s"(x_plane), "s"(x_row)
+    : "v"(xoff[0]), "v"(xoff[1]), "v"(xoff[2]), "v"(xoff[3]), "s"(rsrc), "s"(wptr), "s"(groups),  \
+      "s"(w.koff), "s"(w.fw), "s"(w.fh), "s"(w.FW), "s"(w.FH), "s"(w.row_step), "s"(w.plane_step), \
+      "s"(w.koff_max)
 
 template <int BITS>
 __device__ __forceinline__ void planes_main_loop(v16i (&a)[8], const uint32_t (&xoff)[4], v4i rsrc,
-                                                 const uint32_t *wptr, const uint32_t *kptr, int groups,
-                                                 int x_plane, int x_row);
-template <>
-__device__ __forceinline__ void planes_main_loop<1>(v16i (&a)[8], const uint32_t (&xoff)[4], v4i rsrc,
-                                                    const uint32_t *wptr, const uint32_t *kptr,
-                                                    int groups, int x_plane, int x_row)
-{
-    asm volatile(DS_PLANES_ASM_B1 DS_PLANES_OPERANDS : DS_PLANES_CLOBBERS_B1);
-}
-template <>
-__device__ __forceinline__ void planes_main_loop<2>(v16i (&a)[8], const uint32_t (&xoff)[4], v4i rsrc,
-                                                    const uint32_t *wptr, const uint32_t *kptr,
-                                                    int groups, int x_plane, int x_row)
-{
-    asm volatile(DS_PLANES_ASM_B2 DS_PLANES_OPERANDS : DS_PLANES_CLOBBERS_B2);
-}
-template <>
-__device__ __forceinline__ void planes_main_loop<3>(v16i (&a)[8], const uint32_t (&xoff)[4], v4i rsrc,
-                                                    const uint32_t *wptr, const uint32_t *kptr,
-                                                    int groups, int x_plane, int x_row)
-{
-    asm volatile(DS_PLANES_ASM_B3 DS_PLANES_OPERANDS : DS_PLANES_CLOBBERS_B3);
-}
-template <>
-__device__ __forceinline__ void planes_main_loop<4>(v16i (&a)[8], const uint32_t (&xoff)[4], v4i rsrc,
-                                                    const uint32_t *wptr, const uint32_t *kptr,
-                                                    int groups, int x_plane, int x_row)
-{
-    asm volatile(DS_PLANES_ASM_B4 DS_PLANES_OPERANDS : DS_PLANES_CLOBBERS_B4);
-}
+                                                 const uint32_t *wptr, int groups, const PlaneWalk &w);
+#define DS_PLANES_SPECIALISE(B)                                                                    \
+    template <>                                                                                    \
+    __device__ __forceinline__ void planes_main_loop<B>(v16i (&a)[8], const uint32_t (&xoff)[4],  \
+                                                        v4i rsrc, const uint32_t *wptr, int groups, \
+                                                        const PlaneWalk &w)                        \
+    {                                                                                              \
+        asm volatile(DS_PLANES_ASM_B##B DS_PLANES_OPERANDS : DS_PLANES_CLOBBERS_B##B);             \
+    }
+DS_PLANES_SPECIALISE(1)
+DS_PLANES_SPECIALISE(2)
+DS_PLANES_SPECIALISE(3)
+DS_PLANES_SPECIALISE(4)
 
+// One segment of work of the shift-plane kernel: K groups [g_begin, g_end) of the tile made of the 32
+// channels of `ntile` and the R*64 pixels starting at m0.  `atomic` selects accumulation into a
+// pre-filled output (several segments share the tile) or a plain store of acc + bias.
 template <int BITS>
-__global__ __launch_bounds__(256) void shift_planes_kernel(const ShiftArgs p)
+__device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, int m0, int g_begin,
+                                               int g_end, bool atomic)
 {
     constexpr int NUM = 32 / (BITS + 1);
     constexpr int R = 4, J = 32;
     const int lane = threadIdx.x & (kWave - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int bid = blockIdx.x;
-    const int tile = (bid & 7) * p.blocks_per_xcd + (bid >> 3);
-    if (tile >= p.tiles_m4 * p.tiles_n) return;
-    const int ntile = tile % p.tiles_n;
-    const int mtile = (tile / p.tiles_n) * 4 + wave;
-    const int m0 = mtile * (R * kWave);
-    if (m0 >= p.M) return;
 
     uint32_t xoff[R], yoff[R];
     bool live[R];
@@ -300,9 +287,6 @@ __global__ __launch_bounds__(256) void shift_planes_kernel(const ShiftArgs p)
         yoff[r] = 4u * (uint32_t)(img * p.y_img_stride + rem * p.y_pix_stride);
     }
 
-    const int g_begin = blockIdx.y * p.groups_per_split;
-    int g_end = g_begin + p.groups_per_split;
-    if (g_end > p.comm) g_end = p.comm;
     const int full_groups = p.K / NUM;
     const int g_full_end = g_end < full_groups ? g_end : full_groups;
     const uint32_t *wrow = p.wt + (size_t)ntile * p.comm * kTileWords;
@@ -317,8 +301,18 @@ __global__ __launch_bounds__(256) void shift_planes_kernel(const ShiftArgs p)
         rsrc.y = (int32_t)(uint32_t)(xaddr >> 32);  // stride 0: raw buffer
         rsrc.z = (int32_t)p.x_bytes;
         rsrc.w = 0x00020000;
-        planes_main_loop<BITS>(a, xoff, rsrc, wrow + (size_t)g_begin * kTileWords,
-                               p.ktab + (size_t)g_begin * NUM, g_full_end - g_begin, p.x_plane, p.x_row);
+        PlaneWalk w;
+        const int k0 = g_begin * NUM, ff = p.FH * p.FW;
+        const int ic = k0 / ff, rem = k0 - ic * ff;
+        w.fh = rem / p.FW;
+        w.fw = rem - w.fh * p.FW;
+        w.koff = ic * p.x_plane + w.fh * p.x_row + w.fw;
+        w.FW = p.FW;
+        w.FH = p.FH;
+        w.row_step = p.x_row - p.FW;
+        w.plane_step = p.x_plane - p.FH * p.x_row;
+        w.koff_max = (p.K / ff - 1) * p.x_plane + (p.FH - 1) * p.x_row + p.FW - 1;
+        planes_main_loop<BITS>(a, xoff, rsrc, wrow + (size_t)g_begin * kTileWords, g_full_end - g_begin, w);
     }
 
     int32_t acc[R][J];
@@ -330,7 +324,7 @@ __global__ __launch_bounds__(256) void shift_planes_kernel(const ShiftArgs p)
     // partial last group (codes with k >= K read as x = 0)
     const __amdgpu_buffer_rsrc_t xrsrc =
         __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, (int)p.x_bytes, 0x00020000);
-    for (int g = g_full_end; g < g_end; ++g) {
+    for (int g = g_full_end > g_begin ? g_full_end : g_begin; g < g_end; ++g) {
         uint32_t w[J];
 #pragma unroll
         for (int j = 0; j < J; ++j) w[j] = wrow[(size_t)g * kTileWords + j];
@@ -351,7 +345,7 @@ __global__ __launch_bounds__(256) void shift_planes_kernel(const ShiftArgs p)
         const int n = n0 + j;
         if (n >= p.N) break;
         int32_t *yc = p.y + (size_t)n * p.y_ch_stride;
-        if (p.atomic_out) {
+        if (atomic) {
 #pragma unroll
             for (int r = 0; r < R; ++r)
                 if (live[r]) atomicAdd(at_lane(yc, yoff[r]), acc[r][j]);
@@ -361,6 +355,50 @@ __global__ __launch_bounds__(256) void shift_planes_kernel(const ShiftArgs p)
             for (int r = 0; r < R; ++r)
                 if (live[r]) *at_lane(yc, yoff[r]) = acc[r][j] + add;
         }
+    }
+}
+
+// Tile-per-wave launch: gridDim.y K-slices per tile.
+template <int BITS>
+__global__ __launch_bounds__(256) void shift_planes_kernel(const ShiftArgs p)
+{
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int bid = blockIdx.x;
+    const int tile = (bid & 7) * p.blocks_per_xcd + (bid >> 3);
+    if (tile >= p.tiles_m4 * p.tiles_n) return;
+    const int ntile = tile % p.tiles_n;
+    const int m0 = ((tile / p.tiles_n) * 4 + wave) * (4 * kWave);
+    if (m0 >= p.M) return;
+    const int g_begin = blockIdx.y * p.groups_per_split;
+    int g_end = g_begin + p.groups_per_split;
+    if (g_end > p.comm) g_end = p.comm;
+    planes_segment<BITS>(p, ntile, m0, g_begin, g_end, p.atomic_out != 0);
+}
+
+// Work-balanced launch: the (tile, K group) iteration space is cut into one equal contiguous share
+// per wave, so every wave of the launch does the same number of group iterations whatever the tile
+// count (each wave touches at most a few tiles; tiles shared between waves are combined with
+// atomic adds onto the pre-filled output).  tiles_m4 holds the number of 256-pixel tiles here.
+template <int BITS>
+__global__ __launch_bounds__(256) void shift_planes_balanced_kernel(const ShiftArgs p)
+{
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int bid = blockIdx.x;
+    // waves of one XCD (workgroup ids congruent mod 8) take a contiguous range of shares
+    const long w = ((long)(bid & 7) * (gridDim.x >> 3) + (bid >> 3)) * 4 + wave;
+    const long waves = (long)gridDim.x * 4;
+    const long total = (long)p.tiles_m4 * p.tiles_n * p.comm;
+    long it = w * total / waves;
+    const long it_end = (w + 1) * total / waves;
+    while (it < it_end) {
+        const int tile = (int)(it / p.comm);
+        const int g_begin = (int)(it - (long)tile * p.comm);
+        long g_end = g_begin + (it_end - it);
+        if (g_end > p.comm) g_end = p.comm;
+        const int ntile = tile % p.tiles_n;
+        const int m0 = (tile / p.tiles_n) * (4 * kWave);
+        planes_segment<BITS>(p, ntile, m0, g_begin, (int)g_end, true);
+        it += g_end - g_begin;
     }
 }
 
@@ -417,7 +455,7 @@ static TileChoice choose_tile(const ShiftArgs &a)
     if (a.N <= 16) { c.R = 4; c.J = 16; }                   // few channels: more pixels per lane
     else if (a.M <= 64) { c.R = 1; c.J = 32; }              // a single wave of rows
     else if (a.comm <= 32 && a.N >= 64) { c.R = 4; c.J = 16; }  // short reduction (e.g. 7x7x3 stem)
-    else if (a.x_col_stride > 1) { c.R = 3; c.J = 16; }     // strided pixels: half-used cache lines
+    else if (a.x_col_stride > 1 && a.OW > 8) { c.R = 3; c.J = 16; }  // strided pixels: half-used lines
     const long tiles = (long)ceil_div(a.M, c.R * kWave) * ceil_div(a.N, c.J);
     const long simds = 1024;
     const double per_simd = (double)tiles / simds;
@@ -436,20 +474,27 @@ template <int BITS>
 static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
 {
     constexpr int R = 4, J = 32;
-    a.tiles_m4 = ceil_div(ceil_div(a.M, R * kWave), 4);
     a.tiles_n = ceil_div(a.N, J);
+    const long total = (long)a.M * a.N;
+    int fill_blocks = (int)((total + 255) / 256);
+    if (fill_blocks > 65536) fill_blocks = 65536;
+    if (nsplit <= 0 && a.comm > 0) {
+        // balanced launch: one share of the iteration space per wave slot (2 waves per SIMD)
+        a.tiles_m4 = ceil_div(a.M, R * kWave);
+        a.atomic_out = 1;
+        hipLaunchKernelGGL(fill_bias_kernel, dim3(fill_blocks), dim3(256), 0, st, a);
+        int blocks = 512 * (nsplit < 0 ? -nsplit : 1);
+        hipLaunchKernelGGL((shift_planes_balanced_kernel<BITS>), dim3(blocks), dim3(256), 0, st, a);
+        return launch_status();
+    }
+    a.tiles_m4 = ceil_div(ceil_div(a.M, R * kWave), 4);
     const int tiles = a.tiles_m4 * a.tiles_n;
     a.blocks_per_xcd = ceil_div(tiles, 8);
     if (nsplit < 1 || a.comm == 0) nsplit = 1;
     a.groups_per_split = a.comm == 0 ? 1 : ceil_div(a.comm, nsplit);
     nsplit = a.comm == 0 ? 1 : ceil_div(a.comm, a.groups_per_split);
     a.atomic_out = nsplit > 1;
-    if (a.atomic_out) {
-        const long total = (long)a.M * a.N;
-        int blocks = (int)((total + 255) / 256);
-        if (blocks > 65536) blocks = 65536;
-        hipLaunchKernelGGL(fill_bias_kernel, dim3(blocks), dim3(256), 0, st, a);
-    }
+    if (a.atomic_out) hipLaunchKernelGGL(fill_bias_kernel, dim3(fill_blocks), dim3(256), 0, st, a);
     dim3 grid(a.blocks_per_xcd * 8, nsplit);
     hipLaunchKernelGGL((shift_planes_kernel<BITS>), grid, dim3(256), 0, st, a);
     return launch_status();
@@ -459,9 +504,19 @@ template <int BITS, bool GENERAL>
 static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
 {
     if constexpr (!GENERAL && BITS <= 4) {
+        // Shift-plane kernel with the work-balanced launch: measured 6..10 % faster than the
+        // two-instruction kernel on long stride-1 reductions (ResNet 3x3 layers, large GEMMs); the
+        // short, strided and few-channel layers stay on the kernel above.
         const char *t = getenv("DS_TUNE_PLANES");
-        if (t && atoi(t) > 0) {
-            int nsplit = 1;
+        const long iters = (long)ceil_div(a.M, 256) * ceil_div(a.N, 32) * a.comm;
+        bool planes = a.comm >= 48 && iters >= 2048L * 24 && (a.N % 32 == 0 || a.N >= 256);
+        if (t) planes = atoi(t) > 0;
+        if (planes) {
+            // 2 waves per SIMD fit (2048 slots): one tile per wave when the tiles fill whole rounds
+            // of slots (no atomics, no pre-fill), otherwise equal shares of the iteration space
+            const long tiles = (long)ceil_div(a.M, 256) * ceil_div(a.N, 32);
+            const long rounds = (tiles + 2047) / 2048;
+            int nsplit = (tiles >= 2048 && (double)tiles / (2048.0 * rounds) >= 0.93) ? 1 : 0;
             if (const char *sp = getenv("DS_TUNE_SPLIT")) nsplit = atoi(sp);
             return launch_planes<BITS>(a, nsplit, st);
         }
@@ -556,6 +611,7 @@ DS_EXPORT int ds_conv2d_tiled_i32(const int32_t *x, const void *tiled, const int
     a.y_img_stride = O * OH * OW; a.y_pix_stride = 1; a.y_ch_stride = OH * OW;
     a.ktab = tiled_ktab(tiled, g);
     a.x_plane = Hp * Wp; a.x_row = Wp;
+    a.FH = FH; a.FW = FW;
     a.nbase = -base;
     return dispatch_bits(a, bits, base != 0 || bits == 6, (hipStream_t)stream);
 }
@@ -625,6 +681,7 @@ DS_EXPORT int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled,
     a.y_img_stride = 0; a.y_pix_stride = N; a.y_ch_stride = 1;
     a.ktab = tiled_ktab(tiled, g);
     a.x_plane = ldx; a.x_row = 1;
+    a.FH = 1; a.FW = 1;
     a.nbase = -base;
     return dispatch_bits(a, bits, base != 0 || bits == 6, (hipStream_t)stream);
 }

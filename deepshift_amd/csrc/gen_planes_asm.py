@@ -14,58 +14,52 @@ VGPR-relative addressing (s_set_gpr_idx_*), which needs a fixed register map:
 so a shift-add term costs 1 + 2^BITS/32 vector instructions instead of 2.
 
 Register map (R = 4 pixels per lane, J = 32 channels, NUM = 32 // (BITS + 1) codes per word):
-    v[8 + 4*i + r]                       prefetched activation of reduction slot i, row r
-    v[8 + 4*NUM + P*r + s]               plane[r][s], P = 2^BITS
-    v[96 + 32*r + j]                     acc[r][j]                       (asm operands %0..%7)
-    s[4:35] packed words of the 32 channels, s[36:67] the next group's words (loading),
-    s[68:83] next group's k-table entries, s84..s93 temps
-Operands: %8..%11 per-row byte offsets (VGPR), %12 buffer descriptor, %13 word pointer, %14 k-table
-pointer, %15 number of K groups, %16 / %17 plane and row pitch of the activations (elements).
+    v[8 + 4*i + r]            prefetched activation of reduction slot i, row r (loaded one K group ahead)
+    v[8 + 4*NUM + P*r + s]    plane[r][s], P = 2^BITS
+    v[96 + 32*r + j]          acc[r][j]                                   (asm operands %0..%7)
+    s[36:67]                  packed words of the 32 channels for the group being accumulated
+    s[68:99]                  the next group's words (in flight while this group is accumulated)
+    s4..s6                    walk over the reduction index: element offset, fw, fh of the next k to load
+    s7..s15                   temporaries, loop counter, word pointer
+Operands: %8..%11 per-row byte offsets (VGPR), %12 buffer descriptor, %13 word pointer, %14 number of
+K groups, %15..%17 initial walk state (offset, fw, fh), %18 FW, %19 FH, %20 offset step when fw wraps,
+%21 offset step when fh wraps, %22 largest valid offset (the walk runs one group ahead and is clamped).
 """
 import os
 
 R, J = 4, 32
 ACC = 96
 XP = 8
-W = 4           # s[4:35]   words of the group being accumulated
-WS = 36         # s[36:67]  words of the next group (in flight while this one is accumulated)
-KT = 68         # s[68:83]
-CNT, T0, WP, KP, T1, IDX, MASK, KOFF = 84, 85, 86, 88, 90, 91, 92, 93
+W = 36
+WS = 68
+KOFF, FWC, FHC = 4, 5, 6
+CNT, T0, T1, IDX, MASK, KB = 7, 8, 9, 10, 11, 12
+WP = 14
 
 
-def sload(dst, n, ptr, off):
-    return "s_load_dword%s s[%d:%d], s[%d:%d], 0x%x" % ("x%d" % n if n > 1 else "", dst, dst + n - 1,
-                                                         ptr, ptr + 1, off) if n > 1 else \
-        "s_load_dword s%d, s[%d:%d], 0x%x" % (dst, ptr, ptr + 1, off)
+def load_words():
+    return ["s_load_dwordx16 s[%d:%d], s[%d:%d], 0x0" % (WS, WS + 15, WP, WP + 1),
+            "s_load_dwordx16 s[%d:%d], s[%d:%d], 0x40" % (WS + 16, WS + 31, WP, WP + 1)]
 
 
-def load_ktab(num):
-    """Scalar loads of `num` consecutive k-table entries into s[KT..]."""
-    out, done = [], 0
-    for n in (16, 8, 4, 2, 1):
-        while num - done >= n:
-            out.append(sload(KT + done, n, KP, done * 4))
-            done += n
-    return out
-
-
-def koff(i):
-    """KOFF <- 4 * (ic * plane + fh * row + fw) for k-table entry i (ic << 10 | fh << 5 | fw)."""
-    v = KT + i
-    return [
-        "s_lshr_b32 s%d, s%d, 10" % (T0, v),
-        "s_mul_i32 s%d, s%d, %%16" % (T0, T0),
-        "s_bfe_u32 s%d, s%d, 0x50005" % (T1, v),
-        "s_mul_i32 s%d, s%d, %%17" % (T1, T1),
-        "s_add_u32 s%d, s%d, s%d" % (T0, T0, T1),
-        "s_and_b32 s%d, s%d, 31" % (T1, v),
-        "s_add_u32 s%d, s%d, s%d" % (T0, T0, T1),
-        "s_lshl_b32 s%d, s%d, 2" % (KOFF, T0),
-    ]
-
-
-def issue_loads(i):
-    return ["buffer_load_dword v%d, %%%d, %%12, s%d offen" % (XP + 4 * i + r, 8 + r, KOFF) for r in range(R)]
+def walk_and_load(i):
+    """Issue the R loads of the walk's current k into slot i, then step the walk to k + 1."""
+    L = ["s_min_u32 s%d, s%d, %%22" % (T0, KOFF),
+         "s_lshl_b32 s%d, s%d, 2" % (KB, T0)]
+    L += ["buffer_load_dword v%d, %%%d, %%12, s%d offen" % (XP + 4 * i + r, 8 + r, KB) for r in range(R)]
+    L += ["s_add_u32 s%d, s%d, 1" % (FWC, FWC),
+          "s_add_u32 s%d, s%d, 1" % (KOFF, KOFF),
+          "s_cmp_eq_u32 s%d, %%18" % FWC,
+          "s_cselect_b32 s%d, 0, s%d" % (FWC, FWC),
+          "s_cselect_b32 s%d, %%20, 0" % T0,
+          "s_cselect_b32 s%d, 1, 0" % T1,
+          "s_add_u32 s%d, s%d, s%d" % (KOFF, KOFF, T0),
+          "s_add_u32 s%d, s%d, s%d" % (FHC, FHC, T1),
+          "s_cmp_eq_u32 s%d, %%19" % FHC,
+          "s_cselect_b32 s%d, 0, s%d" % (FHC, FHC),
+          "s_cselect_b32 s%d, %%21, 0" % T0,
+          "s_add_u32 s%d, s%d, s%d" % (KOFF, KOFF, T0)]
+    return L
 
 
 def body(bits):
@@ -75,37 +69,29 @@ def body(bits):
     PL = XP + 4 * num
     assert PL + P * R <= ACC
     L = []
-    # ---- prologue: copies of the mutable inputs, first group's activation loads
-    L += ["s_mov_b32 s%d, %%15" % CNT,
+    # ---- prologue: mutable copies of the inputs, the first group's activation loads and words
+    L += ["s_mov_b32 s%d, %%14" % CNT,
           "s_mov_b64 s[%d:%d], %%13" % (WP, WP + 1),
-          "s_mov_b64 s[%d:%d], %%14" % (KP, KP + 1)]
-    L += load_ktab(num)
-    L += ["s_waitcnt lgkmcnt(0)"]
+          "s_mov_b32 s%d, %%15" % KOFF, "s_mov_b32 s%d, %%16" % FWC, "s_mov_b32 s%d, %%17" % FHC]
+    L += load_words()
     for i in range(num):
-        L += koff(i) + issue_loads(i)
-    L += ["s_add_u32 s%d, s%d, %d" % (KP, KP, num * 4), "s_addc_u32 s%d, s%d, 0" % (KP + 1, KP + 1)]
+        L += walk_and_load(i)
     L += ["s_mov_b32 s%d, 0" % IDX, "s_set_gpr_idx_on s%d, 0x1" % IDX]  # src0 of vector ops is M0-relative
-    # first group's words and second group's k-table entries: in flight into the staging registers
-    L += [sload(WS, 16, WP, 0), sload(WS + 16, 16, WP, 64)] + load_ktab(num)
     # ---- one K group per iteration
     L += ["1:"]
     L += ["s_add_u32 s%d, s%d, 128" % (WP, WP), "s_addc_u32 s%d, s%d, 0" % (WP + 1, WP + 1),
-          "s_add_u32 s%d, s%d, %d" % (KP, KP, num * 4), "s_addc_u32 s%d, s%d, 0" % (KP + 1, KP + 1),
           "s_waitcnt lgkmcnt(0)"]
-    # this group's words move out of the staging registers, which then receive the next group's
-    # (one group past the end reads the padding that follows the words in the weight blob)
+    # this group's words leave the staging registers, which then receive the next group's (one group
+    # past the end reads the padding that follows the words in the weight blob)
     L += ["s_mov_b64 s[%d:%d], s[%d:%d]" % (W + 2 * q, W + 2 * q + 1, WS + 2 * q, WS + 2 * q + 1)
           for q in range(16)]
-    L += ["s_mov_b64 s[%d:%d], s[%d:%d]" % (KT2 + 2 * q, KT2 + 2 * q + 1, KT + 2 * q, KT + 2 * q + 1)
-          for q in range((num + 1) // 2)]
-    L += [sload(WS, 16, WP, 0), sload(WS + 16, 16, WP, 64)] + load_ktab(num)
+    L += load_words()
     for i in range(num):
-        L += koff(i)
         L += ["s_waitcnt vmcnt(%d)" % (4 * (num - 1))]
         # plane 0 = the activation itself (a shift by 0 keeps src0 a constant: not M0-relative)
         for r in range(R):
             L += ["v_ashrrev_i32 v%d, 0, v%d" % (PL + P * r, XP + 4 * i + r)]
-        L += issue_loads(i)  # same slot of the next group
+        L += walk_and_load(i)  # the same slot of the next group
         for s in range(1, P):
             for r in range(R):
                 L += ["v_ashrrev_i32 v%d, %d, v%d" % (PL + P * r + s, s, PL + P * r)]
@@ -117,8 +103,8 @@ def body(bits):
                 a = ACC + 32 * r + j
                 L += ["v_xad_u32 v%d, v%d, s%d, v%d" % (a, PL + P * r, MASK, a)]
     L += ["s_sub_u32 s%d, s%d, 1" % (CNT, CNT), "s_cmp_lg_u32 s%d, 0" % CNT, "s_cbranch_scc1 1b"]
-    # ---- drain the loads issued for the group after the last one, leave relative addressing
-    L += ["s_set_gpr_idx_off", "s_waitcnt vmcnt(0)"]
+    # ---- leave relative addressing, drain the loads issued for the group after the last one
+    L += ["s_set_gpr_idx_off", "s_waitcnt vmcnt(0) lgkmcnt(0)"]
     return L
 
 
@@ -126,7 +112,7 @@ def clobbers(bits):
     num = 32 // (bits + 1)
     P = 1 << bits
     v = ['"v%d"' % n for n in range(XP, XP + 4 * num + P * R)]
-    s = ['"s%d"' % n for n in range(W, KOFF + 1)]
+    s = ['"s%d"' % n for n in list(range(4, 16)) + list(range(W, WS + 32))]
     return ", ".join(v + s + ['"scc"', '"memory"'])
 
 
