@@ -37,7 +37,7 @@ def is_stale():
     if not os.path.exists(LIB_PATH):
         return True
     built = os.path.getmtime(LIB_PATH)
-    deps = sources() + glob.glob(os.path.join(CSRC, "*.h")) + \
+    deps = sources() + glob.glob(os.path.join(CSRC, "*.h")) + glob.glob(os.path.join(CSRC, "*.py")) + \
         glob.glob(os.path.join(_HERE, "..", "include", "*.h"))
     return any(os.path.getmtime(p) > built for p in deps)
 
@@ -45,6 +45,8 @@ def is_stale():
 def build(verbose=True):
     """Compile every .hip translation unit (in parallel) and link the shared library."""
     os.makedirs(LIB_DIR, exist_ok=True)
+    # the asm main loop of the shift-plane kernel is generated text (csrc/ds_planes_asm.inc)
+    subprocess.check_call([sys.executable, os.path.join(CSRC, "gen_planes_asm.py")])
     obj_dir = os.path.join(_HERE, "build")
     os.makedirs(obj_dir, exist_ok=True)
     procs = []
