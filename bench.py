@@ -328,15 +328,16 @@ def main():
         "shift_layers_images_per_s": BATCH / kernel_s,
         "roofline": {
             "bound": "valu",
-            "kernel": "ds::shift_kernel (20 conv launches + 1 FC launch per step)",
+            "kernel": "ds::shift_planes_balanced_kernel<4> (16 launches) + ds::shift_kernel (5 launches) per step",
             "achieved": pairs / kernel_s / 1e12,
             "peak": PEAK_PAIRS / 1e12,
             "unit": "Tpair/s",
             "frac": pairs / kernel_s / PEAK_PAIRS,
             # HBM bytes of one launch of the dominant shape (layer1 3x3 conv, 8 of the 21 launches are
-            # this size): 56.7 MB read + 411 MB of split-K atomic adds, from the FETCH_SIZE / WRITE_SIZE
-            # runs summarised in profiles/shift_kernel_layer1_conv_counters.md (106.6 MB algorithmic)
-            "traffic": 468.0e6,
+            # this size): 106.9 MB read + 117.4 MB of atomic partial sums, from the FETCH_SIZE /
+            # WRITE_SIZE runs summarised in profiles/shift_kernel_layer1_conv_counters.md
+            # (106.6 MB algorithmic)
+            "traffic": 224.3e6,
             "avg_launch_us": kernel_s / len(layers) * 1e6,
             "peak_calibrated": peak_cal / 1e12 if peak_cal else None,
             "frac_of_calibrated": pairs / kernel_s / peak_cal if peak_cal else None,
