@@ -24,9 +24,14 @@ inline int launch_status() { return hip_status(hipGetLastError()); }
 //   negcount[ntiles*32]               negative codes per channel
 //   ktab    [(comm+1)*num]            reduction index k -> (ic << 10 | fh << 5 | fw); zero past K,
 //                                     with one spare group so that a prefetch of group comm is valid
+//   words16 [ntiles][comm*num/2][32]  (bits <= 4 only) the same codes pre-decoded for the shift-plane
+//                                     kernel, two 16-bit codes per word (k even | k odd << 16):
+//                                     bits 3:0 shift field, bit 8 negative, bits 15:12 = 0001 so
+//                                     that the half-word is a ready M0 value for relative addressing
+//                                     (index in 7:0, "src0 is relative" in 15:12); one spare row
 struct TiledGeom {
     int num, comm, ntiles;
-    size_t word_count, negcount_offset, ktab_offset, ktab_count, bytes;
+    size_t word_count, negcount_offset, ktab_offset, ktab_count, words16_offset, words16_count, bytes;
 };
 inline TiledGeom tiled_geom(int N, int K, int bits)
 {
@@ -38,12 +43,18 @@ inline TiledGeom tiled_geom(int N, int K, int bits)
     g.negcount_offset = align_up(g.word_count * 4, 256);
     g.ktab_offset = g.negcount_offset + align_up((size_t)g.ntiles * kTileWords * 4, 256);
     g.ktab_count = (size_t)(g.comm + 1) * g.num;
-    g.bytes = g.ktab_offset + align_up(g.ktab_count * 4, 256);
+    g.words16_offset = g.ktab_offset + align_up(g.ktab_count * 4, 256);
+    g.words16_count = bits <= 4 ? ((size_t)g.ntiles * g.comm * (g.num / 2) + 1) * kTileWords : 0;
+    g.bytes = g.words16_offset + align_up(g.words16_count * 4, 256);
     return g;
 }
 inline const int32_t *tiled_negcount(const void *tiled, const TiledGeom &g)
 {
     return (const int32_t *)((const char *)tiled + g.negcount_offset);
+}
+inline const uint32_t *tiled_words16(const void *tiled, const TiledGeom &g)
+{
+    return (const uint32_t *)((const char *)tiled + g.words16_offset);
 }
 inline const uint32_t *tiled_ktab(const void *tiled, const TiledGeom &g)
 {

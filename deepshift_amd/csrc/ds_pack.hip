@@ -116,6 +116,37 @@ __global__ void ktab_kernel(uint32_t *ktab, int K, int count, int FH, int FW)
     ktab[k] = v;
 }
 
+// words16[t][g*(num/2) + h][j]: codes k = g*num + 2h and k + 1 of channel t*32 + j as 16-bit M0-ready
+// values (see TiledGeom).  Codes past K and padding channels are (field 0, positive).
+__global__ void tile16_kernel(const int32_t *__restrict__ w_ref, uint32_t *__restrict__ w16, int N, int K,
+                              int comm, int bits, int num, long words)
+{
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= words) return;
+    const int half = num / 2;
+    const int j = (int)(idx % kTileWords);
+    const long rest = idx / kTileWords;
+    const long rows = (long)comm * half;
+    const int row = (int)(rest % rows);
+    const int t = (int)(rest / rows);
+    const int g = row / half, h = row - g * half;
+    const int n = t * kTileWords + j;
+    uint32_t out = 0x10001000u;
+    if (n < N) {
+        const uint32_t in = (uint32_t)w_ref[(long)n * comm + g];
+        const int cb = bits + 1;
+        const uint32_t fmask = (1u << bits) - 1u;
+        for (int c = 0; c < 2; ++c) {
+            const int i = 2 * h + c;
+            if (g * num + i >= K) continue;
+            const uint32_t code = in >> (i * cb);
+            const uint32_t neg = ((code >> bits) & 1u) ^ 1u;
+            out |= ((code & fmask) | (neg << 8)) << (16 * c);
+        }
+    }
+    w16[idx] = out;
+}
+
 int launch_tile(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW, int bits,
                 hipStream_t st)
 {
@@ -133,6 +164,12 @@ int launch_tile(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW,
     }
     hipLaunchKernelGGL(ktab_kernel, dim3(ceil_div((int)g.ktab_count, 256)), dim3(256), 0, st,
                        (uint32_t *)tiled_ktab(tiled, g), K, (int)g.ktab_count, FH, FW);
+    if (g.words16_count) {
+        const long blocks = ((long)g.words16_count + 255) / 256;
+        hipLaunchKernelGGL(tile16_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w_ref,
+                           (uint32_t *)tiled_words16(tiled, g), N, K, g.comm, bits, g.num,
+                           (long)g.words16_count);
+    }
     return launch_status();
 }
 

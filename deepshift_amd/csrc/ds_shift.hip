@@ -30,7 +30,8 @@ namespace ds {
 
 struct ShiftArgs {
     const int32_t *x;       // activations
-    const uint32_t *wt;     // tiled words [ntiles16][comm][16]
+    const uint32_t *wt;     // tiled words [ntiles][comm][32]
+    const uint32_t *wt16;   // 16-bit pre-decoded codes [ntiles][comm*num/2][32] (fields of <= 4 bits)
     const int32_t *negcnt;  // per channel: number of negative codes
     const int32_t *bias;    // per channel or nullptr
     const uint32_t *ktab;   // [(comm+1)*num] k -> ic << 10 | fh << 5 | fw (0 past K)
@@ -312,7 +313,9 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
         w.row_step = p.x_row - p.FW;
         w.plane_step = p.x_plane - p.FH * p.x_row;
         w.koff_max = (p.K / ff - 1) * p.x_plane + (p.FH - 1) * p.x_row + p.FW - 1;
-        planes_main_loop<BITS>(a, xoff, rsrc, wrow + (size_t)g_begin * kTileWords, g_full_end - g_begin, w);
+        planes_main_loop<BITS>(a, xoff, rsrc,
+                               p.wt16 + ((size_t)ntile * p.comm + g_begin) * (NUM / 2) * kTileWords,
+                               g_full_end - g_begin, w);
     }
 
     int32_t acc[R][J];
@@ -602,6 +605,7 @@ DS_EXPORT int ds_conv2d_tiled_i32(const int32_t *x, const void *tiled, const int
     a.x = x;
     a.x_bytes = (uint32_t)x_bytes;
     a.wt = (const uint32_t *)tiled;
+    a.wt16 = tiled_words16(tiled, g);
     a.negcnt = tiled_negcount(tiled, g);
     a.bias = bias;
     a.y = y;
@@ -672,6 +676,7 @@ DS_EXPORT int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled,
     a.x = xT;
     a.x_bytes = (uint32_t)x_bytes;
     a.wt = (const uint32_t *)tiled;
+    a.wt16 = tiled_words16(tiled, g);
     a.negcnt = tiled_negcount(tiled, g);
     a.bias = bias;
     a.y = y;

@@ -8,7 +8,7 @@ VGPR-relative addressing (s_set_gpr_idx_*), which needs a fixed register map:
 
     per reduction index k and pixel row r:  plane[r][s] = x >> s  for every shift amount s < 2^BITS
                                             (2^BITS vector shifts, shared by all 32 output channels)
-    per (k, channel j):                     M0 <- shift field of the code (scalar), mask <- sign
+    per (k, channel j):                     M0 <- the code's 16-bit pre-decoded form (scalar), mask <- sign
                                             acc[r][j] = (plane[r][M0] ^ mask) + acc[r][j]   (v_xad_u32)
 
 so a shift-add term costs 1 + 2^BITS/32 vector instructions instead of 2.
@@ -17,8 +17,8 @@ Register map (R = 4 pixels per lane, J = 32 channels, NUM = 32 // (BITS + 1) cod
     v[8 + 4*i + r]            prefetched activation of reduction slot i, row r (loaded one K group ahead)
     v[8 + 4*NUM + P*r + s]    plane[r][s], P = 2^BITS
     v[96 + 32*r + j]          acc[r][j]                                   (asm operands %0..%7)
-    s[36:67]                  packed words of the 32 channels for the group being accumulated
-    s[68:99]                  the next group's words (in flight while this group is accumulated)
+    s[36:67]                  16-bit codes of the 32 channels for the two reduction slots being accumulated
+    s[68:99]                  the next two slots' codes (in flight meanwhile)
     s4..s6                    walk over the reduction index: element offset, fw, fh of the next k to load
     s7..s15                   temporaries, loop counter, word pointer
 Operands: %8..%11 per-row byte offsets (VGPR), %12 buffer descriptor, %13 word pointer, %14 number of
@@ -77,16 +77,17 @@ def body(bits):
     for i in range(num):
         L += walk_and_load(i)
     L += ["s_mov_b32 s%d, 0" % IDX, "s_set_gpr_idx_on s%d, 0x1" % IDX]  # src0 of vector ops is M0-relative
-    # ---- one K group per iteration
+    # ---- one K group per iteration, two reduction slots (one row of 16-bit codes) at a time
     L += ["1:"]
-    L += ["s_add_u32 s%d, s%d, 128" % (WP, WP), "s_addc_u32 s%d, s%d, 0" % (WP + 1, WP + 1),
-          "s_waitcnt lgkmcnt(0)"]
-    # this group's words leave the staging registers, which then receive the next group's (one group
-    # past the end reads the padding that follows the words in the weight blob)
-    L += ["s_mov_b64 s[%d:%d], s[%d:%d]" % (W + 2 * q, W + 2 * q + 1, WS + 2 * q, WS + 2 * q + 1)
-          for q in range(16)]
-    L += load_words()
     for i in range(num):
+        if i % 2 == 0:
+            # this row's codes leave the staging registers, which then receive the next row's (one
+            # row past the end reads the spare row that follows the codes in the weight blob)
+            L += ["s_add_u32 s%d, s%d, 128" % (WP, WP), "s_addc_u32 s%d, s%d, 0" % (WP + 1, WP + 1),
+                  "s_waitcnt lgkmcnt(0)"]
+            L += ["s_mov_b64 s[%d:%d], s[%d:%d]" % (W + 2 * q, W + 2 * q + 1, WS + 2 * q, WS + 2 * q + 1)
+                  for q in range(16)]
+            L += load_words()
         L += ["s_waitcnt vmcnt(%d)" % (4 * (num - 1))]
         # plane 0 = the activation itself (a shift by 0 keeps src0 a constant: not M0-relative)
         for r in range(R):
@@ -96,9 +97,12 @@ def body(bits):
             for r in range(R):
                 L += ["v_ashrrev_i32 v%d, %d, v%d" % (PL + P * r + s, s, PL + P * r)]
         for j in range(J):
-            L += ["s_bfe_u32 s%d, s%d, 0x%x" % (IDX, W + j, (bits << 16) | (i * cb)),
-                  "s_set_gpr_idx_idx s%d" % IDX,
-                  "s_bfe_i32 s%d, s%d, 0x%x" % (MASK, W + j, (1 << 16) | (i * cb + bits))]
+            # the 16-bit code is a ready M0 value: plane index in 7:0, "src0 relative" in 15:12
+            if i % 2 == 0:
+                L += ["s_mov_b32 m0, s%d" % (W + j)]
+            else:
+                L += ["s_lshr_b32 m0, s%d, 16" % (W + j)]
+            L += ["s_bfe_i32 s%d, s%d, 0x%x" % (MASK, W + j, (1 << 16) | (16 * (i % 2) + 8))]
             for r in range(R):
                 a = ACC + 32 * r + j
                 L += ["v_xad_u32 v%d, v%d, s%d, v%d" % (a, PL + P * r, MASK, a)]

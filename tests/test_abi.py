@@ -39,10 +39,13 @@ def test_version_and_status_strings():
 def test_size_queries():
     L = _lib.lib()
     # bits 4 -> 6 codes per word; N=64,K=576 -> comm 96; 64 channels = 4 tiles of 16 words
-    # words [2 tiles][96][32] + negcount[64] + k table [(96+1)*6], each part padded to 256 bytes
-    assert L.ds_tiled_bytes(64, 576, 4) == 2 * 96 * 32 * 4 + 256 + 2560
+    # words [2 tiles][96][32] + negcount[64] + k table [(96+1)*6] + 16-bit codes [2*96*3 + 1][32],
+    # each part padded to 256 bytes
+    assert L.ds_tiled_bytes(64, 576, 4) == 2 * 96 * 32 * 4 + 256 + 2560 + (2 * 96 * 3 + 1) * 128 + 128
     # channels are padded to a multiple of 32
-    assert L.ds_tiled_bytes(10, 6, 4) == 256 + 256 + 256
+    assert L.ds_tiled_bytes(10, 6, 4) == 256 + 256 + 256 + (1 * 1 * 3 + 1) * 128
+    # fields wider than 4 bits carry no 16-bit code section
+    assert L.ds_tiled_bytes(10, 6, 5) == 256 + 256 + 256
     assert L.ds_tiled_bytes(64, 576, 7) == 0
     assert L.ds_conv2d_tiled_workspace_bytes(1, 64, 58, 58, 64, 3, 3, 1, 1, 4) == 0
     assert L.ds_conv2d_workspace_bytes(1, 64, 58, 58, 64, 3, 3, 1, 1, 4) == L.ds_tiled_bytes(64, 576, 4)
