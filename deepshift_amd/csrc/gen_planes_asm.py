@@ -35,6 +35,7 @@ WS = 68
 KOFF, FWC, FHC = 4, 5, 6
 CNT, T0, T1, IDX, MASK, KB = 7, 8, 9, 10, 11, 12
 WP = 14
+PRIO = 13
 
 
 def load_words():
@@ -70,7 +71,8 @@ def body(bits):
     assert PL + P * R <= ACC
     L = []
     # ---- prologue: mutable copies of the inputs, the first group's activation loads and words
-    L += ["s_mov_b32 s%d, %%14" % CNT,
+    L += ["s_getreg_b32 s%d, hwreg(HW_REG_HW_ID, 0, 1)" % PRIO,  # parity of the wave slot on its SIMD
+          "s_mov_b32 s%d, %%14" % CNT,
           "s_mov_b64 s[%d:%d], %%13" % (WP, WP + 1),
           "s_mov_b32 s%d, %%15" % KOFF, "s_mov_b32 s%d, %%16" % FWC, "s_mov_b32 s%d, %%17" % FHC]
     L += load_words()
@@ -79,6 +81,10 @@ def body(bits):
     L += ["s_mov_b32 s%d, 0" % IDX, "s_set_gpr_idx_on s%d, 0x1" % IDX]  # src0 of vector ops is M0-relative
     # ---- one K group per iteration, two reduction slots (one row of 16-bit codes) at a time
     L += ["1:"]
+    # the two waves that share a SIMD swap issue priority every group: a fixed order (the arbiter
+    # favours the older wave) would let one wave finish early and leave the other alone on the SIMD
+    L += ["s_xor_b32 s%d, s%d, 1" % (PRIO, PRIO), "s_cmp_eq_u32 s%d, 0" % PRIO, "s_cbranch_scc0 3f",
+          "s_setprio 2", "s_branch 4f", "3:", "s_setprio 0", "4:"]
     for i in range(num):
         if i % 2 == 0:
             # this row's codes leave the staging registers, which then receive the next row's (one
@@ -108,7 +114,7 @@ def body(bits):
                 L += ["v_xad_u32 v%d, v%d, s%d, v%d" % (a, PL + P * r, MASK, a)]
     L += ["s_sub_u32 s%d, s%d, 1" % (CNT, CNT), "s_cmp_lg_u32 s%d, 0" % CNT, "s_cbranch_scc1 1b"]
     # ---- leave relative addressing, drain the loads issued for the group after the last one
-    L += ["s_set_gpr_idx_off", "s_waitcnt vmcnt(0) lgkmcnt(0)"]
+    L += ["s_set_gpr_idx_off", "s_setprio 0", "s_waitcnt vmcnt(0) lgkmcnt(0)"]
     return L
 
 
