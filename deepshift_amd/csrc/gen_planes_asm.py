@@ -36,6 +36,7 @@ KOFF, FWC, FHC = 4, 5, 6
 CNT, T0, T1, IDX, MASK, KB = 7, 8, 9, 10, 11, 12
 WP = 14
 PRIO = 13
+TIME = 34
 
 
 def load_words():
@@ -76,24 +77,30 @@ def body(bits):
           "s_mov_b64 s[%d:%d], %%13" % (WP, WP + 1),
           "s_mov_b32 s%d, %%15" % KOFF, "s_mov_b32 s%d, %%16" % FWC, "s_mov_b32 s%d, %%17" % FHC]
     L += load_words()
+    L += ["s_memrealtime s[%d:%d]" % (TIME, TIME + 1)]
     for i in range(num):
         L += walk_and_load(i)
     L += ["s_mov_b32 s%d, 0" % IDX, "s_set_gpr_idx_on s%d, 0x1" % IDX]  # src0 of vector ops is M0-relative
     # ---- one K group per iteration, two reduction slots (one row of 16-bit codes) at a time
     L += ["1:"]
-    # the two waves that share a SIMD swap issue priority every group: a fixed order (the arbiter
-    # favours the older wave) would let one wave finish early and leave the other alone on the SIMD
-    L += ["s_xor_b32 s%d, s%d, 1" % (PRIO, PRIO), "s_cmp_eq_u32 s%d, 0" % PRIO, "s_cbranch_scc0 3f",
-          "s_setprio 2", "s_branch 4f", "3:", "s_setprio 0", "4:"]
     for i in range(num):
         if i % 2 == 0:
             # this row's codes leave the staging registers, which then receive the next row's (one
             # row past the end reads the spare row that follows the codes in the weight blob)
             L += ["s_add_u32 s%d, s%d, 128" % (WP, WP), "s_addc_u32 s%d, s%d, 0" % (WP + 1, WP + 1),
                   "s_waitcnt lgkmcnt(0)"]
+            # The two waves that share a SIMD take turns at the higher issue priority, by the clock:
+            # bit 12 of the 100 MHz counter (41 us each) against the parity of the wave's slot.  With
+            # equal priorities the arbiter favours the older wave, which then finishes early and
+            # leaves the other alone on the SIMD.  The turn is checked every row, because the wave
+            # that should take over is the one that is running slowly.
+            L += ["s_bfe_u32 s%d, s%d, 0x1000c" % (T0, TIME), "s_cmp_eq_u32 s%d, s%d" % (T0, PRIO),
+                  "s_cbranch_scc0 %df" % (3 + i), "s_setprio 2", "s_branch %df" % (4 + i),
+                  "%d:" % (3 + i), "s_setprio 0", "%d:" % (4 + i)]
             L += ["s_mov_b64 s[%d:%d], s[%d:%d]" % (W + 2 * q, W + 2 * q + 1, WS + 2 * q, WS + 2 * q + 1)
                   for q in range(16)]
             L += load_words()
+            L += ["s_memrealtime s[%d:%d]" % (TIME, TIME + 1)]  # read when the next row arrives
         L += ["s_waitcnt vmcnt(%d)" % (4 * (num - 1))]
         # plane 0 = the activation itself (a shift by 0 keeps src0 a constant: not M0-relative)
         for r in range(R):
@@ -122,7 +129,7 @@ def clobbers(bits):
     num = 32 // (bits + 1)
     P = 1 << bits
     v = ['"v%d"' % n for n in range(XP, XP + 4 * num + P * R)]
-    s = ['"s%d"' % n for n in list(range(4, 16)) + list(range(W, WS + 32))]
+    s = ['"s%d"' % n for n in list(range(4, 16)) + list(range(W, WS + 32)) + [TIME, TIME + 1]]
     return ", ".join(v + s + ['"scc"', '"memory"'])
 
 
