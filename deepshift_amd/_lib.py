@@ -39,6 +39,7 @@ SIGNATURES = {
     "ds_transpose_i32": (_c_int, [_ptr, _ptr, _c_int, _c_int, _c_int, _ptr]),
     "ds_dequantize_i32_f32": (_c_int, [_ptr, _ptr, _c_i64, _c_int, _ptr]),
     "ds_dequantize_affine_i32_f32": (_c_int, [_ptr] * 5 + [_c_int] * 5 + [_ptr]),
+    "ds_requantize_affine_pad_i32": (_c_int, [_ptr] * 6 + [_c_int] * 11 + [_ptr]),
     "ds_valu_calibrate": (_c_int, [_ptr, _c_int, _c_int, _ptr]),
     "ds_copy_i32": (_c_int, [_ptr, _ptr, _c_i64, _ptr]),
 }

@@ -180,6 +180,18 @@ __global__ void dequantize_kernel(const int32_t *__restrict__ y, float *__restri
 // out = act(float(y) / 2^F * scale[c] + shift[c] (+ residual)): the dequantisation of a shift layer
 // fused with an inference-mode per-channel affine (a folded BatchNorm), a residual add and ReLU.
 // One thread per 4 consecutive pixels of one (image, channel) plane when HW % 4 == 0.
+// The float value that follows a shift layer: act(float(y) / 2^F * a + b (+ r)).  One definition, with
+// contraction off, so that every kernel that needs it rounds the same way.
+__device__ __forceinline__ float affine_one(int32_t y, float inv, float a, float b, const float *r,
+                                            int relu)
+{
+#pragma clang fp contract(off)
+    float v = ((float)y * inv) * a + b;
+    if (r) v += *r;
+    if (relu) v = v > 0.0f ? v : 0.0f;
+    return v;
+}
+
 template <int VEC>
 __global__ void dequantize_affine_kernel(const int32_t *__restrict__ y, float *__restrict__ out,
                                          const float *__restrict__ scale, const float *__restrict__ shift,
@@ -195,12 +207,40 @@ __global__ void dequantize_affine_kernel(const int32_t *__restrict__ y, float *_
         float v[VEC];
 #pragma unroll
         for (int t = 0; t < VEC; ++t) {
-            v[t] = ((float)y[e + t] * inv) * a + b;
-            if (residual) v[t] += residual[e + t];
-            if (relu) v[t] = v[t] > 0.0f ? v[t] : 0.0f;
+            v[t] = affine_one(y[e + t], inv, a, b, residual ? residual + e + t : nullptr, relu);
         }
 #pragma unroll
         for (int t = 0; t < VEC; ++t) out[e + t] = v[t];
+    }
+}
+
+// dequantize_affine followed by the next shift layer's input conversion (round to the I.F grid,
+// cast, zero padding) in one pass: one thread per element of the padded int32 output q; the float
+// value is also stored to out when the caller needs it (a later residual add, a non-shift consumer).
+__global__ void requantize_affine_pad_kernel(const int32_t *__restrict__ y, float *__restrict__ out,
+                                             int32_t *__restrict__ q, const float *__restrict__ scale,
+                                             const float *__restrict__ shift,
+                                             const float *__restrict__ residual, uint32_t planes, int C,
+                                             int H, int W, int ph, int pw, float inv, int relu,
+                                             QuantSpec spec)
+{
+    const uint32_t Hp = H + 2 * ph, Wp = W + 2 * pw;
+    const uint32_t total = planes * Hp * Wp;
+    for (uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+        const uint32_t plane = idx / (Hp * Wp);
+        const uint32_t rem = idx - plane * Hp * Wp;
+        const uint32_t hp = rem / Wp;
+        const int h = (int)hp - ph, w = (int)(rem - hp * Wp) - pw;
+        int32_t v = 0;
+        if ((unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W) {
+            const uint32_t src = (plane * H + h) * W + w;
+            const uint32_t c = plane % (uint32_t)C;
+            const float f = affine_one(y[src], inv, scale ? scale[c] : 1.0f, shift ? shift[c] : 0.0f,
+                                       residual ? residual + src : nullptr, relu);
+            if (out) out[src] = f;
+            v = quantize_one(f, spec);
+        }
+        q[idx] = v;
     }
 }
 
@@ -317,6 +357,24 @@ DS_EXPORT int ds_dequantize_affine_i32_f32(const int32_t *y, float *out, const f
     else
         hipLaunchKernelGGL((dequantize_affine_kernel<1>), dim3(grid_for(n)), dim3(256), 0,
                            (hipStream_t)stream, y, out, scale, shift, residual, n, C, HW, inv, relu);
+    return launch_status();
+}
+
+DS_EXPORT int ds_requantize_affine_pad_i32(const int32_t *y, float *out, int32_t *q, const float *scale,
+                                           const float *shift, const float *residual, int Nb, int C,
+                                           int H, int W, int ph, int pw, int F_in, int relu, int I, int F,
+                                           int mode, ds_stream_t stream)
+{
+    int rc = check_fixed(I, F, mode);
+    if (rc) return rc;
+    if (Nb < 0 || C < 0 || H < 0 || W < 0 || ph < 0 || pw < 0 || F_in < 0 || F_in > 31) return DS_EINVAL;
+    const long total = (long)Nb * C * (H + 2 * ph) * (W + 2 * pw);
+    if (total == 0) return DS_OK;
+    if (total * 4 >= (1L << 31)) return DS_ETOOLARGE;
+    if (!q || (!y && (long)Nb * C * H * W > 0)) return DS_EINVAL;
+    hipLaunchKernelGGL(requantize_affine_pad_kernel, dim3(grid_for(total)), dim3(256), 0,
+                       (hipStream_t)stream, y, out, q, scale, shift, residual, (uint32_t)(Nb * C), C, H, W,
+                       ph, pw, ldexpf(1.0f, -F_in), relu, make_spec(I, F, mode));
     return launch_status();
 }
 

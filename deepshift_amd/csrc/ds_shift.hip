@@ -409,12 +409,47 @@ __global__ __launch_bounds__(256) void shift_planes_balanced_kernel(const ShiftA
 // are dense, so the flat index is the address and n = (idx / y_ch_stride) % N.
 __global__ void fill_bias_kernel(const ShiftArgs p)
 {
-    const long total = (long)p.M * p.N;
-    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-         idx += (long)gridDim.x * blockDim.x) {
-        const int n = (int)((idx / p.y_ch_stride) % p.N);
+    const uint32_t total = (uint32_t)p.M * (uint32_t)p.N;  // < 2^29: tensors are below 2 GiB
+    for (uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+        const int n = (int)((idx / (uint32_t)p.y_ch_stride) % (uint32_t)p.N);
         p.y[idx] = p.negcnt[n] + (p.bias ? p.bias[n] : 0);
     }
+}
+
+// The same, four outputs per lane: needs a 16-byte aligned y and runs of four that either share
+// their channel (y_ch_stride % 4 == 0) or step through channels (y_ch_stride == 1, N % 4 == 0).
+__global__ void fill_bias4_kernel(const ShiftArgs p)
+{
+    const uint32_t total4 = ((uint32_t)p.M * (uint32_t)p.N) >> 2;
+    int4 *y4 = (int4 *)p.y;
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < total4; i += gridDim.x * blockDim.x) {
+        const uint32_t idx = i << 2;
+        const int n = (int)((idx / (uint32_t)p.y_ch_stride) % (uint32_t)p.N);
+        int4 v;
+        if (p.y_ch_stride != 1) {
+            v.x = v.y = v.z = v.w = p.negcnt[n] + (p.bias ? p.bias[n] : 0);
+        } else {
+            v.x = p.negcnt[n] + (p.bias ? p.bias[n] : 0);
+            v.y = p.negcnt[n + 1] + (p.bias ? p.bias[n + 1] : 0);
+            v.z = p.negcnt[n + 2] + (p.bias ? p.bias[n + 2] : 0);
+            v.w = p.negcnt[n + 3] + (p.bias ? p.bias[n + 3] : 0);
+        }
+        y4[i] = v;
+    }
+}
+
+static void launch_fill(const ShiftArgs &a, hipStream_t st)
+{
+    const long total = (long)a.M * a.N;
+    const bool vec = ((uintptr_t)a.y & 15) == 0 && total % 4 == 0 &&
+                     (a.y_ch_stride % 4 == 0 || (a.y_ch_stride == 1 && a.N % 4 == 0));
+    long blocks = vec ? (total / 4 + 255) / 256 : (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    if (blocks < 1) blocks = 1;
+    if (vec)
+        hipLaunchKernelGGL(fill_bias4_kernel, dim3((unsigned)blocks), dim3(256), 0, st, a);
+    else
+        hipLaunchKernelGGL(fill_bias_kernel, dim3((unsigned)blocks), dim3(256), 0, st, a);
 }
 
 template <int BITS, bool GENERAL, int R, int J>
@@ -428,12 +463,7 @@ static int launch_shift(ShiftArgs a, int nsplit, hipStream_t st)
     a.groups_per_split = a.comm == 0 ? 1 : ceil_div(a.comm, nsplit);
     nsplit = a.comm == 0 ? 1 : ceil_div(a.comm, a.groups_per_split);
     a.atomic_out = nsplit > 1;
-    if (a.atomic_out) {
-        const long total = (long)a.M * a.N;
-        int blocks = (int)((total + 255) / 256);
-        if (blocks > 65536) blocks = 65536;
-        hipLaunchKernelGGL(fill_bias_kernel, dim3(blocks), dim3(256), 0, st, a);
-    }
+    if (a.atomic_out) launch_fill(a, st);
     dim3 grid(a.blocks_per_xcd * 8, nsplit);
     hipLaunchKernelGGL((shift_kernel<BITS, GENERAL, R, J>), grid, dim3(256), 0, st, a);
     return launch_status();
@@ -478,14 +508,11 @@ static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
 {
     constexpr int R = 4, J = 32;
     a.tiles_n = ceil_div(a.N, J);
-    const long total = (long)a.M * a.N;
-    int fill_blocks = (int)((total + 255) / 256);
-    if (fill_blocks > 65536) fill_blocks = 65536;
     if (nsplit <= 0 && a.comm > 0) {
         // balanced launch: one share of the iteration space per wave slot (2 waves per SIMD)
         a.tiles_m4 = ceil_div(a.M, R * kWave);
         a.atomic_out = 1;
-        hipLaunchKernelGGL(fill_bias_kernel, dim3(fill_blocks), dim3(256), 0, st, a);
+        launch_fill(a, st);
         int blocks = 512 * (nsplit < 0 ? -nsplit : 1);
         hipLaunchKernelGGL((shift_planes_balanced_kernel<BITS>), dim3(blocks), dim3(256), 0, st, a);
         return launch_status();
@@ -497,7 +524,7 @@ static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
     a.groups_per_split = a.comm == 0 ? 1 : ceil_div(a.comm, nsplit);
     nsplit = a.comm == 0 ? 1 : ceil_div(a.comm, a.groups_per_split);
     a.atomic_out = nsplit > 1;
-    if (a.atomic_out) hipLaunchKernelGGL(fill_bias_kernel, dim3(fill_blocks), dim3(256), 0, st, a);
+    if (a.atomic_out) launch_fill(a, st);
     dim3 grid(a.blocks_per_xcd * 8, nsplit);
     hipLaunchKernelGGL((shift_planes_kernel<BITS>), grid, dim3(256), 0, st, a);
     return launch_status();

@@ -9,6 +9,11 @@ into one :class:`FusedConv2dShift` call: the int32 result of the shift kernel is
 scaled and shifted per channel (the folded BatchNorm), added to the residual and clamped at zero
 in a single pass (``ds_dequantize_affine_i32_f32``) instead of four.  The shift arithmetic itself
 is untouched; the float glue differs from the unfused ops by fp32 rounding only.
+
+Where a fused convolution feeds another one (zero padding), the same pass also writes the consumer's
+fixed-point input -- rounded to the consumer's I.F grid and zero padded -- so the consumer skips its
+own conversion pass, and the float tensor is not written at all when nothing else reads it
+(``ds_requantize_affine_pad_i32``).  This is bit-identical to the two passes it replaces.
 """
 import operator
 
@@ -33,6 +38,8 @@ class FusedConv2dShift(nn.Module):
         super().__init__()
         self.conv = conv
         self.relu = relu
+        self.prequantized = False  # the input is this layer's int32 padded input, made by its producer
+        self.emit = None           # (padding, I, F, want_float) of the consumers' input to produce
         if bn is not None:
             if bn.training or not bn.track_running_stats:
                 raise ValueError("only an eval-mode BatchNorm with running statistics can be folded")
@@ -54,7 +61,7 @@ class FusedConv2dShift(nn.Module):
         elif conv.conc_weight is None:
             modules.pack_module_weights(conv)
         return modules.conv_kernel_forward(conv, input, conv.conc_weight, self.scale, self.shift,
-                                           residual, self.relu)
+                                           residual, self.relu, self.prequantized, self.emit)
 
 
 class _Tracer(fx.Tracer):
@@ -81,9 +88,10 @@ def _sole_user(node):
     return users[0] if len(users) == 1 else None
 
 
-def fuse_conv_epilogues(model):
+def fuse_conv_epilogues(model, handoff=True):
     """Return a ``torch.fx.GraphModule`` equivalent to ``model`` (eval mode) with every kernel-mode
-    shift convolution fused with the BatchNorm / residual add / ReLU that consume its output."""
+    shift convolution fused with the BatchNorm / residual add / ReLU that consume its output.
+    ``handoff``: fused convolutions that feed each other pass the fixed-point tensor directly."""
     model.eval()
     graph = _Tracer().trace(model)
     gm = fx.GraphModule(model, graph)
@@ -126,6 +134,55 @@ def fuse_conv_epilogues(model):
         chain[-1].replace_all_uses_with(new)
         for old in reversed(chain):
             gm.graph.erase_node(old)
+    if handoff:
+        _hand_off_fixed_point(gm)
     gm.graph.lint()
     gm.recompile()
     return gm
+
+
+def _input_key(conv):
+    """What a kernel-mode convolution needs of its int32 input, or None if it pads by itself."""
+    if conv.padding_mode != 'zeros' or not conv.use_kernel:
+        return None
+    return (tuple(conv.padding), conv.act_integer_bits, conv.act_fraction_bits)
+
+
+def _hand_off_fixed_point(gm):
+    """Second pass: a fused convolution whose result feeds fused convolutions also writes their
+    fixed-point padded input, and they read that instead of converting the float tensor again."""
+    mods = dict(gm.named_modules())
+
+    def fused(n):
+        m = mods.get(n.target) if n.op == "call_module" else None
+        return m if isinstance(m, FusedConv2dShift) else None
+
+    for node in list(gm.graph.nodes):
+        producer = fused(node)
+        if producer is None or producer.emit is not None:
+            continue
+        key, takers = None, []
+        for user in node.users:
+            consumer = fused(user)
+            if consumer is None or user.args[0] is not node or consumer.prequantized:
+                continue
+            k = _input_key(consumer.conv)
+            if k is None or (key is not None and k != key):
+                continue
+            key = k
+            takers.append(user)
+        if not takers:
+            continue
+        # the float result is still needed by any other use, including a taker's residual operand
+        want_float = any(u not in takers or node in u.args[1:] for u in node.users)
+        producer.emit = key + (want_float,)
+        if want_float:
+            with gm.graph.inserting_after(node):
+                q = gm.graph.call_function(operator.getitem, (node, 1))
+                f = gm.graph.call_function(operator.getitem, (node, 0))
+            node.replace_all_uses_with(f, delete_user_cb=lambda u: u is not f and u is not q)
+        else:
+            q = node
+        for user in takers:
+            user.args = (q,) + tuple(user.args[1:])
+            fused(user).prequantized = True

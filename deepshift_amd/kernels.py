@@ -205,6 +205,33 @@ def dequantize_affine(y, fraction_bits=16, scale=None, shift=None, residual=None
     return out
 
 
+def requantize_affine_pad(y, fraction_bits_in, scale, shift, residual, relu, padding,
+                          integer_bits=16, fraction_bits=16, want_float=True):
+    """:func:`dequantize_affine` and the next shift convolution's :func:`quantize_pad` in one pass.
+
+    Returns ``(out, q)``: the float32 result (``None`` unless ``want_float``) and its round-to-fixed,
+    zero padded int32 form, bit-identical to the two separate calls."""
+    y = _require_device_i32("y", y)
+    if y.dim() != 4:
+        raise TypeError("requantize_affine_pad expects a 4-D int32 GPU tensor")
+    Nb, C, H, W = y.shape
+    ph, pw = _pair(padding)
+    for name, t in (("scale", scale), ("shift", shift)):
+        if t is not None and (t.dtype != torch.float32 or t.numel() != C or not t.is_contiguous()):
+            raise ValueError("%s must be a contiguous float32 tensor of %d elements" % (name, C))
+    if residual is not None:
+        if residual.shape != y.shape or residual.dtype != torch.float32:
+            raise ValueError("residual must be float32 with the shape of y")
+        residual = residual.contiguous()
+    out = torch.empty(y.shape, dtype=torch.float32, device=y.device) if want_float else None
+    q = torch.empty([Nb, C, H + 2 * ph, W + 2 * pw], dtype=torch.int32, device=y.device)
+    _lib.call("ds_requantize_affine_pad_i32", _lib.ptr(y), _lib.ptr(out), _lib.ptr(q), _lib.ptr(scale),
+              _lib.ptr(shift), _lib.ptr(residual), Nb, C, H, W, ph, pw, fraction_bits_in,
+              int(bool(relu)), integer_bits, fraction_bits, _lib.DS_Q_ROUND_TO_FIXED,
+              _lib.current_stream(y.device))
+    return out, q
+
+
 # ---------------------------------------------------------------------------------------------
 # LinearShift / Conv2dShift kernels
 # ---------------------------------------------------------------------------------------------

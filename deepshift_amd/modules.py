@@ -196,29 +196,43 @@ def _circular_pad(x, padding):
     return F.pad(x, expanded, mode='circular')
 
 
-def conv_kernel_forward(module, input, conc_weight, scale=None, shift=None, residual=None, relu=False):
+def conv_kernel_forward(module, input, conc_weight, scale=None, shift=None, residual=None, relu=False,
+                        prequantized=False, emit=None):
     """Fixed-point shift convolution of a float NCHW input (modules.py:152-162,317-337).
 
     ``scale``/``shift`` (per output channel), ``residual`` and ``relu`` describe what follows the
     layer (a folded BatchNorm, a shortcut add, ReLU); when any is given it is applied in the same
-    pass that converts the int32 result back to float."""
+    pass that converts the int32 result back to float.
+
+    ``prequantized``: ``input`` is already the layer's round-to-fixed, zero padded int32 input (made
+    by the layer before it).  ``emit = (padding, integer_bits, fraction_bits, want_float)``: also
+    produce that form of the result for the next shift convolution; the return value is then
+    ``(out, q)``, or ``q`` alone when ``want_float`` is false."""
     if not module.use_cuda:
         kernels._no_cpu_kernel()
     if module.dilation != (1, 1) or module.groups != 1:
         raise NotImplementedError("the shift kernel supports dilation=1 and groups=1 only")
     I, Fb = module.act_integer_bits, module.act_fraction_bits
-    padding = module.padding
-    input = input.float()
-    if module.padding_mode == 'circular':
-        input = _circular_pad(input, padding)
-        padding = (0, 0)
-    # round_to_fixed + cast + zero padding in one pass
-    xq = kernels.quantize_pad(input, padding, I, Fb, round_to_fixed=True)
+    if prequantized:
+        xq = input
+    else:
+        padding = module.padding
+        input = input.float()
+        if module.padding_mode == 'circular':
+            input = _circular_pad(input, padding)
+            padding = (0, 0)
+        # round_to_fixed + cast + zero padding in one pass
+        xq = kernels.quantize_pad(input, padding, I, Fb, round_to_fixed=True)
     bias = module._fixed_bias.get(module.bias, I, Fb, round_to_fixed=True)
     tiled = kernels._tiled_of(conc_weight, module.out_channels, module.in_channels,
                               module.kernel_size[0], module.kernel_size[1])
     out = kernels.conv2d_tiled(xq, tiled, bias, module.out_channels, module.kernel_size,
                                module.stride, conc_weight.bits, conc_weight.base)
+    if emit is not None:
+        next_padding, next_I, next_F, want_float = emit
+        f, q = kernels.requantize_affine_pad(out, Fb, scale, shift, residual, relu, next_padding,
+                                             next_I, next_F, want_float)
+        return (f, q) if want_float else q
     if scale is None and shift is None and residual is None and not relu:
         return kernels.dequantize(out, Fb)
     return kernels.dequantize_affine(out, Fb, scale, shift, residual, relu)

@@ -150,6 +150,17 @@ int ds_dequantize_affine_i32_f32(const int32_t *y, float *out, const float *scal
                                  const float *residual, int Nb, int C, int HW, int F, int relu,
                                  ds_stream_t stream);
 
+/* ds_dequantize_affine_i32_f32 followed by the next shift layer's ds_quantize_pad_f32_i32, in one
+ * pass: v = act(float(y) / 2^F_in * scale[c] + shift[c] + residual) is rounded to the I.F grid
+ * (mode as in ds_quantize_f32_i32) and written, zero padded by (ph, pw), to q [Nb][C][H+2ph][W+2pw];
+ * when out is not NULL v is also stored there ([Nb][C][H][W], float).  Bit-identical to the two
+ * calls it replaces.  No counterpart in the reference (modules.py:161-162 then :152-153 of the next
+ * layer, with the PyTorch ops in between). */
+int ds_requantize_affine_pad_i32(const int32_t *y, float *out, int32_t *q, const float *scale,
+                                 const float *shift, const float *residual, int Nb, int C, int H, int W,
+                                 int ph, int pw, int F_in, int relu, int I, int F, int mode,
+                                 ds_stream_t stream);
+
 /* ---- measurement ----------------------------------------------------------------------- */
 
 /* VALU calibration: every lane of `blocks` x 256 threads runs `iters` x 64 independent

@@ -230,6 +230,45 @@ def test_fused_epilogues_match_unfused_model():
         assert (got - want).abs().max().item() <= 2e-3 * scale + 1e-4, cls.__name__
 
 
+def test_fixed_point_handoff_is_bit_identical():
+    """Fused convolutions that feed each other pass the fixed-point tensor directly
+    (ds_requantize_affine_pad_i32): the network output must not change by a single bit."""
+    from deepshift_amd import fuse
+    for cls, shape in [(workloads.ResNet18, (2, 3, 64, 64)), (workloads.ResNet20, (3, 3, 32, 32)),
+                       (workloads.ResNet50, (1, 3, 64, 64))]:
+        g = torch.Generator().manual_seed(11)
+        model = workloads.randomize_batchnorm(cls(), g).eval()
+        model, n = convert.convert_to_shift(model, 1000, 'PS', convert_weights=True, use_kernel=True)
+        model = model.to(DEV)
+        x = torch.randn(*shape, generator=g).to(DEV)
+        with torch.no_grad():
+            plain = fuse.fuse_conv_epilogues(model, handoff=False)
+            want = plain(x)
+            direct = fuse.fuse_conv_epilogues(model, handoff=True)
+            got = direct(x)
+        takers = [m for m in direct.modules() if isinstance(m, fuse.FusedConv2dShift) and m.prequantized]
+        assert len(takers) >= n // 2, cls.__name__
+        assert not any(m.prequantized or m.emit for m in plain.modules()
+                       if isinstance(m, fuse.FusedConv2dShift))
+        assert torch.equal(got, want), cls.__name__
+
+
+def test_requantize_affine_pad_matches_the_two_passes(rng):
+    for (Nb, C, H, W), pad in [((3, 5, 7, 4), (1, 1)), ((2, 3, 5, 9), (0, 2)), ((1, 4, 6, 6), (0, 0))]:
+        y = torch.from_numpy(rng.integers(-2 ** 27, 2 ** 27, size=(Nb, C, H, W)).astype(np.int32)).to(DEV)
+        scale = torch.rand(C, device=DEV) + 0.5
+        shift = torch.randn(C, device=DEV)
+        res = torch.randn(Nb, C, H, W, device=DEV) * 100
+        for sc, sh, r, relu, I, F in [(scale, shift, res, True, 16, 16), (scale, None, None, False, 8, 8),
+                                      (None, None, res, True, 12, 4), (None, None, None, False, 16, 16)]:
+            f_want = kernels.dequantize_affine(y, 16, sc, sh, r, relu)
+            q_want = kernels.quantize_pad(f_want, pad, I, F, round_to_fixed=True)
+            f, q = kernels.requantize_affine_pad(y, 16, sc, sh, r, relu, pad, I, F, want_float=True)
+            assert torch.equal(f, f_want) and torch.equal(q, q_want)
+            f, q = kernels.requantize_affine_pad(y, 16, sc, sh, r, relu, pad, I, F, want_float=False)
+            assert f is None and torch.equal(q, q_want)
+
+
 def test_dequantize_affine_matches_torch(rng):
     Nb, C, H, W = 3, 5, 7, 4
     y = torch.from_numpy(rng.integers(-2 ** 24, 2 ** 24, size=(Nb, C, H, W)).astype(np.int32)).to(DEV)

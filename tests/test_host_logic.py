@@ -140,3 +140,23 @@ def test_workload_pair_counts():
         pairs = sum(l["M"] * l["K"] * l["N"] for l in shapes)
         assert abs(pairs - want) / want < 2e-3
     assert deepshift_amd.__version__
+
+
+def test_fused_graph_hands_fixed_point_tensors_on():
+    """Structure of the fused ResNet-18 graph (no kernel runs): every block's first convolution
+    takes its producer's int32 tensor, and the float result is kept only where a shortcut needs it."""
+    from deepshift_amd import convert, fuse, modules, workloads
+    model = workloads.ResNet18()
+    model, n = convert.convert_to_shift(model, 1000, 'PS', convert_weights=False, use_kernel=False)
+    for m in model.modules():
+        if isinstance(m, (modules.Conv2dShift, modules.LinearShift)):
+            m.use_kernel = True
+    gm = fuse.fuse_conv_epilogues(model)
+    fused = [m for m in gm.modules() if isinstance(m, fuse.FusedConv2dShift)]
+    assert len(fused) == 20
+    assert sum(m.prequantized for m in fused) == 15          # 8 second convolutions + 7 block inputs
+    emits = [m.emit for m in fused if m.emit is not None]
+    assert len(emits) == 15 and sum(e[3] for e in emits) == 7  # float kept for the 7 block outputs
+    assert all(e[:3] == ((1, 1), 16, 16) for e in emits)
+    plain = fuse.fuse_conv_epilogues(model, handoff=False)
+    assert not any(m.prequantized or m.emit for m in plain.modules() if isinstance(m, fuse.FusedConv2dShift))
