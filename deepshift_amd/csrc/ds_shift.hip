@@ -486,7 +486,7 @@ static TileChoice choose_tile(const ShiftArgs &a)
 {
     TileChoice c{2, 32, 1};
     if (a.N <= 16) { c.R = 4; c.J = 16; }                   // few channels: more pixels per lane
-    else if (a.M <= 64) { c.R = 1; c.J = 32; }              // a single wave of rows
+    else if (a.M <= 64) { c.R = 1; c.J = a.N >= 256 ? 8 : 32; }  // a single wave of rows: many narrow tiles
     else if (a.comm <= 32 && a.N >= 64) { c.R = 4; c.J = 16; }  // short reduction (e.g. 7x7x3 stem)
     else if (a.x_col_stride > 1 && a.OW > 8) { c.R = 3; c.J = 16; }  // strided pixels: half-used lines
     const long tiles = (long)ceil_div(a.M, c.R * kWave) * ceil_div(a.N, c.J);
@@ -534,12 +534,13 @@ template <int BITS, bool GENERAL>
 static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
 {
     if constexpr (!GENERAL && BITS <= 4) {
-        // Shift-plane kernel with the work-balanced launch: measured 6..10 % faster than the
-        // two-instruction kernel on long stride-1 reductions (ResNet 3x3 layers, large GEMMs); the
-        // short, strided and few-channel layers stay on the kernel above.
+        // Shift-plane kernel with the work-balanced launch: measured 10..25 % faster than the
+        // two-instruction kernel when every wave slot gets at least 24 K groups of work and a tile
+        // spans at least 24 (ResNet 3x3 and 7x7 layers, large GEMMs); the 1x1 shortcuts, small
+        // batches and few-channel layers stay on the kernel above.
         const char *t = getenv("DS_TUNE_PLANES");
         const long iters = (long)ceil_div(a.M, 256) * ceil_div(a.N, 32) * a.comm;
-        bool planes = a.comm >= 48 && iters >= 2048L * 24 && (a.N % 32 == 0 || a.N >= 256);
+        bool planes = a.comm >= 24 && iters >= 2048L * 24 && (a.N % 32 == 0 || a.N >= 256);
         if (t) planes = atoi(t) > 0;
         if (planes) {
             // 2 waves per SIMD fit (2048 slots): one tile per wave when the tiles fill whole rounds
@@ -557,6 +558,7 @@ static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
     if (c.R == 4 && c.J == 16) return launch_shift<BITS, GENERAL, 4, 16>(a, c.nsplit, st);
     if (c.R == 3 && c.J == 16) return launch_shift<BITS, GENERAL, 3, 16>(a, c.nsplit, st);
     if (c.R == 1 && c.J == 32) return launch_shift<BITS, GENERAL, 1, 32>(a, c.nsplit, st);
+    if (c.R == 1 && c.J == 8) return launch_shift<BITS, GENERAL, 1, 8>(a, c.nsplit, st);
     return launch_shift<BITS, GENERAL, 2, 32>(a, c.nsplit, st);
 }
 
