@@ -328,7 +328,7 @@ def main():
         "shift_layers_images_per_s": BATCH / kernel_s,
         "roofline": {
             "bound": "valu",
-            "kernel": "ds::shift_planes_balanced_kernel<4> (16 launches) + ds::shift_kernel (5 launches) per step",
+            "kernel": "ds::shift_planes_balanced_kernel<4> (17 launches) + ds::shift_kernel (4 launches) per step",
             "achieved": pairs / kernel_s / 1e12,
             "peak": PEAK_PAIRS / 1e12,
             "unit": "Tpair/s",
