@@ -217,7 +217,7 @@ __global__ __launch_bounds__(256) void shift_kernel(const ShiftArgs p)
 }
 
 // ---------------------------------------------------------------------------------------------
-// Shift-plane variant of the kernel (R = 4 pixels x J = 32 channels per lane, fields of <= 4 bits).
+// Shift-plane variant of the kernel (R = 3 pixels x J = 32 channels per lane, fields of <= 4 bits).
 //
 // For one reduction index k and one pixel the 32 channels only ever ask for the 2^BITS values
 // x >> 0 .. x >> (2^BITS - 1).  The kernel computes these "planes" once (2^BITS vector shifts per
@@ -239,19 +239,22 @@ struct PlaneWalk {
     int koff, fw, fh, FW, FH, row_step, plane_step, koff_max;
 };
 
+constexpr int kPlaneRows = 3;      // pixels per lane (R of gen_planes_asm.py)
+constexpr int kPlaneSlots = 3072;  // wave slots of the machine at 3 waves per SIMD (256 CUs x 4 SIMDs)
+
 #define DS_PLANES_OPERANDS                                                                        \
-    : "+{v[96:111]}"(a[0]), "+{v[112:127]}"(a[1]), "+{v[128:143]}"(a[2]), "+{v[144:159]}"(a[3]),  \
-      "+{v[160:175]}"(a[4]), "+{v[176:191]}"(a[5]), "+{v[192:207]}"(a[6]), "+{v[208:223]}"(a[7])  \
-    : "v"(xoff[0]), "v"(xoff[1]), "v"(xoff[2]), "v"(xoff[3]), "s"(rsrc), "s"(wptr), "s"(groups),  \
-      "s"(w.koff), "s"(w.fw), "s"(w.fh), "s"(w.FW), "s"(w.FH), "s"(w.row_step), "s"(w.plane_step), \
+    : "+{v[66:81]}"(a[0]), "+{v[82:97]}"(a[1]), "+{v[98:113]}"(a[2]), "+{v[114:129]}"(a[3]),      \
+      "+{v[130:145]}"(a[4]), "+{v[146:161]}"(a[5])                                                \
+    : "v"(xoff[0]), "v"(xoff[1]), "v"(xoff[2]), "s"(rsrc), "s"(wptr), "s"(groups), "s"(w.koff),   \
+      "s"(w.fw), "s"(w.fh), "s"(w.FW), "s"(w.FH), "s"(w.row_step), "s"(w.plane_step),             \
       "s"(w.koff_max)
 
 template <int BITS>
-__device__ __forceinline__ void planes_main_loop(v16i (&a)[8], const uint32_t (&xoff)[4], v4i rsrc,
+__device__ __forceinline__ void planes_main_loop(v16i (&a)[6], const uint32_t (&xoff)[3], v4i rsrc,
                                                  const uint32_t *wptr, int groups, const PlaneWalk &w);
 #define DS_PLANES_SPECIALISE(B)                                                                    \
     template <>                                                                                    \
-    __device__ __forceinline__ void planes_main_loop<B>(v16i (&a)[8], const uint32_t (&xoff)[4],  \
+    __device__ __forceinline__ void planes_main_loop<B>(v16i (&a)[6], const uint32_t (&xoff)[3],  \
                                                         v4i rsrc, const uint32_t *wptr, int groups, \
                                                         const PlaneWalk &w)                        \
     {                                                                                              \
@@ -270,7 +273,7 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
                                                int g_end, bool atomic)
 {
     constexpr int NUM = 32 / (BITS + 1);
-    constexpr int R = 4, J = 32;
+    constexpr int R = kPlaneRows, J = 32;
     const int lane = threadIdx.x & (kWave - 1);
 
     uint32_t xoff[R], yoff[R];
@@ -292,9 +295,9 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
     const int g_full_end = g_end < full_groups ? g_end : full_groups;
     const uint32_t *wrow = p.wt + (size_t)ntile * p.comm * kTileWords;
 
-    v16i a[8];
+    v16i a[2 * R];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) a[i] = (v16i)(0);
+    for (int i = 0; i < 2 * R; ++i) a[i] = (v16i)(0);
     if (g_begin < g_full_end) {
         const uint64_t xaddr = (uint64_t)p.x;
         v4i rsrc;
@@ -363,14 +366,15 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
 
 // Tile-per-wave launch: gridDim.y K-slices per tile.
 template <int BITS>
-__global__ __launch_bounds__(256) void shift_planes_kernel(const ShiftArgs p)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void shift_planes_kernel(
+    const ShiftArgs p)
 {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int bid = blockIdx.x;
     const int tile = (bid & 7) * p.blocks_per_xcd + (bid >> 3);
     if (tile >= p.tiles_m4 * p.tiles_n) return;
     const int ntile = tile % p.tiles_n;
-    const int m0 = ((tile / p.tiles_n) * 4 + wave) * (4 * kWave);
+    const int m0 = ((tile / p.tiles_n) * 4 + wave) * (kPlaneRows * kWave);
     if (m0 >= p.M) return;
     const int g_begin = blockIdx.y * p.groups_per_split;
     int g_end = g_begin + p.groups_per_split;
@@ -381,9 +385,10 @@ __global__ __launch_bounds__(256) void shift_planes_kernel(const ShiftArgs p)
 // Work-balanced launch: the (tile, K group) iteration space is cut into one equal contiguous share
 // per wave, so every wave of the launch does the same number of group iterations whatever the tile
 // count (each wave touches at most a few tiles; tiles shared between waves are combined with
-// atomic adds onto the pre-filled output).  tiles_m4 holds the number of 256-pixel tiles here.
+// atomic adds onto the pre-filled output).  tiles_m4 holds the number of 192-pixel tiles here.
 template <int BITS>
-__global__ __launch_bounds__(256) void shift_planes_balanced_kernel(const ShiftArgs p)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void shift_planes_balanced_kernel(
+    const ShiftArgs p)
 {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int bid = blockIdx.x;
@@ -399,7 +404,7 @@ __global__ __launch_bounds__(256) void shift_planes_balanced_kernel(const ShiftA
         long g_end = g_begin + (it_end - it);
         if (g_end > p.comm) g_end = p.comm;
         const int ntile = tile % p.tiles_n;
-        const int m0 = (tile / p.tiles_n) * (4 * kWave);
+        const int m0 = (tile / p.tiles_n) * (kPlaneRows * kWave);
         planes_segment<BITS>(p, ntile, m0, g_begin, (int)g_end, true);
         it += g_end - g_begin;
     }
@@ -506,14 +511,14 @@ static TileChoice choose_tile(const ShiftArgs &a)
 template <int BITS>
 static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
 {
-    constexpr int R = 4, J = 32;
+    constexpr int R = kPlaneRows, J = 32;
     a.tiles_n = ceil_div(a.N, J);
     if (nsplit <= 0 && a.comm > 0) {
-        // balanced launch: one share of the iteration space per wave slot (2 waves per SIMD)
+        // balanced launch: one share of the iteration space per wave slot (3 waves per SIMD)
         a.tiles_m4 = ceil_div(a.M, R * kWave);
         a.atomic_out = 1;
         launch_fill(a, st);
-        int blocks = 512 * (nsplit < 0 ? -nsplit : 1);
+        int blocks = (kPlaneSlots / 4) * (nsplit < 0 ? -nsplit : 1);
         hipLaunchKernelGGL((shift_planes_balanced_kernel<BITS>), dim3(blocks), dim3(256), 0, st, a);
         return launch_status();
     }
@@ -539,15 +544,15 @@ static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
         // spans at least 24 (ResNet 3x3 and 7x7 layers, large GEMMs); the 1x1 shortcuts, small
         // batches and few-channel layers stay on the kernel above.
         const char *t = getenv("DS_TUNE_PLANES");
-        const long iters = (long)ceil_div(a.M, 256) * ceil_div(a.N, 32) * a.comm;
-        bool planes = a.comm >= 24 && iters >= 2048L * 24 && (a.N % 32 == 0 || a.N >= 256);
+        const long tiles = (long)ceil_div(a.M, kPlaneRows * kWave) * ceil_div(a.N, 32);
+        const long iters = tiles * a.comm;
+        bool planes = a.comm >= 24 && iters >= (long)kPlaneSlots * 16 && (a.N % 32 == 0 || a.N >= 256);
         if (t) planes = atoi(t) > 0;
         if (planes) {
-            // 2 waves per SIMD fit (2048 slots): one tile per wave when the tiles fill whole rounds
+            // 3 waves per SIMD fit (3072 slots): one tile per wave when the tiles fill whole rounds
             // of slots (no atomics, no pre-fill), otherwise equal shares of the iteration space
-            const long tiles = (long)ceil_div(a.M, 256) * ceil_div(a.N, 32);
-            const long rounds = (tiles + 2047) / 2048;
-            int nsplit = (tiles >= 2048 && (double)tiles / (2048.0 * rounds) >= 0.93) ? 1 : 0;
+            const long rounds = (tiles + kPlaneSlots - 1) / kPlaneSlots;
+            int nsplit = (tiles >= kPlaneSlots && (double)tiles / ((double)kPlaneSlots * rounds) >= 0.93) ? 1 : 0;
             if (const char *sp = getenv("DS_TUNE_SPLIT")) nsplit = atoi(sp);
             return launch_planes<BITS>(a, nsplit, st);
         }

@@ -13,22 +13,27 @@ VGPR-relative addressing (s_set_gpr_idx_*), which needs a fixed register map:
 
 so a shift-add term costs 1 + 2^BITS/32 vector instructions instead of 2.
 
-Register map (R = 4 pixels per lane, J = 32 channels, NUM = 32 // (BITS + 1) codes per word):
-    v[8 + 4*i + r]            prefetched activation of reduction slot i, row r (loaded one K group ahead)
-    v[8 + 4*NUM + P*r + s]    plane[r][s], P = 2^BITS
-    v[96 + 32*r + j]          acc[r][j]                                   (asm operands %0..%7)
+Register map (R = 3 pixels per lane, J = 32 channels, NUM = 32 // (BITS + 1) codes per word, D = depth
+of the activation prefetch ring in reduction slots, a divisor of NUM):
+    v[8 + R*(i % D) + r]      prefetched activation of reduction slot i, row r (loaded D slots ahead)
+    v[8 + R*D + P*r + s]      plane[r][s], P = 2^BITS
+    v[66 + 32*r + j]          acc[r][j]                                   (asm operands %0..%5)
+162 registers for 4-bit fields, which with the few the surrounding C++ needs stays within the 168 that
+let three waves share a SIMD.
     s[36:67]                  16-bit codes of the 32 channels for the two reduction slots being accumulated
     s[68:99]                  the next two slots' codes (in flight meanwhile)
     s4..s6                    walk over the reduction index: element offset, fw, fh of the next k to load
     s7..s15                   temporaries, loop counter, word pointer
-Operands: %8..%11 per-row byte offsets (VGPR), %12 buffer descriptor, %13 word pointer, %14 number of
-K groups, %15..%17 initial walk state (offset, fw, fh), %18 FW, %19 FH, %20 offset step when fw wraps,
-%21 offset step when fh wraps, %22 largest valid offset (the walk runs one group ahead and is clamped).
+Operands: %6..%8 per-row byte offsets (VGPR), %9 buffer descriptor, %10 word pointer, %11 number of
+K groups, %12..%14 initial walk state (offset, fw, fh), %15 FW, %16 FH, %17 offset step when fw wraps,
+%18 offset step when fh wraps, %19 largest valid offset (the walk runs D slots ahead and is clamped).
 """
 import os
 
-R, J = 4, 32
-ACC = 96
+R, J = 3, 32
+ACC = 66
+DEPTH = {1: 4, 2: 5, 3: 4, 4: 3}
+OP_XOFF, OP_RSRC, OP_WPTR, OP_GROUPS, OP_WALK = 6, 9, 10, 11, 12
 XP = 8
 W = 36
 WS = 68
@@ -44,41 +49,71 @@ def load_words():
             "s_load_dwordx16 s[%d:%d], s[%d:%d], 0x40" % (WS + 16, WS + 31, WP, WP + 1)]
 
 
-def walk_and_load(i):
-    """Issue the R loads of the walk's current k into slot i, then step the walk to k + 1."""
-    L = ["s_min_u32 s%d, s%d, %%22" % (T0, KOFF),
+def walk_and_load(slot):
+    """Issue the R loads of the walk's current k into ring slot `slot`, then step the walk to k + 1."""
+    fw_end, fh_end, row_step, plane_step, koff_max = (OP_WALK + 3, OP_WALK + 4, OP_WALK + 5, OP_WALK + 6,
+                                                      OP_WALK + 7)
+    L = ["s_min_u32 s%d, s%d, %%%d" % (T0, KOFF, koff_max),
          "s_lshl_b32 s%d, s%d, 2" % (KB, T0)]
-    L += ["buffer_load_dword v%d, %%%d, %%12, s%d offen" % (XP + 4 * i + r, 8 + r, KB) for r in range(R)]
+    L += ["buffer_load_dword v%d, %%%d, %%%d, s%d offen" % (XP + R * slot + r, OP_XOFF + r, OP_RSRC, KB)
+          for r in range(R)]
     L += ["s_add_u32 s%d, s%d, 1" % (FWC, FWC),
           "s_add_u32 s%d, s%d, 1" % (KOFF, KOFF),
-          "s_cmp_eq_u32 s%d, %%18" % FWC,
+          "s_cmp_eq_u32 s%d, %%%d" % (FWC, fw_end),
           "s_cselect_b32 s%d, 0, s%d" % (FWC, FWC),
-          "s_cselect_b32 s%d, %%20, 0" % T0,
+          "s_cselect_b32 s%d, %%%d, 0" % (T0, row_step),
           "s_cselect_b32 s%d, 1, 0" % T1,
           "s_add_u32 s%d, s%d, s%d" % (KOFF, KOFF, T0),
           "s_add_u32 s%d, s%d, s%d" % (FHC, FHC, T1),
-          "s_cmp_eq_u32 s%d, %%19" % FHC,
+          "s_cmp_eq_u32 s%d, %%%d" % (FHC, fh_end),
           "s_cselect_b32 s%d, 0, s%d" % (FHC, FHC),
-          "s_cselect_b32 s%d, %%21, 0" % T0,
+          "s_cselect_b32 s%d, %%%d, 0" % (T0, plane_step),
           "s_add_u32 s%d, s%d, s%d" % (KOFF, KOFF, T0)]
     return L
+
+
+def take_turn(tag):
+    """The waves that share a SIMD take turns at the issue priorities 2, 1, 0, by the clock: with equal
+    priorities the arbiter favours the oldest wave, which then finishes early and leaves the others
+    with a SIMD they cannot fill (a wave cannot overlap its own scalar and vector work).  The turn is
+    41 us (bit 12 of the 100 MHz counter) and is checked with every code row, because the wave that
+    should take over is the one that is running slowly."""
+    hi, mid, end = "%d" % (20 + tag), "%d" % (40 + tag), "%d" % (60 + tag)
+    return ["s_bfe_u32 s%d, s%d, 0xe000c" % (T0, TIME),          # 14 bits of turn counter
+            "s_mul_i32 s%d, s%d, 0x5556" % (T1, T0),
+            "s_lshr_b32 s%d, s%d, 16" % (T1, T1),                # turn counter / 3
+            "s_mul_i32 s%d, s%d, 3" % (T1, T1),
+            "s_sub_u32 s%d, s%d, s%d" % (T0, T0, T1),            # turn = counter mod 3
+            "s_sub_i32 s%d, s%d, s%d" % (T0, PRIO, T0),          # wave slot relative to the turn
+            "s_cmp_lt_i32 s%d, 0" % T0,
+            "s_cselect_b32 s%d, 3, 0" % T1,
+            "s_add_u32 s%d, s%d, s%d" % (T0, T0, T1),
+            "s_cmp_eq_u32 s%d, 0" % T0, "s_cbranch_scc1 %sf" % hi,
+            "s_cmp_eq_u32 s%d, 1" % T0, "s_cbranch_scc1 %sf" % mid,
+            "s_setprio 0", "s_branch %sf" % end,
+            hi + ":", "s_setprio 2", "s_branch %sf" % end,
+            mid + ":", "s_setprio 1",
+            end + ":"]
 
 
 def body(bits):
     cb = bits + 1
     num = 32 // cb
     P = 1 << bits
-    PL = XP + 4 * num
+    D = DEPTH[bits]
+    assert num % D == 0 and num % 2 == 0
+    PL = XP + R * D
     assert PL + P * R <= ACC
     L = []
-    # ---- prologue: mutable copies of the inputs, the first group's activation loads and words
-    L += ["s_getreg_b32 s%d, hwreg(HW_REG_HW_ID, 0, 1)" % PRIO,  # parity of the wave slot on its SIMD
-          "s_mov_b32 s%d, %%14" % CNT,
-          "s_mov_b64 s[%d:%d], %%13" % (WP, WP + 1),
-          "s_mov_b32 s%d, %%15" % KOFF, "s_mov_b32 s%d, %%16" % FWC, "s_mov_b32 s%d, %%17" % FHC]
+    # ---- prologue: mutable copies of the inputs, the first activation loads and code row
+    L += ["s_getreg_b32 s%d, hwreg(HW_REG_HW_ID, 0, 4)" % PRIO,  # the wave's slot on its SIMD
+          "s_mov_b32 s%d, %%%d" % (CNT, OP_GROUPS),
+          "s_mov_b64 s[%d:%d], %%%d" % (WP, WP + 1, OP_WPTR),
+          "s_mov_b32 s%d, %%%d" % (KOFF, OP_WALK), "s_mov_b32 s%d, %%%d" % (FWC, OP_WALK + 1),
+          "s_mov_b32 s%d, %%%d" % (FHC, OP_WALK + 2)]
     L += load_words()
     L += ["s_memrealtime s[%d:%d]" % (TIME, TIME + 1)]
-    for i in range(num):
+    for i in range(D):
         L += walk_and_load(i)
     L += ["s_mov_b32 s%d, 0" % IDX, "s_set_gpr_idx_on s%d, 0x1" % IDX]  # src0 of vector ops is M0-relative
     # ---- one K group per iteration, two reduction slots (one row of 16-bit codes) at a time
@@ -89,23 +124,17 @@ def body(bits):
             # row past the end reads the spare row that follows the codes in the weight blob)
             L += ["s_add_u32 s%d, s%d, 128" % (WP, WP), "s_addc_u32 s%d, s%d, 0" % (WP + 1, WP + 1),
                   "s_waitcnt lgkmcnt(0)"]
-            # The two waves that share a SIMD take turns at the higher issue priority, by the clock:
-            # bit 12 of the 100 MHz counter (41 us each) against the parity of the wave's slot.  With
-            # equal priorities the arbiter favours the older wave, which then finishes early and
-            # leaves the other alone on the SIMD.  The turn is checked every row, because the wave
-            # that should take over is the one that is running slowly.
-            L += ["s_bfe_u32 s%d, s%d, 0x1000c" % (T0, TIME), "s_cmp_eq_u32 s%d, s%d" % (T0, PRIO),
-                  "s_cbranch_scc0 %df" % (3 + i), "s_setprio 2", "s_branch %df" % (4 + i),
-                  "%d:" % (3 + i), "s_setprio 0", "%d:" % (4 + i)]
+            L += take_turn(i // 2)
             L += ["s_mov_b64 s[%d:%d], s[%d:%d]" % (W + 2 * q, W + 2 * q + 1, WS + 2 * q, WS + 2 * q + 1)
                   for q in range(16)]
             L += load_words()
             L += ["s_memrealtime s[%d:%d]" % (TIME, TIME + 1)]  # read when the next row arrives
-        L += ["s_waitcnt vmcnt(%d)" % (4 * (num - 1))]
+        slot = i % D
+        L += ["s_waitcnt vmcnt(%d)" % (R * (D - 1))]
         # plane 0 = the activation itself (a shift by 0 keeps src0 a constant: not M0-relative)
         for r in range(R):
-            L += ["v_ashrrev_i32 v%d, 0, v%d" % (PL + P * r, XP + 4 * i + r)]
-        L += walk_and_load(i)  # the same slot of the next group
+            L += ["v_ashrrev_i32 v%d, 0, v%d" % (PL + P * r, XP + R * slot + r)]
+        L += walk_and_load(slot)  # the ring slot is free again: load reduction slot i + D into it
         for s in range(1, P):
             for r in range(R):
                 L += ["v_ashrrev_i32 v%d, %d, v%d" % (PL + P * r + s, s, PL + P * r)]
@@ -120,7 +149,7 @@ def body(bits):
                 a = ACC + 32 * r + j
                 L += ["v_xad_u32 v%d, v%d, s%d, v%d" % (a, PL + P * r, MASK, a)]
     L += ["s_sub_u32 s%d, s%d, 1" % (CNT, CNT), "s_cmp_lg_u32 s%d, 0" % CNT, "s_cbranch_scc1 1b"]
-    # ---- leave relative addressing, drain the loads issued for the group after the last one
+    # ---- leave relative addressing, drain the loads that ran ahead of the last slot
     L += ["s_set_gpr_idx_off", "s_setprio 0", "s_waitcnt vmcnt(0) lgkmcnt(0)"]
     return L
 
@@ -128,7 +157,7 @@ def body(bits):
 def clobbers(bits):
     num = 32 // (bits + 1)
     P = 1 << bits
-    v = ['"v%d"' % n for n in range(XP, XP + 4 * num + P * R)]
+    v = ['"v%d"' % n for n in range(XP, XP + R * DEPTH[bits] + P * R)]
     s = ['"s%d"' % n for n in list(range(4, 16)) + list(range(W, WS + 32)) + [TIME, TIME + 1]]
     return ", ".join(v + s + ['"scc"', '"memory"'])
 
