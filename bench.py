@@ -337,7 +337,7 @@ def main():
             # this size): 106.9 MB read + 117.4 MB of atomic partial sums, from the FETCH_SIZE /
             # WRITE_SIZE runs summarised in profiles/shift_kernel_layer1_conv_counters.md
             # (106.6 MB algorithmic)
-            "traffic": 224.3e6,
+            "traffic": 257.4e6,
             "avg_launch_us": kernel_s / len(layers) * 1e6,
             "peak_calibrated": peak_cal / 1e12 if peak_cal else None,
             "frac_of_calibrated": pairs / kernel_s / peak_cal if peak_cal else None,
