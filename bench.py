@@ -334,10 +334,13 @@ def main():
             "unit": "Tpair/s",
             "frac": pairs / kernel_s / PEAK_PAIRS,
             # HBM bytes of one launch of the dominant shape (layer1 3x3 conv, 8 of the 21 launches are
-            # this size): 106.9 MB read + 117.4 MB of atomic partial sums, from the FETCH_SIZE /
+            # this size): 125.3 MB read + 132.1 MB of atomic partial sums, from the FETCH_SIZE /
             # WRITE_SIZE runs summarised in profiles/shift_kernel_layer1_conv_counters.md
             # (106.6 MB algorithmic)
             "traffic": 257.4e6,
+            # vector instructions the dominant kernel issues per pair (SQ_INSTS_VALU, same profile):
+            # `peak` prices a pair at 2 instructions, so its fraction can exceed 1
+            "valu_instr_per_pair": 1.53,
             "avg_launch_us": kernel_s / len(layers) * 1e6,
             "peak_calibrated": peak_cal / 1e12 if peak_cal else None,
             "frac_of_calibrated": pairs / kernel_s / peak_cal if peak_cal else None,
