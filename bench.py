@@ -165,6 +165,13 @@ def config2(device, reps=10):
     t = timeit(lambda: kernels.conv2d_tiled(xq, tiled, None, 64, (3, 3), (1, 1), cw.bits, cw.base))
     pairs = 32 * 56 * 56 * 576 * 64
     out["conv3x3_64x64_32x56x56"] = dict(ms=t * 1e3, gops=2 * pairs / t / 1e9, valu_frac=pairs / t / PEAK_PAIRS)
+    # the float multiply-accumulate comparator on the same shape (kernel only, padded input resident)
+    from deepshift_amd.unoptimized import kernels as float_kernels
+    import torch.nn.functional as F
+    wf = torch.randn(64, 64, 3, 3, generator=g).to(device)
+    xp = F.pad(x, (1, 1, 1, 1))
+    tf = timeit(lambda: float_kernels.conv2d(xp, wf, None, (1, 1), (1, 1)))
+    out["conv3x3_64x64_32x56x56"].update(float_multiply_ms=tf * 1e3, shift_over_float_multiply=t / tf)
 
     x = torch.randn(4096, 4096, generator=g).clamp_min(0).to(device)
     shift, sign = codes((4096, 4096))
@@ -174,6 +181,9 @@ def config2(device, reps=10):
     t = timeit(lambda: kernels.linear_tiled(xT, 4096, tiled, None, 4096, cw.bits, cw.base))
     pairs = 4096 ** 3
     out["gemm_4096"] = dict(ms=t * 1e3, gops=2 * pairs / t / 1e9, valu_frac=pairs / t / PEAK_PAIRS)
+    wf = torch.randn(4096, 4096, generator=g).to(device)
+    tf = timeit(lambda: float_kernels.linear(x, wf, None))  # includes its input transpose
+    out["gemm_4096"].update(float_multiply_ms=tf * 1e3, shift_over_float_multiply=t / tf)
     return out
 
 

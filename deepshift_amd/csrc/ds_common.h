@@ -67,5 +67,7 @@ int launch_pack(const int32_t *s, const int32_t *sign, int32_t *out, int O, int 
 int launch_tile(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW, int bits,
                 hipStream_t st);
 int launch_transpose(const int32_t *x, int32_t *xT, int M, int K, int ldx, hipStream_t st);
+// the same with rows of x ldin elements apart
+int launch_transpose_strided(const int32_t *x, int ldin, int32_t *xT, int M, int K, int ldx, hipStream_t st);
 
 }  // namespace ds

@@ -127,14 +127,14 @@ __global__ __launch_bounds__(256) void quantize_transpose_kernel(const float *__
 
 __global__ __launch_bounds__(256) void transpose_i32_kernel(const int32_t *__restrict__ x,
                                                             int32_t *__restrict__ xT, int M, int K,
-                                                            int ldx)
+                                                            int ldx, int ldin)
 {
     __shared__ int32_t tile[64][65];
     const int k0 = blockIdx.x * 64, m0 = blockIdx.y * 64;
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
     for (int r = ty; r < 64; r += 4) {
         const int m = m0 + r, k = k0 + tx;
-        tile[r][tx] = (m < M && k < K) ? x[(long)m * K + k] : 0;
+        tile[r][tx] = (m < M && k < K) ? x[(long)m * ldin + k] : 0;
     }
     __syncthreads();
     for (int r = ty; r < 64; r += 4) {
@@ -146,7 +146,14 @@ __global__ __launch_bounds__(256) void transpose_i32_kernel(const int32_t *__res
 int launch_transpose(const int32_t *x, int32_t *xT, int M, int K, int ldx, hipStream_t st)
 {
     dim3 grid(ceil_div(K, 64), ceil_div(ldx, 64));
-    hipLaunchKernelGGL(transpose_i32_kernel, grid, dim3(256), 0, st, x, xT, M, K, ldx);
+    hipLaunchKernelGGL(transpose_i32_kernel, grid, dim3(256), 0, st, x, xT, M, K, ldx, K);
+    return launch_status();
+}
+
+int launch_transpose_strided(const int32_t *x, int ldin, int32_t *xT, int M, int K, int ldx, hipStream_t st)
+{
+    dim3 grid(ceil_div(K, 64), ceil_div(ldx, 64));
+    hipLaunchKernelGGL(transpose_i32_kernel, grid, dim3(256), 0, st, x, xT, M, K, ldx, ldin);
     return launch_status();
 }
 

@@ -49,7 +49,25 @@ struct ShiftArgs {
     int tiles_n;                          // number of channel tiles
     int blocks_per_xcd;                   // ceil(tiles / 8)
     int atomic_out;                       // 1: y pre-filled with bias, accumulate atomically
+    // LinearShift only: channel-major scratch [N][alt_ld] for launches that combine partial sums.
+    // y[M][N] puts the 64 rows of a wave 4*N bytes apart, one cache line per lane and atomic; the
+    // scratch keeps them adjacent, and a transpose writes y afterwards.
+    int32_t *alt_y;
+    int alt_ld;
+    uint32_t y_elems;                     // elements the pre-fill covers
 };
+
+// Redirects an atomic LinearShift launch to its channel-major scratch; returns the final y or nullptr.
+static int32_t *redirect_to_scratch(ShiftArgs &a)
+{
+    if (!a.alt_y) return nullptr;
+    int32_t *final_y = a.y;
+    a.y = a.alt_y;
+    a.y_pix_stride = 1;
+    a.y_ch_stride = a.alt_ld;
+    a.y_elems = (uint32_t)a.N * (uint32_t)a.alt_ld;
+    return final_y;
+}
 
 // (t ^ mask) + acc in ONE vector instruction with the wave-uniform mask read from a scalar
 // register.  Spelled as v_xad_u32 because the compiler otherwise re-associates pairs of terms into
@@ -414,7 +432,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 // are dense, so the flat index is the address and n = (idx / y_ch_stride) % N.
 __global__ void fill_bias_kernel(const ShiftArgs p)
 {
-    const uint32_t total = (uint32_t)p.M * (uint32_t)p.N;  // < 2^29: tensors are below 2 GiB
+    const uint32_t total = p.y_elems;  // < 2^29: tensors are below 2 GiB
     for (uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
         const int n = (int)((idx / (uint32_t)p.y_ch_stride) % (uint32_t)p.N);
         p.y[idx] = p.negcnt[n] + (p.bias ? p.bias[n] : 0);
@@ -425,7 +443,7 @@ __global__ void fill_bias_kernel(const ShiftArgs p)
 // their channel (y_ch_stride % 4 == 0) or step through channels (y_ch_stride == 1, N % 4 == 0).
 __global__ void fill_bias4_kernel(const ShiftArgs p)
 {
-    const uint32_t total4 = ((uint32_t)p.M * (uint32_t)p.N) >> 2;
+    const uint32_t total4 = p.y_elems >> 2;
     int4 *y4 = (int4 *)p.y;
     for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < total4; i += gridDim.x * blockDim.x) {
         const uint32_t idx = i << 2;
@@ -445,7 +463,7 @@ __global__ void fill_bias4_kernel(const ShiftArgs p)
 
 static void launch_fill(const ShiftArgs &a, hipStream_t st)
 {
-    const long total = (long)a.M * a.N;
+    const long total = (long)a.y_elems;
     const bool vec = ((uintptr_t)a.y & 15) == 0 && total % 4 == 0 &&
                      (a.y_ch_stride % 4 == 0 || (a.y_ch_stride == 1 && a.N % 4 == 0));
     long blocks = vec ? (total / 4 + 255) / 256 : (total + 255) / 256;
@@ -468,9 +486,14 @@ static int launch_shift(ShiftArgs a, int nsplit, hipStream_t st)
     a.groups_per_split = a.comm == 0 ? 1 : ceil_div(a.comm, nsplit);
     nsplit = a.comm == 0 ? 1 : ceil_div(a.comm, a.groups_per_split);
     a.atomic_out = nsplit > 1;
-    if (a.atomic_out) launch_fill(a, st);
+    int32_t *final_y = nullptr;
+    if (a.atomic_out) {
+        final_y = redirect_to_scratch(a);
+        launch_fill(a, st);
+    }
     dim3 grid(a.blocks_per_xcd * 8, nsplit);
     hipLaunchKernelGGL((shift_kernel<BITS, GENERAL, R, J>), grid, dim3(256), 0, st, a);
+    if (final_y) return launch_transpose_strided(a.y, a.alt_ld, final_y, a.N, a.M, a.N, st);
     return launch_status();
 }
 
@@ -517,9 +540,11 @@ static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
         // balanced launch: one share of the iteration space per wave slot (3 waves per SIMD)
         a.tiles_m4 = ceil_div(a.M, R * kWave);
         a.atomic_out = 1;
+        int32_t *final_y = redirect_to_scratch(a);
         launch_fill(a, st);
         int blocks = (kPlaneSlots / 4) * (nsplit < 0 ? -nsplit : 1);
         hipLaunchKernelGGL((shift_planes_balanced_kernel<BITS>), dim3(blocks), dim3(256), 0, st, a);
+        if (final_y) return launch_transpose_strided(a.y, a.alt_ld, final_y, a.N, a.M, a.N, st);
         return launch_status();
     }
     a.tiles_m4 = ceil_div(ceil_div(a.M, R * kWave), 4);
@@ -529,9 +554,14 @@ static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
     a.groups_per_split = a.comm == 0 ? 1 : ceil_div(a.comm, nsplit);
     nsplit = a.comm == 0 ? 1 : ceil_div(a.comm, a.groups_per_split);
     a.atomic_out = nsplit > 1;
-    if (a.atomic_out) launch_fill(a, st);
+    int32_t *final_y = nullptr;
+    if (a.atomic_out) {
+        final_y = redirect_to_scratch(a);
+        launch_fill(a, st);
+    }
     dim3 grid(a.blocks_per_xcd * 8, nsplit);
     hipLaunchKernelGGL((shift_planes_kernel<BITS>), grid, dim3(256), 0, st, a);
+    if (final_y) return launch_transpose_strided(a.y, a.alt_ld, final_y, a.N, a.M, a.N, st);
     return launch_status();
 }
 
@@ -647,6 +677,7 @@ DS_EXPORT int ds_conv2d_tiled_i32(const int32_t *x, const void *tiled, const int
     a.pix_per_img = OH * OW; a.OW = OW;
     a.x_img_stride = C * Hp * Wp; a.x_row_stride = sh * Wp; a.x_col_stride = sw;
     a.y_img_stride = O * OH * OW; a.y_pix_stride = 1; a.y_ch_stride = OH * OW;
+    a.y_elems = (uint32_t)a.M * (uint32_t)a.N;
     a.ktab = tiled_ktab(tiled, g);
     a.x_plane = Hp * Wp; a.x_row = Wp;
     a.FH = FH; a.FW = FW;
@@ -678,27 +709,38 @@ DS_EXPORT int ds_conv2d_i32(const int32_t *x, const int32_t *w_ref, const int32_
 // LinearShift
 // ---------------------------------------------------------------------------------------------
 
+// Channel-major scratch for launches that combine partial sums (see ShiftArgs::alt_y); a single
+// wave of rows never needs it.
+static size_t linear_scratch_bytes(int M, int N)
+{
+    if (M <= kWave || N <= 0) return 0;
+    return align_up((size_t)N * align_up((size_t)M, 64) * 4, 256);
+}
+
 DS_EXPORT size_t ds_linear_tiled_workspace_bytes(int M, int K, int N, int bits)
 {
-    (void)M; (void)K; (void)N; (void)bits;
-    return 0;  // the tiled entry point needs no scratch memory
+    (void)K;
+    if (bits < 1 || bits > 6 || M < 0 || N < 0) return 0;
+    return linear_scratch_bytes(M, N);
 }
 
 DS_EXPORT size_t ds_linear_workspace_bytes(int M, int K, int N, int bits)
 {
     if (bits < 1 || bits > 6 || M < 0 || K < 0 || N < 0) return 0;
     const size_t ldx = align_up((size_t)M, 64);
-    return align_up(tiled_geom(N, K, bits).bytes, 256) + align_up(ldx * K * 4, 256);
+    return align_up(tiled_geom(N, K, bits).bytes, 256) + align_up(ldx * K * 4, 256) +
+           linear_scratch_bytes(M, N);
 }
 
 DS_EXPORT int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled, const int32_t *bias,
                                   int32_t *y, int M, int K, int N, int bits, int base,
                                   void *workspace, size_t workspace_bytes, ds_stream_t stream)
 {
-    (void)workspace; (void)workspace_bytes;
     int rc = check_common(bits, base);
     if (rc) return rc;
     if (M < 0 || K < 0 || N < 0 || ldx < M) return DS_EINVAL;
+    const size_t scratch = linear_scratch_bytes(M, N);
+    if (scratch && (!workspace || workspace_bytes < scratch)) return DS_EWORKSPACE;
     if (M == 0 || N == 0) return DS_OK;
     if (!tiled || !y || (!xT && K > 0)) return DS_EINVAL;
     const size_t x_bytes = (size_t)ldx * K * 4;
@@ -718,6 +760,11 @@ DS_EXPORT int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled,
     a.pix_per_img = M; a.OW = M;
     a.x_img_stride = 0; a.x_row_stride = 0; a.x_col_stride = 1;
     a.y_img_stride = 0; a.y_pix_stride = N; a.y_ch_stride = 1;
+    a.y_elems = (uint32_t)M * (uint32_t)N;
+    if (scratch && (size_t)N * align_up((size_t)M, 64) * 4 < kMaxBytes) {
+        a.alt_y = (int32_t *)workspace;
+        a.alt_ld = (int)align_up((size_t)M, 64);
+    }
     a.ktab = tiled_ktab(tiled, g);
     a.x_plane = ldx; a.x_row = 1;
     a.FH = 1; a.FW = 1;
@@ -749,5 +796,8 @@ DS_EXPORT int ds_linear_i32(const int32_t *x, const int32_t *w_ref, const int32_
         rc = launch_transpose(x, xT, M, K, ldx, st);
         if (rc) return rc;
     }
-    return ds_linear_tiled_i32(xT, ldx, tiled, bias, y, M, K, N, bits, base, nullptr, 0, stream);
+    const size_t scratch = linear_scratch_bytes(M, N);
+    return ds_linear_tiled_i32(xT, ldx, tiled, bias, y, M, K, N, bits, base,
+                               scratch ? (char *)xT + align_up((size_t)ldx * K * 4, 256) : nullptr, scratch,
+                               stream);
 }

@@ -161,6 +161,30 @@ int ds_requantize_affine_pad_i32(const int32_t *y, float *out, int32_t *q, const
                                  int ph, int pw, int F_in, int relu, int I, int F, int mode,
                                  ds_stream_t stream);
 
+/* ---- float multiply comparator -------------------------------------------------------------
+ * The reference ships plain float multiply-accumulate kernels of the same structure as its shift
+ * kernels to compare "shift against multiply" on one machine (UNOPTIMIZED_LINEAR /
+ * UNOPTIMIZED_CONV, kernels/cuda/unoptimized_cuda.cpp:20-51, unoptimized.cu:63-103).  These entry
+ * points are that comparator: the data movement of the shift kernel with one fused multiply-add
+ * per term.  fp32 accumulation in reduction order k = 0..K-1 per output element. */
+
+/* Bytes of the tiled float weights for ds_mul_*_f32 (0 for non-positive N or K). */
+size_t ds_mul_tiled_bytes(int N, int K);
+
+/* w [N][C*FH*FW] float (nn.Linear / nn.Conv2d weight, flattened) -> tiled blob. */
+int ds_mul_tile_weights_f32(const float *w, void *tiled, int N, int C, int FH, int FW,
+                            ds_stream_t stream);
+
+/* Replaces UNOPTIMIZED_CONV (unoptimized_cuda.cpp:34-46): x_padded [Nb][C][Hp][Wp] float (already
+ * padded, as unoptimized/modules/conv.py:87 passes it), y [Nb][O][OH][OW], bias [O] or NULL. */
+int ds_mul_conv2d_f32(const float *x_padded, const void *tiled, const float *bias, float *y, int Nb,
+                      int C, int Hp, int Wp, int O, int FH, int FW, int sh, int sw, ds_stream_t stream);
+
+/* Replaces UNOPTIMIZED_LINEAR (unoptimized_cuda.cpp:20-32): xT [K][ldx] float (transposed
+ * activations, ldx >= M; ds_transpose_i32 moves the 32-bit patterns), y [M][N], bias [N] or NULL. */
+int ds_mul_linear_f32(const float *xT, int ldx, const void *tiled, const float *bias, float *y, int M,
+                      int K, int N, ds_stream_t stream);
+
 /* ---- measurement ----------------------------------------------------------------------- */
 
 /* VALU calibration: every lane of `blocks` x 256 threads runs `iters` x 64 independent

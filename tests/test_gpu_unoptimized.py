@@ -1,0 +1,83 @@
+"""The float multiply-accumulate comparator (deepshift_amd.unoptimized) against PyTorch's own fp32
+linear / conv2d.  The kernel accumulates in reduction order k = 0..K-1 in fp32, PyTorch in another
+order, so the comparison allows K * eps_fp32 relative to the magnitude of the terms."""
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+pytestmark = pytest.mark.gpu
+
+if not torch.cuda.is_available():  # pragma: no cover
+    pytest.skip("needs a GPU", allow_module_level=True)
+
+from deepshift_amd import unoptimized, workloads  # noqa: E402
+from deepshift_amd.unoptimized import kernels as uk  # noqa: E402
+
+DEV = torch.device("cuda:0")
+
+
+def _tol(K, x, w):
+    # |sum of K products| rounding: each of the K additions may lose 2^-24 of the running magnitude
+    return K * 2.0 ** -23 * float(x.abs().max()) * float(w.detach().abs().max()) * 4 + 1e-6
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 1, 1), (64, 784, 512), (100, 37, 10), (7, 130, 33), (300, 64, 96),
+                                   (65, 3, 1000)])
+def test_linear_matches_torch(M, K, N):
+    g = torch.Generator().manual_seed(M * 131 + K)
+    x = torch.randn(M, K, generator=g).to(DEV)
+    w = torch.randn(N, K, generator=g).to(DEV)
+    b = torch.randn(N, generator=g).to(DEV)
+    got = uk.linear(x, w, b)
+    want = F.linear(x.double(), w.double(), b.double())
+    assert (got.double() - want).abs().max().item() <= _tol(K, x, w)
+    got = uk.linear(x, w, None)
+    want = F.linear(x.double(), w.double())
+    assert (got.double() - want).abs().max().item() <= _tol(K, x, w)
+
+
+@pytest.mark.parametrize("Nb,C,H,W,O,FH,FW,stride,pad", [
+    (2, 3, 32, 32, 16, 3, 3, 1, 1), (1, 3, 37, 29, 8, 7, 7, 2, 3), (3, 16, 14, 14, 40, 1, 1, 2, 0),
+    (2, 5, 9, 11, 33, 3, 2, 1, 0), (1, 64, 8, 8, 64, 3, 3, 1, 1), (4, 1, 5, 5, 1, 5, 5, 1, 2)])
+def test_conv2d_matches_torch(Nb, C, H, W, O, FH, FW, stride, pad):
+    g = torch.Generator().manual_seed(C * 17 + O)
+    conv = nn.Conv2d(C, O, (FH, FW), stride=stride, padding=pad).to(DEV)
+    x = torch.randn(Nb, C, H, W, generator=g).to(DEV)
+    mine = unoptimized.UnoptimizedConv2d(C, O, (FH, FW), stride=stride, padding=pad).to(DEV)
+    mine.weight, mine.bias = conv.weight, conv.bias
+    with torch.no_grad():
+        got = mine(x)
+        want = F.conv2d(x.double(), conv.weight.double(), conv.bias.double(), stride=stride, padding=pad)
+    assert got.shape == want.shape
+    assert (got.double() - want).abs().max().item() <= _tol(C * FH * FW, x, conv.weight)
+
+
+def test_non_finite_inputs_do_not_leak_through_the_reduction_tail():
+    """K = 5 is not a multiple of the kernel's group of 4: the padded reduction rows must not read x."""
+    x = torch.full((70, 5), float("inf"), device=DEV)
+    x[:, 1:] = 1.0
+    w = torch.zeros(3, 5, device=DEV)
+    w[:, 1:] = 2.0
+    got = uk.linear(x, w, None)  # inf * 0 = nan only in column 0, which is real data
+    assert torch.isnan(got).all()
+    x[:, 0] = 3.0
+    assert torch.equal(uk.linear(x, w, None), torch.full((70, 3), 8.0, device=DEV))
+
+
+def test_convert_to_unoptimized_keeps_the_model_function():
+    g = torch.Generator().manual_seed(3)
+    model = workloads.randomize_batchnorm(workloads.ResNet20(), g).eval().to(DEV)
+    x = torch.randn(4, 3, 32, 32, generator=g).to(DEV)
+    with torch.no_grad():
+        want = model(x)
+        n_layers = sum(isinstance(m, (nn.Conv2d, nn.Linear)) for m in model.modules())
+        conv = unoptimized.convert_to_unoptimized(model)
+        got = conv(x)
+    assert sum(isinstance(m, (unoptimized.UnoptimizedConv2d, unoptimized.UnoptimizedLinear))
+               for m in conv.modules()) == n_layers
+    assert not any(type(m) in (nn.Conv2d, nn.Linear) for m in conv.modules())
+    torch.testing.assert_close(got, want, rtol=1e-4, atol=1e-4)
+    with pytest.raises(NotImplementedError):
+        unoptimized.convert_to_unoptimized(nn.Sequential(nn.Linear(4, 4)))(torch.zeros(2, 4))
