@@ -709,11 +709,10 @@ DS_EXPORT int ds_conv2d_i32(const int32_t *x, const int32_t *w_ref, const int32_
 // LinearShift
 // ---------------------------------------------------------------------------------------------
 
-// Channel-major scratch for launches that combine partial sums (see ShiftArgs::alt_y); a single
-// wave of rows never needs it.
+// Channel-major scratch for launches that combine partial sums (see ShiftArgs::alt_y).
 static size_t linear_scratch_bytes(int M, int N)
 {
-    if (M <= kWave || N <= 0) return 0;
+    if (M <= 0 || N <= 0) return 0;
     return align_up((size_t)N * align_up((size_t)M, 64) * 4, 256);
 }
 
