@@ -246,6 +246,80 @@ def test_conv_split_k_path(oracle, rng):
     np.testing.assert_array_equal(abi_conv(xp, w, bias, O, 3, 3, (1, 1), 4), want)
 
 
+# ----------------------------------------------------------------------------- kernel variants
+
+class _Tune:
+    """Forces a kernel variant through the library's DS_TUNE_* environment overrides."""
+
+    def __init__(self, **kv):
+        self.kv = {k: str(v) for k, v in kv.items()}
+
+    def __enter__(self):
+        self.old = {k: os.environ.get(k) for k in self.kv}
+        os.environ.update(self.kv)
+
+    def __exit__(self, *exc):
+        for k, v in self.old.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+
+
+# split 0: equal shares of the (tile, K group) space; 1: one tile per wave; 3: tiles with K cut in 3
+@pytest.mark.parametrize("split", [0, 1, 3])
+@pytest.mark.parametrize("bits", [1, 2, 3, 4])
+def test_shift_plane_kernel_every_field_width_and_launch(oracle, rng, bits, split):
+    """The shift-plane kernel is normally chosen for large layers only; force it on shapes with ragged
+    pixel counts, channel counts that do not fill a tile and reductions with a partial last word."""
+    with _Tune(DS_TUNE_PLANES=1, DS_TUNE_SPLIT=split):
+        # convolution, stride 2, 40 channels (a 32-channel tile and a quarter), K = 5*3*3 = 45
+        Nb, C, Hp, Wp, O = 3, 5, 21, 17, 40
+        xp = random_activations(rng, (Nb, C, Hp, Wp))
+        s, sign = random_codes(rng, (O, C, 3, 3), max_s=2 ** bits - 1)
+        bias = rng.integers(-2 ** 31, 2 ** 31 - 1, size=O, dtype=np.int64).astype(np.int32)
+        w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)
+        want = oracle.conv2d(xp, -s, sign, bias, (2, 2), nthreads=NTHREADS)
+        np.testing.assert_array_equal(abi_conv(xp, w, bias, O, 3, 3, (2, 2), bits), want)
+        # convolution, 1x1 and 5x2 filters, several pixel tiles
+        for (FH, FW, stride) in [(1, 1, (1, 1)), (5, 2, (1, 2))]:
+            Nb, C, Hp, Wp, O = 2, 19, 23, 20, 33
+            xp = random_activations(rng, (Nb, C, Hp, Wp))
+            s, sign = random_codes(rng, (O, C, FH, FW), max_s=2 ** bits - 1)
+            w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)
+            want = oracle.conv2d(xp, -s, sign, None, stride, nthreads=NTHREADS)
+            np.testing.assert_array_equal(abi_conv(xp, w, None, O, FH, FW, stride, bits), want)
+        # GEMM with every dimension ragged
+        M, K, N = 333, 517, 71
+        x = random_activations(rng, (M, K))
+        s, sign = random_codes(rng, (N, K), max_s=2 ** bits - 1)
+        bias = rng.integers(-2 ** 20, 2 ** 20, size=N).astype(np.int32)
+        w, _ = oracle.pack_words(s, sign, bits)
+        want = oracle.linear(x, -s, sign, bias, nthreads=NTHREADS)
+        np.testing.assert_array_equal(abi_linear(x, w, bias, N, bits), want)
+
+
+@pytest.mark.parametrize("tile", ["2x32", "4x16", "3x16", "1x32", "1x8"])
+@pytest.mark.parametrize("split", [1, 4])
+def test_two_instruction_kernel_every_tile_shape(oracle, rng, tile, split):
+    with _Tune(DS_TUNE_PLANES=0, DS_TUNE_TILE=tile, DS_TUNE_SPLIT=split):
+        Nb, C, Hp, Wp, O = 2, 11, 19, 22, 45
+        xp = random_activations(rng, (Nb, C, Hp, Wp))
+        s, sign = random_codes(rng, (O, C, 3, 3), max_s=15)
+        bias = rng.integers(-2 ** 31, 2 ** 31 - 1, size=O, dtype=np.int64).astype(np.int32)
+        w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), 4)
+        want = oracle.conv2d(xp, -s, sign, bias, (1, 2), nthreads=NTHREADS)
+        np.testing.assert_array_equal(abi_conv(xp, w, bias, O, 3, 3, (1, 2), 4), want)
+        M, K, N = 130, 200, 77
+        x = random_activations(rng, (M, K))
+        s, sign = random_codes(rng, (N, K), max_s=31, zero_frac=0.2)  # ternary: the general variant
+        s_z = np.where(sign == 0, 32, s).astype(np.int32)
+        sign_z = np.where(sign == 0, 1, sign).astype(np.int32)
+        w = so.np_pack_words(s_z, sign_z, 6)
+        want = oracle.linear(x, -s, sign, None, nthreads=NTHREADS)
+        np.testing.assert_array_equal(abi_linear(x, w, None, N, 6), want)
+
+
 # ----------------------------------------------------------------------------- fixed point
 
 def _float_samples(rng, n):
