@@ -282,3 +282,49 @@ def test_dequantize_affine_matches_torch(rng):
     y2 = y[:, :, :, :3].contiguous()  # HW not a multiple of 4: scalar path
     got = kernels.dequantize_affine(y2, 16, scale, None, None, relu=False)
     torch.testing.assert_close(got, y2.float() / 65536 * scale.view(1, -1, 1, 1), rtol=1e-6, atol=1e-6)
+
+
+def test_packed_export_round_trip(tmp_path):
+    """export.save_packed / load_packed: a freshly built model that only receives the packed words
+    (its float shift/sign parameters are different random values) reproduces the outputs bit for bit."""
+    from deepshift_amd import export
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(3, 3, 32, 32, generator=g).to(DEV)
+    src = workloads.randomize_batchnorm(workloads.ResNet20(), g).eval()
+    src, n = convert.convert_to_shift(src, 1000, 'PS', convert_weights=True, use_kernel=True)
+    src = src.to(DEV)
+    with torch.no_grad():
+        want = src(x)
+    path = str(tmp_path / "packed.pt")
+    export.save_packed(src, path)
+    blob = torch.load(path, weights_only=True)
+    n = sum(isinstance(m, (modules.Conv2dShift, modules.LinearShift)) for m in src.modules())
+    assert blob["format"] == export.FORMAT and len(blob["layers"]) == n == 20
+    dst = workloads.ResNet20().eval()
+    dst, _ = convert.convert_to_shift(dst, 1000, 'PS', convert_weights=True, use_kernel=False)
+    dst.load_state_dict({k: v for k, v in src.state_dict().items() if "shift" not in k and "sign" not in k},
+                        strict=False)  # BatchNorm statistics and biases; not the shift/sign parameters
+    dst = dst.to(DEV)
+    assert export.load_packed(dst, path) == n
+    with torch.no_grad():
+        got = dst(x)
+    assert torch.equal(got, want)
+
+
+def test_evaluate_cli_runs_the_three_modes(tmp_path, capsys):
+    from deepshift_amd import evaluate
+    r = evaluate.main(["-e", "-a", "mlp", "--use-kernel", "True", "--iterations", "2", "--json"])
+    assert r["converted_layers"] == 3 and r["mode"] == "shift kernels"
+    assert r["max_abs_diff_vs_float_shift_path"] <= 784 * 2.0 ** -16 * 4 + 1e-3 * r["output_scale"]
+    packed = str(tmp_path / "p.pt")
+    r = evaluate.main(["-e", "-a", "resnet20", "--use-kernel", "True", "--batch-size", "4", "--iterations", "1",
+                       "--export-packed", packed, "--json"])
+    assert r["converted_layers"] == 20 and r["images_per_s"] > 0
+    assert r["max_abs_diff_vs_float_shift_path"] <= 0.02 * r["output_scale"] + 1e-3
+    r2 = evaluate.main(["-e", "-a", "resnet20", "--use-kernel", "True", "--batch-size", "4", "--iterations", "1",
+                        "--packed", packed, "--json"])
+    assert r2["packed_layers_loaded"] == 20
+    r = evaluate.main(["-e", "-a", "resnet20", "--use-kernel", "True", "--shift-depth", "0", "--batch-size", "4",
+                       "--iterations", "1", "--json"])
+    assert r["mode"] == "float multiply comparator" and r["max_abs_diff_vs_pytorch"] < 1e-3
+    capsys.readouterr()

@@ -160,3 +160,28 @@ def test_fused_graph_hands_fixed_point_tensors_on():
     assert all(e[:3] == ((1, 1), 16, 16) for e in emits)
     plain = fuse.fuse_conv_epilogues(model, handoff=False)
     assert not any(m.prequantized or m.emit for m in plain.modules() if isinstance(m, fuse.FusedConv2dShift))
+
+
+def test_evaluate_cli_arguments_and_refusals():
+    from deepshift_amd import evaluate
+    args = evaluate.build_parser().parse_args(["-e", "-a", "resnet20", "--use-kernel", "True", "-wb", "3",
+                                               "-ab", "3", "5", "--shift-depth", "0"])
+    assert args.evaluate and args.use_kernel is True and args.activation_bits == [3, 5]
+    assert args.arch == "resnet20" and args.shift_depth == 0 and args.weight_bits == 3
+    with pytest.raises(SystemExit) as e:
+        evaluate.main([])
+    assert "evaluate" in str(e.value)
+    if not torch.cuda.is_available():
+        with pytest.raises(SystemExit) as e:
+            evaluate.main(["-e"])
+        assert "GPU" in str(e.value)
+
+
+def test_packed_export_rejects_foreign_files(tmp_path):
+    from deepshift_amd import export, workloads
+    torch.save({"format": "something else", "layers": {}}, tmp_path / "x.pt")
+    with pytest.raises(ValueError):
+        export.load_packed(workloads.MLP(), str(tmp_path / "x.pt"))
+    torch.save({"format": export.FORMAT, "layers": {"nope": {}}}, tmp_path / "y.pt")
+    with pytest.raises(KeyError):
+        export.load_packed(workloads.MLP(), str(tmp_path / "y.pt"))
