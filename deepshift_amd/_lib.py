@@ -40,6 +40,7 @@ SIGNATURES = {
     "ds_dequantize_i32_f32": (_c_int, [_ptr, _ptr, _c_i64, _c_int, _ptr]),
     "ds_dequantize_affine_i32_f32": (_c_int, [_ptr] * 5 + [_c_int] * 5 + [_ptr]),
     "ds_requantize_affine_pad_i32": (_c_int, [_ptr] * 6 + [_c_int] * 11 + [_ptr]),
+    "ds_requantize_affine_maxpool_i32": (_c_int, [_ptr] * 5 + [_c_int] * 14 + [_ptr]),
     "ds_mul_tiled_bytes": (_size, [_c_int, _c_int]),
     "ds_mul_tile_weights_f32": (_c_int, [_ptr, _ptr] + [_c_int] * 4 + [_ptr]),
     "ds_mul_conv2d_f32": (_c_int, [_ptr] * 4 + [_c_int] * 9 + [_ptr]),

@@ -251,6 +251,46 @@ __global__ void requantize_affine_pad_kernel(const int32_t *__restrict__ y, floa
     }
 }
 
+// The same with a max pooling between the affine/ReLU and the conversion (the ResNet stem):
+// f[oh][ow] = max over the pk x pk window (stride ps, implicit -inf padding pp, as nn.MaxPool2d) of
+// affine_one(y); one thread per element of the padded int32 output (or of out when q is NULL, with
+// ph = pw = 0).  y is [planes][H][W], out [planes][OH][OW], q [planes][OH+2ph][OW+2pw].
+__global__ void requantize_affine_maxpool_kernel(const int32_t *__restrict__ y, float *__restrict__ out,
+                                                 int32_t *__restrict__ q, const float *__restrict__ scale,
+                                                 const float *__restrict__ shift, uint32_t planes, int C,
+                                                 int H, int W, int OH, int OW, int pk, int ps, int pp,
+                                                 int ph, int pw, float inv, int relu, QuantSpec spec)
+{
+    const uint32_t Hp = OH + 2 * ph, Wp = OW + 2 * pw;
+    const uint32_t total = planes * Hp * Wp;
+    for (uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+        const uint32_t plane = idx / (Hp * Wp);
+        const uint32_t rem = idx - plane * Hp * Wp;
+        const uint32_t hp = rem / Wp;
+        const int oh = (int)hp - ph, ow = (int)(rem - hp * Wp) - pw;
+        int32_t v = 0;
+        if ((unsigned)oh < (unsigned)OH && (unsigned)ow < (unsigned)OW) {
+            const uint32_t c = plane % (uint32_t)C;
+            const float a = scale ? scale[c] : 1.0f, b = shift ? shift[c] : 0.0f;
+            const int32_t *yp = y + (size_t)plane * H * W;
+            float best = -__builtin_inff();
+            for (int i = 0; i < pk; ++i) {
+                const int ih = oh * ps - pp + i;
+                if ((unsigned)ih >= (unsigned)H) continue;
+                for (int j = 0; j < pk; ++j) {
+                    const int iw = ow * ps - pp + j;
+                    if ((unsigned)iw >= (unsigned)W) continue;
+                    const float f = affine_one(yp[ih * W + iw], inv, a, b, nullptr, relu);
+                    best = f > best ? f : best;
+                }
+            }
+            if (out) out[((size_t)plane * OH + oh) * OW + ow] = best;
+            v = quantize_one(best, spec);
+        }
+        if (q) q[idx] = v;
+    }
+}
+
 __global__ void copy_kernel(const int4 *__restrict__ src, int4 *__restrict__ dst, long n4)
 {
     const long stride = (long)gridDim.x * blockDim.x;
@@ -382,6 +422,28 @@ DS_EXPORT int ds_requantize_affine_pad_i32(const int32_t *y, float *out, int32_t
     hipLaunchKernelGGL(requantize_affine_pad_kernel, dim3(grid_for(total)), dim3(256), 0,
                        (hipStream_t)stream, y, out, q, scale, shift, residual, (uint32_t)(Nb * C), C, H, W,
                        ph, pw, ldexpf(1.0f, -F_in), relu, make_spec(I, F, mode));
+    return launch_status();
+}
+
+DS_EXPORT int ds_requantize_affine_maxpool_i32(const int32_t *y, float *out, int32_t *q, const float *scale,
+                                               const float *shift, int Nb, int C, int H, int W, int pk,
+                                               int ps, int pp, int ph, int pw, int F_in, int relu, int I,
+                                               int F, int mode, ds_stream_t stream)
+{
+    int rc = check_fixed(I, F, mode);
+    if (rc) return rc;
+    if (Nb < 0 || C < 0 || H < 0 || W < 0 || ph < 0 || pw < 0 || F_in < 0 || F_in > 31) return DS_EINVAL;
+    if (pk < 1 || ps < 1 || pp < 0 || 2 * pp > pk) return DS_EINVAL;  // nn.MaxPool2d's own rule
+    if (!q && (ph || pw)) return DS_EINVAL;
+    if (H + 2 * pp < pk || W + 2 * pp < pk) return DS_EINVAL;
+    const int OH = (H + 2 * pp - pk) / ps + 1, OW = (W + 2 * pp - pk) / ps + 1;
+    const long total = (long)Nb * C * (OH + 2 * ph) * (OW + 2 * pw);
+    if (total == 0) return DS_OK;
+    if (total * 4 >= (1L << 31) || (long)Nb * C * H * W * 4 >= (1L << 31)) return DS_ETOOLARGE;
+    if (!y || (!q && !out)) return DS_EINVAL;
+    hipLaunchKernelGGL(requantize_affine_maxpool_kernel, dim3(grid_for(total)), dim3(256), 0,
+                       (hipStream_t)stream, y, out, q, scale, shift, (uint32_t)(Nb * C), C, H, W, OH, OW, pk,
+                       ps, pp, ph, pw, ldexpf(1.0f, -F_in), relu, make_spec(I, F, mode));
     return launch_status();
 }
 

@@ -40,6 +40,7 @@ class FusedConv2dShift(nn.Module):
         self.relu = relu
         self.prequantized = False  # the input is this layer's int32 padded input, made by its producer
         self.emit = None           # (padding, I, F, want_float) of the consumers' input to produce
+        self.pool = None           # (kernel, stride, padding) of a max pooling that follows the ReLU
         if bn is not None:
             if bn.training or not bn.track_running_stats:
                 raise ValueError("only an eval-mode BatchNorm with running statistics can be folded")
@@ -61,7 +62,7 @@ class FusedConv2dShift(nn.Module):
         elif conv.conc_weight is None:
             modules.pack_module_weights(conv)
         return modules.conv_kernel_forward(conv, input, conv.conc_weight, self.scale, self.shift,
-                                           residual, self.relu, self.prequantized, self.emit)
+                                           residual, self.relu, self.prequantized, self.emit, self.pool)
 
 
 class _Tracer(fx.Tracer):
@@ -75,6 +76,37 @@ def _is_relu(node, mods):
     if node.op == "call_method" and node.target in ("relu", "relu_"):
         return True
     return node.op == "call_module" and isinstance(mods.get(node.target), nn.ReLU)
+
+
+def _square(v):
+    if isinstance(v, (tuple, list)):
+        return int(v[0]) if len(v) == 1 or (len(v) == 2 and v[0] == v[1]) else None
+    return int(v) if isinstance(v, int) else None
+
+
+def _max_pool_of(node, mods):
+    """(kernel, stride, padding) if ``node`` is a plain square 2-D max pooling, else None."""
+    if node.op == "call_module" and isinstance(mods.get(node.target), nn.MaxPool2d):
+        m = mods[node.target]
+        spec = dict(kernel_size=m.kernel_size, stride=m.stride, padding=m.padding, dilation=m.dilation,
+                    ceil_mode=m.ceil_mode, return_indices=m.return_indices)
+    elif node.op == "call_function" and node.target is F.max_pool2d:
+        names = ("kernel_size", "stride", "padding", "dilation", "ceil_mode", "return_indices")
+        spec = dict(stride=None, padding=0, dilation=1, ceil_mode=False, return_indices=False)
+        spec.update(zip(names, node.args[1:]))
+        spec.update(node.kwargs)
+        if "kernel_size" not in spec:
+            return None
+    else:
+        return None
+    if spec["ceil_mode"] or spec["return_indices"] or _square(spec["dilation"]) != 1:
+        return None
+    k = _square(spec["kernel_size"])
+    st = k if spec["stride"] in (None, ()) else _square(spec["stride"])
+    pd = _square(spec["padding"])
+    if k is None or st is None or pd is None or 2 * pd > k:
+        return None
+    return (k, st, pd)
 
 
 def _is_add(node):
@@ -123,11 +155,18 @@ def fuse_conv_epilogues(model, handoff=True):
         if nxt is not None and _is_relu(nxt, mods):
             relu = True
             chain.append(nxt)
+            nxt = _sole_user(nxt)
+        pool = None
+        if nxt is not None and residual is None and len(chain) > 1 and nxt.args and nxt.args[0] is chain[-1]:
+            pool = _max_pool_of(nxt, mods)
+            if pool is not None:
+                chain.append(nxt)
         if len(chain) == 1:
             continue  # nothing to fuse
         name = "fused_%d" % count
         count += 1
         gm.add_module(name, FusedConv2dShift(conv, bn, relu))
+        gm.get_submodule(name).pool = pool
         with gm.graph.inserting_after(chain[-1]):
             args = (node.args[0],) if residual is None else (node.args[0], residual)
             new = gm.graph.call_module(name, args)

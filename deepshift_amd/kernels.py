@@ -232,6 +232,32 @@ def requantize_affine_pad(y, fraction_bits_in, scale, shift, residual, relu, pad
     return out, q
 
 
+def requantize_affine_maxpool(y, fraction_bits_in, scale, shift, relu, pool, padding=None,
+                              integer_bits=16, fraction_bits=16, want_float=True):
+    """:func:`dequantize_affine`, ``max_pool2d(kernel, stride, padding)`` and -- when ``padding`` (of
+    the next shift convolution) is given -- its :func:`quantize_pad`, in one pass.
+    ``pool = (kernel, stride, padding)``.  Returns ``(out, q)``; either may be ``None``."""
+    y = _require_device_i32("y", y)
+    if y.dim() != 4:
+        raise TypeError("requantize_affine_maxpool expects a 4-D int32 GPU tensor")
+    Nb, C, H, W = y.shape
+    pk, ps, pp = (int(v) for v in pool)
+    OH, OW = (H + 2 * pp - pk) // ps + 1, (W + 2 * pp - pk) // ps + 1
+    for name, t in (("scale", scale), ("shift", shift)):
+        if t is not None and (t.dtype != torch.float32 or t.numel() != C or not t.is_contiguous()):
+            raise ValueError("%s must be a contiguous float32 tensor of %d elements" % (name, C))
+    if padding is None and not want_float:
+        raise ValueError("nothing to produce")
+    ph, pw = _pair(padding) if padding is not None else (0, 0)
+    out = torch.empty([Nb, C, OH, OW], dtype=torch.float32, device=y.device) if want_float else None
+    q = torch.empty([Nb, C, OH + 2 * ph, OW + 2 * pw], dtype=torch.int32, device=y.device) \
+        if padding is not None else None
+    _lib.call("ds_requantize_affine_maxpool_i32", _lib.ptr(y), _lib.ptr(out), _lib.ptr(q), _lib.ptr(scale),
+              _lib.ptr(shift), Nb, C, H, W, pk, ps, pp, ph, pw, fraction_bits_in, int(bool(relu)),
+              integer_bits, fraction_bits, _lib.DS_Q_ROUND_TO_FIXED, _lib.current_stream(y.device))
+    return out, q
+
+
 # ---------------------------------------------------------------------------------------------
 # LinearShift / Conv2dShift kernels
 # ---------------------------------------------------------------------------------------------

@@ -197,7 +197,7 @@ def _circular_pad(x, padding):
 
 
 def conv_kernel_forward(module, input, conc_weight, scale=None, shift=None, residual=None, relu=False,
-                        prequantized=False, emit=None):
+                        prequantized=False, emit=None, pool=None):
     """Fixed-point shift convolution of a float NCHW input (modules.py:152-162,317-337).
 
     ``scale``/``shift`` (per output channel), ``residual`` and ``relu`` describe what follows the
@@ -207,7 +207,8 @@ def conv_kernel_forward(module, input, conc_weight, scale=None, shift=None, resi
     ``prequantized``: ``input`` is already the layer's round-to-fixed, zero padded int32 input (made
     by the layer before it).  ``emit = (padding, integer_bits, fraction_bits, want_float)``: also
     produce that form of the result for the next shift convolution; the return value is then
-    ``(out, q)``, or ``q`` alone when ``want_float`` is false."""
+    ``(out, q)``, or ``q`` alone when ``want_float`` is false.  ``pool = (kernel, stride, padding)``:
+    a max pooling follows the ReLU (no residual) and runs in the same pass."""
     if not module.use_cuda:
         kernels._no_cpu_kernel()
     if module.dilation != (1, 1) or module.groups != 1:
@@ -228,6 +229,15 @@ def conv_kernel_forward(module, input, conc_weight, scale=None, shift=None, resi
                               module.kernel_size[0], module.kernel_size[1])
     out = kernels.conv2d_tiled(xq, tiled, bias, module.out_channels, module.kernel_size,
                                module.stride, conc_weight.bits, conc_weight.base)
+    if pool is not None:
+        if residual is not None:
+            raise ValueError("a fused max pooling cannot follow a residual add")
+        if emit is None:
+            return kernels.requantize_affine_maxpool(out, Fb, scale, shift, relu, pool)[0]
+        next_padding, next_I, next_F, want_float = emit
+        f, q = kernels.requantize_affine_maxpool(out, Fb, scale, shift, relu, pool, next_padding,
+                                                 next_I, next_F, want_float)
+        return (f, q) if want_float else q
     if emit is not None:
         next_padding, next_I, next_F, want_float = emit
         f, q = kernels.requantize_affine_pad(out, Fb, scale, shift, residual, relu, next_padding,

@@ -161,6 +161,15 @@ int ds_requantize_affine_pad_i32(const int32_t *y, float *out, int32_t *q, const
                                  int ph, int pw, int F_in, int relu, int I, int F, int mode,
                                  ds_stream_t stream);
 
+/* The same with a max pooling (window pk x pk, stride ps, implicit -inf padding pp, floor mode, as
+ * nn.MaxPool2d) between the affine/ReLU and the conversion -- the ResNet stem: y [Nb][C][H][W],
+ * out [Nb][C][OH][OW] float or NULL, q [Nb][C][OH+2ph][OW+2pw] or NULL (then ph = pw = 0),
+ * OH = (H + 2pp - pk) / ps + 1.  No counterpart in the reference. */
+int ds_requantize_affine_maxpool_i32(const int32_t *y, float *out, int32_t *q, const float *scale,
+                                     const float *shift, int Nb, int C, int H, int W, int pk, int ps,
+                                     int pp, int ph, int pw, int F_in, int relu, int I, int F, int mode,
+                                     ds_stream_t stream);
+
 /* ---- float multiply comparator -------------------------------------------------------------
  * The reference ships plain float multiply-accumulate kernels of the same structure as its shift
  * kernels to compare "shift against multiply" on one machine (UNOPTIMIZED_LINEAR /

@@ -269,6 +269,24 @@ def test_requantize_affine_pad_matches_the_two_passes(rng):
             assert f is None and torch.equal(q, q_want)
 
 
+def test_requantize_affine_maxpool_matches_the_three_passes(rng):
+    import torch.nn.functional as F
+    for (Nb, C, H, W), pool, pad in [((2, 5, 12, 12), (3, 2, 1), (1, 1)), ((1, 3, 9, 7), (2, 2, 0), (0, 0)),
+                                     ((3, 4, 11, 13), (3, 1, 1), (2, 1)), ((1, 2, 5, 5), (5, 5, 2), (1, 1))]:
+        y = torch.from_numpy(rng.integers(-2 ** 27, 2 ** 27, size=(Nb, C, H, W)).astype(np.int32)).to(DEV)
+        scale = torch.rand(C, device=DEV) - 0.3          # some channels flip the order of the values
+        shift = torch.randn(C, device=DEV)
+        for sc, sh, relu in [(scale, shift, True), (scale, None, False), (None, None, False)]:
+            f_want = F.max_pool2d(kernels.dequantize_affine(y, 16, sc, sh, None, relu), *pool)
+            q_want = kernels.quantize_pad(f_want, pad, 16, 16, round_to_fixed=True)
+            f, q = kernels.requantize_affine_maxpool(y, 16, sc, sh, relu, pool, pad, 16, 16, want_float=True)
+            assert torch.equal(f, f_want) and torch.equal(q, q_want)
+            f, q = kernels.requantize_affine_maxpool(y, 16, sc, sh, relu, pool, pad, 16, 16, want_float=False)
+            assert f is None and torch.equal(q, q_want)
+            f, q = kernels.requantize_affine_maxpool(y, 16, sc, sh, relu, pool)
+            assert q is None and torch.equal(f, f_want)
+
+
 def test_dequantize_affine_matches_torch(rng):
     Nb, C, H, W = 3, 5, 7, 4
     y = torch.from_numpy(rng.integers(-2 ** 24, 2 ** 24, size=(Nb, C, H, W)).astype(np.int32)).to(DEV)

@@ -154,9 +154,10 @@ def test_fused_graph_hands_fixed_point_tensors_on():
     gm = fuse.fuse_conv_epilogues(model)
     fused = [m for m in gm.modules() if isinstance(m, fuse.FusedConv2dShift)]
     assert len(fused) == 20
-    assert sum(m.prequantized for m in fused) == 15          # 8 second convolutions + 7 block inputs
+    assert sum(m.prequantized for m in fused) == 16          # 8 second convolutions + 8 block inputs
     emits = [m.emit for m in fused if m.emit is not None]
-    assert len(emits) == 15 and sum(e[3] for e in emits) == 7  # float kept for the 7 block outputs
+    assert len(emits) == 16 and sum(e[3] for e in emits) == 8  # float kept for the 8 block inputs
+    assert [m.pool for m in fused if m.pool] == [(3, 2, 1)]    # the stem's max pooling rides along
     assert all(e[:3] == ((1, 1), 16, 16) for e in emits)
     plain = fuse.fuse_conv_epilogues(model, handoff=False)
     assert not any(m.prequantized or m.emit for m in plain.modules() if isinstance(m, fuse.FusedConv2dShift))
