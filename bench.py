@@ -238,7 +238,27 @@ def cpu_baseline(shapes):
 
     t_multi = run(threads, batch)
     t_single = run(1, 1)
+
+    # The reference's own CPU kernel (oracle/_ref, compiled from its shift_cpu.cpp) on one layer, beside
+    # the port on the same data: it confirms that the port is a fair stand-in.  Its time includes the
+    # pybind conversion of nested Python lists, which is how the reference calls it.
+    check = None
+    ref = shift_oracle.load_reference_cpu_kernel()
+    if ref is not None:
+        x = rng.integers(0, 2 ** 20, size=(1, 64, 58, 58)).astype(np.int32)
+        s = rng.integers(-15, 1, size=(64, 64, 3, 3)).astype(np.int32)
+        sg = rng.choice(np.array([-1, 1], np.int32), size=s.shape)
+        lists = (x.tolist(), s.tolist(), sg.tolist(), [0] * 64)
+        t0 = time.perf_counter()
+        y_ref = ref.convolution_kernel(*lists, (1, 1), (0, 0))
+        t_ref = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        y_port = oracle.conv2d(x, s.astype(np.int8), sg, None, (1, 1), nthreads=1)
+        t_port = time.perf_counter() - t0
+        check = {"layer": "3x3 conv 64->64, 56x56, batch 1 (one thread)", "reference_s": t_ref, "port_s": t_port,
+                 "identical": bool(np.array_equal(np.array(y_ref, np.int64).astype(np.int32), y_port))}
     return {
+        "reference_kernel_check": check,
         "value": batch / t_multi, "unit": "images/s", "cores": threads, "kind": "port",
         "sample": "all 21 shift layers of ResNet-18 at batch %d (one image per thread), kernel time "
                   "only, int32 inputs resident in host memory; single thread on 1 image: %.3f images/s"
