@@ -569,20 +569,29 @@ template <int BITS, bool GENERAL>
 static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
 {
     if constexpr (!GENERAL && BITS <= 4) {
-        // Shift-plane kernel with the work-balanced launch: measured 10..25 % faster than the
-        // two-instruction kernel when every wave slot gets at least 24 K groups of work and a tile
-        // spans at least 24 (ResNet 3x3 and 7x7 layers, large GEMMs); the 1x1 shortcuts, small
-        // batches and few-channel layers stay on the kernel above.
+        // Shift-plane kernel.  Two launch regimes, from sweeps over the ResNet-18/50 shapes:
+        //  * tiles >= 1.3 x the 3072 wave slots: one tile per wave, plain stores.  The hardware hands
+        //    out workgroups as slots free up, the waves of a pixel range run through K in step (they
+        //    share its activations in L2) and nothing is written twice; wins from 7 K groups up
+        //    (1x1 convolutions on large images, stems), where output traffic decides.
+        //  * fewer tiles: equal shares of the (tile, K group) space per wave slot, combined with
+        //    atomics -- needs long reductions (>= 24 K groups per tile, >= 16 per slot) to pay for
+        //    the pre-fill.  Tiles that already fill whole rounds of slots keep one tile per wave.
+        // The 1x1 shortcuts of small images, single-wave batches and layers with few channels stay on
+        // the two-instruction kernel.
         const char *t = getenv("DS_TUNE_PLANES");
         const long tiles = (long)ceil_div(a.M, kPlaneRows * kWave) * ceil_div(a.N, 32);
         const long iters = tiles * a.comm;
-        bool planes = a.comm >= 24 && iters >= (long)kPlaneSlots * 16 && (a.N % 32 == 0 || a.N >= 256);
+        const bool n_ok = a.N % 32 == 0 || a.N >= 256;
+        const bool many_tiles = tiles * 10 >= (long)kPlaneSlots * 13;
+        bool planes = n_ok && ((many_tiles && a.comm >= 6) || (a.comm >= 24 && iters >= (long)kPlaneSlots * 16));
         if (t) planes = atoi(t) > 0;
         if (planes) {
-            // 3 waves per SIMD fit (3072 slots): one tile per wave when the tiles fill whole rounds
-            // of slots (no atomics, no pre-fill), otherwise equal shares of the iteration space
             const long rounds = (tiles + kPlaneSlots - 1) / kPlaneSlots;
-            int nsplit = (tiles >= kPlaneSlots && (double)tiles / ((double)kPlaneSlots * rounds) >= 0.93) ? 1 : 0;
+            const bool whole_rounds = tiles >= kPlaneSlots && (double)tiles / ((double)kPlaneSlots * rounds) >= 0.93;
+            // (a very long reduction with many tiles, e.g. an 8192^3 GEMM, is compute-heavy enough for
+            // the equal shares to win again)
+            int nsplit = ((many_tiles && a.comm <= 128) || whole_rounds) ? 1 : 0;
             if (const char *sp = getenv("DS_TUNE_SPLIT")) nsplit = atoi(sp);
             return launch_planes<BITS>(a, nsplit, st);
         }
