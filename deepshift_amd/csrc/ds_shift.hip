@@ -589,9 +589,13 @@ static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
         if (planes) {
             const long rounds = (tiles + kPlaneSlots - 1) / kPlaneSlots;
             const bool whole_rounds = tiles >= kPlaneSlots && (double)tiles / ((double)kPlaneSlots * rounds) >= 0.93;
-            // (a very long reduction with many tiles, e.g. an 8192^3 GEMM, is compute-heavy enough for
-            // the equal shares to win again)
-            int nsplit = ((many_tiles && a.comm <= 128) || whole_rounds) ? 1 : 0;
+            // With many tiles the equal shares still win when the reduction is long and the rounds of
+            // slots fill badly (3x3 layers with 1.4 rounds of tiles, an 8192^3 GEMM), unless many
+            // channel tiles share each pixel range: their waves then start at staggered K offsets
+            // and evict each other's activations from L2.
+            const double fill = (double)tiles / ((double)kPlaneSlots * rounds);
+            const bool per_tile = many_tiles && (a.comm < 24 || (a.comm <= 128 && (fill >= 0.85 || ceil_div(a.N, 32) >= 8)));
+            int nsplit = (per_tile || whole_rounds) ? 1 : 0;
             if (const char *sp = getenv("DS_TUNE_SPLIT")) nsplit = atoi(sp);
             return launch_planes<BITS>(a, nsplit, st);
         }
