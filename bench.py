@@ -7,7 +7,7 @@ One step = one forward pass of ResNet-18 (every conv and the FC replaced by shif
 weight_bits 5, activations 16.16) over one synthetic batch of 64 x 3 x 224 x 224 that is already
 resident in HBM.  Prints ONE JSON line: images/s for the whole forward pass, the shift kernel's
 rate against the VALU roofline (timed live with HIP events on the launch stream), the 4096^3
-shift GEMM and the 3x3 conv of BASELINE config 2, and the CPU restatement of the reference's
+shift GEMM and the 3x3 conv of benchmark configuration 2, and the CPU restatement of the reference's
 shift kernel timed on this host's cores.
 """
 import argparse
@@ -137,7 +137,7 @@ def calibrate_valu(device):
 
 
 def config2(device, reps=10):
-    """BASELINE config 2: the 3x3 conv (32x64x56x56, 64 -> 64) and the 4096^3 shift GEMM."""
+    """Benchmark configuration 2: the 3x3 conv (32x64x56x56, 64 -> 64) and the 4096^3 shift GEMM."""
     from deepshift_amd import kernels, utils
     g = torch.Generator().manual_seed(0)
     out = {}
@@ -348,7 +348,7 @@ def main():
         "dtype": "int32",
         "data": "synthetic",
         "config": {"workload": "ResNet-18, batch 64 x 3x224x224, all 20 conv + FC as shift layers "
-                               "(BASELINE configs[3]); weight_bits 5 (4-bit shift + sign, 6 codes per "
+                               "(benchmark configuration 4); weight_bits 5 (4-bit shift + sign, 6 codes per "
                                "word), activations 16.16; BatchNorm/residual/ReLU folded into each "
                                "conv's dequantisation pass, pooling fp32 PyTorch",
                    "batch": BATCH, "shift_layers": 21, "pairs_per_step": pairs},

@@ -1,4 +1,4 @@
-"""GPU: BASELINE.json's full-size cases.  The oracle is too slow for a whole tensor here, so parity
+"""GPU: the benchmark configurations at full size.  The oracle is too slow for a whole tensor here, so parity
 is checked on slices the oracle finishes in seconds plus size-independent properties."""
 import os
 

@@ -152,7 +152,7 @@ def test_q_modules_and_circular_padding():
 
 
 def test_mlp_config1_end_to_end(oracle):
-    """BASELINE config 1: 784-512-512-10, batch 64, ternary sign, shift in [-15, 0], 16.16."""
+    """Benchmark configuration 1 (MLP): 784-512-512-10, batch 64, ternary sign, shift in [-15, 0], 16.16."""
     g = torch.Generator().manual_seed(0)
     x = torch.rand(64, 784, generator=g)
     model = workloads.MLP()
@@ -174,7 +174,7 @@ def test_mlp_config1_end_to_end(oracle):
 
 
 def test_resnet20_config3_kernel_vs_float_path():
-    """BASELINE config 3 at a reduced batch: every conv + FC shift-kernelised; the kernel model and
+    """Benchmark configuration 3 (ResNet-20) at a reduced batch: every conv + FC shift-kernelised; the kernel model and
     the float model agree layer by layer within the fixed-point bound on the same inputs."""
     g = torch.Generator().manual_seed(3)
     model = workloads.randomize_batchnorm(workloads.ResNet20(), g).eval()
