@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libdeepshift_hip.so")
 
 DS_Q_ROUND_TO_FIXED = 0
 DS_Q_CAST = 1
+DS_BITS_ZERO_TOP = 0x100
 
 _c_int = ctypes.c_int
 _c_i64 = ctypes.c_int64
@@ -24,6 +25,7 @@ SIGNATURES = {
     "ds_pack_i32": (_c_int, [_ptr, _ptr, _ptr, _c_int, _c_int, _c_int, _c_int, _ptr]),
     "ds_tiled_bytes": (_size, [_c_int, _c_int, _c_int]),
     "ds_tile_weights_i32": (_c_int, [_ptr, _ptr] + [_c_int] * 6 + [_ptr]),
+    "ds_tile_weights_zero_top_i32": (_c_int, [_ptr, _ptr] + [_c_int] * 5 + [_ptr]),
     "ds_linear_workspace_bytes": (_size, [_c_int] * 4),
     "ds_linear_i32": (_c_int, [_ptr] * 4 + [_c_int] * 5 + [_ptr, _size, _ptr]),
     "ds_linear_tiled_workspace_bytes": (_size, [_c_int] * 4),

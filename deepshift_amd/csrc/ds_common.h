@@ -64,8 +64,9 @@ inline const uint32_t *tiled_ktab(const void *tiled, const TiledGeom &g)
 // Launchers implemented across the .hip files.
 int launch_pack(const int32_t *s, const int32_t *sign, int32_t *out, int O, int K, int bits,
                 int base, hipStream_t st);
-int launch_tile(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW, int bits,
-                hipStream_t st);
+// in_bits: field width of the reference words (0: the same as bits); zero_top: see ds_pack.hip
+int launch_tile(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW, int bits, hipStream_t st,
+                int in_bits = 0, int zero_top = 0);
 int launch_transpose(const int32_t *x, int32_t *xT, int M, int K, int ldx, hipStream_t st);
 // the same with rows of x ldin elements apart
 int launch_transpose_strided(const int32_t *x, int ldin, int32_t *xT, int M, int K, int ldx, hipStream_t st);

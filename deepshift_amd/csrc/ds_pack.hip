@@ -44,14 +44,46 @@ int launch_pack(const int32_t *s, const int32_t *sign, int32_t *out, int O, int 
     return launch_status();
 }
 
-// Reference-format words [N][comm] -> tiled words [ntiles][comm][32].
-//   * code sign bit inverted: 1 = negative (the compute kernel sign-extends it into an xor mask);
-//   * codes past K, and every code of a padding channel, become (field 0, positive): with the
-//     activation read as 0 they add nothing;
-//   * zero-weight codes (field >= 32, bits == 6 only) are made positive so that they neither add
-//     nor need the negative-count correction.
+// One code of the reference format: shift field and "positive" bit of reduction index k, channel n.
+struct RefCode {
+    uint32_t field, positive;
+};
+
+__device__ __forceinline__ RefCode ref_code(const int32_t *__restrict__ w_ref, long n, int k, int in_comm,
+                                            int in_bits)
+{
+    const int num = codes_per_word(in_bits);
+    const uint32_t in = (uint32_t)w_ref[n * in_comm + k / num];
+    const uint32_t code = in >> ((k % num) * (in_bits + 1));
+    return RefCode{code & ((1u << in_bits) - 1u), (code >> in_bits) & 1u};
+}
+
+// Field and sign of a code in the private formats.  Sign bit inverted: 1 = negative (the compute
+// kernel sign-extends it into an xor mask).  Zero-weight codes (field >= 32, 6-bit reference words
+// only) are made positive so that they neither add nor need the negative-count correction; with
+// `zero_top` they become the highest field value of the narrower output width, whose shift plane
+// the kernel holds at 0 (the other fields must be below it: the caller vouches for that).
+struct OwnCode {
+    uint32_t field, neg;
+};
+
+__device__ __forceinline__ OwnCode own_code(RefCode c, int out_bits, int zero_top)
+{
+    OwnCode o{c.field, c.positive ^ 1u};
+    if (c.field >= 32u) {
+        o.neg = 0;
+        if (zero_top) o.field = (1u << out_bits) - 1u;
+    }
+    o.field &= (1u << out_bits) - 1u;
+    return o;
+}
+
+// Reference-format words [N][in_comm] -> tiled words [ntiles][comm][32] of `bits`-wide fields
+// (bits == in_bits unless zero_top re-packs 6-bit ternary words into a narrower width).  Codes past
+// K, and every code of a padding channel, become (field 0, positive): with the activation read as
+// 0 they add nothing.
 __global__ void tile_kernel(const int32_t *__restrict__ w_ref, uint32_t *__restrict__ wt, int N, int K,
-                            int comm, int bits, int num, long words)
+                            int comm, int bits, int num, long words, int in_bits, int in_comm, int zero_top)
 {
     const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= words) return;
@@ -62,17 +94,12 @@ __global__ void tile_kernel(const int32_t *__restrict__ w_ref, uint32_t *__restr
     const int n = t * kTileWords + j;
     uint32_t out = 0;
     const int cb = bits + 1;
-    const uint32_t fmask = (1u << bits) - 1u;
     if (n < N) {
-        const uint32_t in = (uint32_t)w_ref[(long)n * comm + g];
         for (int i = 0; i < num; ++i) {
             const int k = g * num + i;
             if (k >= K) break;
-            const uint32_t code = in >> (i * cb);
-            const uint32_t field = code & fmask;
-            uint32_t neg = ((code >> bits) & 1u) ^ 1u;
-            if (field >= 32u) neg = 0;
-            out |= (field | (neg << bits)) << (i * cb);
+            const OwnCode c = own_code(ref_code(w_ref, n, k, in_comm, in_bits), bits, zero_top);
+            out |= (c.field | (c.neg << bits)) << (i * cb);
         }
     }
     wt[idx] = out;
@@ -119,7 +146,7 @@ __global__ void ktab_kernel(uint32_t *ktab, int K, int count, int FH, int FW)
 // words16[t][g*(num/2) + h][j]: codes k = g*num + 2h and k + 1 of channel t*32 + j as 16-bit M0-ready
 // values (see TiledGeom).  Codes past K and padding channels are (field 0, positive).
 __global__ void tile16_kernel(const int32_t *__restrict__ w_ref, uint32_t *__restrict__ w16, int N, int K,
-                              int comm, int bits, int num, long words)
+                              int comm, int bits, int num, long words, int in_bits, int in_comm, int zero_top)
 {
     const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= words) return;
@@ -133,34 +160,33 @@ __global__ void tile16_kernel(const int32_t *__restrict__ w_ref, uint32_t *__res
     const int n = t * kTileWords + j;
     uint32_t out = 0x10001000u;
     if (n < N) {
-        const uint32_t in = (uint32_t)w_ref[(long)n * comm + g];
-        const int cb = bits + 1;
-        const uint32_t fmask = (1u << bits) - 1u;
         for (int c = 0; c < 2; ++c) {
-            const int i = 2 * h + c;
-            if (g * num + i >= K) continue;
-            const uint32_t code = in >> (i * cb);
-            const uint32_t neg = ((code >> bits) & 1u) ^ 1u;
-            out |= ((code & fmask) | (neg << 8)) << (16 * c);
+            const int k = g * num + 2 * h + c;
+            if (k >= K) continue;
+            const OwnCode o = own_code(ref_code(w_ref, n, k, in_comm, in_bits), bits, zero_top);
+            out |= (o.field | (o.neg << 8)) << (16 * c);
         }
     }
     w16[idx] = out;
 }
 
 int launch_tile(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW, int bits,
-                hipStream_t st)
+                hipStream_t st, int in_bits, int zero_top)
 {
     const int K = C * FH * FW;
+    if (in_bits == 0) in_bits = bits;
+    const int in_num = codes_per_word(in_bits), in_comm = ceil_div(K, in_num);
     const TiledGeom g = tiled_geom(N, K, bits);
     if (g.word_count) {
         const long blocks = ((long)g.word_count + 255) / 256;
         hipLaunchKernelGGL(tile_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w_ref,
-                           (uint32_t *)tiled, N, K, g.comm, bits, g.num, (long)g.word_count);
+                           (uint32_t *)tiled, N, K, g.comm, bits, g.num, (long)g.word_count, in_bits, in_comm,
+                           zero_top);
     }
     const int Npad = g.ntiles * kTileWords;
     if (Npad) {
         hipLaunchKernelGGL(negcount_kernel, dim3(ceil_div(Npad, 64)), dim3(64), 0, st, w_ref,
-                           (int32_t *)tiled_negcount(tiled, g), N, Npad, K, g.comm, bits, g.num);
+                           (int32_t *)tiled_negcount(tiled, g), N, Npad, K, in_comm, in_bits, in_num);
     }
     hipLaunchKernelGGL(ktab_kernel, dim3(ceil_div((int)g.ktab_count, 256)), dim3(256), 0, st,
                        (uint32_t *)tiled_ktab(tiled, g), K, (int)g.ktab_count, FH, FW);
@@ -168,7 +194,7 @@ int launch_tile(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW,
         const long blocks = ((long)g.words16_count + 255) / 256;
         hipLaunchKernelGGL(tile16_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w_ref,
                            (uint32_t *)tiled_words16(tiled, g), N, K, g.comm, bits, g.num,
-                           (long)g.words16_count);
+                           (long)g.words16_count, in_bits, in_comm, zero_top);
     }
     return launch_status();
 }
@@ -204,4 +230,15 @@ DS_EXPORT int ds_tile_weights_i32(const int32_t *w_ref, void *tiled, int N, int 
     if (N == 0) return DS_OK;
     if (!tiled || (!w_ref && C > 0)) return DS_EINVAL;
     return launch_tile(w_ref, tiled, N, C, FH, FW, bits, (hipStream_t)stream);
+}
+
+DS_EXPORT int ds_tile_weights_zero_top_i32(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW,
+                                           int field_bits, ds_stream_t stream)
+{
+    if (field_bits < 1 || field_bits > 4) return DS_EBITS;
+    if (N < 0 || C < 0 || FH < 1 || FW < 1) return DS_EINVAL;
+    if (C >= (1 << 22) || FH > 31 || FW > 31 || (size_t)C * FH * FW >= (1u << 24)) return DS_ETOOLARGE;
+    if (N == 0) return DS_OK;
+    if (!tiled || (!w_ref && C > 0)) return DS_EINVAL;
+    return launch_tile(w_ref, tiled, N, C, FH, FW, field_bits, (hipStream_t)stream, 6, 1);
 }

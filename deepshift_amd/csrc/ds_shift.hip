@@ -55,6 +55,7 @@ struct ShiftArgs {
     int32_t *alt_y;
     int alt_ld;
     uint32_t y_elems;                     // elements the pre-fill covers
+    int zero_top;                         // the highest field value is a zero weight (ternary blobs)
 };
 
 // Redirects an atomic LinearShift launch to its channel-major scratch; returns the final y or nullptr.
@@ -122,6 +123,25 @@ __device__ __forceinline__ void accumulate_code(int32_t (&acc)[R][J], const int3
             }
             acc[r][j] = xor_add(t, mask, acc[r][j]);
         }
+    }
+}
+
+// The same for blobs whose highest field value stands for a zero weight (partial last K group of the
+// shift-plane kernel only: three vector instructions per term).
+template <int BITS, int R, int J>
+__device__ __forceinline__ void accumulate_code_zero_top(int32_t (&acc)[R][J], const int32_t (&xv)[R],
+                                                         const uint32_t (&w)[J], const int i)
+{
+    constexpr int CB = BITS + 1;
+    constexpr uint32_t TOP = (1u << BITS) - 1u;
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        const uint32_t code = w[j] >> (i * CB);
+        const int32_t mask = -(int32_t)((code >> BITS) & 1u);
+        const uint32_t field = code & TOP;
+        const int32_t keep = field == TOP ? 0 : -1;
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[r][j] = xor_add((xv[r] >> field) & keep, mask, acc[r][j]);
     }
 }
 
@@ -267,16 +287,24 @@ constexpr int kPlaneSlots = 3072;  // wave slots of the machine at 3 waves per S
       "s"(w.fw), "s"(w.fh), "s"(w.FW), "s"(w.FH), "s"(w.row_step), "s"(w.plane_step),             \
       "s"(w.koff_max)
 
-template <int BITS>
+// ZT: the blob's highest field value stands for a zero weight (its plane is held at 0).
+template <int BITS, bool ZT>
 __device__ __forceinline__ void planes_main_loop(v16i (&a)[6], const uint32_t (&xoff)[3], v4i rsrc,
                                                  const uint32_t *wptr, int groups, const PlaneWalk &w);
 #define DS_PLANES_SPECIALISE(B)                                                                    \
     template <>                                                                                    \
-    __device__ __forceinline__ void planes_main_loop<B>(v16i (&a)[6], const uint32_t (&xoff)[3],  \
-                                                        v4i rsrc, const uint32_t *wptr, int groups, \
-                                                        const PlaneWalk &w)                        \
+    __device__ __forceinline__ void planes_main_loop<B, false>(v16i (&a)[6], const uint32_t (&xoff)[3], \
+                                                               v4i rsrc, const uint32_t *wptr, int groups, \
+                                                               const PlaneWalk &w)                 \
     {                                                                                              \
         asm volatile(DS_PLANES_ASM_B##B DS_PLANES_OPERANDS : DS_PLANES_CLOBBERS_B##B);             \
+    }                                                                                              \
+    template <>                                                                                    \
+    __device__ __forceinline__ void planes_main_loop<B, true>(v16i (&a)[6], const uint32_t (&xoff)[3], \
+                                                              v4i rsrc, const uint32_t *wptr, int groups, \
+                                                              const PlaneWalk &w)                  \
+    {                                                                                              \
+        asm volatile(DS_PLANES_ASM_B##B##Z DS_PLANES_OPERANDS : DS_PLANES_CLOBBERS_B##B);          \
     }
 DS_PLANES_SPECIALISE(1)
 DS_PLANES_SPECIALISE(2)
@@ -286,7 +314,7 @@ DS_PLANES_SPECIALISE(4)
 // One segment of work of the shift-plane kernel: K groups [g_begin, g_end) of the tile made of the 32
 // channels of `ntile` and the R*64 pixels starting at m0.  `atomic` selects accumulation into a
 // pre-filled output (several segments share the tile) or a plain store of acc + bias.
-template <int BITS>
+template <int BITS, bool ZT>
 __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, int m0, int g_begin,
                                                int g_end, bool atomic)
 {
@@ -334,7 +362,7 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
         w.row_step = p.x_row - p.FW;
         w.plane_step = p.x_plane - p.FH * p.x_row;
         w.koff_max = (p.K / ff - 1) * p.x_plane + (p.FH - 1) * p.x_row + p.FW - 1;
-        planes_main_loop<BITS>(a, xoff, rsrc,
+        planes_main_loop<BITS, ZT>(a, xoff, rsrc,
                                p.wt16 + ((size_t)ntile * p.comm + g_begin) * (NUM / 2) * kTileWords,
                                g_full_end - g_begin, w);
     }
@@ -359,7 +387,8 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
             const bool real = g * NUM + i < p.K;
 #pragma unroll
             for (int r = 0; r < R; ++r) xt[i][r] = real ? xt[i][r] : 0;
-            accumulate_code<BITS, false, R, J>(acc, xt[i], w, i, 0);
+            if (ZT) accumulate_code_zero_top<BITS, R, J>(acc, xt[i], w, i);
+            else accumulate_code<BITS, false, R, J>(acc, xt[i], w, i, 0);
         }
     }
 
@@ -383,7 +412,7 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
 }
 
 // Tile-per-wave launch: gridDim.y K-slices per tile.
-template <int BITS>
+template <int BITS, bool ZT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void shift_planes_kernel(
     const ShiftArgs p)
 {
@@ -397,14 +426,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     const int g_begin = blockIdx.y * p.groups_per_split;
     int g_end = g_begin + p.groups_per_split;
     if (g_end > p.comm) g_end = p.comm;
-    planes_segment<BITS>(p, ntile, m0, g_begin, g_end, p.atomic_out != 0);
+    planes_segment<BITS, ZT>(p, ntile, m0, g_begin, g_end, p.atomic_out != 0);
 }
 
 // Work-balanced launch: the (tile, K group) iteration space is cut into one equal contiguous share
 // per wave, so every wave of the launch does the same number of group iterations whatever the tile
 // count (each wave touches at most a few tiles; tiles shared between waves are combined with
 // atomic adds onto the pre-filled output).  tiles_m4 holds the number of 192-pixel tiles here.
-template <int BITS>
+template <int BITS, bool ZT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void shift_planes_balanced_kernel(
     const ShiftArgs p)
 {
@@ -423,7 +452,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         if (g_end > p.comm) g_end = p.comm;
         const int ntile = tile % p.tiles_n;
         const int m0 = (tile / p.tiles_n) * (kPlaneRows * kWave);
-        planes_segment<BITS>(p, ntile, m0, g_begin, (int)g_end, true);
+        planes_segment<BITS, ZT>(p, ntile, m0, g_begin, (int)g_end, true);
         it += g_end - g_begin;
     }
 }
@@ -531,7 +560,7 @@ static TileChoice choose_tile(const ShiftArgs &a)
     return c;
 }
 
-template <int BITS>
+template <int BITS, bool ZT>
 static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
 {
     constexpr int R = kPlaneRows, J = 32;
@@ -543,7 +572,11 @@ static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
         int32_t *final_y = redirect_to_scratch(a);
         launch_fill(a, st);
         int blocks = (kPlaneSlots / 4) * (nsplit < 0 ? -nsplit : 1);
-        hipLaunchKernelGGL((shift_planes_balanced_kernel<BITS>), dim3(blocks), dim3(256), 0, st, a);
+        // small layers: at least 8 K groups per wave (the workgroup count stays a multiple of 8)
+        const long iters = (long)a.tiles_m4 * a.tiles_n * a.comm;
+        const long fit = (iters / 32) / 8 * 8;
+        if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
+        hipLaunchKernelGGL((shift_planes_balanced_kernel<BITS, ZT>), dim3(blocks), dim3(256), 0, st, a);
         if (final_y) return launch_transpose_strided(a.y, a.alt_ld, final_y, a.N, a.M, a.N, st);
         return launch_status();
     }
@@ -560,9 +593,43 @@ static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
         launch_fill(a, st);
     }
     dim3 grid(a.blocks_per_xcd * 8, nsplit);
-    hipLaunchKernelGGL((shift_planes_kernel<BITS>), grid, dim3(256), 0, st, a);
+    hipLaunchKernelGGL((shift_planes_kernel<BITS, ZT>), grid, dim3(256), 0, st, a);
     if (final_y) return launch_transpose_strided(a.y, a.alt_ld, final_y, a.N, a.M, a.N, st);
     return launch_status();
+}
+
+// Launch regime of the shift-plane kernel for a layer: 1 = one tile per wave, 0 = equal shares,
+// -1 = the layer is better off on the two-instruction kernel.
+static int plane_regime(const ShiftArgs &a)
+{
+    const long tiles = (long)ceil_div(a.M, kPlaneRows * kWave) * ceil_div(a.N, 32);
+    const long iters = tiles * a.comm;
+    const bool n_ok = a.N % 32 == 0 || a.N >= 256;
+    const bool many_tiles = tiles * 10 >= (long)kPlaneSlots * 13;
+    const long rounds = (tiles + kPlaneSlots - 1) / kPlaneSlots;
+    const double fill = (double)tiles / ((double)kPlaneSlots * (double)(rounds > 0 ? rounds : 1));
+    const bool whole_rounds = tiles >= kPlaneSlots && fill >= 0.93;
+    // With many tiles the equal shares still win when the reduction is long and the rounds of slots
+    // fill badly (3x3 layers with 1.4 rounds of tiles, an 8192^3 GEMM), unless many channel tiles
+    // share each pixel range: their waves then start at staggered K offsets and evict each other's
+    // activations from L2.
+    const bool per_tile =
+        many_tiles && (a.comm < 24 || (a.comm <= 128 && (fill >= 0.85 || ceil_div(a.N, 32) >= 8)));
+    const int regime = (per_tile || whole_rounds) ? 1 : 0;
+    const bool eligible =
+        n_ok && ((many_tiles && a.comm >= 6) || (a.comm >= 24 && iters >= (long)kPlaneSlots * 16));
+    return eligible ? regime : -1 - regime;
+}
+
+// Blobs whose highest field value is a zero weight run on the shift-plane kernel whatever the shape
+// (the two-instruction kernel has no form for them).
+template <int BITS>
+static int dispatch_zero_top(const ShiftArgs &a, hipStream_t st)
+{
+    const int r = plane_regime(a);
+    int nsplit = (r >= 0 ? r : -1 - r) > 0 ? 1 : 0;
+    if (const char *sp = getenv("DS_TUNE_SPLIT")) nsplit = atoi(sp);
+    return launch_planes<BITS, true>(a, nsplit, st);
 }
 
 template <int BITS, bool GENERAL>
@@ -580,24 +647,12 @@ static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
         // The 1x1 shortcuts of small images, single-wave batches and layers with few channels stay on
         // the two-instruction kernel.
         const char *t = getenv("DS_TUNE_PLANES");
-        const long tiles = (long)ceil_div(a.M, kPlaneRows * kWave) * ceil_div(a.N, 32);
-        const long iters = tiles * a.comm;
-        const bool n_ok = a.N % 32 == 0 || a.N >= 256;
-        const bool many_tiles = tiles * 10 >= (long)kPlaneSlots * 13;
-        bool planes = n_ok && ((many_tiles && a.comm >= 6) || (a.comm >= 24 && iters >= (long)kPlaneSlots * 16));
+        bool planes = plane_regime(a) >= 0;
         if (t) planes = atoi(t) > 0;
         if (planes) {
-            const long rounds = (tiles + kPlaneSlots - 1) / kPlaneSlots;
-            const bool whole_rounds = tiles >= kPlaneSlots && (double)tiles / ((double)kPlaneSlots * rounds) >= 0.93;
-            // With many tiles the equal shares still win when the reduction is long and the rounds of
-            // slots fill badly (3x3 layers with 1.4 rounds of tiles, an 8192^3 GEMM), unless many
-            // channel tiles share each pixel range: their waves then start at staggered K offsets
-            // and evict each other's activations from L2.
-            const double fill = (double)tiles / ((double)kPlaneSlots * rounds);
-            const bool per_tile = many_tiles && (a.comm < 24 || (a.comm <= 128 && (fill >= 0.85 || ceil_div(a.N, 32) >= 8)));
-            int nsplit = (per_tile || whole_rounds) ? 1 : 0;
+            int nsplit = plane_regime(a) > 0 ? 1 : 0;
             if (const char *sp = getenv("DS_TUNE_SPLIT")) nsplit = atoi(sp);
-            return launch_planes<BITS>(a, nsplit, st);
+            return launch_planes<BITS, false>(a, nsplit, st);
         }
     }
     TileChoice c = choose_tile(a);
@@ -612,6 +667,15 @@ static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
 
 static int dispatch_bits(const ShiftArgs &a, int bits, bool general, hipStream_t st)
 {
+    if (a.zero_top) {
+        switch (bits) {
+        case 1: return dispatch_zero_top<1>(a, st);
+        case 2: return dispatch_zero_top<2>(a, st);
+        case 3: return dispatch_zero_top<3>(a, st);
+        case 4: return dispatch_zero_top<4>(a, st);
+        default: return DS_EBITS;
+        }
+    }
     switch (bits) {
     case 1: return general ? dispatch_shape<1, true>(a, st) : dispatch_shape<1, false>(a, st);
     case 2: return general ? dispatch_shape<2, true>(a, st) : dispatch_shape<2, false>(a, st);
@@ -621,6 +685,16 @@ static int dispatch_bits(const ShiftArgs &a, int bits, bool general, hipStream_t
     case 6: return dispatch_shape<6, true>(a, st);
     default: return DS_EBITS;
     }
+}
+
+// Splits the zero-top flag off `bits` (tiled entry points only).
+static int take_zero_top(int &bits, int base)
+{
+    if (!(bits & DS_BITS_ZERO_TOP)) return 0;
+    bits &= ~DS_BITS_ZERO_TOP;
+    if (bits < 1 || bits > 4) bits = 0;  // rejected by check_common
+    if (base != 0) bits = 0;
+    return 1;
 }
 
 static int check_common(int bits, int base)
@@ -663,6 +737,7 @@ DS_EXPORT int ds_conv2d_tiled_i32(const int32_t *x, const void *tiled, const int
                                   size_t workspace_bytes, ds_stream_t stream)
 {
     (void)workspace; (void)workspace_bytes;
+    const int zero_top = take_zero_top(bits, base);
     int rc = check_common(bits, base);
     if (rc) return rc;
     if (Nb < 0 || C < 0 || O < 0 || FH < 1 || FW < 1 || sh < 1 || sw < 1 || Hp < FH || Wp < FW)
@@ -695,6 +770,7 @@ DS_EXPORT int ds_conv2d_tiled_i32(const int32_t *x, const void *tiled, const int
     a.x_plane = Hp * Wp; a.x_row = Wp;
     a.FH = FH; a.FW = FW;
     a.nbase = -base;
+    a.zero_top = zero_top;
     return dispatch_bits(a, bits, base != 0 || bits == 6, (hipStream_t)stream);
 }
 
@@ -732,6 +808,7 @@ static size_t linear_scratch_bytes(int M, int N)
 DS_EXPORT size_t ds_linear_tiled_workspace_bytes(int M, int K, int N, int bits)
 {
     (void)K;
+    bits &= ~DS_BITS_ZERO_TOP;
     if (bits < 1 || bits > 6 || M < 0 || N < 0) return 0;
     return linear_scratch_bytes(M, N);
 }
@@ -748,6 +825,7 @@ DS_EXPORT int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled,
                                   int32_t *y, int M, int K, int N, int bits, int base,
                                   void *workspace, size_t workspace_bytes, ds_stream_t stream)
 {
+    const int zero_top = take_zero_top(bits, base);
     int rc = check_common(bits, base);
     if (rc) return rc;
     if (M < 0 || K < 0 || N < 0 || ldx < M) return DS_EINVAL;
@@ -781,6 +859,7 @@ DS_EXPORT int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled,
     a.x_plane = ldx; a.x_row = 1;
     a.FH = 1; a.FW = 1;
     a.nbase = -base;
+    a.zero_top = zero_top;
     return dispatch_bits(a, bits, base != 0 || bits == 6, (hipStream_t)stream);
 }
 

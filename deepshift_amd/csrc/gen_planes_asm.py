@@ -11,7 +11,9 @@ VGPR-relative addressing (s_set_gpr_idx_*), which needs a fixed register map:
     per (k, channel j):                     M0 <- the code's 16-bit pre-decoded form (scalar), mask <- sign
                                             acc[r][j] = (plane[r][M0] ^ mask) + acc[r][j]   (v_xad_u32)
 
-so a shift-add term costs 1 + 2^BITS/32 vector instructions instead of 2.
+so a shift-add term costs 1 + 2^BITS/32 vector instructions instead of 2.  Every width also comes in
+a "zero top" form (DS_PLANES_ASM_B<n>Z) for ternary weights: the highest field value stands for a
+zero weight and its plane is 0 instead of x >> (2^BITS - 1).
 
 Register map (R = 3 pixels per lane, J = 32 channels, NUM = 32 // (BITS + 1) codes per word, D = depth
 of the activation prefetch ring in reduction slots, a divisor of NUM):
@@ -96,7 +98,7 @@ def take_turn(tag):
             end + ":"]
 
 
-def body(bits):
+def body(bits, zero_top=False):
     cb = bits + 1
     num = 32 // cb
     P = 1 << bits
@@ -137,7 +139,11 @@ def body(bits):
         L += walk_and_load(slot)  # the ring slot is free again: load reduction slot i + D into it
         for s in range(1, P):
             for r in range(R):
-                L += ["v_ashrrev_i32 v%d, %d, v%d" % (PL + P * r + s, s, PL + P * r)]
+                if zero_top and s == P - 1:
+                    # the highest field value encodes a zero weight: its plane is 0
+                    L += ["v_mov_b32 v%d, 0" % (PL + P * r + s)]
+                else:
+                    L += ["v_ashrrev_i32 v%d, %d, v%d" % (PL + P * r + s, s, PL + P * r)]
         for j in range(J):
             # the 16-bit code is a ready M0 value: plane index in 7:0, "src0 relative" in 15:12
             if i % 2 == 0:
@@ -166,10 +172,11 @@ def main():
     here = os.path.dirname(os.path.abspath(__file__))
     out = ["// Generated by gen_planes_asm.py -- do not edit by hand.", ""]
     for bits in (1, 2, 3, 4):
-        lines = body(bits)
-        out.append("#define DS_PLANES_ASM_B%d \\" % bits)
-        out.append(" \\\n".join('    "%s\\n"' % line for line in lines))
-        out.append("")
+        for zero_top, tag in ((False, ""), (True, "Z")):
+            lines = body(bits, zero_top)
+            out.append("#define DS_PLANES_ASM_B%d%s \\" % (bits, tag))
+            out.append(" \\\n".join('    "%s\\n"' % line for line in lines))
+            out.append("")
         out.append("#define DS_PLANES_CLOBBERS_B%d %s" % (bits, clobbers(bits)))
         out.append("")
     with open(os.path.join(here, "ds_planes_asm.inc"), "w") as f:

@@ -33,7 +33,8 @@ def packed_state(model):
     for name, m in _shift_layers(model):
         cw = _pack(m)
         shape = list((m.shift if hasattr(m, "shift") else m.weight).shape)
-        entry = {"words": cw.data.detach().cpu(), "bits": int(cw.bits), "base": int(cw.base), "shape": shape}
+        entry = {"words": cw.data.detach().cpu(), "bits": int(cw.bits), "base": int(cw.base), "shape": shape,
+                 "zero_top_bits": int(getattr(cw, "zero_top_bits", 0))}
         if m.bias is not None:
             entry["bias"] = m.bias.detach().float().cpu()
         layers[name] = entry
@@ -71,7 +72,7 @@ def load_packed(model, path_or_state, device=None):
         words = entry["words"].to(dev, torch.int32).contiguous()
         if words.numel() != param.shape[0] * comm:
             raise ValueError("%s: %d packed words, expected %d" % (name, words.numel(), param.shape[0] * comm))
-        m.conc_weight = utils.ConcWeight(words, base, bits)
+        m.conc_weight = utils.ConcWeight(words, base, bits, int(entry.get("zero_top_bits", 0)))
         m.use_kernel = True
         if "bias" in entry and m.bias is not None:
             with torch.no_grad():

@@ -119,13 +119,41 @@ def tile_weights(packed, N, C, FH, FW, bits, base=0):
     return blob
 
 
+def tile_weights_zero_top(packed, N, C, FH, FW, field_bits):
+    """6-bit reference words of a ternary layer whose non-zero fields are all below
+    ``2**field_bits - 1`` -> a tiled blob of ``field_bits``-wide codes whose highest value means
+    "zero weight" (pass ``field_bits | DS_BITS_ZERO_TOP`` as ``bits`` to the tiled kernels)."""
+    packed = _require_device_i32("packed", packed)
+    K = C * FH * FW
+    if packed.numel() != N * ((K + 3) // 4):
+        raise ValueError("packed weight has %d words, expected %d" % (packed.numel(), N * ((K + 3) // 4)))
+    nbytes = _lib.lib().ds_tiled_bytes(N, K, field_bits)
+    blob = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=packed.device)
+    _lib.call("ds_tile_weights_zero_top_i32", _lib.ptr(packed), _lib.ptr(blob), N, C, FH, FW,
+              int(field_bits), _lib.current_stream(packed.device))
+    return blob
+
+
+def kernel_bits(conc_weight):
+    """The ``bits`` argument of the tiled kernels for the blob :func:`_tiled_of` builds."""
+    width = getattr(conc_weight, "zero_top_bits", 0)
+    if width and conc_weight.bits == 6 and conc_weight.base == 0:
+        return width | _lib.DS_BITS_ZERO_TOP
+    return conc_weight.bits
+
+
 def _tiled_of(conc_weight, N, C, FH=1, FW=1):
     """The tiled blob of a ConcWeight, built once and cached on the object."""
     data = conc_weight.data
-    key = (data.data_ptr(), data._version, N, C, FH, FW, conc_weight.bits, conc_weight.base)
+    kbits = kernel_bits(conc_weight)
+    key = (data.data_ptr(), data._version, N, C, FH, FW, kbits, conc_weight.base)
     cached = getattr(conc_weight, "_tiled", None)
     if cached is None or cached[0] != key:
-        cached = (key, tile_weights(data, N, C, FH, FW, conc_weight.bits, conc_weight.base))
+        if kbits & _lib.DS_BITS_ZERO_TOP:
+            blob = tile_weights_zero_top(data, N, C, FH, FW, kbits & ~_lib.DS_BITS_ZERO_TOP)
+        else:
+            blob = tile_weights(data, N, C, FH, FW, conc_weight.bits, conc_weight.base)
+        cached = (key, blob)
         conc_weight._tiled = cached
     return cached[1]
 
@@ -300,7 +328,7 @@ def linear(input, shift, sign, bias=None, conc_weight=None, use_cuda=True):
     xT = torch.empty([K, ldx], dtype=torch.int32, device=input.device)
     _lib.call("ds_transpose_i32", _lib.ptr(input), _lib.ptr(xT), M, K, ldx,
               _lib.current_stream(input.device))
-    return linear_tiled(xT, M, tiled, bias, N, conc_weight.bits, conc_weight.base)
+    return linear_tiled(xT, M, tiled, bias, N, kernel_bits(conc_weight), conc_weight.base)
 
 
 def conv2d_tiled(x_padded, tiled, bias, O, kernel_size, stride, bits, base=0):
@@ -353,4 +381,4 @@ def conv2d(input, shift, sign, bias=None, conc_weight=None, stride=1, padding=0,
     else:
         xp = input
     tiled = _tiled_of(conc_weight, O, C, FH, FW)
-    return conv2d_tiled(xp, tiled, bias, O, (FH, FW), stride, conc_weight.bits, conc_weight.base)
+    return conv2d_tiled(xp, tiled, bias, O, (FH, FW), stride, kernel_bits(conc_weight), conc_weight.base)

@@ -106,7 +106,7 @@ class LinearShift(nn.Module):
         xT = kernels.quantize_transpose(x2d, I, Fb, round_to_fixed=False)
         bias = self._fixed_bias.get(self.bias, I, Fb, round_to_fixed=False)
         tiled = kernels._tiled_of(self.conc_weight, self.out_features, self.in_features)
-        out = kernels.linear_tiled(xT, M, tiled, bias, self.out_features, self.conc_weight.bits,
+        out = kernels.linear_tiled(xT, M, tiled, bias, self.out_features, kernels.kernel_bits(self.conc_weight),
                                    self.conc_weight.base)
         return kernels.dequantize(out, Fb).reshape(*lead, self.out_features)
 
@@ -228,7 +228,7 @@ def conv_kernel_forward(module, input, conc_weight, scale=None, shift=None, resi
     tiled = kernels._tiled_of(conc_weight, module.out_channels, module.in_channels,
                               module.kernel_size[0], module.kernel_size[1])
     out = kernels.conv2d_tiled(xq, tiled, bias, module.out_channels, module.kernel_size,
-                               module.stride, conc_weight.bits, conc_weight.base)
+                               module.stride, kernels.kernel_bits(conc_weight), conc_weight.base)
     if pool is not None:
         if residual is not None:
             raise ValueError("a fused max pooling cannot follow a residual add")

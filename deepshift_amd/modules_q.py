@@ -80,7 +80,7 @@ class LinearShiftQ(nn.Module):
         xT = kernels.quantize_transpose(x2d, I, Fb, round_to_fixed=True)
         bias = self._fixed_bias.get(self.bias, I, Fb, round_to_fixed=True)
         tiled = kernels._tiled_of(self.conc_weight, self.out_features, self.in_features)
-        out = kernels.linear_tiled(xT, M, tiled, bias, self.out_features, self.conc_weight.bits,
+        out = kernels.linear_tiled(xT, M, tiled, bias, self.out_features, kernels.kernel_bits(self.conc_weight),
                                    self.conc_weight.base)
         return kernels.dequantize(out, Fb).reshape(*lead, self.out_features)
 

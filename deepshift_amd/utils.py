@@ -71,10 +71,14 @@ class ConcWeight():
     reference's row-major word format, ``base`` (0 or the negative minimum of -shift) and ``bits``
     (width of the shift field; a code takes ``bits + 1`` bits)."""
 
-    def __init__(self, data=None, base=0, bits=8):
+    def __init__(self, data=None, base=0, bits=8, zero_top_bits=0):
         self.data = data
         self.base = base
         self.bits = bits
+        # Not in the reference: for 6-bit words that only need them for the zero code (ternary
+        # weights), the field width into which the non-zero shifts fit with one value to spare;
+        # the kernels then run the layer from a narrower private blob (0: not applicable).
+        self.zero_top_bits = zero_top_bits
 
 
 def shift_field_bits(min_shift):
@@ -132,6 +136,14 @@ def compress_bits(shift, sign):
     num = int(32 / (conc_weight.bits + 1))
     row_length = int((shift.shape[1] * shift.shape[2] * shift.shape[3] + num - 1) / num)
     size = row_length * shift.shape[0]
+
+    if conc_weight.bits == 6 and conc_weight.base == 0:
+        real = s[s < ZERO_SHIFT]
+        top = int(real.max()) if real.numel() else 0
+        for width in (1, 2, 3, 4):
+            if top <= 2 ** width - 2:
+                conc_weight.zero_top_bits = width
+                break
 
     conc_weight.data = kernels.compress_sign_and_shift(
         s.int().cuda(), sign.int().cuda(), size, conc_weight.base, conc_weight.bits, row_length, num)

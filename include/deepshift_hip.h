@@ -66,6 +66,21 @@ size_t ds_tiled_bytes(int N, int K, int bits);
 int ds_tile_weights_i32(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW, int bits,
                         int base, ds_stream_t stream);
 
+/* Ternary weights.  The reference encodes a zero weight as shift -32, which forces 6-bit fields
+ * (utils.py:68-72, four codes per word) on every layer that has one -- every DeepShift-PS layer with
+ * a ternary sign.  When the non-zero shifts of such a layer fit field_bits (1..4) with one value to
+ * spare -- all fields <= 2^field_bits - 2, e.g. weight_bits 5 whose shift range [-14, 0] the
+ * reference reserves exactly for this, modules.py:88 -- this call re-packs its 6-bit reference words
+ * (base 0) into a blob of field_bits-wide codes in which the highest field value stands for "zero
+ * weight".  ds_tiled_bytes(N, K, field_bits) sizes it; the tiled compute entry points take it with
+ * bits = field_bits | DS_BITS_ZERO_TOP and base = 0, and run it on the shift-plane kernel (the zero
+ * code selects a plane held at 0): same results as the 6-bit blob at the speed of a 4-bit layer.
+ * The caller vouches for the field range (deepshift_amd.utils.compress_bits checks it when it
+ * packs).  No counterpart in the reference. */
+#define DS_BITS_ZERO_TOP 0x100
+int ds_tile_weights_zero_top_i32(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW,
+                                 int field_bits, ds_stream_t stream);
+
 /* ---- LinearShift ----------------------------------------------------------------------- */
 
 /* Workspace bytes ds_linear_i32 needs (transposed activations, tiled weights, offset table). */

@@ -392,3 +392,62 @@ def test_quantize_pad_transpose_dequantize(oracle, rng):
     yd = dev(y)
     _lib.call("ds_dequantize_i32_f32", _lib.ptr(yd), _lib.ptr(out), y.size, 16, stream())
     np.testing.assert_array_equal(out.cpu().numpy(), y.astype(np.float32) / np.float32(65536.0))
+
+
+# ----------------------------------------------------------------------------- ternary blobs
+
+def _ternary_case(rng, shape, max_s, zero_frac=0.3):
+    s, sign = random_codes(rng, shape, max_s=max_s, zero_frac=zero_frac)
+    s_z = np.where(sign == 0, 32, s).astype(np.int32)
+    sign_z = np.where(sign == 0, 1, sign).astype(np.int32)
+    return s, sign, s_z, sign_z
+
+
+@pytest.mark.parametrize("split", [None, 0, 1, 3])
+@pytest.mark.parametrize("width", [1, 2, 3, 4])
+def test_zero_top_blob_matches_oracle(oracle, rng, width, split):
+    """6-bit ternary words re-packed into `width`-bit codes whose highest value means zero
+    (ds_tile_weights_zero_top_i32) give the results of the 6-bit path, on every launch mode."""
+    from deepshift_amd import kernels
+    L = _lib.lib()
+    flag = width | _lib.DS_BITS_ZERO_TOP
+    env = {} if split is None else {"DS_TUNE_SPLIT": split}
+    with _Tune(**env):
+        # GEMM, ragged in every dimension
+        M, K, N = 333, 517, 71
+        x = random_activations(rng, (M, K))
+        s, sign, s_z, sign_z = _ternary_case(rng, (N, K), 2 ** width - 2)
+        bias = rng.integers(-2 ** 20, 2 ** 20, size=N).astype(np.int32)
+        want = oracle.linear(x, -s, sign, bias, nthreads=NTHREADS)
+        w6 = dev(so.np_pack_words(s_z, sign_z, 6))
+        blob = kernels.tile_weights_zero_top(w6.reshape(-1), N, K, 1, 1, width)
+        xT = dev(np.ascontiguousarray(np.pad(x, ((0, (-M) % 64), (0, 0))).T))
+        got = kernels.linear_tiled(xT, M, blob, dev(bias), N, flag, 0)
+        np.testing.assert_array_equal(got.cpu().numpy(), want)
+        # convolution, stride 2, 40 channels, partial last word
+        Nb, C, Hp, Wp, O = 3, 5, 21, 17, 40
+        xp = random_activations(rng, (Nb, C, Hp, Wp))
+        s, sign, s_z, sign_z = _ternary_case(rng, (O, C, 3, 3), 2 ** width - 2)
+        want = oracle.conv2d(xp, -s, sign, None, (2, 2), nthreads=NTHREADS)
+        w6 = dev(so.np_pack_words(s_z.reshape(O, -1), sign_z.reshape(O, -1), 6))
+        blob = kernels.tile_weights_zero_top(w6.reshape(-1), O, C, 3, 3, width)
+        got = kernels.conv2d_tiled(dev(xp), blob, None, O, (3, 3), (2, 2), flag, 0)
+        np.testing.assert_array_equal(got.cpu().numpy(), want)
+    one = ctypes.c_void_p(16)
+    assert L.ds_tile_weights_zero_top_i32(one, one, 4, 4, 1, 1, 5, None) == -2
+    assert L.ds_linear_tiled_i32(one, 64, one, None, one, 4, 4, 4, 5 | _lib.DS_BITS_ZERO_TOP, 0, one, 1 << 20, None) == -2
+    assert L.ds_linear_tiled_i32(one, 64, one, None, one, 4, 4, 4, flag, -1, one, 1 << 20, None) == -2
+    assert L.ds_linear_i32(one, one, None, one, 4, 4, 4, flag, 0, one, 1 << 20, None) == -2
+
+
+def test_compress_bits_finds_the_zero_top_width(rng):
+    from deepshift_amd import kernels, utils
+    for max_s, want in [(0, 1), (2, 2), (3, 3), (6, 3), (7, 4), (14, 4), (15, 0), (31, 0)]:
+        s, sign = random_codes(rng, (8, 40), max_s=max_s, zero_frac=0.25)
+        s[0, 0], sign[0, 0] = max_s, 1
+        cw = utils.compress_bits(torch.from_numpy(-s).float(), torch.from_numpy(sign).float())
+        assert cw.bits == 6 and cw.zero_top_bits == want, (max_s, cw.zero_top_bits)
+        assert kernels.kernel_bits(cw) == ((want | _lib.DS_BITS_ZERO_TOP) if want else 6)
+    s, sign = random_codes(rng, (8, 40), max_s=14)  # no zero weight: plain 4-bit fields
+    cw = utils.compress_bits(torch.from_numpy(-s).float(), torch.from_numpy(sign).float())
+    assert cw.bits == 4 and cw.zero_top_bits == 0
