@@ -105,17 +105,21 @@ __global__ void tile_kernel(const int32_t *__restrict__ w_ref, uint32_t *__restr
     wt[idx] = out;
 }
 
-// negcount[n] = number of real, non-zero, negative codes of channel n (0 for padding channels)
-__global__ void negcount_kernel(const int32_t *__restrict__ w_ref, int32_t *__restrict__ negcount,
-                                int N, int Npad, int K, int comm, int bits, int num)
+// negcount[n] = number of real, non-zero, negative codes of channel n (0 for padding channels).
+// One wave per channel: the lanes stride over the channel's words and the counts are summed
+// across the wave.
+__global__ __launch_bounds__(256) void negcount_kernel(const int32_t *__restrict__ w_ref,
+                                                       int32_t *__restrict__ negcount, int N, int Npad,
+                                                       int K, int comm, int bits, int num)
 {
-    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int n = blockIdx.x * (blockDim.x / kWave) + (threadIdx.x / kWave);
     if (n >= Npad) return;
     int count = 0;
     if (n < N) {
         const int cb = bits + 1;
         const uint32_t fmask = (1u << bits) - 1u;
-        for (int g = 0; g < comm; ++g) {
+        for (int g = lane; g < comm; g += kWave) {
             const uint32_t in = (uint32_t)w_ref[(long)n * comm + g];
             for (int i = 0; i < num; ++i) {
                 if (g * num + i >= K) break;
@@ -124,7 +128,8 @@ __global__ void negcount_kernel(const int32_t *__restrict__ w_ref, int32_t *__re
             }
         }
     }
-    negcount[n] = count;
+    for (int off = kWave / 2; off > 0; off >>= 1) count += __shfl_down(count, off, kWave);
+    if (lane == 0) negcount[n] = count;
 }
 
 // ktab[k] = ic << 10 | fh << 5 | fw for k = (ic, fh, fw) < K, 0 beyond: the geometry-independent
@@ -185,7 +190,7 @@ int launch_tile(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW,
     }
     const int Npad = g.ntiles * kTileWords;
     if (Npad) {
-        hipLaunchKernelGGL(negcount_kernel, dim3(ceil_div(Npad, 64)), dim3(64), 0, st, w_ref,
+        hipLaunchKernelGGL(negcount_kernel, dim3(ceil_div(Npad, 4)), dim3(256), 0, st, w_ref,
                            (int32_t *)tiled_negcount(tiled, g), N, Npad, K, in_comm, in_bits, in_num);
     }
     hipLaunchKernelGGL(ktab_kernel, dim3(ceil_div((int)g.ktab_count, 256)), dim3(256), 0, st,
