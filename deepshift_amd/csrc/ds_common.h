@@ -16,6 +16,28 @@ __host__ __device__ constexpr int codes_per_word(int bits) { return 32 / (bits +
 __host__ __device__ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
+// Exact unsigned 32-bit division by a launch-invariant divisor in five integer instructions
+// (Granlund-Montgomery round-up form): the element-wise kernels turn a flat index into
+// (plane, row, column) with it instead of the ~25-instruction emulated divide.
+struct FastDiv {
+    uint32_t d, m, s1, s2;
+};
+inline FastDiv fast_div(uint32_t d)
+{
+    FastDiv f{d ? d : 1u, 1u, 0u, 0u};
+    uint32_t l = 0;
+    while (l < 32 && (1ull << l) < f.d) ++l;  // l = ceil(log2 d)
+    f.m = (uint32_t)((((1ull << l) - f.d) << 32) / f.d + 1);
+    f.s1 = l < 1 ? l : 1;
+    f.s2 = l > 1 ? l - 1 : 0;
+    return f;
+}
+__device__ __forceinline__ uint32_t div_by(uint32_t n, const FastDiv &f)
+{
+    const uint32_t t = __umulhi(f.m, n);
+    return (t + ((n - t) >> f.s1)) >> f.s2;
+}
+
 inline int hip_status(hipError_t e) { return e == hipSuccess ? DS_OK : DS_EHIP - (int)e; }
 inline int launch_status() { return hip_status(hipGetLastError()); }
 

@@ -82,21 +82,19 @@ __global__ void quantize_kernel(const float *__restrict__ x, int32_t *__restrict
 
 // One thread per padded output element; rows of the padded image are written contiguously.
 template <bool FROM_FLOAT>
-__global__ void pad_kernel(const void *__restrict__ xin, int32_t *__restrict__ q, long planes, int H,
-                           int W, int ph, int pw, QuantSpec spec)
+__global__ void pad_kernel(const void *__restrict__ xin, int32_t *__restrict__ q, uint32_t planes, int H,
+                           int W, int ph, int pw, QuantSpec spec, FastDiv by_plane, FastDiv by_row)
 {
-    const int Hp = H + 2 * ph, Wp = W + 2 * pw;
-    const long total = planes * Hp * Wp;
-    const long stride = (long)gridDim.x * blockDim.x;
-    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
-        const long plane = idx / ((long)Hp * Wp);
-        const int rem = (int)(idx - plane * Hp * Wp);
-        const int hp = rem / Wp;
-        const int wp = rem - hp * Wp;
-        const int h = hp - ph, w = wp - pw;
+    const uint32_t Hp = H + 2 * ph, Wp = W + 2 * pw;
+    const uint32_t total = planes * Hp * Wp;  // < 2^29: tensors are below 2 GiB
+    for (uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+        const uint32_t plane = div_by(idx, by_plane);
+        const uint32_t rem = idx - plane * Hp * Wp;
+        const uint32_t hp = div_by(rem, by_row);
+        const int h = (int)hp - ph, w = (int)(rem - hp * Wp) - pw;
         int32_t v = 0;
         if ((unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W) {
-            const long src = (plane * H + h) * W + w;
+            const uint32_t src = (plane * H + h) * W + w;
             if (FROM_FLOAT) v = quantize_one(((const float *)xin)[src], spec);
             else v = ((const int32_t *)xin)[src];
         }
@@ -229,19 +227,20 @@ __global__ void requantize_affine_pad_kernel(const int32_t *__restrict__ y, floa
                                              const float *__restrict__ shift,
                                              const float *__restrict__ residual, uint32_t planes, int C,
                                              int H, int W, int ph, int pw, float inv, int relu,
-                                             QuantSpec spec)
+                                             QuantSpec spec, FastDiv by_plane, FastDiv by_row,
+                                             FastDiv by_channels)
 {
     const uint32_t Hp = H + 2 * ph, Wp = W + 2 * pw;
     const uint32_t total = planes * Hp * Wp;
     for (uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
-        const uint32_t plane = idx / (Hp * Wp);
+        const uint32_t plane = div_by(idx, by_plane);
         const uint32_t rem = idx - plane * Hp * Wp;
-        const uint32_t hp = rem / Wp;
+        const uint32_t hp = div_by(rem, by_row);
         const int h = (int)hp - ph, w = (int)(rem - hp * Wp) - pw;
         int32_t v = 0;
         if ((unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W) {
             const uint32_t src = (plane * H + h) * W + w;
-            const uint32_t c = plane % (uint32_t)C;
+            const uint32_t c = plane - div_by(plane, by_channels) * (uint32_t)C;
             const float f = affine_one(y[src], inv, scale ? scale[c] : 1.0f, shift ? shift[c] : 0.0f,
                                        residual ? residual + src : nullptr, relu);
             if (out) out[src] = f;
@@ -259,31 +258,59 @@ __global__ void requantize_affine_maxpool_kernel(const int32_t *__restrict__ y, 
                                                  int32_t *__restrict__ q, const float *__restrict__ scale,
                                                  const float *__restrict__ shift, uint32_t planes, int C,
                                                  int H, int W, int OH, int OW, int pk, int ps, int pp,
-                                                 int ph, int pw, float inv, int relu, QuantSpec spec)
+                                                 int ph, int pw, float inv, int relu, QuantSpec spec,
+                                                 FastDiv by_plane, FastDiv by_row, FastDiv by_channels)
 {
     const uint32_t Hp = OH + 2 * ph, Wp = OW + 2 * pw;
     const uint32_t total = planes * Hp * Wp;
     for (uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
-        const uint32_t plane = idx / (Hp * Wp);
+        const uint32_t plane = div_by(idx, by_plane);
         const uint32_t rem = idx - plane * Hp * Wp;
-        const uint32_t hp = rem / Wp;
+        const uint32_t hp = div_by(rem, by_row);
         const int oh = (int)hp - ph, ow = (int)(rem - hp * Wp) - pw;
         int32_t v = 0;
         if ((unsigned)oh < (unsigned)OH && (unsigned)ow < (unsigned)OW) {
-            const uint32_t c = plane % (uint32_t)C;
+            const uint32_t c = plane - div_by(plane, by_channels) * (uint32_t)C;
             const float a = scale ? scale[c] : 1.0f, b = shift ? shift[c] : 0.0f;
             const int32_t *yp = y + (size_t)plane * H * W;
-            float best = -__builtin_inff();
-            for (int i = 0; i < pk; ++i) {
-                const int ih = oh * ps - pp + i;
-                if ((unsigned)ih >= (unsigned)H) continue;
-                for (int j = 0; j < pk; ++j) {
-                    const int iw = ow * ps - pp + j;
-                    if ((unsigned)iw >= (unsigned)W) continue;
-                    const float f = affine_one(yp[ih * W + iw], inv, a, b, nullptr, relu);
-                    best = f > best ? f : best;
+            // affine_one is monotonic in y (non-decreasing for a >= 0, non-increasing for a < 0: every
+            // rounding step is), so the maximum of the window is affine_one of its largest / smallest
+            // int32 -- one conversion per output instead of one per window element
+            const bool flip = a < 0.0f;
+            int32_t ext = flip ? INT32_MAX : INT32_MIN;
+            if (pk == 3) {
+                // the usual 3x3 window: nine independent loads from clamped coordinates (no branch
+                // between them, so they are all in flight together), masked afterwards
+                int32_t v[9];
+                bool ok[9];
+#pragma unroll
+                for (int i = 0; i < 3; ++i) {
+                    const int ih = oh * ps - pp + i;
+                    const int ihc = ih < 0 ? 0 : (ih >= H ? H - 1 : ih);
+#pragma unroll
+                    for (int j = 0; j < 3; ++j) {
+                        const int iw = ow * ps - pp + j;
+                        const int iwc = iw < 0 ? 0 : (iw >= W ? W - 1 : iw);
+                        ok[i * 3 + j] = ih == ihc && iw == iwc;
+                        v[i * 3 + j] = yp[ihc * W + iwc];
+                    }
+                }
+#pragma unroll
+                for (int t = 0; t < 9; ++t)
+                    if (ok[t]) ext = flip ? (v[t] < ext ? v[t] : ext) : (v[t] > ext ? v[t] : ext);
+            } else {
+                for (int i = 0; i < pk; ++i) {
+                    const int ih = oh * ps - pp + i;
+                    if ((unsigned)ih >= (unsigned)H) continue;
+                    for (int j = 0; j < pk; ++j) {
+                        const int iw = ow * ps - pp + j;
+                        if ((unsigned)iw >= (unsigned)W) continue;
+                        const int32_t v = yp[ih * W + iw];
+                        ext = flip ? (v < ext ? v : ext) : (v > ext ? v : ext);
+                    }
                 }
             }
+            const float best = affine_one(ext, inv, a, b, nullptr, relu);
             if (out) out[((size_t)plane * OH + oh) * OW + ow] = best;
             v = quantize_one(best, spec);
         }
@@ -337,9 +364,11 @@ DS_EXPORT int ds_quantize_pad_f32_i32(const float *x, int32_t *q, int Nb, int C,
     if (Nb < 0 || C < 0 || H < 0 || W < 0 || ph < 0 || pw < 0) return DS_EINVAL;
     const long total = (long)Nb * C * (H + 2 * ph) * (W + 2 * pw);
     if (total == 0) return DS_OK;
+    if (total * 4 >= (1L << 31)) return DS_ETOOLARGE;  // like every tensor of the compute kernels
     if (!x || !q) return DS_EINVAL;
     hipLaunchKernelGGL((pad_kernel<true>), dim3(grid_for(total)), dim3(256), 0, (hipStream_t)stream,
-                       (const void *)x, q, (long)Nb * C, H, W, ph, pw, make_spec(I, F, mode));
+                       (const void *)x, q, (uint32_t)(Nb * C), H, W, ph, pw, make_spec(I, F, mode),
+                       fast_div((uint32_t)((H + 2 * ph) * (W + 2 * pw))), fast_div((uint32_t)(W + 2 * pw)));
     return launch_status();
 }
 
@@ -349,9 +378,11 @@ DS_EXPORT int ds_pad_i32(const int32_t *x, int32_t *xp, int Nb, int C, int H, in
     if (Nb < 0 || C < 0 || H < 0 || W < 0 || ph < 0 || pw < 0) return DS_EINVAL;
     const long total = (long)Nb * C * (H + 2 * ph) * (W + 2 * pw);
     if (total == 0) return DS_OK;
+    if (total * 4 >= (1L << 31)) return DS_ETOOLARGE;
     if (!x || !xp) return DS_EINVAL;
     hipLaunchKernelGGL((pad_kernel<false>), dim3(grid_for(total)), dim3(256), 0, (hipStream_t)stream,
-                       (const void *)x, xp, (long)Nb * C, H, W, ph, pw, make_spec(16, 16, 0));
+                       (const void *)x, xp, (uint32_t)(Nb * C), H, W, ph, pw, make_spec(16, 16, 0),
+                       fast_div((uint32_t)((H + 2 * ph) * (W + 2 * pw))), fast_div((uint32_t)(W + 2 * pw)));
     return launch_status();
 }
 
@@ -421,7 +452,9 @@ DS_EXPORT int ds_requantize_affine_pad_i32(const int32_t *y, float *out, int32_t
     if (!q || (!y && (long)Nb * C * H * W > 0)) return DS_EINVAL;
     hipLaunchKernelGGL(requantize_affine_pad_kernel, dim3(grid_for(total)), dim3(256), 0,
                        (hipStream_t)stream, y, out, q, scale, shift, residual, (uint32_t)(Nb * C), C, H, W,
-                       ph, pw, ldexpf(1.0f, -F_in), relu, make_spec(I, F, mode));
+                       ph, pw, ldexpf(1.0f, -F_in), relu, make_spec(I, F, mode),
+                       fast_div((uint32_t)((H + 2 * ph) * (W + 2 * pw))), fast_div((uint32_t)(W + 2 * pw)),
+                       fast_div((uint32_t)C));
     return launch_status();
 }
 
@@ -443,7 +476,9 @@ DS_EXPORT int ds_requantize_affine_maxpool_i32(const int32_t *y, float *out, int
     if (!y || (!q && !out)) return DS_EINVAL;
     hipLaunchKernelGGL(requantize_affine_maxpool_kernel, dim3(grid_for(total)), dim3(256), 0,
                        (hipStream_t)stream, y, out, q, scale, shift, (uint32_t)(Nb * C), C, H, W, OH, OW, pk,
-                       ps, pp, ph, pw, ldexpf(1.0f, -F_in), relu, make_spec(I, F, mode));
+                       ps, pp, ph, pw, ldexpf(1.0f, -F_in), relu, make_spec(I, F, mode),
+                       fast_div((uint32_t)((OH + 2 * ph) * (OW + 2 * pw))), fast_div((uint32_t)(OW + 2 * pw)),
+                       fast_div((uint32_t)C));
     return launch_status();
 }
 
