@@ -384,9 +384,7 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
         load_group<NUM, R>(xt, xrsrc, xoff, p, g);
 #pragma unroll
         for (int i = 0; i < NUM; ++i) {
-            const bool real = g * NUM + i < p.K;
-#pragma unroll
-            for (int r = 0; r < R; ++r) xt[i][r] = real ? xt[i][r] : 0;
+            if (g * NUM + i >= p.K) break;  // the codes past K trail the word: nothing left to add
             if (ZT) accumulate_code_zero_top<BITS, R, J>(acc, xt[i], w, i);
             else accumulate_code<BITS, false, R, J>(acc, xt[i], w, i, 0);
         }
