@@ -544,13 +544,20 @@ static TileChoice choose_tile(const ShiftArgs &a)
     else if (a.M <= 64) { c.R = 1; c.J = a.N >= 256 ? 8 : 32; }  // a single wave of rows: many narrow tiles
     else if (a.comm <= 32 && a.N >= 64) { c.R = 4; c.J = 16; }  // short reduction (e.g. 7x7x3 stem)
     else if (a.x_col_stride > 1 && a.OW > 8) { c.R = 3; c.J = 16; }  // strided pixels: half-used lines
-    const long tiles = (long)ceil_div(a.M, c.R * kWave) * ceil_div(a.N, c.J);
     const long simds = 1024;
+    // short layers (the 1x1 shortcuts of small images): with fewer than two 128-pixel tiles per SIMD
+    // the launch is set by its start-up and the fullest SIMD; single-row tiles double the waves
+    if (c.R > 1 && a.N >= 32 && (long)ceil_div(a.M, 2 * kWave) * ceil_div(a.N, 32) < 2 * simds) {
+        c.R = 1;
+        c.J = 32;
+    }
+    const long tiles = (long)ceil_div(a.M, c.R * kWave) * ceil_div(a.N, c.J);
     const double per_simd = (double)tiles / simds;
     const double balance = per_simd / (double)((tiles + simds - 1) / simds);
     if (tiles >= 12 * simds || (tiles >= 4 * simds && balance >= 0.94)) return c;
     long want = (24 * simds + tiles / 2) / tiles;
-    const long max_by_k = a.comm / 12 > 0 ? a.comm / 12 : 1;
+    const long min_groups = c.R == 1 ? 10 : 12;
+    const long max_by_k = a.comm / min_groups > 0 ? a.comm / min_groups : 1;
     if (want > max_by_k) want = max_by_k;
     if (want > 32) want = 32;
     if (want < 1) want = 1;
