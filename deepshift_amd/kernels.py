@@ -13,7 +13,6 @@ Differences from the reference, all deliberate:
   kernels.py:32-33, swaps them; identical for square padding).
 * weights that have to stay zero contribute exactly 0 (see ``utils.compress_bits``).
 """
-import ctypes
 
 import torch
 

@@ -13,7 +13,6 @@ evidently intends.
 """
 import math
 
-import torch
 import torch.nn as nn
 import torch.nn.functional as F
 from torch.nn import init

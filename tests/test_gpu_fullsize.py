@@ -7,7 +7,6 @@ import pytest
 import torch
 
 from deepshift_amd import kernels, utils
-from oracle import shift_oracle as so
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"

@@ -1,7 +1,6 @@
 """The float multiply-accumulate comparator (deepshift_amd.unoptimized) against PyTorch's own fp32
 linear / conv2d.  The kernel accumulates in reduction order k = 0..K-1 in fp32, PyTorch in another
 order, so the comparison allows K * eps_fp32 relative to the magnitude of the terms."""
-import numpy as np
 import pytest
 import torch
 import torch.nn as nn
