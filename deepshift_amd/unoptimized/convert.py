@@ -1,26 +1,30 @@
 """``convert_to_unoptimized`` (unoptimized/convert.py:8-30 in the reference): every ``nn.Linear`` /
-``nn.Conv2d`` becomes its comparator counterpart, sharing the original parameters."""
+``nn.Conv2d`` of a model becomes its comparator counterpart and keeps its parameters."""
 import torch.nn as nn
 
 from .modules import UnoptimizedConv2d, UnoptimizedLinear
 
 
+def _as_comparator(layer):
+    """The comparator module for an exact ``nn.Linear`` / ``nn.Conv2d`` (subclasses are left alone),
+    sharing the layer's parameter objects; ``None`` for anything else."""
+    if type(layer) is nn.Linear:
+        twin = UnoptimizedLinear(layer.in_features, layer.out_features, bias=layer.bias is not None)
+    elif type(layer) is nn.Conv2d:
+        twin = UnoptimizedConv2d(layer.in_channels, layer.out_channels, layer.kernel_size, layer.stride,
+                                 layer.padding, layer.dilation, layer.groups, layer.bias is not None,
+                                 layer.padding_mode)
+    else:
+        return None
+    twin.weight, twin.bias = layer.weight, layer.bias
+    return twin.to(layer.weight.device)
+
+
 def convert_to_unoptimized(model):
-    for name, module in model._modules.items():
-        if module is None:
-            continue
-        if len(list(module.children())) > 0:
-            model._modules[name] = convert_to_unoptimized(model=module)
-        if type(module) == nn.Linear:
-            new = UnoptimizedLinear(module.in_features, module.out_features, module.bias is not None)
-            new.weight = module.weight
-            new.bias = module.bias
-            model._modules[name] = new
-        if type(module) == nn.Conv2d:
-            new = UnoptimizedConv2d(module.in_channels, module.out_channels, module.kernel_size,
-                                    module.stride, module.padding, module.dilation, module.groups,
-                                    module.bias is not None, module.padding_mode)
-            new.weight = module.weight
-            new.bias = module.bias
-            model._modules[name] = new
+    for name, child in list(model.named_children()):
+        twin = _as_comparator(child)
+        if twin is not None:
+            setattr(model, name, twin)
+        else:
+            convert_to_unoptimized(child)
     return model

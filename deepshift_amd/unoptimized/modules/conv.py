@@ -1,59 +1,21 @@
-"""``UnoptimizedConv2d`` (unoptimized/modules/conv.py:12-93 in the reference): zero padding with
-``F.pad``, then the float multiply-accumulate kernel on the padded input."""
-import math
-
-import torch
+"""``UnoptimizedConv2d``: an ``nn.Conv2d`` whose forward pass pads with zeros and runs the
+comparator's float multiply-accumulate kernel on the padded input (the role of
+unoptimized/modules/conv.py:12-93 in the reference)."""
 import torch.nn as nn
 import torch.nn.functional as F
-from torch.nn import init
-from torch.nn.modules.utils import _pair
 
 from .. import kernels
 
 
-class UnoptimizedConv2d(nn.Module):
-    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
-                 groups=1, bias=True, padding_mode='zeros'):
-        super().__init__()
-        if in_channels % groups != 0:
-            raise ValueError('in_channels must be divisible by groups')
-        if out_channels % groups != 0:
-            raise ValueError('out_channels must be divisible by groups')
-        self.in_channels = in_channels
-        self.out_channels = out_channels
-        self.kernel_size = _pair(kernel_size)
-        self.stride = _pair(stride)
-        self.padding = _pair(padding)
-        self.dilation = _pair(dilation)
-        self.groups = groups
-        self.padding_mode = padding_mode
-        self.weight = nn.Parameter(torch.empty(out_channels, in_channels // groups, *self.kernel_size))
-        if bias:
-            self.bias = nn.Parameter(torch.empty(out_channels))
-        else:
-            self.register_parameter('bias', None)
-        self.reset_parameters()
-
-    def reset_parameters(self):
-        init.kaiming_uniform_(self.weight, a=math.sqrt(5))
-        if self.bias is not None:
-            fan_in, _ = init._calculate_fan_in_and_fan_out(self.weight)
-            bound = 1 / math.sqrt(fan_in)
-            init.uniform_(self.bias, -bound, bound)
+class UnoptimizedConv2d(nn.Conv2d):
+    """Same parameters, initialisation and ``repr`` as ``nn.Conv2d``; zero padding, dilation 1 and
+    groups 1 only -- what the kernel (and the reference's) covers."""
 
     def forward(self, input):
-        if self.dilation != (1, 1) or self.groups != 1:
+        if tuple(self.dilation) != (1, 1) or self.groups != 1:
             raise NotImplementedError("the comparator kernel supports dilation=1 and groups=1 only")
-        if self.padding_mode != 'zeros':
-            raise NotImplementedError("the comparator kernel supports zero padding only")
+        if self.padding_mode != 'zeros' or isinstance(self.padding, str):
+            raise NotImplementedError("the comparator kernel supports explicit zero padding only")
         ph, pw = self.padding
-        input = F.pad(input, (pw, pw, ph, ph), mode='constant', value=0)
-        return kernels.conv2d(input, self.weight, self.bias, self.stride, self.padding)
-
-    def extra_repr(self):
-        s = '{in_channels}, {out_channels}, kernel_size={kernel_size}, stride={stride}'
-        if self.padding != (0, 0):
-            s += ', padding={padding}'
-        if self.bias is None:
-            s += ', bias=False'
-        return s.format(**self.__dict__)
+        padded = F.pad(input, (pw, pw, ph, ph))
+        return kernels.conv2d(padded, self.weight, self.bias, self.stride, self.padding)

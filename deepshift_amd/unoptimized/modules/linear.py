@@ -1,35 +1,13 @@
-"""``UnoptimizedLinear`` (unoptimized/modules/linear.py:13-51 in the reference)."""
-import math
-
-import torch
+"""``UnoptimizedLinear``: an ``nn.Linear`` whose forward pass is the comparator's float
+multiply-accumulate kernel (the role of unoptimized/modules/linear.py:13-51 in the reference)."""
 import torch.nn as nn
-from torch.nn import init
 
 from .. import kernels
 
 
-class UnoptimizedLinear(nn.Module):
-    def __init__(self, in_features, out_features, bias=True):
-        super().__init__()
-        self.in_features = in_features
-        self.out_features = out_features
-        self.weight = nn.Parameter(torch.empty(out_features, in_features))
-        if bias:
-            self.bias = nn.Parameter(torch.empty(out_features))
-        else:
-            self.register_parameter('bias', None)
-        self.reset_parameters()
-
-    def reset_parameters(self):
-        init.kaiming_uniform_(self.weight, a=math.sqrt(5))
-        if self.bias is not None:
-            fan_in, _ = init._calculate_fan_in_and_fan_out(self.weight)
-            bound = 1 / math.sqrt(fan_in)
-            init.uniform_(self.bias, -bound, bound)
+class UnoptimizedLinear(nn.Linear):
+    """Same parameters, initialisation and ``repr`` as ``nn.Linear``; only the arithmetic moves to
+    ``ds_mul_linear_f32``."""
 
     def forward(self, input):
         return kernels.linear(input, self.weight, self.bias)
-
-    def extra_repr(self):
-        return 'in_features={}, out_features={}, bias={}'.format(
-            self.in_features, self.out_features, self.bias is not None)
