@@ -51,6 +51,10 @@ inline int launch_status() { return hip_status(hipGetLastError()); }
 //                                     bits 3:0 shift field, bit 8 negative, bits 15:12 = 0001 so
 //                                     that the half-word is a ready M0 value for relative addressing
 //                                     (index in 7:0, "src0 is relative" in 15:12); one spare row
+//                                     When tiled_wide(N, K, bits) the section is laid out for the
+//                                     64-channel form of that kernel instead:
+//           [ntiles/2][comm*num][32]  word j = code of channel j | code of channel j + 32 << 16 of
+//                                     one reduction index (same size, one spare row)
 struct TiledGeom {
     int num, comm, ntiles;
     size_t word_count, negcount_offset, ktab_offset, ktab_count, words16_offset, words16_count, bytes;
@@ -73,6 +77,12 @@ inline TiledGeom tiled_geom(int N, int K, int bits)
 inline const int32_t *tiled_negcount(const void *tiled, const TiledGeom &g)
 {
     return (const int32_t *)((const char *)tiled + g.negcount_offset);
+}
+// Layers whose channel count is a multiple of 64 (fields of <= 4 bits) use the 64-channel form.
+inline bool tiled_wide(int N, int K, int bits)
+{
+    (void)K;
+    return bits <= 4 && N > 0 && N % 64 == 0;
 }
 inline const uint32_t *tiled_words16(const void *tiled, const TiledGeom &g)
 {

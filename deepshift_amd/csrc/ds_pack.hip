@@ -175,6 +175,31 @@ __global__ void tile16_kernel(const int32_t *__restrict__ w_ref, uint32_t *__res
     w16[idx] = out;
 }
 
+// The 64-channel layout of the same section: words16[t64][k][j] = code (k, channel t64*64 + j) |
+// code (k, channel t64*64 + 32 + j) << 16.
+__global__ void tile16_wide_kernel(const int32_t *__restrict__ w_ref, uint32_t *__restrict__ w16, int N, int K,
+                                   int comm, int bits, int num, long words, int in_bits, int in_comm,
+                                   int zero_top)
+{
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= words) return;
+    const int j = (int)(idx % kTileWords);
+    const long rest = idx / kTileWords;
+    const long rows = (long)comm * num;  // one row per reduction slot, K rounded up to whole groups
+    const int k = (int)(rest % rows);
+    const int t = (int)(rest / rows);
+    uint32_t out = 0x10001000u;
+    if (k < K) {
+        for (int c = 0; c < 2; ++c) {
+            const int n = t * 64 + 32 * c + j;
+            if (n >= N) continue;
+            const OwnCode o = own_code(ref_code(w_ref, n, k, in_comm, in_bits), bits, zero_top);
+            out |= (o.field | (o.neg << 8)) << (16 * c);
+        }
+    }
+    w16[idx] = out;
+}
+
 int launch_tile(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW, int bits,
                 hipStream_t st, int in_bits, int zero_top)
 {
@@ -197,9 +222,14 @@ int launch_tile(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW,
                        (uint32_t *)tiled_ktab(tiled, g), K, (int)g.ktab_count, FH, FW);
     if (g.words16_count) {
         const long blocks = ((long)g.words16_count + 255) / 256;
-        hipLaunchKernelGGL(tile16_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w_ref,
-                           (uint32_t *)tiled_words16(tiled, g), N, K, g.comm, bits, g.num,
-                           (long)g.words16_count, in_bits, in_comm, zero_top);
+        if (tiled_wide(N, K, bits))
+            hipLaunchKernelGGL(tile16_wide_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w_ref,
+                               (uint32_t *)tiled_words16(tiled, g), N, K, g.comm, bits, g.num,
+                               (long)g.words16_count, in_bits, in_comm, zero_top);
+        else
+            hipLaunchKernelGGL(tile16_kernel, dim3((unsigned)blocks), dim3(256), 0, st, w_ref,
+                               (uint32_t *)tiled_words16(tiled, g), N, K, g.comm, bits, g.num,
+                               (long)g.words16_count, in_bits, in_comm, zero_top);
     }
     return launch_status();
 }

@@ -25,6 +25,7 @@
 #include "ds_common.h"
 #include <cstdio>
 #include <cstdlib>
+#include <type_traits>
 
 namespace ds {
 
@@ -269,6 +270,7 @@ __global__ __launch_bounds__(256) void shift_kernel(const ShiftArgs p)
 #include "ds_planes_asm.inc"
 
 typedef int32_t v16i __attribute__((ext_vector_type(16)));
+typedef int32_t v32i __attribute__((ext_vector_type(32)));
 typedef int32_t v4i __attribute__((ext_vector_type(4)));
 
 // Walk over the reduction index handed to the asm loop: offset / fw / fh of the first k, the filter
@@ -280,46 +282,61 @@ struct PlaneWalk {
 constexpr int kPlaneRows = 3;      // pixels per lane (R of gen_planes_asm.py)
 constexpr int kPlaneSlots = 3072;  // wave slots of the machine at 3 waves per SIMD (256 CUs x 4 SIMDs)
 
-#define DS_PLANES_OPERANDS                                                                        \
-    : "+{v[66:81]}"(a[0]), "+{v[82:97]}"(a[1]), "+{v[98:113]}"(a[2]), "+{v[114:129]}"(a[3]),      \
-      "+{v[130:145]}"(a[4]), "+{v[146:161]}"(a[5])                                                \
+constexpr int kPlaneSlotsWide = 2048;  // the 64-channel form holds 246 registers: 2 waves per SIMD
+
+#define DS_PLANES_INPUTS                                                                          \
     : "v"(xoff[0]), "v"(xoff[1]), "v"(xoff[2]), "s"(rsrc), "s"(wptr), "s"(groups), "s"(w.koff),   \
       "s"(w.fw), "s"(w.fh), "s"(w.FW), "s"(w.FH), "s"(w.row_step), "s"(w.plane_step),             \
       "s"(w.koff_max)
+#define DS_PLANES_OPERANDS                                                                        \
+    : "+{v[66:81]}"(a[0]), "+{v[82:97]}"(a[1]), "+{v[98:113]}"(a[2]), "+{v[114:129]}"(a[3]),      \
+      "+{v[130:145]}"(a[4]), "+{v[146:161]}"(a[5])                                                \
+    DS_PLANES_INPUTS
+// (six 32-register operands: an asm statement takes at most 30 operands, tied ones counted twice)
+#define DS_PLANES_OPERANDS_WIDE                                                                   \
+    : "+{v[64:95]}"(a[0]), "+{v[96:127]}"(a[1]), "+{v[128:159]}"(a[2]), "+{v[160:191]}"(a[3]),    \
+      "+{v[192:223]}"(a[4]), "+{v[224:255]}"(a[5])                                                \
+    DS_PLANES_INPUTS
 
+// Main loop of the 32-channel form (six 16-register accumulator vectors) and of the 64-channel form
+// (six of 32 registers).
 // ZT: the blob's highest field value stands for a zero weight (its plane is held at 0).
 template <int BITS, bool ZT>
 __device__ __forceinline__ void planes_main_loop(v16i (&a)[6], const uint32_t (&xoff)[3], v4i rsrc,
                                                  const uint32_t *wptr, int groups, const PlaneWalk &w);
-#define DS_PLANES_SPECIALISE(B)                                                                    \
+template <int BITS, bool ZT>
+__device__ __forceinline__ void planes_main_loop(v32i (&a)[6], const uint32_t (&xoff)[3], v4i rsrc,
+                                                 const uint32_t *wptr, int groups, const PlaneWalk &w);
+#define DS_PLANES_ONE(B, ZT, VEC, ASM, OPERANDS, CLOBBERS)                                         \
     template <>                                                                                    \
-    __device__ __forceinline__ void planes_main_loop<B, false>(v16i (&a)[6], const uint32_t (&xoff)[3], \
-                                                               v4i rsrc, const uint32_t *wptr, int groups, \
-                                                               const PlaneWalk &w)                 \
+    __device__ __forceinline__ void planes_main_loop<B, ZT>(VEC (&a)[6], const uint32_t (&xoff)[3], \
+                                                            v4i rsrc, const uint32_t *wptr, int groups, \
+                                                            const PlaneWalk &w)                    \
     {                                                                                              \
-        asm volatile(DS_PLANES_ASM_B##B DS_PLANES_OPERANDS : DS_PLANES_CLOBBERS_B##B);             \
-    }                                                                                              \
-    template <>                                                                                    \
-    __device__ __forceinline__ void planes_main_loop<B, true>(v16i (&a)[6], const uint32_t (&xoff)[3], \
-                                                              v4i rsrc, const uint32_t *wptr, int groups, \
-                                                              const PlaneWalk &w)                  \
-    {                                                                                              \
-        asm volatile(DS_PLANES_ASM_B##B##Z DS_PLANES_OPERANDS : DS_PLANES_CLOBBERS_B##B);          \
+        asm volatile(ASM OPERANDS : CLOBBERS);                                                     \
     }
+#define DS_PLANES_SPECIALISE(B)                                                                    \
+    DS_PLANES_ONE(B, false, v16i, DS_PLANES_ASM_B##B, DS_PLANES_OPERANDS, DS_PLANES_CLOBBERS_B##B)   \
+    DS_PLANES_ONE(B, true, v16i, DS_PLANES_ASM_B##B##Z, DS_PLANES_OPERANDS, DS_PLANES_CLOBBERS_B##B) \
+    DS_PLANES_ONE(B, false, v32i, DS_PLANES_ASM_B##B##W, DS_PLANES_OPERANDS_WIDE, DS_PLANES_CLOBBERS_B##B##W) \
+    DS_PLANES_ONE(B, true, v32i, DS_PLANES_ASM_B##B##ZW, DS_PLANES_OPERANDS_WIDE, DS_PLANES_CLOBBERS_B##B##W)
 DS_PLANES_SPECIALISE(1)
 DS_PLANES_SPECIALISE(2)
 DS_PLANES_SPECIALISE(3)
 DS_PLANES_SPECIALISE(4)
 
-// One segment of work of the shift-plane kernel: K groups [g_begin, g_end) of the tile made of the 32
+// One segment of work of the shift-plane kernel: K groups [g_begin, g_end) of the tile made of the J
 // channels of `ntile` and the R*64 pixels starting at m0.  `atomic` selects accumulation into a
-// pre-filled output (several segments share the tile) or a plain store of acc + bias.
-template <int BITS, bool ZT>
+// pre-filled output (several segments share the tile) or a plain store of acc + bias.  WIDE: the
+// 64-channel form (layers with N % 64 == 0).
+template <int BITS, bool ZT, bool WIDE>
 __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, int m0, int g_begin,
                                                int g_end, bool atomic)
 {
     constexpr int NUM = 32 / (BITS + 1);
-    constexpr int R = kPlaneRows, J = 32;
+    constexpr int R = kPlaneRows, J = WIDE ? 64 : 32;
+    constexpr int VEC = WIDE ? 32 : 16;  // registers per accumulator operand of the asm loop
+    using acc_vec = typename std::conditional<WIDE, v32i, v16i>::type;
     const int lane = threadIdx.x & (kWave - 1);
 
     uint32_t xoff[R], yoff[R];
@@ -339,11 +356,9 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
 
     const int full_groups = p.K / NUM;
     const int g_full_end = g_end < full_groups ? g_end : full_groups;
-    const uint32_t *wrow = p.wt + (size_t)ntile * p.comm * kTileWords;
-
-    v16i a[2 * R];
+    acc_vec a[6];
 #pragma unroll
-    for (int i = 0; i < 2 * R; ++i) a[i] = (v16i)(0);
+    for (int i = 0; i < 6; ++i) a[i] = (acc_vec)(0);
     if (g_begin < g_full_end) {
         const uint64_t xaddr = (uint64_t)p.x;
         v4i rsrc;
@@ -362,31 +377,37 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
         w.row_step = p.x_row - p.FW;
         w.plane_step = p.x_plane - p.FH * p.x_row;
         w.koff_max = (p.K / ff - 1) * p.x_plane + (p.FH - 1) * p.x_row + p.FW - 1;
+        // rows of 16-bit codes per K group: NUM/2 (two slots per row) or NUM (one slot, 64 channels)
+        constexpr int ROWS = WIDE ? NUM : NUM / 2;
         planes_main_loop<BITS, ZT>(a, xoff, rsrc,
-                               p.wt16 + ((size_t)ntile * p.comm + g_begin) * (NUM / 2) * kTileWords,
-                               g_full_end - g_begin, w);
+                                   p.wt16 + ((size_t)ntile * p.comm + g_begin) * ROWS * kTileWords,
+                                   __builtin_amdgcn_readfirstlane(g_full_end - g_begin), w);
     }
 
     int32_t acc[R][J];
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
-        for (int j = 0; j < J; ++j) acc[r][j] = a[2 * r + j / 16][j % 16];
+        for (int j = 0; j < J; ++j) acc[r][j] = a[(J / VEC) * r + j / VEC][j % VEC];
 
-    // partial last group (codes with k >= K read as x = 0)
-    const __amdgpu_buffer_rsrc_t xrsrc =
-        __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, (int)p.x_bytes, 0x00020000);
-    for (int g = g_full_end > g_begin ? g_full_end : g_begin; g < g_end; ++g) {
-        uint32_t w[J];
+    {
+        // partial last group, from the packed words (rows of 32 channels: a 64-channel tile has two)
+        const uint32_t *wrow = p.wt + (size_t)ntile * (J / kTileWords) * p.comm * kTileWords;
+        const __amdgpu_buffer_rsrc_t xrsrc =
+            __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, (int)p.x_bytes, 0x00020000);
+        for (int g = g_full_end > g_begin ? g_full_end : g_begin; g < g_end; ++g) {
+            uint32_t w[J];
 #pragma unroll
-        for (int j = 0; j < J; ++j) w[j] = wrow[(size_t)g * kTileWords + j];
-        int32_t xt[NUM][R];
-        load_group<NUM, R>(xt, xrsrc, xoff, p, g);
+            for (int j = 0; j < J; ++j)
+                w[j] = wrow[((size_t)(j / kTileWords) * p.comm + g) * kTileWords + j % kTileWords];
+            int32_t xt[NUM][R];
+            load_group<NUM, R>(xt, xrsrc, xoff, p, g);
 #pragma unroll
-        for (int i = 0; i < NUM; ++i) {
-            if (g * NUM + i >= p.K) break;  // the codes past K trail the word: nothing left to add
-            if (ZT) accumulate_code_zero_top<BITS, R, J>(acc, xt[i], w, i);
-            else accumulate_code<BITS, false, R, J>(acc, xt[i], w, i, 0);
+            for (int i = 0; i < NUM; ++i) {
+                if (g * NUM + i >= p.K) break;  // the codes past K trail the word: nothing left to add
+                if (ZT) accumulate_code_zero_top<BITS, R, J>(acc, xt[i], w, i);
+                else accumulate_code<BITS, false, R, J>(acc, xt[i], w, i, 0);
+            }
         }
     }
 
@@ -410,9 +431,8 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
 }
 
 // Tile-per-wave launch: gridDim.y K-slices per tile.
-template <int BITS, bool ZT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void shift_planes_kernel(
-    const ShiftArgs p)
+template <int BITS, bool ZT, bool WIDE>
+__device__ __forceinline__ void planes_tile_body(const ShiftArgs &p)
 {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int bid = blockIdx.x;
@@ -424,35 +444,61 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     const int g_begin = blockIdx.y * p.groups_per_split;
     int g_end = g_begin + p.groups_per_split;
     if (g_end > p.comm) g_end = p.comm;
-    planes_segment<BITS, ZT>(p, ntile, m0, g_begin, g_end, p.atomic_out != 0);
+    planes_segment<BITS, ZT, WIDE>(p, ntile, m0, g_begin, g_end, p.atomic_out != 0);
 }
 
 // Work-balanced launch: the (tile, K group) iteration space is cut into one equal contiguous share
 // per wave, so every wave of the launch does the same number of group iterations whatever the tile
 // count (each wave touches at most a few tiles; tiles shared between waves are combined with
 // atomic adds onto the pre-filled output).  tiles_m4 holds the number of 192-pixel tiles here.
-template <int BITS, bool ZT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void shift_planes_balanced_kernel(
-    const ShiftArgs p)
+template <int BITS, bool ZT, bool WIDE>
+__device__ __forceinline__ void planes_balanced_body(const ShiftArgs &p)
 {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int bid = blockIdx.x;
     // waves of one XCD (workgroup ids congruent mod 8) take a contiguous range of shares
-    const long w = ((long)(bid & 7) * (gridDim.x >> 3) + (bid >> 3)) * 4 + wave;
-    const long waves = (long)gridDim.x * 4;
+    const int w = ((bid & 7) * (int)(gridDim.x >> 3) + (bid >> 3)) * 4 + wave;
+    const int waves = (int)gridDim.x * 4;
+    // (tile, K group) iterations: below 2^31 because every tensor is below 2^31 bytes
     const long total = (long)p.tiles_m4 * p.tiles_n * p.comm;
-    long it = w * total / waves;
-    const long it_end = (w + 1) * total / waves;
+    int it = (int)(w * total / waves);
+    const int it_end = (int)((w + 1) * total / waves);
     while (it < it_end) {
-        const int tile = (int)(it / p.comm);
-        const int g_begin = (int)(it - (long)tile * p.comm);
-        long g_end = g_begin + (it_end - it);
+        const int tile = it / p.comm;
+        const int g_begin = it - tile * p.comm;
+        int g_end = g_begin + (it_end - it);
         if (g_end > p.comm) g_end = p.comm;
         const int ntile = tile % p.tiles_n;
         const int m0 = (tile / p.tiles_n) * (kPlaneRows * kWave);
-        planes_segment<BITS, ZT>(p, ntile, m0, g_begin, (int)g_end, true);
+        planes_segment<BITS, ZT, WIDE>(p, ntile, m0, g_begin, g_end, true);
         it += g_end - g_begin;
     }
+}
+
+// 32-channel form: 168 registers, three waves per SIMD; 64-channel form: 256 registers, two.
+template <int BITS, bool ZT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void shift_planes_kernel(
+    const ShiftArgs p)
+{
+    planes_tile_body<BITS, ZT, false>(p);
+}
+template <int BITS, bool ZT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void shift_planes_balanced_kernel(
+    const ShiftArgs p)
+{
+    planes_balanced_body<BITS, ZT, false>(p);
+}
+template <int BITS, bool ZT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void shift_planes_wide_kernel(
+    const ShiftArgs p)
+{
+    planes_tile_body<BITS, ZT, true>(p);
+}
+template <int BITS, bool ZT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void shift_planes_wide_balanced_kernel(const ShiftArgs p)
+{
+    planes_balanced_body<BITS, ZT, true>(p);
 }
 
 // y = bias[n] + negcnt[n] for the split-K path.  Both output layouts ([img][n][pix] and [m][n])
@@ -565,10 +611,11 @@ static TileChoice choose_tile(const ShiftArgs &a)
     return c;
 }
 
-template <int BITS, bool ZT>
+template <int BITS, bool ZT, bool WIDE>
 static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
 {
-    constexpr int R = kPlaneRows, J = 32;
+    constexpr int R = kPlaneRows, J = WIDE ? 64 : 32;
+    constexpr int kSlots = WIDE ? kPlaneSlotsWide : kPlaneSlots;
     a.tiles_n = ceil_div(a.N, J);
     if (nsplit <= 0 && a.comm > 0) {
         // balanced launch: one share of the iteration space per wave slot (3 waves per SIMD)
@@ -576,12 +623,15 @@ static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
         a.atomic_out = 1;
         int32_t *final_y = redirect_to_scratch(a);
         launch_fill(a, st);
-        int blocks = (kPlaneSlots / 4) * (nsplit < 0 ? -nsplit : 1);
+        int blocks = (kSlots / 4) * (nsplit < 0 ? -nsplit : 1);
         // small layers: at least 8 K groups per wave (the workgroup count stays a multiple of 8)
         const long iters = (long)a.tiles_m4 * a.tiles_n * a.comm;
         const long fit = (iters / 32) / 8 * 8;
         if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
-        hipLaunchKernelGGL((shift_planes_balanced_kernel<BITS, ZT>), dim3(blocks), dim3(256), 0, st, a);
+        if (WIDE)
+            hipLaunchKernelGGL((shift_planes_wide_balanced_kernel<BITS, ZT>), dim3(blocks), dim3(256), 0, st, a);
+        else
+            hipLaunchKernelGGL((shift_planes_balanced_kernel<BITS, ZT>), dim3(blocks), dim3(256), 0, st, a);
         if (final_y) return launch_transpose_strided(a.y, a.alt_ld, final_y, a.N, a.M, a.N, st);
         return launch_status();
     }
@@ -598,31 +648,35 @@ static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
         launch_fill(a, st);
     }
     dim3 grid(a.blocks_per_xcd * 8, nsplit);
-    hipLaunchKernelGGL((shift_planes_kernel<BITS, ZT>), grid, dim3(256), 0, st, a);
+    if (WIDE)
+        hipLaunchKernelGGL((shift_planes_wide_kernel<BITS, ZT>), grid, dim3(256), 0, st, a);
+    else
+        hipLaunchKernelGGL((shift_planes_kernel<BITS, ZT>), grid, dim3(256), 0, st, a);
     if (final_y) return launch_transpose_strided(a.y, a.alt_ld, final_y, a.N, a.M, a.N, st);
     return launch_status();
 }
 
 // Launch regime of the shift-plane kernel for a layer: 1 = one tile per wave, 0 = equal shares,
 // -1 = the layer is better off on the two-instruction kernel.
-static int plane_regime(const ShiftArgs &a)
+static int plane_regime(const ShiftArgs &a, bool wide)
 {
-    const long tiles = (long)ceil_div(a.M, kPlaneRows * kWave) * ceil_div(a.N, 32);
+    const long slots = wide ? kPlaneSlotsWide : kPlaneSlots;
+    const int J = wide ? 64 : 32;
+    const long tiles = (long)ceil_div(a.M, kPlaneRows * kWave) * ceil_div(a.N, J);
     const long iters = tiles * a.comm;
     const bool n_ok = a.N % 32 == 0 || a.N >= 256;
-    const bool many_tiles = tiles * 10 >= (long)kPlaneSlots * 13;
-    const long rounds = (tiles + kPlaneSlots - 1) / kPlaneSlots;
-    const double fill = (double)tiles / ((double)kPlaneSlots * (double)(rounds > 0 ? rounds : 1));
-    const bool whole_rounds = tiles >= kPlaneSlots && fill >= 0.93;
+    const bool many_tiles = tiles * 10 >= slots * 13;
+    const long rounds = (tiles + slots - 1) / slots;
+    const double fill = (double)tiles / ((double)slots * (double)(rounds > 0 ? rounds : 1));
+    const bool whole_rounds = tiles >= slots && fill >= 0.93;
     // With many tiles the equal shares still win when the reduction is long and the rounds of slots
     // fill badly (3x3 layers with 1.4 rounds of tiles, an 8192^3 GEMM), unless many channel tiles
     // share each pixel range: their waves then start at staggered K offsets and evict each other's
     // activations from L2.
     const bool per_tile =
-        many_tiles && (a.comm < 24 || (a.comm <= 128 && (fill >= 0.85 || ceil_div(a.N, 32) >= 8)));
+        many_tiles && (a.comm < 24 || (a.comm <= 128 && (fill >= 0.85 || ceil_div(a.N, J) >= 8)));
     const int regime = (per_tile || whole_rounds) ? 1 : 0;
-    const bool eligible =
-        n_ok && ((many_tiles && a.comm >= 6) || (a.comm >= 24 && iters >= (long)kPlaneSlots * 16));
+    const bool eligible = n_ok && ((many_tiles && a.comm >= 6) || (a.comm >= 24 && iters >= slots * 16));
     return eligible ? regime : -1 - regime;
 }
 
@@ -631,10 +685,11 @@ static int plane_regime(const ShiftArgs &a)
 template <int BITS>
 static int dispatch_zero_top(const ShiftArgs &a, hipStream_t st)
 {
-    const int r = plane_regime(a);
+    const bool wide = tiled_wide(a.N, a.K, BITS);
+    const int r = plane_regime(a, wide);
     int nsplit = (r >= 0 ? r : -1 - r) > 0 ? 1 : 0;
     if (const char *sp = getenv("DS_TUNE_SPLIT")) nsplit = atoi(sp);
-    return launch_planes<BITS, true>(a, nsplit, st);
+    return wide ? launch_planes<BITS, true, true>(a, nsplit, st) : launch_planes<BITS, true, false>(a, nsplit, st);
 }
 
 template <int BITS, bool GENERAL>
@@ -652,12 +707,14 @@ static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
         // The 1x1 shortcuts of small images, single-wave batches and layers with few channels stay on
         // the two-instruction kernel.
         const char *t = getenv("DS_TUNE_PLANES");
-        bool planes = plane_regime(a) >= 0;
+        const bool wide = tiled_wide(a.N, a.K, BITS);  // decided by the shape alone, as at tiling time
+        bool planes = plane_regime(a, wide) >= 0;
         if (t) planes = atoi(t) > 0;
         if (planes) {
-            int nsplit = plane_regime(a) > 0 ? 1 : 0;
+            int nsplit = plane_regime(a, wide) > 0 ? 1 : 0;
             if (const char *sp = getenv("DS_TUNE_SPLIT")) nsplit = atoi(sp);
-            return launch_planes<BITS, false>(a, nsplit, st);
+            return wide ? launch_planes<BITS, false, true>(a, nsplit, st)
+                        : launch_planes<BITS, false, false>(a, nsplit, st);
         }
     }
     TileChoice c = choose_tile(a);

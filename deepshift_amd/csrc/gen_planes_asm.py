@@ -26,16 +26,37 @@ let three waves share a SIMD.
     s[68:99]                  the next two slots' codes (in flight meanwhile)
     s4..s6                    walk over the reduction index: element offset, fw, fh of the next k to load
     s7..s15                   temporaries, loop counter, word pointer
+
+Every loop also comes in a "wide" form (suffix W) for layers whose channel count is a multiple of 64:
+J = 64 channels per lane, so the planes are shared by twice as many terms (1 + 2^BITS/64 vector
+instructions per term).  It keeps 192 accumulators in v[64 + 64*r + j], needs 246 registers for 4-bit
+fields (two waves per SIMD), reads one code row per reduction slot -- word j holds the codes of
+channels j (low half) and j + 32 (high half) -- and alternates between the two SGPR sets instead of
+copying.
 Operands: %6..%8 per-row byte offsets (VGPR), %9 buffer descriptor, %10 word pointer, %11 number of
 K groups, %12..%14 initial walk state (offset, fw, fh), %15 FW, %16 FH, %17 offset step when fw wraps,
 %18 offset step when fh wraps, %19 largest valid offset (the walk runs D slots ahead and is clamped).
 """
 import os
 
-R, J = 3, 32
-ACC = 66
-DEPTH = {1: 4, 2: 5, 3: 4, 4: 3}
-OP_XOFF, OP_RSRC, OP_WPTR, OP_GROUPS, OP_WALK = 6, 9, 10, 11, 12
+R = 3
+DEPTH = {1: 4, 2: 5, 3: 4, 4: 3}        # prefetch ring depth, 32-channel form
+DEPTH_WIDE = {1: 4, 2: 5, 3: 4, 4: 2}   # 64-channel form: 4-bit fields leave room for two slots only
+
+
+class Form:
+    """Register and operand layout of the 32-channel (wide=False) or 64-channel loop."""
+
+    def __init__(self, bits, wide):
+        self.J = 64 if wide else 32
+        self.acc = 64 if wide else 66
+        self.depth = (DEPTH_WIDE if wide else DEPTH)[bits]
+        self.waves = 2 if wide else 3
+        nacc = 2 * R                            # accumulator operands %0..%5, 16 or 32 registers each
+        self.op_xoff, self.op_rsrc, self.op_wptr, self.op_groups, self.op_walk = (
+            nacc, nacc + R, nacc + R + 1, nacc + R + 2, nacc + R + 3)
+
+
 XP = 8
 W = 36
 WS = 68
@@ -46,13 +67,14 @@ PRIO = 13
 TIME = 34
 
 
-def load_words():
-    return ["s_load_dwordx16 s[%d:%d], s[%d:%d], 0x0" % (WS, WS + 15, WP, WP + 1),
-            "s_load_dwordx16 s[%d:%d], s[%d:%d], 0x40" % (WS + 16, WS + 31, WP, WP + 1)]
+def load_words(dst=WS):
+    return ["s_load_dwordx16 s[%d:%d], s[%d:%d], 0x0" % (dst, dst + 15, WP, WP + 1),
+            "s_load_dwordx16 s[%d:%d], s[%d:%d], 0x40" % (dst + 16, dst + 31, WP, WP + 1)]
 
 
-def walk_and_load(slot):
+def walk_and_load(slot, f):
     """Issue the R loads of the walk's current k into ring slot `slot`, then step the walk to k + 1."""
+    OP_XOFF, OP_RSRC, OP_WALK = f.op_xoff, f.op_rsrc, f.op_walk
     fw_end, fh_end, row_step, plane_step, koff_max = (OP_WALK + 3, OP_WALK + 4, OP_WALK + 5, OP_WALK + 6,
                                                       OP_WALK + 7)
     L = ["s_min_u32 s%d, s%d, %%%d" % (T0, KOFF, koff_max),
@@ -74,13 +96,21 @@ def walk_and_load(slot):
     return L
 
 
-def take_turn(tag):
-    """The waves that share a SIMD take turns at the issue priorities 2, 1, 0, by the clock: with equal
+def take_turn(tag, waves):
+    """The waves that share a SIMD take turns at the issue priorities, by the clock: with equal
     priorities the arbiter favours the oldest wave, which then finishes early and leaves the others
-    with a SIMD they cannot fill (a wave cannot overlap its own scalar and vector work).  The turn is
-    41 us (bit 12 of the 100 MHz counter) and is checked with every code row, because the wave that
-    should take over is the one that is running slowly."""
+    with a SIMD they cannot fill (a wave cannot overlap its own scalar and vector work).  A turn is
+    41 us (bit 12 of the 100 MHz counter up) and is checked with every code row, because the wave that
+    should take over is the one that is running slowly.  Three waves rotate through priorities 2, 1,
+    0; two waves swap 2 and 0."""
     hi, mid, end = "%d" % (20 + tag), "%d" % (40 + tag), "%d" % (60 + tag)
+    if waves == 2:
+        return ["s_bfe_u32 s%d, s%d, 0x1000c" % (T0, TIME),
+                "s_and_b32 s%d, s%d, 1" % (T1, PRIO),
+                "s_cmp_eq_u32 s%d, s%d" % (T0, T1), "s_cbranch_scc1 %sf" % hi,
+                "s_setprio 0", "s_branch %sf" % end,
+                hi + ":", "s_setprio 2",
+                end + ":"]
     return ["s_bfe_u32 s%d, s%d, 0xe000c" % (T0, TIME),          # 14 bits of turn counter
             "s_mul_i32 s%d, s%d, 0x5556" % (T1, T0),
             "s_lshr_b32 s%d, s%d, 16" % (T1, T1),                # turn counter / 3
@@ -98,45 +128,59 @@ def take_turn(tag):
             end + ":"]
 
 
-def body(bits, zero_top=False):
+def body(bits, zero_top=False, wide=False):
+    f = Form(bits, wide)
     cb = bits + 1
     num = 32 // cb
     P = 1 << bits
-    D = DEPTH[bits]
+    D, ACC = f.depth, f.acc
     assert num % D == 0 and num % 2 == 0
     PL = XP + R * D
-    assert PL + P * R <= ACC
+    assert PL + P * R <= ACC and ACC + R * f.J <= 256
     L = []
     # ---- prologue: mutable copies of the inputs, the first activation loads and code row
     L += ["s_getreg_b32 s%d, hwreg(HW_REG_HW_ID, 0, 4)" % PRIO,  # the wave's slot on its SIMD
-          "s_mov_b32 s%d, %%%d" % (CNT, OP_GROUPS),
-          "s_mov_b64 s[%d:%d], %%%d" % (WP, WP + 1, OP_WPTR),
-          "s_mov_b32 s%d, %%%d" % (KOFF, OP_WALK), "s_mov_b32 s%d, %%%d" % (FWC, OP_WALK + 1),
-          "s_mov_b32 s%d, %%%d" % (FHC, OP_WALK + 2)]
-    L += load_words()
+          "s_mov_b32 s%d, %%%d" % (CNT, f.op_groups),
+          "s_mov_b64 s[%d:%d], %%%d" % (WP, WP + 1, f.op_wptr),
+          "s_mov_b32 s%d, %%%d" % (KOFF, f.op_walk), "s_mov_b32 s%d, %%%d" % (FWC, f.op_walk + 1),
+          "s_mov_b32 s%d, %%%d" % (FHC, f.op_walk + 2)]
+    L += load_words(W if wide else WS)
     L += ["s_memrealtime s[%d:%d]" % (TIME, TIME + 1)]
     for i in range(D):
-        L += walk_and_load(i)
+        L += walk_and_load(i, f)
     L += ["s_mov_b32 s%d, 0" % IDX, "s_set_gpr_idx_on s%d, 0x1" % IDX]  # src0 of vector ops is M0-relative
-    # ---- one K group per iteration, two reduction slots (one row of 16-bit codes) at a time
+    # ---- one K group per iteration
     L += ["1:"]
     for i in range(num):
-        if i % 2 == 0:
-            # this row's codes leave the staging registers, which then receive the next row's (one
+        if wide:
+            # one code row per reduction slot; the two SGPR sets alternate (NUM is even, so the set
+            # of slot 0 is the same in every group), the other set receives the next slot's row (one
             # row past the end reads the spare row that follows the codes in the weight blob)
+            cur, nxt = (W, WS) if i % 2 == 0 else (WS, W)
             L += ["s_add_u32 s%d, s%d, 128" % (WP, WP), "s_addc_u32 s%d, s%d, 0" % (WP + 1, WP + 1),
                   "s_waitcnt lgkmcnt(0)"]
-            L += take_turn(i // 2)
+            if i % 2 == 0:
+                L += take_turn(i // 2, f.waves)
+            L += load_words(nxt)
+            if i % 2 == 1:
+                L += ["s_memrealtime s[%d:%d]" % (TIME, TIME + 1)]  # read at the next turn check
+        elif i % 2 == 0:
+            # one code row per two reduction slots: this row's codes leave the staging registers,
+            # which then receive the next row's
+            cur = W
+            L += ["s_add_u32 s%d, s%d, 128" % (WP, WP), "s_addc_u32 s%d, s%d, 0" % (WP + 1, WP + 1),
+                  "s_waitcnt lgkmcnt(0)"]
+            L += take_turn(i // 2, f.waves)
             L += ["s_mov_b64 s[%d:%d], s[%d:%d]" % (W + 2 * q, W + 2 * q + 1, WS + 2 * q, WS + 2 * q + 1)
                   for q in range(16)]
-            L += load_words()
+            L += load_words(WS)
             L += ["s_memrealtime s[%d:%d]" % (TIME, TIME + 1)]  # read when the next row arrives
         slot = i % D
         L += ["s_waitcnt vmcnt(%d)" % (R * (D - 1))]
         # plane 0 = the activation itself (a shift by 0 keeps src0 a constant: not M0-relative)
         for r in range(R):
             L += ["v_ashrrev_i32 v%d, 0, v%d" % (PL + P * r, XP + R * slot + r)]
-        L += walk_and_load(slot)  # the ring slot is free again: load reduction slot i + D into it
+        L += walk_and_load(slot, f)  # the ring slot is free again: load reduction slot i + D into it
         for s in range(1, P):
             for r in range(R):
                 if zero_top and s == P - 1:
@@ -144,26 +188,30 @@ def body(bits, zero_top=False):
                     L += ["v_mov_b32 v%d, 0" % (PL + P * r + s)]
                 else:
                     L += ["v_ashrrev_i32 v%d, %d, v%d" % (PL + P * r + s, s, PL + P * r)]
-        for j in range(J):
-            # the 16-bit code is a ready M0 value: plane index in 7:0, "src0 relative" in 15:12
-            if i % 2 == 0:
-                L += ["s_mov_b32 m0, s%d" % (W + j)]
-            else:
-                L += ["s_lshr_b32 m0, s%d, 16" % (W + j)]
-            L += ["s_bfe_i32 s%d, s%d, 0x%x" % (MASK, W + j, (1 << 16) | (16 * (i % 2) + 8))]
-            for r in range(R):
-                a = ACC + 32 * r + j
-                L += ["v_xad_u32 v%d, v%d, s%d, v%d" % (a, PL + P * r, MASK, a)]
+        # the 16-bit code is a ready M0 value: plane index in 7:0, "src0 relative" in 15:12.  32-channel
+        # form: low / high half = even / odd slot of the row; 64-channel form: channel j / j + 32.
+        halves = (0, 1) if wide else (i % 2,)
+        for half in halves:
+            for j in range(32):
+                if half == 0:
+                    L += ["s_mov_b32 m0, s%d" % (cur + j)]
+                else:
+                    L += ["s_lshr_b32 m0, s%d, 16" % (cur + j)]
+                L += ["s_bfe_i32 s%d, s%d, 0x%x" % (MASK, cur + j, (1 << 16) | (16 * half + 8))]
+                ch = j + 32 * half if wide else j
+                for r in range(R):
+                    a = ACC + f.J * r + ch
+                    L += ["v_xad_u32 v%d, v%d, s%d, v%d" % (a, PL + P * r, MASK, a)]
     L += ["s_sub_u32 s%d, s%d, 1" % (CNT, CNT), "s_cmp_lg_u32 s%d, 0" % CNT, "s_cbranch_scc1 1b"]
     # ---- leave relative addressing, drain the loads that ran ahead of the last slot
     L += ["s_set_gpr_idx_off", "s_setprio 0", "s_waitcnt vmcnt(0) lgkmcnt(0)"]
     return L
 
 
-def clobbers(bits):
-    num = 32 // (bits + 1)
+def clobbers(bits, wide=False):
+    f = Form(bits, wide)
     P = 1 << bits
-    v = ['"v%d"' % n for n in range(XP, XP + R * DEPTH[bits] + P * R)]
+    v = ['"v%d"' % n for n in range(XP, XP + R * f.depth + P * R)]
     s = ['"s%d"' % n for n in list(range(4, 16)) + list(range(W, WS + 32)) + [TIME, TIME + 1]]
     return ", ".join(v + s + ['"scc"', '"memory"'])
 
@@ -171,14 +219,15 @@ def clobbers(bits):
 def main():
     here = os.path.dirname(os.path.abspath(__file__))
     out = ["// Generated by gen_planes_asm.py -- do not edit by hand.", ""]
-    for bits in (1, 2, 3, 4):
-        for zero_top, tag in ((False, ""), (True, "Z")):
-            lines = body(bits, zero_top)
-            out.append("#define DS_PLANES_ASM_B%d%s \\" % (bits, tag))
-            out.append(" \\\n".join('    "%s\\n"' % line for line in lines))
+    for wide, wtag in ((False, ""), (True, "W")):
+        for bits in (1, 2, 3, 4):
+            for zero_top, tag in ((False, ""), (True, "Z")):
+                lines = body(bits, zero_top, wide)
+                out.append("#define DS_PLANES_ASM_B%d%s%s \\" % (bits, tag, wtag))
+                out.append(" \\\n".join('    "%s\\n"' % line for line in lines))
+                out.append("")
+            out.append("#define DS_PLANES_CLOBBERS_B%d%s %s" % (bits, wtag, clobbers(bits, wide)))
             out.append("")
-        out.append("#define DS_PLANES_CLOBBERS_B%d %s" % (bits, clobbers(bits)))
-        out.append("")
     with open(os.path.join(here, "ds_planes_asm.inc"), "w") as f:
         f.write("\n".join(out))
 

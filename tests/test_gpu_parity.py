@@ -289,6 +289,20 @@ def test_shift_plane_kernel_every_field_width_and_launch(oracle, rng, bits, spli
             w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)
             want = oracle.conv2d(xp, -s, sign, None, stride, nthreads=NTHREADS)
             np.testing.assert_array_equal(abi_conv(xp, w, None, O, FH, FW, stride, bits), want)
+        # channel counts that are multiples of 64 with K a whole number of words: the 64-channel form
+        M, K, N = 333, 480, 128
+        x = random_activations(rng, (M, K))
+        s, sign = random_codes(rng, (N, K), max_s=2 ** bits - 1)
+        bias = rng.integers(-2 ** 20, 2 ** 20, size=N).astype(np.int32)
+        w, _ = oracle.pack_words(s, sign, bits)
+        want = oracle.linear(x, -s, sign, bias, nthreads=NTHREADS)
+        np.testing.assert_array_equal(abi_linear(x, w, bias, N, bits), want)
+        Nb, C, Hp, Wp, O = 2, 80, 13, 11, 64
+        xp = random_activations(rng, (Nb, C, Hp, Wp))
+        s, sign = random_codes(rng, (O, C, 3, 3), max_s=2 ** bits - 1)
+        w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)
+        want = oracle.conv2d(xp, -s, sign, None, (1, 2), nthreads=NTHREADS)
+        np.testing.assert_array_equal(abi_conv(xp, w, None, O, 3, 3, (1, 2), bits), want)
         # GEMM with every dimension ragged
         M, K, N = 333, 517, 71
         x = random_activations(rng, (M, K))
@@ -413,6 +427,16 @@ def test_zero_top_blob_matches_oracle(oracle, rng, width, split):
     flag = width | _lib.DS_BITS_ZERO_TOP
     env = {} if split is None else {"DS_TUNE_SPLIT": split}
     with _Tune(**env):
+        # 64-channel form (N % 64 == 0, K a whole number of words of every width)
+        M, K, N = 200, 480, 64
+        x = random_activations(rng, (M, K))
+        s, sign, s_z, sign_z = _ternary_case(rng, (N, K), 2 ** width - 2)
+        want = oracle.linear(x, -s, sign, None, nthreads=NTHREADS)
+        w6 = dev(so.np_pack_words(s_z, sign_z, 6))
+        blob = kernels.tile_weights_zero_top(w6.reshape(-1), N, K, 1, 1, width)
+        xT = dev(np.ascontiguousarray(np.pad(x, ((0, (-M) % 64), (0, 0))).T))
+        got = kernels.linear_tiled(xT, M, blob, None, N, flag, 0)
+        np.testing.assert_array_equal(got.cpu().numpy(), want)
         # GEMM, ragged in every dimension
         M, K, N = 333, 517, 71
         x = random_activations(rng, (M, K))
