@@ -358,19 +358,19 @@ def main():
         "shift_layers_images_per_s": BATCH / kernel_s,
         "roofline": {
             "bound": "valu",
-            "kernel": "ds::shift_planes_balanced_kernel<4> (17 launches) + ds::shift_kernel (4 launches) per step",
+            "kernel": "ds::shift_planes_wide_balanced_kernel<4> (17 launches) + ds::shift_kernel (4 launches) per step",
             "achieved": pairs / kernel_s / 1e12,
             "peak": PEAK_PAIRS / 1e12,
             "unit": "Tpair/s",
             "frac": pairs / kernel_s / PEAK_PAIRS,
             # HBM bytes of one launch of the dominant shape (layer1 3x3 conv, 8 of the 21 launches are
-            # this size): 125.3 MB read + 132.1 MB of atomic partial sums, from the FETCH_SIZE /
+            # this size): 65.2 MB read + 155.5 MB of atomic partial sums, from the FETCH_SIZE /
             # WRITE_SIZE runs summarised in profiles/shift_kernel_layer1_conv_counters.md
             # (106.6 MB algorithmic)
-            "traffic": 257.4e6,
+            "traffic": 220.7e6,
             # vector instructions the dominant kernel issues per pair (SQ_INSTS_VALU, same profile):
             # `peak` prices a pair at 2 instructions, so its fraction can exceed 1
-            "valu_instr_per_pair": 1.53,
+            "valu_instr_per_pair": 1.29,
             "avg_launch_us": kernel_s / len(layers) * 1e6,
             "peak_calibrated": peak_cal / 1e12 if peak_cal else None,
             "frac_of_calibrated": pairs / kernel_s / peak_cal if peak_cal else None,
