@@ -1,0 +1,78 @@
+"""Seeded random shapes through the C ABI against the oracle: whatever kernel variant and launch the
+dispatch picks for a shape (two-instruction tiles, 32- or 64-channel shift planes, equal shares or
+one tile per wave, ternary blobs) must give the oracle's int32 result."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from deepshift_amd import _lib, kernels, utils
+from oracle import shift_oracle as so
+from tests.conftest import random_activations, random_codes
+from tests.test_gpu_parity import abi_conv, abi_linear, dev
+
+pytestmark = pytest.mark.gpu
+
+NTHREADS = min(16, os.cpu_count() or 1)
+
+
+def _codes(rng, shape, bits, ternary):
+    if ternary:
+        s, sign = random_codes(rng, shape, max_s=2 ** bits - 2, zero_frac=0.3)
+    else:
+        s, sign = random_codes(rng, shape, max_s=2 ** bits - 1)
+    return s, sign
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_linear_layers(oracle, seed):
+    rng = np.random.default_rng(1000 + seed)
+    bits = int(rng.integers(1, 6))
+    M = int(rng.choice([1, 3, 64, 65, 190, 193, 500, 1500]))
+    K = int(rng.integers(1, 700))
+    N = int(rng.choice([1, 31, 32, 64, 96, 128, 200, 256]))
+    x = random_activations(rng, (M, K))
+    s, sign = _codes(rng, (N, K), bits, False)
+    bias = rng.integers(-2 ** 31, 2 ** 31 - 1, size=N, dtype=np.int64).astype(np.int32) if seed % 3 else None
+    w, _ = oracle.pack_words(s, sign, bits)
+    want = oracle.linear(x, -s, sign, bias, nthreads=NTHREADS)
+    np.testing.assert_array_equal(abi_linear(x, w, bias, N, bits), want, err_msg=str((bits, M, K, N)))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_convolutions(oracle, seed):
+    rng = np.random.default_rng(2000 + seed)
+    bits = int(rng.integers(1, 5))
+    FH, FW = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+    sh, sw = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+    Nb = int(rng.integers(1, 9))
+    C = int(rng.choice([1, 3, 16, 37, 64]))
+    O = int(rng.choice([1, 16, 33, 64, 128]))
+    Hp, Wp = FH + int(rng.integers(0, 30)), FW + int(rng.integers(0, 30))
+    xp = random_activations(rng, (Nb, C, Hp, Wp))
+    s, sign = _codes(rng, (O, C, FH, FW), bits, False)
+    bias = rng.integers(-2 ** 20, 2 ** 20, size=O).astype(np.int32) if seed % 2 else None
+    w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)
+    want = oracle.conv2d(xp, -s, sign, bias, (sh, sw), nthreads=NTHREADS)
+    got = abi_conv(xp, w, bias, O, FH, FW, (sh, sw), bits)
+    np.testing.assert_array_equal(got, want, err_msg=str((bits, Nb, C, Hp, Wp, O, FH, FW, sh, sw)))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_ternary_layers_through_compress_bits(oracle, seed):
+    """The Python path a converted model takes: compress_bits (which finds the zero-top width), the
+    tiled blob it implies, the tiled kernels."""
+    rng = np.random.default_rng(3000 + seed)
+    width = int(rng.integers(1, 5))
+    M, K = int(rng.choice([70, 200, 900])), int(rng.integers(8, 400))
+    N = int(rng.choice([10, 64, 128, 130]))
+    x = random_activations(rng, (M, K))
+    s, sign = _codes(rng, (N, K), width, True)
+    s[0, 0], sign[0, 0] = 2 ** width - 2, 1         # the widest real field is present
+    sign[0, 1] = 0                                  # and at least one zero weight
+    cw = utils.compress_bits(torch.from_numpy(-s).float(), torch.from_numpy(sign).float())
+    assert cw.bits == 6 and cw.zero_top_bits == width
+    want = oracle.linear(x, -s, sign, None, nthreads=NTHREADS)
+    got = kernels.linear(dev(x), torch.from_numpy(-s).float(), torch.from_numpy(sign).float(), None, cw)
+    np.testing.assert_array_equal(got.cpu().numpy(), want, err_msg=str((width, M, K, N)))
