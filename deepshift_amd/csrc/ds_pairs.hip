@@ -1,0 +1,495 @@
+// Shift-add convolution on int8 activations for gfx950: two pixels per lane register.
+//
+// The arithmetic is that of ds_shift.hip, y[m][n] = bias[n] + sum_k sgn(n,k) * (x[m,k] >> s(n,k)),
+// for activations that the caller holds as int8 (fixed-point formats of at most 8 bits).  |x >> s| is
+// then at most 128, so 255 terms fit a 16-bit sum, and the vector ALU works on 16-bit halves:
+//   * a lane owns 6 pixels x 64 channels; each of the 64 accumulator registers of row r (r < 3)
+//     holds pixel 2r + 1 and pixel 2r as the ONE number hi * 65536 + lo, so that a full-rate 32-bit
+//     add accumulates both (the packed 16-bit adds run at half rate): a negative lo borrows from the
+//     high half, and the borrow is undone when the sum is split into lo = the sign-extended low
+//     half and hi = (sum - lo) >> 16;
+//   * per reduction index and row the kernel builds the planes  p[f] = (b >> f) * 65536 + (a >> f)
+//     (one packed 16-bit shift and a correction for a negative a), their negations, and keeps one
+//     plane at zero;
+//   * a weight code is a plane index -- f for +, 2^BITS + f for -, 2^(BITS+1) for a zero weight or a
+//     code past K -- that the scalar ALU writes to M0 (one instruction per code), and a term of both
+//     pixels is the single  v_add_u32 acc, plane[M0], acc.
+// (64 + 3*2^BITS + 1) / 128 vector instructions per shift-add term: 0.60 for 2-bit fields against
+// 1.05 of the int32 shift-plane kernel.  After at most 255 reduction indices the halves are
+// widened and added to the int32 output (atomically when the output is shared), which is why a call
+// of the generated loop never runs more than kChunk K groups.  The result is the int32 kernel's,
+// bit for bit.
+#include "ds_common.h"
+#include <cstdlib>
+
+#include "ds_planes_asm.inc"
+
+namespace ds {
+
+typedef int32_t v32i __attribute__((ext_vector_type(32)));
+typedef int32_t v4i __attribute__((ext_vector_type(4)));
+
+struct PairArgs {
+    const int8_t *x;        // padded activations
+    const uint32_t *codes;  // [N/64][comm*num][32] 16-bit plane indices, channel j | channel j+32 << 16
+    const int32_t *bias;    // per channel or nullptr
+    int32_t *y;
+    uint32_t x_bytes;
+    int M, N, K, comm;
+    int pix_per_img, OW;
+    int x_img_stride, x_row_stride, x_col_stride;
+    int y_img_stride, y_ch_stride;
+    int x_plane, x_row;
+    int FH, FW;
+    int tiles_m, tiles_n;
+    int tile_begin, tile_end;  // tiles of this launch (index = pixel tile * tiles_n + channel tile)
+    int whole_tiles;           // workgroup shares end on tile boundaries
+    int blocks_per_xcd;
+    int atomic_out;
+    uint32_t y_elems;
+};
+
+struct PairWalk {
+    int koff, fw, fh, FW, FH, row_step, plane_step, koff_max;
+};
+
+constexpr int kPairRows = 3;               // accumulator rows per lane, two pixels each
+constexpr int kPairPixels = 6 * kWave;     // pixels of a tile
+constexpr int kPairSlots = 2048;           // wave slots of the machine at 2 waves per SIMD
+
+// K groups per call of the asm loop: at most 255 reduction indices (255 * 128 < 2^15)
+__host__ __device__ constexpr int pair_chunk(int bits) { return 255 / codes_per_word(bits); }
+
+#define DS_PAIRS_OPERANDS                                                                         \
+    : "+{v[64:95]}"(a[0]), "+{v[96:127]}"(a[1]), "+{v[128:159]}"(a[2]), "+{v[160:191]}"(a[3]),    \
+      "+{v[192:223]}"(a[4]), "+{v[224:255]}"(a[5])                                                \
+    : "v"(xoff[0]), "v"(xoff[1]), "v"(xoff[2]), "v"(xoff[3]), "v"(xoff[4]), "v"(xoff[5]),         \
+      "s"(rsrc), "s"(wptr), "s"(groups), "s"(w.koff), "s"(w.fw), "s"(w.fh), "s"(w.FW), "s"(w.FH), \
+      "s"(w.row_step), "s"(w.plane_step), "s"(w.koff_max)
+
+template <int BITS>
+__device__ __forceinline__ void pairs_main_loop(v32i (&a)[6], const uint32_t (&xoff)[6], v4i rsrc,
+                                                const uint32_t *wptr, int groups, const PairWalk &w);
+template <>
+__device__ __forceinline__ void pairs_main_loop<1>(v32i (&a)[6], const uint32_t (&xoff)[6], v4i rsrc,
+                                                   const uint32_t *wptr, int groups, const PairWalk &w)
+{
+    asm volatile(DS_PAIRS_ASM_B1 DS_PAIRS_OPERANDS : DS_PAIRS_CLOBBERS_B1);
+}
+template <>
+__device__ __forceinline__ void pairs_main_loop<2>(v32i (&a)[6], const uint32_t (&xoff)[6], v4i rsrc,
+                                                   const uint32_t *wptr, int groups, const PairWalk &w)
+{
+    asm volatile(DS_PAIRS_ASM_B2 DS_PAIRS_OPERANDS : DS_PAIRS_CLOBBERS_B2);
+}
+
+// K groups [g_begin, g_end) (at most pair_chunk of them) of the tile made of the 64 channels of
+// `ntile` and the 384 pixels from m0.
+// OUT selects where the widened sums go: kStore (y = sum + bias), kAtomic (atomic add to a
+// pre-filled y) or kLds (add to the workgroup's tile buffer lds[channel][pixel of the tile]).
+enum { kStore, kAtomic, kLds };
+
+template <int BITS, int OUT>
+__device__ __forceinline__ void pairs_segment(const PairArgs &p, int ntile, int m0, int g_begin, int g_end,
+                                              int32_t *lds)
+{
+    constexpr int NUM = 32 / (BITS + 1);
+    const int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+
+    uint32_t xoff[6];
+#pragma unroll
+    for (int q = 0; q < 6; ++q) {
+        int m = m0 + q * kWave + lane;
+        if (m >= p.M) m = p.M - 1;
+        const int img = m / p.pix_per_img;
+        const int rem = m - img * p.pix_per_img;
+        const int oh = rem / p.OW;
+        const int ow = rem - oh * p.OW;
+        xoff[q] = (uint32_t)(img * p.x_img_stride + oh * p.x_row_stride + ow * p.x_col_stride);
+    }
+
+    v32i a[6];
+#pragma unroll
+    for (int i = 0; i < 6; ++i) a[i] = (v32i)(0);
+    {
+        const uint64_t xaddr = (uint64_t)p.x;
+        v4i rsrc;
+        rsrc.x = (int32_t)(uint32_t)xaddr;
+        rsrc.y = (int32_t)(uint32_t)(xaddr >> 32);  // stride 0: raw buffer
+        rsrc.z = (int32_t)p.x_bytes;
+        rsrc.w = 0x00020000;
+        PairWalk w;
+        const int k0 = g_begin * NUM, ff = p.FH * p.FW;
+        const int ic = k0 / ff, rem = k0 - ic * ff;
+        w.fh = rem / p.FW;
+        w.fw = rem - w.fh * p.FW;
+        w.koff = ic * p.x_plane + w.fh * p.x_row + w.fw;
+        w.FW = p.FW;
+        w.FH = p.FH;
+        w.row_step = p.x_row - p.FW;
+        w.plane_step = p.x_plane - p.FH * p.x_row;
+        // reduction indices past K (the codes there select the zero plane) read the last real one
+        w.koff_max = (p.K / ff - 1) * p.x_plane + (p.FH - 1) * p.x_row + p.FW - 1;
+        pairs_main_loop<BITS>(a, xoff, rsrc,
+                              p.codes + ((size_t)ntile * p.comm + g_begin) * NUM * kTileWords,
+                              __builtin_amdgcn_readfirstlane(g_end - g_begin), w);
+    }
+
+    // split the sums into their halves (v = hi * 65536 + lo) and add them to the output
+    if (OUT == kLds) {
+#pragma unroll
+        for (int j = 0; j < 64; ++j) {
+#pragma unroll
+            for (int r = 0; r < kPairRows; ++r) {
+                const int32_t v = a[2 * r + j / 32][j % 32];
+                const int32_t lo = (int32_t)(int16_t)(v & 0xffff), hi = (v - lo) >> 16;
+                atomicAdd(lds + j * kPairPixels + (2 * r) * kWave + lane, lo);
+                atomicAdd(lds + j * kPairPixels + (2 * r + 1) * kWave + lane, hi);
+            }
+        }
+        return;
+    }
+    uint32_t yoff[6];
+    bool live[6];
+#pragma unroll
+    for (int q = 0; q < 6; ++q) {
+        const int m = m0 + q * kWave + lane;
+        live[q] = m < p.M;
+        const int mc = live[q] ? m : p.M - 1;
+        const int img = mc / p.pix_per_img;
+        yoff[q] = 4u * (uint32_t)(img * p.y_img_stride + (mc - img * p.pix_per_img));
+    }
+    const int n0 = ntile * 64;
+#pragma unroll
+    for (int j = 0; j < 64; ++j) {
+        int32_t *yc = p.y + (size_t)(n0 + j) * p.y_ch_stride;
+        const int32_t add = OUT == kAtomic ? 0 : (p.bias ? p.bias[n0 + j] : 0);
+#pragma unroll
+        for (int r = 0; r < kPairRows; ++r) {
+            const int32_t v = a[2 * r + j / 32][j % 32];
+            const int32_t lo = (int32_t)(int16_t)(v & 0xffff), hi = (v - lo) >> 16;
+            int32_t *dlo = (int32_t *)((char *)yc + yoff[2 * r]), *dhi = (int32_t *)((char *)yc + yoff[2 * r + 1]);
+            if (OUT == kAtomic) {
+                if (live[2 * r]) atomicAdd(dlo, lo);
+                if (live[2 * r + 1]) atomicAdd(dhi, hi);
+            } else {
+                if (live[2 * r]) *dlo = lo + add;
+                if (live[2 * r + 1]) *dhi = hi + add;
+            }
+        }
+    }
+}
+
+// One tile per wave, for reductions of a single chunk: plain stores of acc + bias.
+template <int BITS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void shift_pairs_kernel(
+    const PairArgs p)
+{
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int bid = blockIdx.x;
+    const int tile4 = (bid & 7) * p.blocks_per_xcd + (bid >> 3);
+    const int tile = p.tile_begin + tile4 * 4 + wave;  // neighbouring channel tiles of a pixel range share a workgroup
+    if (tile >= p.tile_end) return;
+    const int mt = tile / p.tiles_n, ntile = tile - mt * p.tiles_n;
+    pairs_segment<BITS, kStore>(p, ntile, mt * kPairPixels, 0, p.comm, nullptr);
+}
+
+// Equal shares of the (tile, K group) space, one per wave slot, as in the int32 kernel.
+template <int BITS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void shift_pairs_balanced_kernel(
+    const PairArgs p)
+{
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int bid = blockIdx.x;
+    const int w = ((bid & 7) * (int)(gridDim.x >> 3) + (bid >> 3)) * 4 + wave;
+    const int waves = (int)gridDim.x * 4;
+    const long total = (long)(p.tile_end - p.tile_begin) * p.comm;
+    int it = (int)(w * total / waves);
+    const int it_end = (int)((w + 1) * total / waves);
+    while (it < it_end) {
+        const int tile = p.tile_begin + it / p.comm;
+        const int g_begin = it - (tile - p.tile_begin) * p.comm;
+        int g_end = g_begin + (it_end - it);
+        if (g_end > p.comm) g_end = p.comm;
+        if (g_end > g_begin + pair_chunk(BITS)) g_end = g_begin + pair_chunk(BITS);
+        const int ntile = tile % p.tiles_n;
+        pairs_segment<BITS, kAtomic>(p, ntile, (tile / p.tiles_n) * kPairPixels, g_begin, g_end, nullptr);
+        it += g_end - g_begin;
+    }
+}
+
+// Workgroup-cooperative launch: equal shares of the (tile, K group) space per workgroup of eight
+// waves (one per compute unit: the tile buffer takes 96 KiB of its LDS).  The waves split the K
+// range of a tile among themselves and add their chunks to the tile buffer with LDS atomics, which
+// cost next to nothing; the combined tile then goes to the output once -- a plain store when the
+// workgroup ran the tile's whole reduction, atomic adds when it shares the tile with a neighbour.
+// Global atomics run at one lane per clock and L2 channel: flushing every chunk through them, as
+// the wave-level shares above do, costs as much as the arithmetic.
+constexpr int kPairCuWaves = 8;
+constexpr int kPairLdsBytes = 64 * kPairPixels * 4;
+
+template <int BITS>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void shift_pairs_cu_kernel(
+    const PairArgs p)
+{
+    extern __shared__ int32_t tile_sums[];  // [64 channels][384 pixels]
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & (kWave - 1);
+    const int bid = blockIdx.x;
+    const int w = (bid & 7) * (int)(gridDim.x >> 3) + (bid >> 3);  // an XCD takes a contiguous range
+    const int ntiles = p.tile_end - p.tile_begin;
+    const long total = (long)ntiles * p.comm;
+    int it, it_end;
+    if (p.whole_tiles) {
+        it = (int)((long)w * ntiles / (long)gridDim.x) * p.comm;
+        it_end = (int)((long)(w + 1) * ntiles / (long)gridDim.x) * p.comm;
+    } else {
+        it = (int)(w * total / (long)gridDim.x);
+        it_end = (int)((w + 1) * total / (long)gridDim.x);
+    }
+    while (it < it_end) {
+        const int tile = p.tile_begin + it / p.comm;
+        const int g0 = it - (tile - p.tile_begin) * p.comm;
+        int g1 = g0 + (it_end - it);
+        if (g1 > p.comm) g1 = p.comm;
+        const int ntile = tile % p.tiles_n, m0 = (tile / p.tiles_n) * kPairPixels;
+        for (int i = threadIdx.x; i < 64 * kPairPixels; i += 512) tile_sums[i] = 0;
+        __syncthreads();
+        const int len = g1 - g0;
+        const int wb = g0 + wave * len / kPairCuWaves, we = g0 + (wave + 1) * len / kPairCuWaves;
+        for (int g = wb; g < we; g += pair_chunk(BITS)) {
+            const int ge = g + pair_chunk(BITS) < we ? g + pair_chunk(BITS) : we;
+            pairs_segment<BITS, kLds>(p, ntile, m0, g, ge, tile_sums);
+        }
+        __syncthreads();
+        const bool whole = len == p.comm;
+        for (int c = 0; c < 64 / kPairCuWaves; ++c) {
+            const int j = wave * (64 / kPairCuWaves) + c, n = ntile * 64 + j;
+            const int32_t add = whole && p.bias ? p.bias[n] : 0;
+            for (int q = 0; q < 6; ++q) {
+                const int m = m0 + q * kWave + lane;
+                if (m >= p.M) break;
+                const int img = m / p.pix_per_img;
+                int32_t *dst = p.y + (size_t)img * p.y_img_stride + (size_t)n * p.y_ch_stride +
+                               (m - img * p.pix_per_img);
+                const int32_t v = tile_sums[j * kPairPixels + q * kWave + lane];
+                if (whole) *dst = v + add;
+                else atomicAdd(dst, v);
+            }
+        }
+        __syncthreads();
+        it += len;
+    }
+}
+
+// y = bias[n] before an accumulating launch; y is [img][n][pix], dense.
+__global__ void pairs_fill_kernel(const PairArgs p)
+{
+    const uint32_t total = p.y_elems;
+    const bool vec = ((uintptr_t)p.y & 15) == 0 && p.y_ch_stride % 4 == 0;
+    if (vec) {
+        int4 *y4 = (int4 *)p.y;
+        for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < (total >> 2); i += gridDim.x * blockDim.x) {
+            const int n = (int)(((i << 2) / (uint32_t)p.y_ch_stride) % (uint32_t)p.N);
+            const int32_t b = p.bias ? p.bias[n] : 0;
+            y4[i] = make_int4(b, b, b, b);
+        }
+    } else {
+        for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
+            const int n = (int)((i / (uint32_t)p.y_ch_stride) % (uint32_t)p.N);
+            p.y[i] = p.bias ? p.bias[n] : 0;
+        }
+    }
+}
+
+template <int BITS>
+static int launch_pairs_cu(const PairArgs &a, int blocks, hipStream_t st)
+{
+    static bool lds_opted_in = false;  // the tile buffer is above the default 64 KiB limit
+    if (!lds_opted_in) {
+        hipError_t e = hipFuncSetAttribute((const void *)shift_pairs_cu_kernel<BITS>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kPairLdsBytes);
+        if (e != hipSuccess) return hip_status(e);
+        lds_opted_in = true;
+    }
+    hipLaunchKernelGGL((shift_pairs_cu_kernel<BITS>), dim3(blocks), dim3(512), kPairLdsBytes, st, a);
+    return launch_status();
+}
+
+template <int BITS>
+static int launch_pairs(PairArgs a, hipStream_t st)
+{
+    a.tiles_m = ceil_div(a.M, kPairPixels);
+    a.tiles_n = a.N / 64;
+    const long tiles = (long)a.tiles_m * a.tiles_n;
+    const long iters = tiles * a.comm;
+    a.tile_begin = 0;
+    a.tile_end = (int)tiles;
+    // regime: 1 = one tile per wave (single chunk, plain stores), 2 = workgroup-cooperative,
+    // 0 = wave-level shares with global atomics
+    int regime = a.comm <= pair_chunk(BITS) ? 1 : 2;
+    if (const char *t = getenv("DS_TUNE_SPLIT")) {
+        regime = atoi(t);
+        if (regime == 1 && a.comm > pair_chunk(BITS)) regime = 0;
+    }
+    if (regime == 1) {
+        // Whole rounds of wave slots run one tile per wave.  A last round that would fill less than
+        // 60 % of the slots goes to the workgroup-cooperative kernel instead, whole tiles per
+        // workgroup (plain stores as well): its waves split each tile's reduction, so the tail of
+        // the launch takes a fraction of a tile time instead of a whole one.
+        const long rounds = tiles / kPairSlots, rest = tiles % kPairSlots;
+        long head = tiles;
+        if (rounds >= 1 && rest > 0 && rest * 10 <= (long)kPairSlots * 6) head = rounds * kPairSlots;
+        if (getenv("DS_TUNE_NOTAIL")) head = tiles;
+        a.atomic_out = 0;
+        a.tile_end = (int)head;
+        a.blocks_per_xcd = ceil_div((int)ceil_div((int)head, 4), 8);
+        hipLaunchKernelGGL((shift_pairs_kernel<BITS>), dim3(a.blocks_per_xcd * 8), dim3(256), 0, st, a);
+        if (head == tiles) return launch_status();
+        a.tile_begin = (int)head;
+        a.tile_end = (int)tiles;
+        a.whole_tiles = 1;
+        const long rest_blocks = (rest + 7) / 8 * 8;
+        return launch_pairs_cu<BITS>(a, rest_blocks < 256 ? (int)rest_blocks : 256, st);
+    }
+    a.atomic_out = 1;
+    long fill_blocks = ((long)a.y_elems / 4 + 255) / 256;
+    if (fill_blocks > 65536) fill_blocks = 65536;
+    if (fill_blocks < 1) fill_blocks = 1;
+    hipLaunchKernelGGL(pairs_fill_kernel, dim3((unsigned)fill_blocks), dim3(256), 0, st, a);
+    if (regime == 2) {
+        int blocks = 256;
+        const long fit = (iters / 64) / 8 * 8;  // small layers: at least 8 K groups per wave
+        if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
+        return launch_pairs_cu<BITS>(a, blocks, st);
+    }
+    int blocks = kPairSlots / 4;
+    const long fit = (iters / 16) / 8 * 8;  // small layers: at least 4 K groups per wave
+    if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
+    hipLaunchKernelGGL((shift_pairs_balanced_kernel<BITS>), dim3(blocks), dim3(256), 0, st, a);
+    return launch_status();
+}
+
+// Weight blob of this kernel: [N/64][comm*num][32] words and one spare row (the loop reads the codes
+// one reduction index ahead).
+struct PairedGeom {
+    int num, comm;
+    size_t rows, bytes;
+};
+static PairedGeom paired_geom(int N, int K, int bits)
+{
+    PairedGeom g;
+    g.num = codes_per_word(bits);
+    g.comm = ceil_div(K, g.num);
+    g.rows = (size_t)(N / 64) * g.comm * g.num + 1;
+    g.bytes = align_up(g.rows * kTileWords * 4, 256);
+    return g;
+}
+
+// Reference-format words [N][in_comm] (fields of in_bits) -> plane indices of `bits`-wide fields:
+// word j of row (t, k) = index(k, channel 64t + j) | index(k, channel 64t + 32 + j) << 16, each with
+// "src0 is relative" (bit 12) set so that the half-word is a ready M0 value.
+__global__ void tile_paired_kernel(const int32_t *__restrict__ w_ref, uint32_t *__restrict__ out, int N,
+                                   int K, int comm, int bits, int num, long words, int in_bits, int in_comm)
+{
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= words) return;
+    const uint32_t P = 1u << bits, zero = 0x1000u | (2u * P);
+    const int j = (int)(idx % kTileWords);
+    const long rest = idx / kTileWords;
+    const long rows = (long)comm * num;
+    const int k = (int)(rest % rows);
+    const long t = rest / rows;
+    uint32_t word = zero | (zero << 16);
+    if (k < K && t * 64 < N) {
+        word = 0;
+        const int in_cb = in_bits + 1, in_num = 32 / in_cb;
+        for (int c = 0; c < 2; ++c) {
+            const long n = t * 64 + 32 * c + j;
+            const uint32_t w = (uint32_t)w_ref[n * in_comm + k / in_num];
+            const uint32_t code = w >> ((k % in_num) * in_cb);
+            const uint32_t field = code & ((1u << in_bits) - 1u);
+            const uint32_t positive = (code >> in_bits) & 1u;
+            uint32_t index = zero;                      // fields >= 32 (6-bit words): zero weight
+            if (field < 32u) index = 0x1000u | ((field & (P - 1u)) + (positive ? 0u : P));
+            word |= index << (16 * c);
+        }
+    }
+    out[idx] = word;
+}
+
+}  // namespace ds
+
+using namespace ds;
+
+static int check_paired(int N, int C, int FH, int FW, int bits)
+{
+    if (bits < 1 || bits > 2) return DS_EBITS;
+    if (N < 0 || C < 0 || FH < 1 || FW < 1 || N % 64 != 0) return DS_EINVAL;
+    if (C >= (1 << 22) || FH > 31 || FW > 31 || (size_t)C * FH * FW >= (1u << 24)) return DS_ETOOLARGE;
+    return DS_OK;
+}
+
+DS_EXPORT size_t ds_paired_bytes(int N, int K, int field_bits)
+{
+    if (field_bits < 1 || field_bits > 2 || N < 0 || K < 0 || N % 64 != 0) return 0;
+    return paired_geom(N, K, field_bits).bytes;
+}
+
+DS_EXPORT int ds_tile_weights_paired_i32(const int32_t *w_ref, void *paired, int N, int C, int FH, int FW,
+                                         int ref_bits, int field_bits, ds_stream_t stream)
+{
+    int rc = check_paired(N, C, FH, FW, field_bits);
+    if (rc) return rc;
+    if (ref_bits != field_bits && ref_bits != 6) return DS_EBITS;
+    if (N == 0) return DS_OK;
+    if (!paired || (!w_ref && C > 0)) return DS_EINVAL;
+    const int K = C * FH * FW;
+    const PairedGeom g = paired_geom(N, K, field_bits);
+    const long words = (long)g.rows * kTileWords;
+    hipLaunchKernelGGL(tile_paired_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, w_ref, (uint32_t *)paired, N, K, g.comm, field_bits, g.num, words,
+                       ref_bits, ceil_div(K, codes_per_word(ref_bits)));
+    return launch_status();
+}
+
+DS_EXPORT int ds_conv2d_paired_i8(const int8_t *x, const void *paired, const int32_t *bias, int32_t *y,
+                                  int Nb, int C, int Hp, int Wp, int O, int FH, int FW, int sh, int sw,
+                                  int field_bits, ds_stream_t stream)
+{
+    int rc = check_paired(O, C, FH, FW, field_bits);
+    if (rc) return rc;
+    if (Nb < 0 || sh < 1 || sw < 1 || Hp < FH || Wp < FW) return DS_EINVAL;
+    const int OH = (Hp - FH) / sh + 1, OW = (Wp - FW) / sw + 1;
+    const size_t M = (size_t)Nb * OH * OW;
+    if (M == 0 || O == 0) return DS_OK;
+    if (!paired || !y || (!x && C > 0)) return DS_EINVAL;
+    const size_t K = (size_t)C * FH * FW;
+    const size_t x_bytes = (size_t)Nb * C * Hp * Wp;
+    if (x_bytes >= ((size_t)1 << 31) || M * O * 4 >= ((size_t)1 << 31)) return DS_ETOOLARGE;
+    const PairedGeom g = paired_geom(O, (int)K, field_bits);
+
+    PairArgs a{};
+    a.x = x;
+    a.x_bytes = (uint32_t)x_bytes;
+    a.codes = (const uint32_t *)paired;
+    a.bias = bias;
+    a.y = y;
+    a.M = (int)M; a.N = O; a.K = (int)K; a.comm = g.comm;
+    a.pix_per_img = OH * OW; a.OW = OW;
+    a.x_img_stride = C * Hp * Wp; a.x_row_stride = sh * Wp; a.x_col_stride = sw;
+    a.y_img_stride = O * OH * OW; a.y_ch_stride = OH * OW;
+    a.y_elems = (uint32_t)(M * O);
+    a.x_plane = Hp * Wp; a.x_row = Wp;
+    a.FH = FH; a.FW = FW;
+    if (K == 0) {
+        // no terms: the output is the bias
+        a.tiles_m = 0;
+        long blocks = ((long)a.y_elems / 4 + 255) / 256;
+        if (blocks > 65536) blocks = 65536;
+        if (blocks < 1) blocks = 1;
+        hipLaunchKernelGGL(pairs_fill_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, a);
+        return launch_status();
+    }
+    return field_bits == 1 ? launch_pairs<1>(a, (hipStream_t)stream) : launch_pairs<2>(a, (hipStream_t)stream);
+}

@@ -81,8 +81,8 @@ __global__ void quantize_kernel(const float *__restrict__ x, int32_t *__restrict
 }
 
 // One thread per padded output element; rows of the padded image are written contiguously.
-template <bool FROM_FLOAT>
-__global__ void pad_kernel(const void *__restrict__ xin, int32_t *__restrict__ q, uint32_t planes, int H,
+template <bool FROM_FLOAT, typename Q = int32_t>
+__global__ void pad_kernel(const void *__restrict__ xin, Q *__restrict__ q, uint32_t planes, int H,
                            int W, int ph, int pw, QuantSpec spec, FastDiv by_plane, FastDiv by_row)
 {
     const uint32_t Hp = H + 2 * ph, Wp = W + 2 * pw;
@@ -98,7 +98,7 @@ __global__ void pad_kernel(const void *__restrict__ xin, int32_t *__restrict__ q
             if (FROM_FLOAT) v = quantize_one(((const float *)xin)[src], spec);
             else v = ((const int32_t *)xin)[src];
         }
-        q[idx] = v;
+        q[idx] = (Q)v;
     }
 }
 
@@ -222,8 +222,9 @@ __global__ void dequantize_affine_kernel(const int32_t *__restrict__ y, float *_
 // dequantize_affine followed by the next shift layer's input conversion (round to the I.F grid,
 // cast, zero padding) in one pass: one thread per element of the padded int32 output q; the float
 // value is also stored to out when the caller needs it (a later residual add, a non-shift consumer).
+template <typename Q>
 __global__ void requantize_affine_pad_kernel(const int32_t *__restrict__ y, float *__restrict__ out,
-                                             int32_t *__restrict__ q, const float *__restrict__ scale,
+                                             Q *__restrict__ q, const float *__restrict__ scale,
                                              const float *__restrict__ shift,
                                              const float *__restrict__ residual, uint32_t planes, int C,
                                              int H, int W, int ph, int pw, float inv, int relu,
@@ -246,7 +247,7 @@ __global__ void requantize_affine_pad_kernel(const int32_t *__restrict__ y, floa
             if (out) out[src] = f;
             v = quantize_one(f, spec);
         }
-        q[idx] = v;
+        q[idx] = (Q)v;
     }
 }
 
@@ -254,8 +255,9 @@ __global__ void requantize_affine_pad_kernel(const int32_t *__restrict__ y, floa
 // f[oh][ow] = max over the pk x pk window (stride ps, implicit -inf padding pp, as nn.MaxPool2d) of
 // affine_one(y); one thread per element of the padded int32 output (or of out when q is NULL, with
 // ph = pw = 0).  y is [planes][H][W], out [planes][OH][OW], q [planes][OH+2ph][OW+2pw].
+template <typename Q>
 __global__ void requantize_affine_maxpool_kernel(const int32_t *__restrict__ y, float *__restrict__ out,
-                                                 int32_t *__restrict__ q, const float *__restrict__ scale,
+                                                 Q *__restrict__ q, const float *__restrict__ scale,
                                                  const float *__restrict__ shift, uint32_t planes, int C,
                                                  int H, int W, int OH, int OW, int pk, int ps, int pp,
                                                  int ph, int pw, float inv, int relu, QuantSpec spec,
@@ -314,7 +316,7 @@ __global__ void requantize_affine_maxpool_kernel(const int32_t *__restrict__ y, 
             if (out) out[((size_t)plane * OH + oh) * OW + ow] = best;
             v = quantize_one(best, spec);
         }
-        if (q) q[idx] = v;
+        if (q) q[idx] = (Q)v;
     }
 }
 
@@ -356,20 +358,46 @@ DS_EXPORT int ds_quantize_f32_i32(const float *x, int32_t *q, int64_t n, int I, 
     return launch_status();
 }
 
+// Formats whose round-to-fixed values fit int8: at most 8 bits, and not the one-bit special case
+// (sign(x) - 1 reaches -2 * 2^F).
+static int check_fixed_i8(int I, int F, int mode)
+{
+    int rc = check_fixed(I, F, mode);
+    if (rc) return rc;
+    if (mode != DS_Q_ROUND_TO_FIXED || I < 2 || I + F > 8) return DS_EINVAL;
+    return DS_OK;
+}
+
+template <typename Q>
+static int quantize_pad_any(const float *x, Q *q, int Nb, int C, int H, int W, int ph, int pw, int I, int F,
+                            int mode, ds_stream_t stream)
+{
+    if (Nb < 0 || C < 0 || H < 0 || W < 0 || ph < 0 || pw < 0) return DS_EINVAL;
+    const long total = (long)Nb * C * (H + 2 * ph) * (W + 2 * pw);
+    if (total == 0) return DS_OK;
+    if (total * (long)sizeof(Q) >= (1L << 31) || (long)Nb * C * H * W * 4 >= (1L << 31))
+        return DS_ETOOLARGE;  // like every tensor of the compute kernels
+    if (!x || !q) return DS_EINVAL;
+    hipLaunchKernelGGL((pad_kernel<true, Q>), dim3(grid_for(total)), dim3(256), 0, (hipStream_t)stream,
+                       (const void *)x, q, (uint32_t)(Nb * C), H, W, ph, pw, make_spec(I, F, mode),
+                       fast_div((uint32_t)((H + 2 * ph) * (W + 2 * pw))), fast_div((uint32_t)(W + 2 * pw)));
+    return launch_status();
+}
+
 DS_EXPORT int ds_quantize_pad_f32_i32(const float *x, int32_t *q, int Nb, int C, int H, int W, int ph,
                                       int pw, int I, int F, int mode, ds_stream_t stream)
 {
     int rc = check_fixed(I, F, mode);
     if (rc) return rc;
-    if (Nb < 0 || C < 0 || H < 0 || W < 0 || ph < 0 || pw < 0) return DS_EINVAL;
-    const long total = (long)Nb * C * (H + 2 * ph) * (W + 2 * pw);
-    if (total == 0) return DS_OK;
-    if (total * 4 >= (1L << 31)) return DS_ETOOLARGE;  // like every tensor of the compute kernels
-    if (!x || !q) return DS_EINVAL;
-    hipLaunchKernelGGL((pad_kernel<true>), dim3(grid_for(total)), dim3(256), 0, (hipStream_t)stream,
-                       (const void *)x, q, (uint32_t)(Nb * C), H, W, ph, pw, make_spec(I, F, mode),
-                       fast_div((uint32_t)((H + 2 * ph) * (W + 2 * pw))), fast_div((uint32_t)(W + 2 * pw)));
-    return launch_status();
+    return quantize_pad_any<int32_t>(x, q, Nb, C, H, W, ph, pw, I, F, mode, stream);
+}
+
+DS_EXPORT int ds_quantize_pad_f32_i8(const float *x, int8_t *q, int Nb, int C, int H, int W, int ph, int pw,
+                                     int I, int F, ds_stream_t stream)
+{
+    int rc = check_fixed_i8(I, F, DS_Q_ROUND_TO_FIXED);
+    if (rc) return rc;
+    return quantize_pad_any<int8_t>(x, q, Nb, C, H, W, ph, pw, I, F, DS_Q_ROUND_TO_FIXED, stream);
 }
 
 DS_EXPORT int ds_pad_i32(const int32_t *x, int32_t *xp, int Nb, int C, int H, int W, int ph, int pw,
@@ -380,7 +408,7 @@ DS_EXPORT int ds_pad_i32(const int32_t *x, int32_t *xp, int Nb, int C, int H, in
     if (total == 0) return DS_OK;
     if (total * 4 >= (1L << 31)) return DS_ETOOLARGE;
     if (!x || !xp) return DS_EINVAL;
-    hipLaunchKernelGGL((pad_kernel<false>), dim3(grid_for(total)), dim3(256), 0, (hipStream_t)stream,
+    hipLaunchKernelGGL((pad_kernel<false, int32_t>), dim3(grid_for(total)), dim3(256), 0, (hipStream_t)stream,
                        (const void *)x, xp, (uint32_t)(Nb * C), H, W, ph, pw, make_spec(16, 16, 0),
                        fast_div((uint32_t)((H + 2 * ph) * (W + 2 * pw))), fast_div((uint32_t)(W + 2 * pw)));
     return launch_status();
@@ -438,6 +466,24 @@ DS_EXPORT int ds_dequantize_affine_i32_f32(const int32_t *y, float *out, const f
     return launch_status();
 }
 
+template <typename Q>
+static int requantize_affine_pad_any(const int32_t *y, float *out, Q *q, const float *scale, const float *shift,
+                                     const float *residual, int Nb, int C, int H, int W, int ph, int pw,
+                                     int F_in, int relu, int I, int F, int mode, ds_stream_t stream)
+{
+    if (Nb < 0 || C < 0 || H < 0 || W < 0 || ph < 0 || pw < 0 || F_in < 0 || F_in > 31) return DS_EINVAL;
+    const long total = (long)Nb * C * (H + 2 * ph) * (W + 2 * pw);
+    if (total == 0) return DS_OK;
+    if (total * (long)sizeof(Q) >= (1L << 31) || (long)Nb * C * H * W * 4 >= (1L << 31)) return DS_ETOOLARGE;
+    if (!q || (!y && (long)Nb * C * H * W > 0)) return DS_EINVAL;
+    hipLaunchKernelGGL((requantize_affine_pad_kernel<Q>), dim3(grid_for(total)), dim3(256), 0,
+                       (hipStream_t)stream, y, out, q, scale, shift, residual, (uint32_t)(Nb * C), C, H, W,
+                       ph, pw, ldexpf(1.0f, -F_in), relu, make_spec(I, F, mode),
+                       fast_div((uint32_t)((H + 2 * ph) * (W + 2 * pw))), fast_div((uint32_t)(W + 2 * pw)),
+                       fast_div((uint32_t)C));
+    return launch_status();
+}
+
 DS_EXPORT int ds_requantize_affine_pad_i32(const int32_t *y, float *out, int32_t *q, const float *scale,
                                            const float *shift, const float *residual, int Nb, int C,
                                            int H, int W, int ph, int pw, int F_in, int relu, int I, int F,
@@ -445,15 +491,40 @@ DS_EXPORT int ds_requantize_affine_pad_i32(const int32_t *y, float *out, int32_t
 {
     int rc = check_fixed(I, F, mode);
     if (rc) return rc;
+    return requantize_affine_pad_any<int32_t>(y, out, q, scale, shift, residual, Nb, C, H, W, ph, pw, F_in,
+                                              relu, I, F, mode, stream);
+}
+
+DS_EXPORT int ds_requantize_affine_pad_i8(const int32_t *y, float *out, int8_t *q, const float *scale,
+                                          const float *shift, const float *residual, int Nb, int C, int H,
+                                          int W, int ph, int pw, int F_in, int relu, int I, int F,
+                                          ds_stream_t stream)
+{
+    int rc = check_fixed_i8(I, F, DS_Q_ROUND_TO_FIXED);
+    if (rc) return rc;
+    return requantize_affine_pad_any<int8_t>(y, out, q, scale, shift, residual, Nb, C, H, W, ph, pw, F_in,
+                                             relu, I, F, DS_Q_ROUND_TO_FIXED, stream);
+}
+
+template <typename Q>
+static int requantize_affine_maxpool_any(const int32_t *y, float *out, Q *q, const float *scale,
+                                         const float *shift, int Nb, int C, int H, int W, int pk, int ps,
+                                         int pp, int ph, int pw, int F_in, int relu, int I, int F, int mode,
+                                         ds_stream_t stream)
+{
     if (Nb < 0 || C < 0 || H < 0 || W < 0 || ph < 0 || pw < 0 || F_in < 0 || F_in > 31) return DS_EINVAL;
-    const long total = (long)Nb * C * (H + 2 * ph) * (W + 2 * pw);
+    if (pk < 1 || ps < 1 || pp < 0 || 2 * pp > pk) return DS_EINVAL;  // nn.MaxPool2d's own rule
+    if (!q && (ph || pw)) return DS_EINVAL;
+    if (H + 2 * pp < pk || W + 2 * pp < pk) return DS_EINVAL;
+    const int OH = (H + 2 * pp - pk) / ps + 1, OW = (W + 2 * pp - pk) / ps + 1;
+    const long total = (long)Nb * C * (OH + 2 * ph) * (OW + 2 * pw);
     if (total == 0) return DS_OK;
-    if (total * 4 >= (1L << 31)) return DS_ETOOLARGE;
-    if (!q || (!y && (long)Nb * C * H * W > 0)) return DS_EINVAL;
-    hipLaunchKernelGGL(requantize_affine_pad_kernel, dim3(grid_for(total)), dim3(256), 0,
-                       (hipStream_t)stream, y, out, q, scale, shift, residual, (uint32_t)(Nb * C), C, H, W,
-                       ph, pw, ldexpf(1.0f, -F_in), relu, make_spec(I, F, mode),
-                       fast_div((uint32_t)((H + 2 * ph) * (W + 2 * pw))), fast_div((uint32_t)(W + 2 * pw)),
+    if (total * 4 >= (1L << 31) || (long)Nb * C * H * W * 4 >= (1L << 31)) return DS_ETOOLARGE;
+    if (!y || (!q && !out)) return DS_EINVAL;
+    hipLaunchKernelGGL((requantize_affine_maxpool_kernel<Q>), dim3(grid_for(total)), dim3(256), 0,
+                       (hipStream_t)stream, y, out, q, scale, shift, (uint32_t)(Nb * C), C, H, W, OH, OW, pk,
+                       ps, pp, ph, pw, ldexpf(1.0f, -F_in), relu, make_spec(I, F, mode),
+                       fast_div((uint32_t)((OH + 2 * ph) * (OW + 2 * pw))), fast_div((uint32_t)(OW + 2 * pw)),
                        fast_div((uint32_t)C));
     return launch_status();
 }
@@ -465,21 +536,19 @@ DS_EXPORT int ds_requantize_affine_maxpool_i32(const int32_t *y, float *out, int
 {
     int rc = check_fixed(I, F, mode);
     if (rc) return rc;
-    if (Nb < 0 || C < 0 || H < 0 || W < 0 || ph < 0 || pw < 0 || F_in < 0 || F_in > 31) return DS_EINVAL;
-    if (pk < 1 || ps < 1 || pp < 0 || 2 * pp > pk) return DS_EINVAL;  // nn.MaxPool2d's own rule
-    if (!q && (ph || pw)) return DS_EINVAL;
-    if (H + 2 * pp < pk || W + 2 * pp < pk) return DS_EINVAL;
-    const int OH = (H + 2 * pp - pk) / ps + 1, OW = (W + 2 * pp - pk) / ps + 1;
-    const long total = (long)Nb * C * (OH + 2 * ph) * (OW + 2 * pw);
-    if (total == 0) return DS_OK;
-    if (total * 4 >= (1L << 31) || (long)Nb * C * H * W * 4 >= (1L << 31)) return DS_ETOOLARGE;
-    if (!y || (!q && !out)) return DS_EINVAL;
-    hipLaunchKernelGGL(requantize_affine_maxpool_kernel, dim3(grid_for(total)), dim3(256), 0,
-                       (hipStream_t)stream, y, out, q, scale, shift, (uint32_t)(Nb * C), C, H, W, OH, OW, pk,
-                       ps, pp, ph, pw, ldexpf(1.0f, -F_in), relu, make_spec(I, F, mode),
-                       fast_div((uint32_t)((OH + 2 * ph) * (OW + 2 * pw))), fast_div((uint32_t)(OW + 2 * pw)),
-                       fast_div((uint32_t)C));
-    return launch_status();
+    return requantize_affine_maxpool_any<int32_t>(y, out, q, scale, shift, Nb, C, H, W, pk, ps, pp, ph, pw,
+                                                  F_in, relu, I, F, mode, stream);
+}
+
+DS_EXPORT int ds_requantize_affine_maxpool_i8(const int32_t *y, float *out, int8_t *q, const float *scale,
+                                              const float *shift, int Nb, int C, int H, int W, int pk, int ps,
+                                              int pp, int ph, int pw, int F_in, int relu, int I, int F,
+                                              ds_stream_t stream)
+{
+    int rc = check_fixed_i8(I, F, DS_Q_ROUND_TO_FIXED);
+    if (rc) return rc;
+    return requantize_affine_maxpool_any<int8_t>(y, out, q, scale, shift, Nb, C, H, W, pk, ps, pp, ph, pw,
+                                                 F_in, relu, I, F, DS_Q_ROUND_TO_FIXED, stream);
 }
 
 DS_EXPORT int ds_copy_i32(const int32_t *src, int32_t *dst, int64_t n, ds_stream_t stream)

@@ -33,6 +33,18 @@ instructions per term).  It keeps 192 accumulators in v[64 + 64*r + j], needs 24
 fields (two waves per SIMD), reads one code row per reduction slot -- word j holds the codes of
 channels j (low half) and j + 32 (high half) -- and alternates between the two SGPR sets instead of
 copying.
+A third family (DS_PAIRS_ASM_B<n>, fields of 1 or 2 bits) serves int8 activations: a lane register
+holds TWO pixels, hi * 65536 + lo, the planes are built with packed 16-bit shifts, the sign of a code
+selects a negated plane instead of an xor mask (plane index = field, 2^BITS + field for a negative
+code, 2^(BITS+1) for a zero weight or a code past K: a plane held at 0), and one 32-bit v_add_u32
+accumulates both pixels: (64 + 3 * 2^BITS + 1) / 128 vector instructions per term.  Each half holds 255
+terms of an int8 activation, so the caller runs at most that many reduction slots per call.
+    v[8 + 6*(i % D) + 2r + h]     prefetched activation of slot i, row r, pixel half h
+    v[8 + 6*D + (2P+1)*r + idx]   planes of row r
+    v[64 + 64*r + j]              acc[r][j], pixel 2r in the low half, pixel 2r + 1 in the high half
+Its operands: %6..%11 per-pixel byte offsets, %12 descriptor, %13 word pointer, %14 groups,
+%15..%22 the walk.
+
 Operands: %6..%8 per-row byte offsets (VGPR), %9 buffer descriptor, %10 word pointer, %11 number of
 K groups, %12..%14 initial walk state (offset, fw, fh), %15 FW, %16 FH, %17 offset step when fw wraps,
 %18 offset step when fh wraps, %19 largest valid offset (the walk runs D slots ahead and is clamped).
@@ -42,19 +54,24 @@ import os
 R = 3
 DEPTH = {1: 4, 2: 5, 3: 4, 4: 3}        # prefetch ring depth, 32-channel form
 DEPTH_WIDE = {1: 4, 2: 5, 3: 4, 4: 2}   # 64-channel form: 4-bit fields leave room for two slots only
+DEPTH_PAIRED = {1: 4, 2: 2}             # int8 form: six activation registers per slot
 
 
 class Form:
     """Register and operand layout of the 32-channel (wide=False) or 64-channel loop."""
 
-    def __init__(self, bits, wide):
+    def __init__(self, bits, wide, paired=False):
+        self.paired = paired
         self.J = 64 if wide else 32
         self.acc = 64 if wide else 66
         self.depth = (DEPTH_WIDE if wide else DEPTH)[bits]
         self.waves = 2 if wide else 3
         nacc = 2 * R                            # accumulator operands %0..%5, 16 or 32 registers each
+        nx = 2 * R if paired else R             # activation offsets: one per pixel held by a lane
+        if paired:
+            self.depth = DEPTH_PAIRED[bits]
         self.op_xoff, self.op_rsrc, self.op_wptr, self.op_groups, self.op_walk = (
-            nacc, nacc + R, nacc + R + 1, nacc + R + 2, nacc + R + 3)
+            nacc, nacc + nx, nacc + nx + 1, nacc + nx + 2, nacc + nx + 3)
 
 
 XP = 8
@@ -77,10 +94,16 @@ def walk_and_load(slot, f):
     OP_XOFF, OP_RSRC, OP_WALK = f.op_xoff, f.op_rsrc, f.op_walk
     fw_end, fh_end, row_step, plane_step, koff_max = (OP_WALK + 3, OP_WALK + 4, OP_WALK + 5, OP_WALK + 6,
                                                       OP_WALK + 7)
-    L = ["s_min_u32 s%d, s%d, %%%d" % (T0, KOFF, koff_max),
-         "s_lshl_b32 s%d, s%d, 2" % (KB, T0)]
-    L += ["buffer_load_dword v%d, %%%d, %%%d, s%d offen" % (XP + R * slot + r, OP_XOFF + r, OP_RSRC, KB)
-          for r in range(R)]
+    if f.paired:
+        # int8 activations: element offsets are byte offsets; two pixels per row
+        L = ["s_min_u32 s%d, s%d, %%%d" % (KB, KOFF, koff_max)]
+        L += ["buffer_load_sbyte v%d, %%%d, %%%d, s%d offen" % (XP + 2 * R * slot + q, OP_XOFF + q, OP_RSRC, KB)
+              for q in range(2 * R)]
+    else:
+        L = ["s_min_u32 s%d, s%d, %%%d" % (T0, KOFF, koff_max),
+             "s_lshl_b32 s%d, s%d, 2" % (KB, T0)]
+        L += ["buffer_load_dword v%d, %%%d, %%%d, s%d offen" % (XP + R * slot + r, OP_XOFF + r, OP_RSRC, KB)
+              for r in range(R)]
     L += ["s_add_u32 s%d, s%d, 1" % (FWC, FWC),
           "s_add_u32 s%d, s%d, 1" % (KOFF, KOFF),
           "s_cmp_eq_u32 s%d, %%%d" % (FWC, fw_end),
@@ -216,6 +239,90 @@ def clobbers(bits, wide=False):
     return ", ".join(v + s + ['"scc"', '"memory"'])
 
 
+def body_paired(bits):
+    """The int8 form: 3 rows x 2 pixels x 64 channels per lane (see the module docstring)."""
+    f = Form(bits, True, paired=True)
+    num = 32 // (bits + 1)
+    P = 1 << bits
+    S = 2 * P + 1                               # planes per row: shifts, negated shifts, zero
+    D, ACC = f.depth, f.acc
+    assert num % D == 0 and num % 2 == 0
+    PL = XP + 2 * R * D
+    assert PL + S * R <= ACC and ACC + R * f.J <= 256
+    L = []
+    L += ["s_getreg_b32 s%d, hwreg(HW_REG_HW_ID, 0, 4)" % PRIO,
+          "s_mov_b32 s%d, %%%d" % (CNT, f.op_groups),
+          "s_mov_b64 s[%d:%d], %%%d" % (WP, WP + 1, f.op_wptr),
+          "s_mov_b32 s%d, %%%d" % (KOFF, f.op_walk), "s_mov_b32 s%d, %%%d" % (FWC, f.op_walk + 1),
+          "s_mov_b32 s%d, %%%d" % (FHC, f.op_walk + 2),
+          "s_mov_b32 s%d, 0x05040100" % MASK]   # v_perm_b32 selector: low halves of (src0, src1)
+    L += load_words(W)
+    L += ["s_memrealtime s[%d:%d]" % (TIME, TIME + 1)]
+    for i in range(D):
+        L += walk_and_load(i, f)
+    for r in range(R):
+        L += ["v_mov_b32 v%d, 0" % (PL + S * r + 2 * P)]
+    L += ["s_mov_b32 s%d, 0" % IDX]
+    L += ["1:"]
+    for i in range(num):
+        cur, nxt = (W, WS) if i % 2 == 0 else (WS, W)
+        L += ["s_add_u32 s%d, s%d, 128" % (WP, WP), "s_addc_u32 s%d, s%d, 0" % (WP + 1, WP + 1),
+              "s_waitcnt lgkmcnt(0)"]
+        if i % 2 == 0:
+            L += take_turn(i // 2, f.waves)
+        L += load_words(nxt)
+        if i % 2 == 1:
+            L += ["s_memrealtime s[%d:%d]" % (TIME, TIME + 1)]
+        slot = i % D
+        L += ["s_waitcnt vmcnt(%d)" % (2 * R * (D - 1))]
+        # The planes, with relative addressing off (these instructions name two vector registers).
+        # A plane holds hi * 65536 + lo as ONE 32-bit number (lo signed), so that the full-rate 32-bit
+        # add accumulates both pixels: borrows of a negative lo run into the high half and come out
+        # again when the sum is split.  Per row: pk = the two activations as 16-bit fields (into the
+        # register of pixel b), c = 65536 where pixel a is negative (into its own register: a >> f has
+        # the sign of a), then p[f] = (pk >> f per half) - c and the negated planes 0 - p[f].
+        L += ["s_set_gpr_idx_off"]
+        for r in range(R):
+            lo, hi = XP + 2 * R * slot + 2 * r, XP + 2 * R * slot + 2 * r + 1
+            L += ["v_perm_b32 v%d, v%d, v%d, s%d" % (hi, hi, lo, MASK),
+                  "v_and_b32 v%d, 0x10000, v%d" % (lo, lo),
+                  "v_sub_u32 v%d, v%d, v%d" % (PL + S * r, hi, lo)]
+        for s in range(1, P):
+            for r in range(R):
+                lo, hi = XP + 2 * R * slot + 2 * r, XP + 2 * R * slot + 2 * r + 1
+                L += ["v_pk_ashrrev_i16 v%d, %d, v%d op_sel_hi:[0,1]" % (PL + S * r + s, s, hi)]
+        for s in range(1, P):
+            for r in range(R):
+                lo = XP + 2 * R * slot + 2 * r
+                L += ["v_sub_u32 v%d, v%d, v%d" % (PL + S * r + s, PL + S * r + s, lo)]
+        for s in range(P):
+            for r in range(R):
+                L += ["v_sub_u32 v%d, 0, v%d" % (PL + S * r + P + s, PL + S * r + s)]
+        L += walk_and_load(slot, f)  # the ring slot is free again
+        L += ["s_set_gpr_idx_on s%d, 0x1" % IDX]
+        # the 16-bit code is the M0 value itself: plane index in 7:0, "src0 relative" in 15:12
+        for half in (0, 1):
+            for j in range(32):
+                if half == 0:
+                    L += ["s_mov_b32 m0, s%d" % (cur + j)]
+                else:
+                    L += ["s_lshr_b32 m0, s%d, 16" % (cur + j)]
+                for r in range(R):
+                    a = ACC + f.J * r + j + 32 * half
+                    L += ["v_add_u32 v%d, v%d, v%d" % (a, PL + S * r, a)]
+    L += ["s_sub_u32 s%d, s%d, 1" % (CNT, CNT), "s_cmp_lg_u32 s%d, 0" % CNT, "s_cbranch_scc1 1b"]
+    L += ["s_set_gpr_idx_off", "s_setprio 0", "s_waitcnt vmcnt(0) lgkmcnt(0)"]
+    return L
+
+
+def clobbers_paired(bits):
+    f = Form(bits, True, paired=True)
+    P = 1 << bits
+    v = ['"v%d"' % n for n in range(XP, XP + 2 * R * f.depth + (2 * P + 1) * R)]
+    s = ['"s%d"' % n for n in list(range(4, 16)) + list(range(W, WS + 32)) + [TIME, TIME + 1]]
+    return ", ".join(v + s + ['"scc"', '"memory"'])
+
+
 def main():
     here = os.path.dirname(os.path.abspath(__file__))
     out = ["// Generated by gen_planes_asm.py -- do not edit by hand.", ""]
@@ -228,6 +335,12 @@ def main():
                 out.append("")
             out.append("#define DS_PLANES_CLOBBERS_B%d%s %s" % (bits, wtag, clobbers(bits, wide)))
             out.append("")
+    for bits in (1, 2):
+        out.append("#define DS_PAIRS_ASM_B%d \\" % bits)
+        out.append(" \\\n".join('    "%s\\n"' % line for line in body_paired(bits)))
+        out.append("")
+        out.append("#define DS_PAIRS_CLOBBERS_B%d %s" % (bits, clobbers_paired(bits)))
+        out.append("")
     with open(os.path.join(here, "ds_planes_asm.inc"), "w") as f:
         f.write("\n".join(out))
 

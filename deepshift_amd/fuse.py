@@ -22,7 +22,7 @@ import torch.fx as fx
 import torch.nn as nn
 import torch.nn.functional as F
 
-from . import modules, modules_q
+from . import kernels, modules, modules_q
 
 __all__ = ["FusedConv2dShift", "fuse_conv_epilogues"]
 
@@ -39,7 +39,7 @@ class FusedConv2dShift(nn.Module):
         self.conv = conv
         self.relu = relu
         self.prequantized = False  # the input is this layer's int32 padded input, made by its producer
-        self.emit = None           # (padding, I, F, want_float) of the consumers' input to produce
+        self.emit = None           # (padding, I, F, want_float, dtype) of the consumers' input to produce
         self.pool = None           # (kernel, stride, padding) of a max pooling that follows the ReLU
         if bn is not None:
             if bn.training or not bn.track_running_stats:
@@ -181,10 +181,19 @@ def fuse_conv_epilogues(model, handoff=True):
 
 
 def _input_key(conv):
-    """What a kernel-mode convolution needs of its int32 input, or None if it pads by itself."""
+    """What a kernel-mode convolution needs of its fixed-point input -- (padding, I, F, dtype) -- or
+    None if it pads by itself."""
     if conv.padding_mode != 'zeros' or not conv.use_kernel:
         return None
-    return (tuple(conv.padding), conv.act_integer_bits, conv.act_fraction_bits)
+    if conv.conc_weight is None and conv.shift.is_cuda:
+        if isinstance(conv, modules_q.Conv2dShiftQ):
+            modules_q.pack_module_weights_q(conv)
+        else:
+            modules.pack_module_weights(conv)
+    paired = kernels.paired_fields(conv.conc_weight, conv.out_channels, conv.act_integer_bits,
+                                   conv.act_fraction_bits)
+    return (tuple(conv.padding), conv.act_integer_bits, conv.act_fraction_bits,
+            torch.int8 if paired else torch.int32)
 
 
 def _hand_off_fixed_point(gm):
@@ -214,7 +223,7 @@ def _hand_off_fixed_point(gm):
             continue
         # the float result is still needed by any other use, including a taker's residual operand
         want_float = any(u not in takers or node in u.args[1:] for u in node.users)
-        producer.emit = key + (want_float,)
+        producer.emit = key[:3] + (want_float, key[3])
         if want_float:
             with gm.graph.inserting_after(node):
                 q = gm.graph.call_function(operator.getitem, (node, 1))

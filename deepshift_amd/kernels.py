@@ -157,6 +157,51 @@ def _tiled_of(conc_weight, N, C, FH=1, FW=1):
     return cached[1]
 
 
+def paired_fields(conc_weight, out_channels, integer_bits, fraction_bits):
+    """``(ref_bits, field_bits)`` when a layer can run on the int8 kernel (two pixels per register),
+    else ``None``: activations of at most 8 bits (and not the one-bit format), a channel count that is a
+    multiple of 64, base 0, and shift fields of at most 2 bits -- either packed that narrow, or 6-bit
+    ternary words whose non-zero fields are that narrow."""
+    if integer_bits < 2 or integer_bits + fraction_bits > 8 or out_channels % 64 != 0:
+        return None
+    if conc_weight is None or conc_weight.base != 0:
+        return None
+    if conc_weight.bits <= 2:
+        return (conc_weight.bits, conc_weight.bits)
+    width = getattr(conc_weight, "zero_top_bits", 0)
+    if conc_weight.bits == 6 and 1 <= width <= 2:
+        return (6, width)
+    return None
+
+
+def tile_weights_paired(packed, N, C, FH, FW, ref_bits, field_bits):
+    """Reference-layout words (fields of ``ref_bits``) -> the blob of the int8 kernel."""
+    packed = _require_device_i32("packed", packed)
+    K = C * FH * FW
+    num = 32 // (ref_bits + 1)
+    if packed.numel() != N * ((K + num - 1) // num):
+        raise ValueError("packed weight has %d words, expected %d" %
+                         (packed.numel(), N * ((K + num - 1) // num)))
+    nbytes = _lib.lib().ds_paired_bytes(N, K, field_bits)
+    if nbytes == 0 and N > 0:
+        raise ValueError("no int8 kernel for N=%d, field_bits=%d" % (N, field_bits))
+    blob = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=packed.device)
+    _lib.call("ds_tile_weights_paired_i32", _lib.ptr(packed), _lib.ptr(blob), N, C, FH, FW, int(ref_bits),
+              int(field_bits), _lib.current_stream(packed.device))
+    return blob
+
+
+def _paired_of(conc_weight, fields, N, C, FH=1, FW=1):
+    """The int8 kernel's blob of a ConcWeight, built once and cached on the object."""
+    data = conc_weight.data
+    key = (data.data_ptr(), data._version, N, C, FH, FW, fields)
+    cached = getattr(conc_weight, "_paired", None)
+    if cached is None or cached[0] != key:
+        cached = (key, tile_weights_paired(data, N, C, FH, FW, fields[0], fields[1]))
+        conc_weight._paired = cached
+    return cached[1]
+
+
 # ---------------------------------------------------------------------------------------------
 # fixed-point conversion
 # ---------------------------------------------------------------------------------------------
@@ -174,14 +219,21 @@ def quantize(x, integer_bits=16, fraction_bits=16, round_to_fixed=True):
     return q
 
 
-def quantize_pad(x, padding, integer_bits=16, fraction_bits=16, round_to_fixed=True):
-    """float32 NCHW -> zero padded int32 NCHW (conversion fused with kernels.py:32-36)."""
+def quantize_pad(x, padding, integer_bits=16, fraction_bits=16, round_to_fixed=True, dtype=torch.int32):
+    """float32 NCHW -> zero padded int32 NCHW (conversion fused with kernels.py:32-36); ``dtype`` int8
+    for the int8 kernel (formats of at most 8 bits, round_to_fixed only)."""
     x = x.contiguous()
     if x.dtype != torch.float32 or not x.is_cuda or x.dim() != 4:
         raise TypeError("quantize_pad expects a 4-D float32 GPU tensor")
     ph, pw = _pair(padding)
     Nb, C, H, W = x.shape
-    q = torch.empty([Nb, C, H + 2 * ph, W + 2 * pw], dtype=torch.int32, device=x.device)
+    q = torch.empty([Nb, C, H + 2 * ph, W + 2 * pw], dtype=dtype, device=x.device)
+    if dtype == torch.int8:
+        if not round_to_fixed:
+            raise ValueError("int8 activations need round_to_fixed")
+        _lib.call("ds_quantize_pad_f32_i8", _lib.ptr(x), _lib.ptr(q), Nb, C, H, W, ph, pw, integer_bits,
+                  fraction_bits, _lib.current_stream(x.device))
+        return q
     _lib.call("ds_quantize_pad_f32_i32", _lib.ptr(x), _lib.ptr(q), Nb, C, H, W, ph, pw,
               integer_bits, fraction_bits,
               _lib.DS_Q_ROUND_TO_FIXED if round_to_fixed else _lib.DS_Q_CAST,
@@ -233,11 +285,11 @@ def dequantize_affine(y, fraction_bits=16, scale=None, shift=None, residual=None
 
 
 def requantize_affine_pad(y, fraction_bits_in, scale, shift, residual, relu, padding,
-                          integer_bits=16, fraction_bits=16, want_float=True):
+                          integer_bits=16, fraction_bits=16, want_float=True, dtype=torch.int32):
     """:func:`dequantize_affine` and the next shift convolution's :func:`quantize_pad` in one pass.
 
     Returns ``(out, q)``: the float32 result (``None`` unless ``want_float``) and its round-to-fixed,
-    zero padded int32 form, bit-identical to the two separate calls."""
+    zero padded int32 (or ``dtype`` int8) form, bit-identical to the two separate calls."""
     y = _require_device_i32("y", y)
     if y.dim() != 4:
         raise TypeError("requantize_affine_pad expects a 4-D int32 GPU tensor")
@@ -251,7 +303,12 @@ def requantize_affine_pad(y, fraction_bits_in, scale, shift, residual, relu, pad
             raise ValueError("residual must be float32 with the shape of y")
         residual = residual.contiguous()
     out = torch.empty(y.shape, dtype=torch.float32, device=y.device) if want_float else None
-    q = torch.empty([Nb, C, H + 2 * ph, W + 2 * pw], dtype=torch.int32, device=y.device)
+    q = torch.empty([Nb, C, H + 2 * ph, W + 2 * pw], dtype=dtype, device=y.device)
+    if dtype == torch.int8:
+        _lib.call("ds_requantize_affine_pad_i8", _lib.ptr(y), _lib.ptr(out), _lib.ptr(q), _lib.ptr(scale),
+                  _lib.ptr(shift), _lib.ptr(residual), Nb, C, H, W, ph, pw, fraction_bits_in,
+                  int(bool(relu)), integer_bits, fraction_bits, _lib.current_stream(y.device))
+        return out, q
     _lib.call("ds_requantize_affine_pad_i32", _lib.ptr(y), _lib.ptr(out), _lib.ptr(q), _lib.ptr(scale),
               _lib.ptr(shift), _lib.ptr(residual), Nb, C, H, W, ph, pw, fraction_bits_in,
               int(bool(relu)), integer_bits, fraction_bits, _lib.DS_Q_ROUND_TO_FIXED,
@@ -260,7 +317,7 @@ def requantize_affine_pad(y, fraction_bits_in, scale, shift, residual, relu, pad
 
 
 def requantize_affine_maxpool(y, fraction_bits_in, scale, shift, relu, pool, padding=None,
-                              integer_bits=16, fraction_bits=16, want_float=True):
+                              integer_bits=16, fraction_bits=16, want_float=True, dtype=torch.int32):
     """:func:`dequantize_affine`, ``max_pool2d(kernel, stride, padding)`` and -- when ``padding`` (of
     the next shift convolution) is given -- its :func:`quantize_pad`, in one pass.
     ``pool = (kernel, stride, padding)``.  Returns ``(out, q)``; either may be ``None``."""
@@ -277,8 +334,13 @@ def requantize_affine_maxpool(y, fraction_bits_in, scale, shift, relu, pool, pad
         raise ValueError("nothing to produce")
     ph, pw = _pair(padding) if padding is not None else (0, 0)
     out = torch.empty([Nb, C, OH, OW], dtype=torch.float32, device=y.device) if want_float else None
-    q = torch.empty([Nb, C, OH + 2 * ph, OW + 2 * pw], dtype=torch.int32, device=y.device) \
+    q = torch.empty([Nb, C, OH + 2 * ph, OW + 2 * pw], dtype=dtype, device=y.device) \
         if padding is not None else None
+    if dtype == torch.int8 and q is not None:
+        _lib.call("ds_requantize_affine_maxpool_i8", _lib.ptr(y), _lib.ptr(out), _lib.ptr(q), _lib.ptr(scale),
+                  _lib.ptr(shift), Nb, C, H, W, pk, ps, pp, ph, pw, fraction_bits_in, int(bool(relu)),
+                  integer_bits, fraction_bits, _lib.current_stream(y.device))
+        return out, q
     _lib.call("ds_requantize_affine_maxpool_i32", _lib.ptr(y), _lib.ptr(out), _lib.ptr(q), _lib.ptr(scale),
               _lib.ptr(shift), Nb, C, H, W, pk, ps, pp, ph, pw, fraction_bits_in, int(bool(relu)),
               integer_bits, fraction_bits, _lib.DS_Q_ROUND_TO_FIXED, _lib.current_stream(y.device))
@@ -347,6 +409,25 @@ def conv2d_tiled(x_padded, tiled, bias, O, kernel_size, stride, bits, base=0):
         _lib.call("ds_conv2d_tiled_i32", _lib.ptr(x_padded), _lib.ptr(tiled), _lib.ptr(bias),
                   _lib.ptr(out), Nb, C, Hp, Wp, O, FH, FW, sh, sw, int(bits), int(base),
                   _lib.ptr(ws), ws_bytes, _lib.current_stream(x_padded.device))
+    return out
+
+
+def conv2d_paired(x_padded, paired, bias, O, kernel_size, stride, field_bits):
+    """Shift convolution on an already padded int8 NCHW input and the blob of
+    :func:`tile_weights_paired`; the int32 result of :func:`conv2d_tiled` on the same values."""
+    if x_padded.dtype != torch.int8 or not x_padded.is_cuda or x_padded.dim() != 4:
+        raise TypeError("x_padded must be a 4-D int8 GPU tensor")
+    x_padded = x_padded.contiguous()
+    Nb, C, Hp, Wp = x_padded.shape
+    FH, FW = _pair(kernel_size)
+    sh, sw = _pair(stride)
+    if Hp < FH or Wp < FW:
+        raise ValueError("padded input %dx%d is smaller than the %dx%d filter" % (Hp, Wp, FH, FW))
+    OH, OW = (Hp - FH) // sh + 1, (Wp - FW) // sw + 1
+    out = torch.empty([Nb, O, OH, OW], dtype=torch.int32, device=x_padded.device)
+    with _Timed("conv", Nb * OH * OW, C * FH * FW, O, x_padded.device):
+        _lib.call("ds_conv2d_paired_i8", _lib.ptr(x_padded), _lib.ptr(paired), _lib.ptr(bias), _lib.ptr(out),
+                  Nb, C, Hp, Wp, O, FH, FW, sh, sw, int(field_bits), _lib.current_stream(x_padded.device))
     return out
 
 

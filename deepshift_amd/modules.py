@@ -206,14 +206,17 @@ def conv_kernel_forward(module, input, conc_weight, scale=None, shift=None, resi
 
     ``prequantized``: ``input`` is already the layer's round-to-fixed, zero padded int32 input (made
     by the layer before it).  ``emit = (padding, integer_bits, fraction_bits, want_float)``: also
-    produce that form of the result for the next shift convolution; the return value is then
-    ``(out, q)``, or ``q`` alone when ``want_float`` is false.  ``pool = (kernel, stride, padding)``:
+    produce that form of the result for the next shift convolution (a fifth element gives its dtype:
+    int8 for a consumer on the int8 kernel); the return value is then ``(out, q)``, or ``q`` alone when
+    ``want_float`` is false.  ``pool = (kernel, stride, padding)``:
     a max pooling follows the ReLU (no residual) and runs in the same pass."""
     if not module.use_cuda:
         kernels._no_cpu_kernel()
     if module.dilation != (1, 1) or module.groups != 1:
         raise NotImplementedError("the shift kernel supports dilation=1 and groups=1 only")
     I, Fb = module.act_integer_bits, module.act_fraction_bits
+    # formats of at most 8 bits on narrow shift fields: int8 activations, two pixels per register
+    fields = kernels.paired_fields(conc_weight, module.out_channels, I, Fb)
     if prequantized:
         xq = input
     else:
@@ -223,12 +226,24 @@ def conv_kernel_forward(module, input, conc_weight, scale=None, shift=None, resi
             input = _circular_pad(input, padding)
             padding = (0, 0)
         # round_to_fixed + cast + zero padding in one pass
-        xq = kernels.quantize_pad(input, padding, I, Fb, round_to_fixed=True)
+        xq = kernels.quantize_pad(input, padding, I, Fb, round_to_fixed=True,
+                                  dtype=torch.int8 if fields else torch.int32)
     bias = module._fixed_bias.get(module.bias, I, Fb, round_to_fixed=True)
-    tiled = kernels._tiled_of(conc_weight, module.out_channels, module.in_channels,
-                              module.kernel_size[0], module.kernel_size[1])
-    out = kernels.conv2d_tiled(xq, tiled, bias, module.out_channels, module.kernel_size,
-                               module.stride, kernels.kernel_bits(conc_weight), conc_weight.base)
+    if xq.dtype == torch.int8:
+        if not fields:
+            raise ValueError("this layer has no int8 kernel; hand it int32 activations")
+        blob = kernels._paired_of(conc_weight, fields, module.out_channels, module.in_channels,
+                                  module.kernel_size[0], module.kernel_size[1])
+        out = kernels.conv2d_paired(xq, blob, bias, module.out_channels, module.kernel_size, module.stride,
+                                    fields[1])
+    else:
+        tiled = kernels._tiled_of(conc_weight, module.out_channels, module.in_channels,
+                                  module.kernel_size[0], module.kernel_size[1])
+        out = kernels.conv2d_tiled(xq, tiled, bias, module.out_channels, module.kernel_size,
+                                   module.stride, kernels.kernel_bits(conc_weight), conc_weight.base)
+    emit_dtype = torch.int32
+    if emit is not None and len(emit) == 5:
+        emit, emit_dtype = emit[:4], emit[4]
     if pool is not None:
         if residual is not None:
             raise ValueError("a fused max pooling cannot follow a residual add")
@@ -236,12 +251,12 @@ def conv_kernel_forward(module, input, conc_weight, scale=None, shift=None, resi
             return kernels.requantize_affine_maxpool(out, Fb, scale, shift, relu, pool)[0]
         next_padding, next_I, next_F, want_float = emit
         f, q = kernels.requantize_affine_maxpool(out, Fb, scale, shift, relu, pool, next_padding,
-                                                 next_I, next_F, want_float)
+                                                 next_I, next_F, want_float, emit_dtype)
         return (f, q) if want_float else q
     if emit is not None:
         next_padding, next_I, next_F, want_float = emit
         f, q = kernels.requantize_affine_pad(out, Fb, scale, shift, residual, relu, next_padding,
-                                             next_I, next_F, want_float)
+                                             next_I, next_F, want_float, emit_dtype)
         return (f, q) if want_float else q
     if scale is None and shift is None and residual is None and not relu:
         return kernels.dequantize(out, Fb)

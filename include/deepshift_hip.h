@@ -81,6 +81,46 @@ int ds_tile_weights_i32(const int32_t *w_ref, void *tiled, int N, int C, int FH,
 int ds_tile_weights_zero_top_i32(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW,
                                  int field_bits, ds_stream_t stream);
 
+/* ---- int8 activations ------------------------------------------------------------------ */
+
+/* Activation formats of at most 8 bits (act_integer_bits + act_fraction_bits <= 8, e.g. the 3.5 format
+ * of the reference's 8-bit runs) can be held as int8.  |x >> s| <= 128 then, 255 terms fit a 16-bit
+ * sum, and the vector ALU handles two pixels per register (packed 16-bit shifts and adds), widening
+ * to the int32 output every 255 reduction indices: the int32 kernels' results, bit for bit, in about
+ * half the vector instructions and a quarter of the activation bytes.  For layers with
+ * O % 64 == 0 and shift fields of 1 or 2 bits (weight_bits <= 3).  No counterpart in the reference,
+ * which always computes on int32 (modules.py:153).
+ *
+ * ds_tile_weights_paired_i32 lays reference-format words w_ref[N][ceil(K / (32 / (ref_bits + 1)))]
+ * (ds_pack_i32's output, base 0) out for that kernel: ds_paired_bytes(N, K, field_bits) bytes.
+ * ref_bits is the field width of the words: field_bits, or 6 for the words of a ternary layer whose
+ * non-zero fields are all below 2^field_bits (zero weights, fields >= 32, then select a plane held
+ * at 0). */
+size_t ds_paired_bytes(int N, int K, int field_bits);
+int ds_tile_weights_paired_i32(const int32_t *w_ref, void *paired, int N, int C, int FH, int FW,
+                               int ref_bits, int field_bits, ds_stream_t stream);
+
+/* Conv2dShift forward on int8 activations: ds_conv2d_tiled_i32 (DEEP_SHIFT_CONV,
+ * kernels/cuda/shift_cuda.cpp:41-53) with x int8 [Nb][C][Hp][Wp], already padded, and the blob of
+ * ds_tile_weights_paired_i32.  y int32 [Nb][O][OH][OW].  DS_EINVAL when O % 64 != 0, DS_EBITS when
+ * field_bits is not 1 or 2. */
+int ds_conv2d_paired_i8(const int8_t *x, const void *paired, const int32_t *bias, int32_t *y, int Nb,
+                        int C, int Hp, int Wp, int O, int FH, int FW, int sh, int sw, int field_bits,
+                        ds_stream_t stream);
+
+/* The conversion passes with an int8 result, for that kernel's input: ds_quantize_pad_f32_i32,
+ * ds_requantize_affine_pad_i32 and ds_requantize_affine_maxpool_i32 with q int8, always in mode
+ * DS_Q_ROUND_TO_FIXED (utils.py:7-21, whose clamp is what bounds the values).  DS_EINVAL unless
+ * 2 <= I and I + F <= 8. */
+int ds_quantize_pad_f32_i8(const float *x, int8_t *q, int Nb, int C, int H, int W, int ph, int pw, int I,
+                           int F, ds_stream_t stream);
+int ds_requantize_affine_pad_i8(const int32_t *y, float *out, int8_t *q, const float *scale,
+                                const float *shift, const float *residual, int Nb, int C, int H, int W,
+                                int ph, int pw, int F_in, int relu, int I, int F, ds_stream_t stream);
+int ds_requantize_affine_maxpool_i8(const int32_t *y, float *out, int8_t *q, const float *scale,
+                                    const float *shift, int Nb, int C, int H, int W, int pk, int ps, int pp,
+                                    int ph, int pw, int F_in, int relu, int I, int F, ds_stream_t stream);
+
 /* ---- LinearShift ----------------------------------------------------------------------- */
 
 /* Workspace bytes ds_linear_i32 needs (transposed activations, tiled weights, offset table). */
