@@ -329,9 +329,9 @@ DS_PLANES_SPECIALISE(4)
 // channels of `ntile` and the R*64 pixels starting at m0.  `atomic` selects accumulation into a
 // pre-filled output (several segments share the tile) or a plain store of acc + bias.  WIDE: the
 // 64-channel form (layers with N % 64 == 0).
-template <int BITS, bool ZT, bool WIDE>
+template <int BITS, bool ZT, bool WIDE, bool TO_LDS = false>
 __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, int m0, int g_begin,
-                                               int g_end, bool atomic)
+                                               int g_end, bool atomic, int32_t *lds = nullptr)
 {
     constexpr int NUM = 32 / (BITS + 1);
     constexpr int R = kPlaneRows, J = WIDE ? 64 : 32;
@@ -411,6 +411,15 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
         }
     }
 
+    if (TO_LDS) {
+        // the workgroup's tile buffer lds[channel][pixel of the tile]: consecutive lanes, consecutive
+        // banks
+#pragma unroll
+        for (int j = 0; j < J; ++j)
+#pragma unroll
+            for (int r = 0; r < R; ++r) atomicAdd(lds + j * (R * kWave) + r * kWave + lane, acc[r][j]);
+        return;
+    }
     const int n0 = ntile * J;
 #pragma unroll
     for (int j = 0; j < J; ++j) {
@@ -499,6 +508,68 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void shift_planes_wide_balanced_kernel(const ShiftArgs p)
 {
     planes_balanced_body<BITS, ZT, true>(p);
+}
+
+// Workgroup-cooperative launch of the 64-channel form: the (tile, K group) space is cut into one
+// equal share per workgroup of eight waves; the waves split the K range of a tile among themselves
+// and combine their sums in a 48 KiB LDS tile (LDS atomics cost next to nothing), and the tile goes
+// to the output once: a plain store of sum + bias when the workgroup ran the tile's whole reduction,
+// atomic adds onto the pre-filled output when it shares the tile with a neighbouring workgroup.
+// Global atomics retire one lane per clock and L2 channel and do not overlap the arithmetic of the
+// waves that wait on them; the wave-level shares above issue one per output and share, this launch
+// one per output and workgroup boundary.
+constexpr int kCuWaves = 8;
+
+template <int BITS, bool ZT>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void shift_planes_wide_cu_kernel(
+    const ShiftArgs p)
+{
+    constexpr int PIX = kPlaneRows * kWave;
+    // Two tile buffers, used alternately, and ONE barrier per tile: a wave adds its sums of tile t to
+    // buffer t % 2, waits for the others, writes out and clears its eight channels of that buffer,
+    // and goes on to tile t + 1 in the other buffer; nobody adds to buffer t % 2 again before the
+    // barrier of tile t + 1, which every wave reaches after it has cleared its channels.
+    extern __shared__ int32_t tile_sums[];  // [2][64 channels][192 pixels]
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & (kWave - 1);
+    const int bid = blockIdx.x;
+    const int w = (bid & 7) * (int)(gridDim.x >> 3) + (bid >> 3);  // an XCD takes a contiguous range
+    const long total = (long)p.tiles_m4 * p.tiles_n * p.comm;
+    int it = (int)(w * total / (long)gridDim.x);
+    const int it_end = (int)((w + 1) * total / (long)gridDim.x);
+    for (int i = threadIdx.x; i < 2 * 64 * PIX; i += 512) tile_sums[i] = 0;
+    __syncthreads();
+    int32_t *buf = tile_sums;
+    while (it < it_end) {
+        const int tile = it / p.comm;
+        const int g0 = it - tile * p.comm;
+        int g1 = g0 + (it_end - it);
+        if (g1 > p.comm) g1 = p.comm;
+        const int ntile = tile % p.tiles_n, m0 = (tile / p.tiles_n) * PIX;
+        const int len = g1 - g0;
+        const int wb = g0 + wave * len / kCuWaves, we = g0 + (wave + 1) * len / kCuWaves;
+        if (wb < we) planes_segment<BITS, ZT, true, true>(p, ntile, m0, wb, we, true, buf);
+        __syncthreads();
+        const bool whole = len == p.comm;
+        for (int c = 0; c < 64 / kCuWaves; ++c) {
+            const int j = wave * (64 / kCuWaves) + c, n = ntile * 64 + j;
+            const int32_t add = whole ? p.negcnt[n] + (p.bias ? p.bias[n] : 0) : 0;
+            for (int r = 0; r < kPlaneRows; ++r) {
+                int32_t *cell = buf + j * PIX + r * kWave + lane;
+                const int32_t v = *cell;
+                *cell = 0;
+                const int m = m0 + r * kWave + lane;
+                if (m >= p.M) continue;
+                const int img = m / p.pix_per_img;
+                int32_t *dst = p.y + (size_t)n * p.y_ch_stride + (size_t)img * p.y_img_stride +
+                               (size_t)(m - img * p.pix_per_img) * p.y_pix_stride;
+                if (whole) *dst = v + add;
+                else atomicAdd(dst, v);
+            }
+        }
+        buf = buf == tile_sums ? tile_sums + 64 * PIX : tile_sums;
+        it += len;
+    }
 }
 
 // y = bias[n] + negcnt[n] for the split-K path.  Both output layouts ([img][n][pix] and [m][n])
@@ -628,7 +699,27 @@ static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
         const long iters = (long)a.tiles_m4 * a.tiles_n * a.comm;
         const long fit = (iters / 32) / 8 * 8;
         if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
-        if (WIDE)
+        // Workgroup-cooperative when three or more wave-level shares would meet in a tile (each
+        // costs a round of global atomics on the tile); layers with more tiles than that keep the
+        // wave-level shares, whose segments are longer.  DS_TUNE_CU=0/1 overrides.
+        bool cooperative = WIDE && (long)a.tiles_m4 * a.tiles_n * 3 <= kSlots;
+        if (const char *t = getenv("DS_TUNE_CU")) cooperative = WIDE && atoi(t) > 0;
+        if (cooperative) {
+            // one workgroup of eight waves per compute unit; small layers: >= 8 K groups per wave
+            int cu_blocks = 256;
+            const long cu_fit = (iters / 64) / 8 * 8;
+            if (cu_fit < cu_blocks) cu_blocks = cu_fit < 8 ? 8 : (int)cu_fit;
+            constexpr int kLdsBytes = 2 * 64 * R * kWave * 4;  // above the default 64 KiB limit
+            static bool lds_opted_in = false;
+            if (!lds_opted_in) {
+                hipError_t e = hipFuncSetAttribute((const void *)shift_planes_wide_cu_kernel<BITS, ZT>,
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+                if (e != hipSuccess) return hip_status(e);
+                lds_opted_in = true;
+            }
+            hipLaunchKernelGGL((shift_planes_wide_cu_kernel<BITS, ZT>), dim3(cu_blocks), dim3(512), kLdsBytes,
+                               st, a);
+        } else if (WIDE)
             hipLaunchKernelGGL((shift_planes_wide_balanced_kernel<BITS, ZT>), dim3(blocks), dim3(256), 0, st, a);
         else
             hipLaunchKernelGGL((shift_planes_balanced_kernel<BITS, ZT>), dim3(blocks), dim3(256), 0, st, a);
