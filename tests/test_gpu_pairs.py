@@ -111,3 +111,67 @@ def test_paired_refusals():
         _lib.call("ds_conv2d_paired_i8", None, None, None, None, 1, 1, 3, 3, 32, 1, 1, 1, 1, 2, stream())
     with pytest.raises(_lib.DeepShiftError):
         _lib.call("ds_conv2d_paired_i8", None, None, None, None, 1, 1, 3, 3, 64, 1, 1, 1, 1, 3, stream())
+
+
+# ----------------------------------------------------------------------------- conversion passes
+
+def test_int8_conversion_passes_match_the_int32_ones(rng):
+    from deepshift_amd import kernels
+    g = torch.Generator().manual_seed(5)
+    for (I, Fb) in [(3, 5), (2, 6), (4, 4), (2, 2)]:
+        x = (torch.randn(2, 5, 9, 7, generator=g) * 3).to(DEV)
+        x.view(-1)[:3] = torch.tensor([100.0, -100.0, float("nan")], device=DEV)
+        want = kernels.quantize_pad(x, (1, 2), I, Fb)
+        got = kernels.quantize_pad(x, (1, 2), I, Fb, dtype=torch.int8)
+        assert got.dtype == torch.int8 and torch.equal(got.to(torch.int32), want)
+
+        y = torch.from_numpy(rng.integers(-2 ** 12, 2 ** 12, size=(2, 5, 9, 7)).astype(np.int32)).to(DEV)
+        scale = torch.rand(5, device=DEV) + 0.5
+        shift = torch.randn(5, device=DEV)
+        res = torch.randn(2, 5, 9, 7, generator=g).to(DEV)
+        f32, q32 = kernels.requantize_affine_pad(y, Fb, scale, shift, res, True, (1, 1), I, Fb, True)
+        f8, q8 = kernels.requantize_affine_pad(y, Fb, scale, shift, res, True, (1, 1), I, Fb, True,
+                                               dtype=torch.int8)
+        assert torch.equal(f8, f32) and torch.equal(q8.to(torch.int32), q32)
+
+        f32, q32 = kernels.requantize_affine_maxpool(y, Fb, scale, shift, True, (3, 2, 1), (1, 1), I, Fb, True)
+        f8, q8 = kernels.requantize_affine_maxpool(y, Fb, scale, shift, True, (3, 2, 1), (1, 1), I, Fb, True,
+                                                   dtype=torch.int8)
+        assert torch.equal(f8, f32) and torch.equal(q8.to(torch.int32), q32)
+
+
+def test_int8_conversions_refuse_wider_formats():
+    from deepshift_amd import kernels
+    x = torch.zeros(1, 1, 4, 4, device=DEV)
+    for (I, Fb) in [(16, 16), (1, 5), (5, 4)]:
+        with pytest.raises(_lib.DeepShiftError):
+            kernels.quantize_pad(x, (0, 0), I, Fb, dtype=torch.int8)
+
+
+# ----------------------------------------------------------------------------- through the modules
+
+def test_models_with_8_bit_activations_take_the_int8_kernel_and_keep_their_output(monkeypatch):
+    """ResNet-50 with weight_bits 3 and 3.5 activations: the fused model runs its 64-channel layers on
+    the int8 kernel; switching that off (int32 kernels on the same values) must not change a bit."""
+    from deepshift_amd import convert, fuse, kernels, workloads
+    g = torch.Generator().manual_seed(3)
+    model = workloads.randomize_batchnorm(workloads.ResNet50(), g).eval()
+    model, n = convert.convert_to_shift(model, 1000, 'PS', convert_weights=True, use_kernel=True,
+                                        weight_bits=3, act_integer_bits=3, act_fraction_bits=5)
+    model = model.to(DEV)
+    x = torch.randn(2, 3, 64, 64, generator=g).to(DEV)
+    calls = []
+    real = kernels.conv2d_paired
+    monkeypatch.setattr(kernels, "conv2d_paired", lambda *a, **k: calls.append(1) or real(*a, **k))
+    with torch.no_grad():
+        fused = fuse.fuse_conv_epilogues(model)
+        got = fused(x)
+        unfused = model(x)
+    assert len(calls) == 2 * 53, "every convolution of ResNet-50 has a multiple of 64 channels"
+    monkeypatch.setattr(kernels, "paired_fields", lambda *a, **k: None)
+    with torch.no_grad():
+        want = fuse.fuse_conv_epilogues(model)(x)
+        want_unfused = model(x)
+    assert len(calls) == 2 * 53
+    assert torch.equal(got, want)
+    assert torch.equal(unfused, want_unfused)

@@ -186,3 +186,24 @@ def test_packed_export_rejects_foreign_files(tmp_path):
     torch.save({"format": export.FORMAT, "layers": {"nope": {}}}, tmp_path / "y.pt")
     with pytest.raises(KeyError):
         export.load_packed(workloads.MLP(), str(tmp_path / "y.pt"))
+
+
+def test_int8_kernel_eligibility():
+    """kernels.paired_fields: activations of at most 8 bits (not the one-bit format), a multiple of 64
+    channels, base 0, shift fields of at most 2 bits (packed that narrow, or ternary 6-bit words whose
+    non-zero fields are)."""
+    from deepshift_amd import kernels
+    from deepshift_amd.utils import ConcWeight
+    narrow = ConcWeight(None, 0, 2)
+    assert kernels.paired_fields(narrow, 64, 3, 5) == (2, 2)
+    assert kernels.paired_fields(ConcWeight(None, 0, 1), 128, 2, 6) == (1, 1)
+    assert kernels.paired_fields(narrow, 64, 16, 16) is None      # 32-bit activations
+    assert kernels.paired_fields(narrow, 64, 1, 7) is None        # sign(x) - 1 reaches -2 * 2^F
+    assert kernels.paired_fields(narrow, 64, 4, 5) is None        # 9 bits
+    assert kernels.paired_fields(narrow, 96, 3, 5) is None        # channels
+    assert kernels.paired_fields(ConcWeight(None, -1, 2), 64, 3, 5) is None
+    assert kernels.paired_fields(ConcWeight(None, 0, 3), 64, 3, 5) is None
+    assert kernels.paired_fields(None, 64, 3, 5) is None
+    assert kernels.paired_fields(ConcWeight(None, 0, 6, 2), 64, 3, 5) == (6, 2)
+    assert kernels.paired_fields(ConcWeight(None, 0, 6, 3), 64, 3, 5) is None
+    assert kernels.paired_fields(ConcWeight(None, 0, 6, 0), 64, 3, 5) is None
