@@ -7,8 +7,8 @@ One step = one forward pass of ResNet-18 (every conv and the FC replaced by shif
 weight_bits 5, activations 16.16) over one synthetic batch of 64 x 3 x 224 x 224 that is already
 resident in HBM.  Prints ONE JSON line: images/s for the whole forward pass, the shift kernel's
 rate against the VALU roofline (timed live with HIP events on the launch stream), the 4096^3
-shift GEMM and the 3x3 conv of benchmark configuration 2, and the CPU restatement of the reference's
-shift kernel timed on this host's cores.
+shift GEMM and the 3x3 conv of benchmark configuration 2, ResNet-50 with 8-bit activations
+(configuration 5), and the CPU restatement of the reference's shift kernel timed on this host's cores.
 """
 import argparse
 import json
@@ -187,6 +187,35 @@ def config2(device, reps=10):
     return out
 
 
+def config5(device, steps=5):
+    """Benchmark configuration 5: ResNet-50, batch 128, weight_bits 3 (2-bit shift fields), activations
+    3.5 (8 bits).  Every convolution has a multiple of 64 channels, so the fused pipeline runs them on
+    the int8 kernel (two pixels per register); the FC stays on the int32 kernel."""
+    from deepshift_amd import convert, fuse, workloads
+    g = torch.Generator().manual_seed(0)
+    model = workloads.ResNet50()
+    for m in model.modules():
+        if isinstance(m, (torch.nn.Conv2d, torch.nn.Linear)):
+            torch.nn.init.kaiming_normal_(m.weight, generator=g)
+    workloads.randomize_batchnorm(model, g)
+    model.eval()
+    model, _ = convert.convert_to_shift(model, 1000, 'PS', convert_weights=True, use_kernel=True,
+                                        weight_bits=3, act_integer_bits=3, act_fraction_bits=5)
+    model = model.to(device)
+    x = torch.randn(128, *CHW, generator=g).to(device)
+    with torch.no_grad():
+        fused = fuse.fuse_conv_epilogues(model)
+    sec = time_steps(fused, x, steps, 2)
+    layers = kernel_timings(fused, x, 3)
+    pairs = sum(L["M"] * L["K"] * L["N"] for L in layers)
+    kernel_s = sum(L["seconds"] for L in layers)
+    return dict(workload="ResNet-50, batch 128 x 3x224x224, weight_bits 3, activations 3.5",
+                ms_per_step=sec * 1e3, images_per_s=128 / sec, shift_layers=len(layers),
+                pairs_per_step=pairs, shift_kernel_ms_per_step=kernel_s * 1e3,
+                shift_tpairs_per_s=pairs / kernel_s / 1e12,
+                frac_of_two_instruction_peak=pairs / kernel_s / PEAK_PAIRS)
+
+
 def pmc_target(device):
     """Counter targets for `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`: a plain copy of 64 MiB (reads
     64 MiB, writes 64 MiB: the scale of the counters) and the dominant shift-kernel launch."""
@@ -334,6 +363,7 @@ def main():
 
     peak_cal = None if args.resnet_only else calibrate_valu(device)
     cfg2 = None if args.resnet_only else config2(device)
+    cfg5 = None if args.resnet_only else config5(device)
     result = {
         "metric": "resnet18_bs64_images_per_s",
         "value": BATCH / sec_per_step,
@@ -358,7 +388,8 @@ def main():
         "shift_layers_images_per_s": BATCH / kernel_s,
         "roofline": {
             "bound": "valu",
-            "kernel": "ds::shift_planes_wide_balanced_kernel<4> (17 launches) + ds::shift_kernel (4 launches) per step",
+            "kernel": "ds::shift_planes_wide_cu_kernel<4> (12 launches) + ds::shift_planes_wide_balanced_kernel<4> "
+                      "(5 launches) + ds::shift_kernel (4 launches) per step",
             "achieved": pairs / kernel_s / 1e12,
             "peak": PEAK_PAIRS / 1e12,
             "unit": "Tpair/s",
@@ -379,6 +410,7 @@ def main():
             "algorithmic_bytes_per_step": alg_bytes,
         },
         "config2": cfg2,
+        "config5": cfg5,
         "shift_gemm_gops": cfg2["gemm_4096"]["gops"] if cfg2 else None,
     }
     if not args.no_cpu:
