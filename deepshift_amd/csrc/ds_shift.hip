@@ -518,18 +518,20 @@ void shift_planes_wide_balanced_kernel(const ShiftArgs p)
 // Global atomics retire one lane per clock and L2 channel and do not overlap the arithmetic of the
 // waves that wait on them; the wave-level shares above issue one per output and share, this launch
 // one per output and workgroup boundary.
-constexpr int kCuWaves = 8;
-
-template <int BITS, bool ZT>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void shift_planes_wide_cu_kernel(
-    const ShiftArgs p)
+// WAVES = 8: one workgroup per compute unit, two tile buffers used alternately and one barrier per
+// tile.  WAVES = 4: two workgroups per compute unit, one buffer each and two barriers per tile; the two
+// waves of a SIMD then belong to different workgroups and are not held at the same barrier.
+template <int BITS, bool ZT, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void shift_planes_wide_cu_kernel(const ShiftArgs p)
 {
     constexpr int PIX = kPlaneRows * kWave;
-    // Two tile buffers, used alternately, and ONE barrier per tile: a wave adds its sums of tile t to
-    // buffer t % 2, waits for the others, writes out and clears its eight channels of that buffer,
-    // and goes on to tile t + 1 in the other buffer; nobody adds to buffer t % 2 again before the
-    // barrier of tile t + 1, which every wave reaches after it has cleared its channels.
-    extern __shared__ int32_t tile_sums[];  // [2][64 channels][192 pixels]
+    constexpr int BUFFERS = WAVES == 8 ? 2 : 1;
+    // With two buffers: a wave adds its sums of tile t to buffer t % 2, waits for the others, writes
+    // out and clears its channels of that buffer, and goes on to tile t + 1 in the other buffer;
+    // nobody adds to buffer t % 2 again before the barrier of tile t + 1, which every wave reaches
+    // after it has cleared its channels.  With one buffer a second barrier follows the clearing.
+    extern __shared__ int32_t tile_sums[];  // [BUFFERS][64 channels][192 pixels]
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & (kWave - 1);
     const int bid = blockIdx.x;
@@ -537,7 +539,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const long total = (long)p.tiles_m4 * p.tiles_n * p.comm;
     int it = (int)(w * total / (long)gridDim.x);
     const int it_end = (int)((w + 1) * total / (long)gridDim.x);
-    for (int i = threadIdx.x; i < 2 * 64 * PIX; i += 512) tile_sums[i] = 0;
+    for (int i = threadIdx.x; i < BUFFERS * 64 * PIX; i += WAVES * 64) tile_sums[i] = 0;
     __syncthreads();
     int32_t *buf = tile_sums;
     while (it < it_end) {
@@ -547,12 +549,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         if (g1 > p.comm) g1 = p.comm;
         const int ntile = tile % p.tiles_n, m0 = (tile / p.tiles_n) * PIX;
         const int len = g1 - g0;
-        const int wb = g0 + wave * len / kCuWaves, we = g0 + (wave + 1) * len / kCuWaves;
+        const int wb = g0 + wave * len / WAVES, we = g0 + (wave + 1) * len / WAVES;
         if (wb < we) planes_segment<BITS, ZT, true, true>(p, ntile, m0, wb, we, true, buf);
         __syncthreads();
         const bool whole = len == p.comm;
-        for (int c = 0; c < 64 / kCuWaves; ++c) {
-            const int j = wave * (64 / kCuWaves) + c, n = ntile * 64 + j;
+        for (int c = 0; c < 64 / WAVES; ++c) {
+            const int j = wave * (64 / WAVES) + c, n = ntile * 64 + j;
             const int32_t add = whole ? p.negcnt[n] + (p.bias ? p.bias[n] : 0) : 0;
             for (int r = 0; r < kPlaneRows; ++r) {
                 int32_t *cell = buf + j * PIX + r * kWave + lane;
@@ -567,9 +569,30 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 else atomicAdd(dst, v);
             }
         }
-        buf = buf == tile_sums ? tile_sums + 64 * PIX : tile_sums;
+        if (BUFFERS == 2) buf = buf == tile_sums ? tile_sums + 64 * PIX : tile_sums;
+        else __syncthreads();
         it += len;
     }
+}
+
+template <int BITS, bool ZT, int WAVES>
+static int launch_planes_cu(const ShiftArgs &a, long iters, hipStream_t st)
+{
+    constexpr int kLdsBytes = (WAVES == 8 ? 2 : 1) * 64 * kPlaneRows * kWave * 4;
+    static bool lds_opted_in = false;  // 96 KiB is above the default limit of a workgroup
+    if (!lds_opted_in) {
+        hipError_t e = hipFuncSetAttribute((const void *)shift_planes_wide_cu_kernel<BITS, ZT, WAVES>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+        if (e != hipSuccess) return hip_status(e);
+        lds_opted_in = true;
+    }
+    // one workgroup per 8 wave slots (2 waves per SIMD); small layers: >= 8 K groups per wave
+    int blocks = kPlaneSlotsWide / WAVES;
+    const long fit = (iters / (8 * WAVES)) / 8 * 8;
+    if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
+    hipLaunchKernelGGL((shift_planes_wide_cu_kernel<BITS, ZT, WAVES>), dim3(blocks), dim3(WAVES * 64), kLdsBytes,
+                       st, a);
+    return launch_status();
 }
 
 // y = bias[n] + negcnt[n] for the split-K path.  Both output layouts ([img][n][pix] and [m][n])
@@ -699,26 +722,22 @@ static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
         const long iters = (long)a.tiles_m4 * a.tiles_n * a.comm;
         const long fit = (iters / 32) / 8 * 8;
         if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
-        // Workgroup-cooperative when three or more wave-level shares would meet in a tile (each
-        // costs a round of global atomics on the tile); layers with more tiles than that keep the
-        // wave-level shares, whose segments are longer.  DS_TUNE_CU=0/1 overrides.
-        bool cooperative = WIDE && (long)a.tiles_m4 * a.tiles_n * 3 <= kSlots;
-        if (const char *t = getenv("DS_TUNE_CU")) cooperative = WIDE && atoi(t) > 0;
+        // Workgroup-cooperative (four waves per workgroup) when a wave's quarter of a tile's reduction
+        // is long enough to carry the extra segment ends: from 64 K groups per tile.  Short reductions
+        // over many tiles (stems, 1x1 layers) keep the wave-level shares.  DS_TUNE_CU=0 / 4 / 8
+        // overrides (8: eight waves per workgroup).
+        bool cooperative = WIDE && a.comm >= 64;
+        int cu_waves = 4;
+        if (const char *t = getenv("DS_TUNE_CU")) {
+            cooperative = WIDE && atoi(t) > 0;
+            cu_waves = atoi(t) == 8 ? 8 : 4;
+        }
         if (cooperative) {
-            // one workgroup of eight waves per compute unit; small layers: >= 8 K groups per wave
-            int cu_blocks = 256;
-            const long cu_fit = (iters / 64) / 8 * 8;
-            if (cu_fit < cu_blocks) cu_blocks = cu_fit < 8 ? 8 : (int)cu_fit;
-            constexpr int kLdsBytes = 2 * 64 * R * kWave * 4;  // above the default 64 KiB limit
-            static bool lds_opted_in = false;
-            if (!lds_opted_in) {
-                hipError_t e = hipFuncSetAttribute((const void *)shift_planes_wide_cu_kernel<BITS, ZT>,
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-                if (e != hipSuccess) return hip_status(e);
-                lds_opted_in = true;
+            if constexpr (WIDE) {
+                const int rc = cu_waves == 4 ? launch_planes_cu<BITS, ZT, 4>(a, iters, st)
+                                             : launch_planes_cu<BITS, ZT, 8>(a, iters, st);
+                if (rc) return rc;
             }
-            hipLaunchKernelGGL((shift_planes_wide_cu_kernel<BITS, ZT>), dim3(cu_blocks), dim3(512), kLdsBytes,
-                               st, a);
         } else if (WIDE)
             hipLaunchKernelGGL((shift_planes_wide_balanced_kernel<BITS, ZT>), dim3(blocks), dim3(256), 0, st, a);
         else
