@@ -305,6 +305,8 @@ def main():
     ap.add_argument("--layers", action="store_true", help="per-layer table on stderr")
     ap.add_argument("--resnet-only", action="store_true",
                     help="skip config 2 and the VALU calibration (clean kernel-trace profiles)")
+    ap.add_argument("--config5-only", action="store_true",
+                    help="only benchmark configuration 5 (ResNet-50, 8-bit activations); prints its JSON object")
     ap.add_argument("--pmc-target", action="store_true",
                     help="only launch the counter targets: a 64 MiB copy kernel and the dominant shift "
                          "kernel (ResNet-18 layer1 3x3 conv, batch 64), 3 times each")
@@ -318,6 +320,9 @@ def main():
 
     if args.pmc_target:
         pmc_target(device)
+        return
+    if args.config5_only:
+        print(json.dumps(config5(device, args.steps)), flush=True)
         return
 
     from deepshift_amd import workloads
@@ -388,20 +393,20 @@ def main():
         "shift_layers_images_per_s": BATCH / kernel_s,
         "roofline": {
             "bound": "valu",
-            "kernel": "ds::shift_planes_wide_cu_kernel<4> (12 launches) + ds::shift_planes_wide_balanced_kernel<4> "
-                      "(5 launches) + ds::shift_kernel (4 launches) per step",
+            "kernel": "ds::shift_planes_wide_cu_kernel<4> (16 launches) + ds::shift_planes_wide_balanced_kernel<4> "
+                      "(1 launch) + ds::shift_kernel (4 launches) per step",
             "achieved": pairs / kernel_s / 1e12,
             "peak": PEAK_PAIRS / 1e12,
             "unit": "Tpair/s",
             "frac": pairs / kernel_s / PEAK_PAIRS,
             # HBM bytes of one launch of the dominant shape (layer1 3x3 conv, 8 of the 21 launches are
-            # this size): 65.2 MB read + 155.5 MB of atomic partial sums, from the FETCH_SIZE /
-            # WRITE_SIZE runs summarised in profiles/shift_kernel_layer1_conv_counters.md
-            # (106.6 MB algorithmic)
-            "traffic": 220.7e6,
+            # this size): 100.4 MB read + 82.7 MB written (tiles shared by two workgroups are combined
+            # with atomic adds), from the FETCH_SIZE / WRITE_SIZE runs summarised in
+            # profiles/shift_kernel_layer1_conv_counters.md (106.6 MB algorithmic)
+            "traffic": 183.1e6,
             # vector instructions the dominant kernel issues per pair (SQ_INSTS_VALU, same profile):
             # `peak` prices a pair at 2 instructions, so its fraction can exceed 1
-            "valu_instr_per_pair": 1.29,
+            "valu_instr_per_pair": 1.31,
             "avg_launch_us": kernel_s / len(layers) * 1e6,
             "peak_calibrated": peak_cal / 1e12 if peak_cal else None,
             "frac_of_calibrated": pairs / kernel_s / peak_cal if peak_cal else None,
