@@ -175,3 +175,23 @@ def test_models_with_8_bit_activations_take_the_int8_kernel_and_keep_their_outpu
     assert len(calls) == 2 * 53
     assert torch.equal(got, want)
     assert torch.equal(unfused, want_unfused)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_int8_convolutions(oracle, seed):
+    rng = np.random.default_rng(4000 + seed)
+    bits = int(rng.integers(1, 3))
+    FH, FW = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+    sh, sw = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+    Nb = int(rng.integers(1, 9))
+    C = int(rng.choice([1, 3, 16, 37, 64, 150]))
+    O = int(rng.choice([64, 128, 192]))
+    Hp, Wp = FH + int(rng.integers(0, 30)), FW + int(rng.integers(0, 30))
+    x8 = random_int8(rng, (Nb, C, Hp, Wp))
+    s, sign = random_codes(rng, (O, C, FH, FW), max_s=2 ** bits - 1)
+    bias = rng.integers(-2 ** 20, 2 ** 20, size=O).astype(np.int32) if seed % 2 else None
+    w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)
+    want = oracle.conv2d(x8.astype(np.int32), -s, sign, bias, (sh, sw), nthreads=NTHREADS)
+    blob = abi_tile_paired(w, O, C, FH, FW, bits, bits)
+    got = abi_conv_paired(x8, blob, bias, O, FH, FW, (sh, sw), bits)
+    np.testing.assert_array_equal(got, want, err_msg=str((bits, Nb, C, Hp, Wp, O, FH, FW, sh, sw)))
