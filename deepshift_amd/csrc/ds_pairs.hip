@@ -17,7 +17,9 @@
 // (64 + 3*2^BITS + 1) / 128 vector instructions per shift-add term: 0.60 for 2-bit fields against
 // 1.05 of the int32 shift-plane kernel.  After at most 255 reduction indices the halves are
 // widened and added to the int32 output (atomically when the output is shared), which is why a call
-// of the generated loop never runs more than kChunk K groups.  The result is the int32 kernel's,
+// of the generated loop never runs more than PairArgs::chunk K groups (the caller may vouch for a
+// smaller bound on |x| -- post-ReLU activations of the 3.5 format stay below 97 -- and get longer
+// chunks).  The result is the int32 kernel's,
 // bit for bit.
 #include "ds_common.h"
 #include <cstdlib>
@@ -44,6 +46,7 @@ struct PairArgs {
     int tiles_m, tiles_n;
     int tile_begin, tile_end;  // tiles of this launch (index = pixel tile * tiles_n + channel tile)
     int whole_tiles;           // workgroup shares end on tile boundaries
+    int chunk;                 // K groups per call of the asm loop (see pair_chunk)
     int blocks_per_xcd;
     int atomic_out;
     uint32_t y_elems;
@@ -57,8 +60,9 @@ constexpr int kPairRows = 3;               // accumulator rows per lane, two pix
 constexpr int kPairPixels = 6 * kWave;     // pixels of a tile
 constexpr int kPairSlots = 2048;           // wave slots of the machine at 2 waves per SIMD
 
-// K groups per call of the asm loop: at most 255 reduction indices (255 * 128 < 2^15)
-__host__ __device__ constexpr int pair_chunk(int bits) { return 255 / codes_per_word(bits); }
+// K groups per call of the asm loop: as many reduction indices as keep a sum of terms of magnitude
+// <= x_bound within 16 bits (255 for x_bound = 128: 255 * 128 < 2^15)
+inline int pair_chunk(int bits, int x_bound) { return (32767 / x_bound) / codes_per_word(bits); }
 
 #define DS_PAIRS_OPERANDS                                                                         \
     : "+{v[64:95]}"(a[0]), "+{v[96:127]}"(a[1]), "+{v[128:159]}"(a[2]), "+{v[160:191]}"(a[3]),    \
@@ -83,7 +87,7 @@ __device__ __forceinline__ void pairs_main_loop<2>(v32i (&a)[6], const uint32_t 
     asm volatile(DS_PAIRS_ASM_B2 DS_PAIRS_OPERANDS : DS_PAIRS_CLOBBERS_B2);
 }
 
-// K groups [g_begin, g_end) (at most pair_chunk of them) of the tile made of the 64 channels of
+// K groups [g_begin, g_end) (at most PairArgs::chunk of them) of the tile made of the 64 channels of
 // `ntile` and the 384 pixels from m0.
 // OUT selects where the widened sums go: kStore (y = sum + bias), kAtomic (atomic add to a
 // pre-filled y) or kLds (add to the workgroup's tile buffer lds[channel][pixel of the tile]).
@@ -211,7 +215,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int g_begin = it - (tile - p.tile_begin) * p.comm;
         int g_end = g_begin + (it_end - it);
         if (g_end > p.comm) g_end = p.comm;
-        if (g_end > g_begin + pair_chunk(BITS)) g_end = g_begin + pair_chunk(BITS);
+        if (g_end > g_begin + p.chunk) g_end = g_begin + p.chunk;
         const int ntile = tile % p.tiles_n;
         pairs_segment<BITS, kAtomic>(p, ntile, (tile / p.tiles_n) * kPairPixels, g_begin, g_end, nullptr);
         it += g_end - g_begin;
@@ -257,8 +261,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         __syncthreads();
         const int len = g1 - g0;
         const int wb = g0 + wave * len / kPairCuWaves, we = g0 + (wave + 1) * len / kPairCuWaves;
-        for (int g = wb; g < we; g += pair_chunk(BITS)) {
-            const int ge = g + pair_chunk(BITS) < we ? g + pair_chunk(BITS) : we;
+        for (int g = wb; g < we; g += p.chunk) {
+            const int ge = g + p.chunk < we ? g + p.chunk : we;
             pairs_segment<BITS, kLds>(p, ntile, m0, g, ge, tile_sums);
         }
         __syncthreads();
@@ -327,10 +331,13 @@ static int launch_pairs(PairArgs a, hipStream_t st)
     a.tile_end = (int)tiles;
     // regime: 1 = one tile per wave (single chunk, plain stores), 2 = workgroup-cooperative,
     // 0 = wave-level shares with global atomics
-    int regime = a.comm <= pair_chunk(BITS) ? 1 : 2;
+    // A wave that has a SIMD to itself issues at well under half the rate of two that share one, so
+    // with fewer tiles than wave slots only short reductions (where the cooperative split would leave
+    // a wave a group or two) stay one tile per wave.
+    int regime = (a.comm <= a.chunk && (tiles >= kPairSlots || a.comm < 16)) ? 1 : 2;
     if (const char *t = getenv("DS_TUNE_SPLIT")) {
         regime = atoi(t);
-        if (regime == 1 && a.comm > pair_chunk(BITS)) regime = 0;
+        if (regime == 1 && a.comm > a.chunk) regime = 0;
     }
     if (regime == 1) {
         // Whole rounds of wave slots run one tile per wave.  A last round that would fill less than
@@ -455,11 +462,11 @@ DS_EXPORT int ds_tile_weights_paired_i32(const int32_t *w_ref, void *paired, int
 
 DS_EXPORT int ds_conv2d_paired_i8(const int8_t *x, const void *paired, const int32_t *bias, int32_t *y,
                                   int Nb, int C, int Hp, int Wp, int O, int FH, int FW, int sh, int sw,
-                                  int field_bits, ds_stream_t stream)
+                                  int field_bits, int x_bound, ds_stream_t stream)
 {
     int rc = check_paired(O, C, FH, FW, field_bits);
     if (rc) return rc;
-    if (Nb < 0 || sh < 1 || sw < 1 || Hp < FH || Wp < FW) return DS_EINVAL;
+    if (Nb < 0 || sh < 1 || sw < 1 || Hp < FH || Wp < FW || x_bound < 1 || x_bound > 128) return DS_EINVAL;
     const int OH = (Hp - FH) / sh + 1, OW = (Wp - FW) / sw + 1;
     const size_t M = (size_t)Nb * OH * OW;
     if (M == 0 || O == 0) return DS_OK;
@@ -482,6 +489,7 @@ DS_EXPORT int ds_conv2d_paired_i8(const int8_t *x, const void *paired, const int
     a.y_elems = (uint32_t)(M * O);
     a.x_plane = Hp * Wp; a.x_row = Wp;
     a.FH = FH; a.FW = FW;
+    a.chunk = pair_chunk(field_bits, x_bound);
     if (K == 0) {
         // no terms: the output is the bias
         a.tiles_m = 0;

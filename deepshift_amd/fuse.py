@@ -39,6 +39,7 @@ class FusedConv2dShift(nn.Module):
         self.conv = conv
         self.relu = relu
         self.prequantized = False  # the input is this layer's int32 padded input, made by its producer
+        self.input_nonneg = False  # ... and that producer ends in a ReLU
         self.emit = None           # (padding, I, F, want_float, dtype) of the consumers' input to produce
         self.pool = None           # (kernel, stride, padding) of a max pooling that follows the ReLU
         if bn is not None:
@@ -62,7 +63,8 @@ class FusedConv2dShift(nn.Module):
         elif conv.conc_weight is None:
             modules.pack_module_weights(conv)
         return modules.conv_kernel_forward(conv, input, conv.conc_weight, self.scale, self.shift,
-                                           residual, self.relu, self.prequantized, self.emit, self.pool)
+                                           residual, self.relu, self.prequantized, self.emit, self.pool,
+                                           self.input_nonneg)
 
 
 class _Tracer(fx.Tracer):
@@ -234,3 +236,4 @@ def _hand_off_fixed_point(gm):
         for user in takers:
             user.args = (q,) + tuple(user.args[1:])
             fused(user).prequantized = True
+            fused(user).input_nonneg = bool(producer.relu)

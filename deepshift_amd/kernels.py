@@ -412,9 +412,11 @@ def conv2d_tiled(x_padded, tiled, bias, O, kernel_size, stride, bits, base=0):
     return out
 
 
-def conv2d_paired(x_padded, paired, bias, O, kernel_size, stride, field_bits):
+def conv2d_paired(x_padded, paired, bias, O, kernel_size, stride, field_bits, x_bound=128):
     """Shift convolution on an already padded int8 NCHW input and the blob of
-    :func:`tile_weights_paired`; the int32 result of :func:`conv2d_tiled` on the same values."""
+    :func:`tile_weights_paired`; the int32 result of :func:`conv2d_tiled` on the same values.
+    ``x_bound``: a bound on ``|x|`` that the caller vouches for (128 always holds); a smaller one lets
+    the kernel widen its 16-bit sums less often."""
     if x_padded.dtype != torch.int8 or not x_padded.is_cuda or x_padded.dim() != 4:
         raise TypeError("x_padded must be a 4-D int8 GPU tensor")
     x_padded = x_padded.contiguous()
@@ -427,7 +429,8 @@ def conv2d_paired(x_padded, paired, bias, O, kernel_size, stride, field_bits):
     out = torch.empty([Nb, O, OH, OW], dtype=torch.int32, device=x_padded.device)
     with _Timed("conv", Nb * OH * OW, C * FH * FW, O, x_padded.device):
         _lib.call("ds_conv2d_paired_i8", _lib.ptr(x_padded), _lib.ptr(paired), _lib.ptr(bias), _lib.ptr(out),
-                  Nb, C, Hp, Wp, O, FH, FW, sh, sw, int(field_bits), _lib.current_stream(x_padded.device))
+                  Nb, C, Hp, Wp, O, FH, FW, sh, sw, int(field_bits), int(x_bound),
+                  _lib.current_stream(x_padded.device))
     return out
 
 

@@ -197,7 +197,7 @@ def _circular_pad(x, padding):
 
 
 def conv_kernel_forward(module, input, conc_weight, scale=None, shift=None, residual=None, relu=False,
-                        prequantized=False, emit=None, pool=None):
+                        prequantized=False, emit=None, pool=None, input_nonneg=False):
     """Fixed-point shift convolution of a float NCHW input (modules.py:152-162,317-337).
 
     ``scale``/``shift`` (per output channel), ``residual`` and ``relu`` describe what follows the
@@ -209,7 +209,9 @@ def conv_kernel_forward(module, input, conc_weight, scale=None, shift=None, resi
     produce that form of the result for the next shift convolution (a fifth element gives its dtype:
     int8 for a consumer on the int8 kernel); the return value is then ``(out, q)``, or ``q`` alone when
     ``want_float`` is false.  ``pool = (kernel, stride, padding)``:
-    a max pooling follows the ReLU (no residual) and runs in the same pass."""
+    a max pooling follows the ReLU (no residual) and runs in the same pass.  ``input_nonneg``: the
+    producer of a prequantized input vouches that it is the output of a ReLU (the int8 kernel then
+    knows a tighter bound on the activations and widens its 16-bit sums less often)."""
     if not module.use_cuda:
         kernels._no_cpu_kernel()
     if module.dilation != (1, 1) or module.groups != 1:
@@ -234,8 +236,11 @@ def conv_kernel_forward(module, input, conc_weight, scale=None, shift=None, resi
             raise ValueError("this layer has no int8 kernel; hand it int32 activations")
         blob = kernels._paired_of(conc_weight, fields, module.out_channels, module.in_channels,
                                   module.kernel_size[0], module.kernel_size[1])
+        # round_to_fixed clamps to [-2^(I-1), 2^(I-1) - 1] (utils.py:7-21): |x| <= 2^(I+F-1), and after
+        # a ReLU x <= (2^(I-1) - 1) * 2^F
+        bound = (2 ** (I - 1) - 1) * 2 ** Fb if (prequantized and input_nonneg) else 2 ** (I + Fb - 1)
         out = kernels.conv2d_paired(xq, blob, bias, module.out_channels, module.kernel_size, module.stride,
-                                    fields[1])
+                                    fields[1], max(1, bound))
     else:
         tiled = kernels._tiled_of(conc_weight, module.out_channels, module.in_channels,
                                   module.kernel_size[0], module.kernel_size[1])

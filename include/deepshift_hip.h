@@ -103,10 +103,15 @@ int ds_tile_weights_paired_i32(const int32_t *w_ref, void *paired, int N, int C,
 /* Conv2dShift forward on int8 activations: ds_conv2d_tiled_i32 (DEEP_SHIFT_CONV,
  * kernels/cuda/shift_cuda.cpp:41-53) with x int8 [Nb][C][Hp][Wp], already padded, and the blob of
  * ds_tile_weights_paired_i32.  y int32 [Nb][O][OH][OW].  DS_EINVAL when O % 64 != 0, DS_EBITS when
- * field_bits is not 1 or 2. */
+ * field_bits is not 1 or 2.
+ * x_bound (1..128): the caller vouches that every |x| <= x_bound.  128 is always true; a smaller
+ * bound lets the kernel run 32767 / x_bound reduction indices between two widenings of its 16-bit
+ * sums -- e.g. 96 for the output of a ReLU in the 3.5 format, whose round-to-fixed clamp
+ * (utils.py:7-21) keeps the values in [0, 96]: a K = 256 layer is then a single chunk.  A value
+ * beyond the bound makes the sums wrap: results are then wrong, nothing else. */
 int ds_conv2d_paired_i8(const int8_t *x, const void *paired, const int32_t *bias, int32_t *y, int Nb,
                         int C, int Hp, int Wp, int O, int FH, int FW, int sh, int sw, int field_bits,
-                        ds_stream_t stream);
+                        int x_bound, ds_stream_t stream);
 
 /* The conversion passes with an int8 result, for that kernel's input: ds_quantize_pad_f32_i32,
  * ds_requantize_affine_pad_i32 and ds_requantize_affine_maxpool_i32 with q int8, always in mode

@@ -25,7 +25,7 @@ def abi_tile_paired(w_ref, O, C, FH, FW, ref_bits, field_bits):
     return blob
 
 
-def abi_conv_paired(x8, blob, bias, O, FH, FW, stride, field_bits):
+def abi_conv_paired(x8, blob, bias, O, FH, FW, stride, field_bits, x_bound=128):
     Nb, C, Hp, Wp = x8.shape
     sh, sw = stride
     OH, OW = (Hp - FH) // sh + 1, (Wp - FW) // sw + 1
@@ -36,7 +36,7 @@ def abi_conv_paired(x8, blob, bias, O, FH, FW, stride, field_bits):
     xd = torch.from_numpy(x8).to(DEV)
     bd = None if bias is None else dev(bias)
     _lib.call("ds_conv2d_paired_i8", _lib.ptr(xd), _lib.ptr(blob), _lib.ptr(bd), ctypes.c_void_p(y.data_ptr()),
-              Nb, C, Hp, Wp, O, FH, FW, sh, sw, field_bits, stream())
+              Nb, C, Hp, Wp, O, FH, FW, sh, sw, field_bits, x_bound, stream())
     torch.cuda.synchronize()
     host = ybuf.cpu().numpy()
     assert (host[:guard] == 0x5A5A5A5A).all() and (host[guard + total:] == 0x5A5A5A5A).all(), \
@@ -108,9 +108,37 @@ def test_paired_refusals():
     assert L.ds_paired_bytes(65, 10, 2) == 0
     assert L.ds_paired_bytes(64, 10, 3) == 0
     with pytest.raises(_lib.DeepShiftError):
-        _lib.call("ds_conv2d_paired_i8", None, None, None, None, 1, 1, 3, 3, 32, 1, 1, 1, 1, 2, stream())
+        _lib.call("ds_conv2d_paired_i8", None, None, None, None, 1, 1, 3, 3, 32, 1, 1, 1, 1, 2, 128, stream())
     with pytest.raises(_lib.DeepShiftError):
-        _lib.call("ds_conv2d_paired_i8", None, None, None, None, 1, 1, 3, 3, 64, 1, 1, 1, 1, 3, stream())
+        _lib.call("ds_conv2d_paired_i8", None, None, None, None, 1, 1, 3, 3, 64, 1, 1, 1, 1, 3, 128, stream())
+    for bound in (0, 129):
+        with pytest.raises(_lib.DeepShiftError):
+            _lib.call("ds_conv2d_paired_i8", None, None, None, None, 1, 1, 3, 3, 64, 1, 1, 1, 1, 2, bound, stream())
+
+
+@pytest.mark.parametrize("bits", [1, 2])
+@pytest.mark.parametrize("bound", [96, 17, 1])
+def test_paired_vouched_bound_lengthens_the_chunks(oracle, rng, bits, bound):
+    """Activations within [-bound, bound], every one at the bound with the same sign where it hurts
+    most: 32767 // bound reduction indices per chunk must still not overflow a half."""
+    O, FH, FW = 64, 1, 1
+    for C in (256, 32767 // bound, 32767 // bound + 7, 1200):
+        C = min(C, 4000)
+        for fill, sgn in ((bound, 1), (bound, -1), (-bound, 1), (-bound, -1)):
+            x8 = np.full((1, C, 20, 21), fill, np.int8)
+            s = np.zeros((O, C, 1, 1), np.int32)
+            sign = np.full((O, C, 1, 1), sgn, np.int32)
+            w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)
+            want = oracle.conv2d(x8.astype(np.int32), -s, sign, None, (1, 1), nthreads=NTHREADS)
+            blob = abi_tile_paired(w, O, C, 1, 1, bits, bits)
+            got = abi_conv_paired(x8, blob, None, O, 1, 1, (1, 1), bits, bound)
+            np.testing.assert_array_equal(got, want, err_msg=str((C, fill, sgn)))
+    x8 = rng.integers(-bound, bound + 1, size=(3, 300, 9, 9)).astype(np.int8)
+    s, sign = random_codes(rng, (128, 300, 3, 3), max_s=2 ** bits - 1)
+    w, _ = oracle.pack_words(s.reshape(128, -1), sign.reshape(128, -1), bits)
+    want = oracle.conv2d(x8.astype(np.int32), -s, sign, None, (1, 1), nthreads=NTHREADS)
+    blob = abi_tile_paired(w, 128, 300, 3, 3, bits, bits)
+    np.testing.assert_array_equal(abi_conv_paired(x8, blob, None, 128, 3, 3, (1, 1), bits, bound), want)
 
 
 # ----------------------------------------------------------------------------- conversion passes
