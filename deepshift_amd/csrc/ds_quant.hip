@@ -251,6 +251,41 @@ __global__ void requantize_affine_pad_kernel(const int32_t *__restrict__ y, floa
     }
 }
 
+// The same without padding (ph = pw = 0: q has the layout of y), four consecutive elements of one
+// (image, channel) plane per thread: 16-byte loads and stores (4-byte for an int8 q).  Needs
+// HW % 4 == 0 and 16-byte aligned y, out, residual (q: 16 / 4-byte aligned).
+template <typename Q>
+__global__ void requantize_affine_flat4_kernel(const int32_t *__restrict__ y, float *__restrict__ out,
+                                               Q *__restrict__ q, const float *__restrict__ scale,
+                                               const float *__restrict__ shift,
+                                               const float *__restrict__ residual, uint32_t total4, int C,
+                                               float inv, int relu, QuantSpec spec, FastDiv by_plane4,
+                                               FastDiv by_channels)
+{
+    for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < total4; i += gridDim.x * blockDim.x) {
+        const uint32_t plane = div_by(i, by_plane4);  // by_plane4 divides by HW / 4
+        const uint32_t c = plane - div_by(plane, by_channels) * (uint32_t)C;
+        const float a = scale ? scale[c] : 1.0f, b = shift ? shift[c] : 0.0f;
+        const int4 v = ((const int4 *)y)[i];
+        float4 r = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (residual) r = ((const float4 *)residual)[i];
+        float4 f;
+        f.x = affine_one(v.x, inv, a, b, residual ? &r.x : nullptr, relu);
+        f.y = affine_one(v.y, inv, a, b, residual ? &r.y : nullptr, relu);
+        f.z = affine_one(v.z, inv, a, b, residual ? &r.z : nullptr, relu);
+        f.w = affine_one(v.w, inv, a, b, residual ? &r.w : nullptr, relu);
+        if (out) ((float4 *)out)[i] = f;
+        const int32_t q0 = quantize_one(f.x, spec), q1 = quantize_one(f.y, spec), q2 = quantize_one(f.z, spec),
+                      q3 = quantize_one(f.w, spec);
+        if (sizeof(Q) == 1) {
+            ((uint32_t *)q)[i] = ((uint32_t)q0 & 0xffu) | (((uint32_t)q1 & 0xffu) << 8) |
+                                 (((uint32_t)q2 & 0xffu) << 16) | ((uint32_t)q3 << 24);
+        } else {
+            ((int4 *)q)[i] = make_int4(q0, q1, q2, q3);
+        }
+    }
+}
+
 // The same with a max pooling between the affine/ReLU and the conversion (the ResNet stem):
 // f[oh][ow] = max over the pk x pk window (stride ps, implicit -inf padding pp, as nn.MaxPool2d) of
 // affine_one(y); one thread per element of the padded int32 output (or of out when q is NULL, with
@@ -476,6 +511,14 @@ static int requantize_affine_pad_any(const int32_t *y, float *out, Q *q, const f
     if (total == 0) return DS_OK;
     if (total * (long)sizeof(Q) >= (1L << 31) || (long)Nb * C * H * W * 4 >= (1L << 31)) return DS_ETOOLARGE;
     if (!q || (!y && (long)Nb * C * H * W > 0)) return DS_EINVAL;
+    const uintptr_t align16 = (uintptr_t)y | (uintptr_t)out | (uintptr_t)residual | (sizeof(Q) == 4 ? (uintptr_t)q : 0);
+    if (ph == 0 && pw == 0 && (H * W) % 4 == 0 && (align16 & 15) == 0 && ((uintptr_t)q & 3) == 0) {
+        hipLaunchKernelGGL((requantize_affine_flat4_kernel<Q>), dim3(grid_for(total / 4)), dim3(256), 0,
+                           (hipStream_t)stream, y, out, q, scale, shift, residual, (uint32_t)(total / 4), C,
+                           ldexpf(1.0f, -F_in), relu, make_spec(I, F, mode), fast_div((uint32_t)(H * W / 4)),
+                           fast_div((uint32_t)C));
+        return launch_status();
+    }
     hipLaunchKernelGGL((requantize_affine_pad_kernel<Q>), dim3(grid_for(total)), dim3(256), 0,
                        (hipStream_t)stream, y, out, q, scale, shift, residual, (uint32_t)(Nb * C), C, H, W,
                        ph, pw, ldexpf(1.0f, -F_in), relu, make_spec(I, F, mode),

@@ -161,6 +161,21 @@ def test_int8_conversion_passes_match_the_int32_ones(rng):
         f8, q8 = kernels.requantize_affine_pad(y, Fb, scale, shift, res, True, (1, 1), I, Fb, True,
                                                dtype=torch.int8)
         assert torch.equal(f8, f32) and torch.equal(q8.to(torch.int32), q32)
+        # unpadded, plane size a multiple of 4: the four-elements-per-thread pass, against the padded
+        # one's interior and the two separate calls
+        y4 = torch.from_numpy(rng.integers(-2 ** 12, 2 ** 12, size=(3, 5, 8, 6)).astype(np.int32)).to(DEV)
+        res4 = torch.randn(3, 5, 8, 6, generator=g).to(DEV)
+        for residual, relu, want_float in [(res4, True, True), (None, False, False), (res4, False, True)]:
+            want_f = kernels.dequantize_affine(y4, Fb, scale, shift, residual, relu)
+            want_q = kernels.quantize_pad(want_f, (0, 0), I, Fb)
+            for dtype in (torch.int32, torch.int8):
+                f, q = kernels.requantize_affine_pad(y4, Fb, scale, shift, residual, relu, (0, 0), I, Fb,
+                                                     want_float, dtype=dtype)
+                assert q.dtype == dtype and torch.equal(q.to(torch.int32), want_q)
+                assert (f is None) == (not want_float) and (f is None or torch.equal(f, want_f))
+                _, qp = kernels.requantize_affine_pad(y4, Fb, scale, shift, residual, relu, (1, 2), I, Fb,
+                                                      False, dtype=dtype)
+                assert torch.equal(qp[:, :, 1:-1, 2:-2], q)
 
         f32, q32 = kernels.requantize_affine_maxpool(y, Fb, scale, shift, True, (3, 2, 1), (1, 1), I, Fb, True)
         f8, q8 = kernels.requantize_affine_maxpool(y, Fb, scale, shift, True, (3, 2, 1), (1, 1), I, Fb, True,
