@@ -306,16 +306,28 @@ __global__ void pairs_fill_kernel(const PairArgs p)
     }
 }
 
+// The tile buffer is above the default 64 KiB limit of a workgroup: opt in, once per device.  Also
+// called when a weight blob is laid out, so that the first convolution launch -- which may be under
+// stream capture -- finds it done.
 template <int BITS>
-static int launch_pairs_cu(const PairArgs &a, int blocks, hipStream_t st)
+static int pairs_opt_in_lds()
 {
-    static bool lds_opted_in = false;  // the tile buffer is above the default 64 KiB limit
-    if (!lds_opted_in) {
+    static bool opted_in[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    if (!opted_in[dev]) {
         hipError_t e = hipFuncSetAttribute((const void *)shift_pairs_cu_kernel<BITS>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kPairLdsBytes);
         if (e != hipSuccess) return hip_status(e);
-        lds_opted_in = true;
+        opted_in[dev] = true;
     }
+    return DS_OK;
+}
+
+template <int BITS>
+static int launch_pairs_cu(const PairArgs &a, int blocks, hipStream_t st)
+{
+    if (int rc = pairs_opt_in_lds<BITS>()) return rc;
     hipLaunchKernelGGL((shift_pairs_cu_kernel<BITS>), dim3(blocks), dim3(512), kPairLdsBytes, st, a);
     return launch_status();
 }
@@ -451,6 +463,8 @@ DS_EXPORT int ds_tile_weights_paired_i32(const int32_t *w_ref, void *paired, int
     if (ref_bits != field_bits && ref_bits != 6) return DS_EBITS;
     if (N == 0) return DS_OK;
     if (!paired || (!w_ref && C > 0)) return DS_EINVAL;
+    rc = field_bits == 1 ? pairs_opt_in_lds<1>() : pairs_opt_in_lds<2>();
+    if (rc) return rc;
     const int K = C * FH * FW;
     const PairedGeom g = paired_geom(N, K, field_bits);
     const long words = (long)g.rows * kTileWords;

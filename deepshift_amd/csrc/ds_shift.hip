@@ -579,12 +579,16 @@ template <int BITS, bool ZT, int WAVES>
 static int launch_planes_cu(const ShiftArgs &a, long iters, hipStream_t st)
 {
     constexpr int kLdsBytes = (WAVES == 8 ? 2 : 1) * 64 * kPlaneRows * kWave * 4;
-    static bool lds_opted_in = false;  // 96 KiB is above the default limit of a workgroup
-    if (!lds_opted_in) {
-        hipError_t e = hipFuncSetAttribute((const void *)shift_planes_wide_cu_kernel<BITS, ZT, WAVES>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-        if (e != hipSuccess) return hip_status(e);
-        lds_opted_in = true;
+    if (kLdsBytes > 64 * 1024) {  // above the default limit of a workgroup: opt in, once per device
+        static bool opted_in[64] = {};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+        if (!opted_in[dev]) {
+            hipError_t e = hipFuncSetAttribute((const void *)shift_planes_wide_cu_kernel<BITS, ZT, WAVES>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+            if (e != hipSuccess) return hip_status(e);
+            opted_in[dev] = true;
+        }
     }
     // one workgroup per 8 wave slots (2 waves per SIMD); small layers: >= 8 K groups per wave
     int blocks = kPlaneSlotsWide / WAVES;

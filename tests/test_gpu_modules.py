@@ -346,3 +346,37 @@ def test_evaluate_cli_runs_the_three_modes(tmp_path, capsys):
                        "--iterations", "1", "--json"])
     assert r["mode"] == "float multiply comparator" and r["max_abs_diff_vs_pytorch"] < 1e-3
     capsys.readouterr()
+
+
+def test_forward_pass_replays_as_a_hip_graph():
+    """The fused pipelines (int32 and int8 activations) captured into a HIP graph: every replay, on new
+    input written into the captured buffer and with eager work in between, must equal the eager result
+    bit for bit (the library clears memory with fill kernels, never with memset nodes)."""
+    from deepshift_amd import fuse
+    cases = [(workloads.ResNet18, (2, 3, 64, 64), dict()),
+             (workloads.ResNet50, (2, 3, 64, 64), dict(weight_bits=3, act_integer_bits=3, act_fraction_bits=5))]
+    for cls, shape, fmt in cases:
+        g = torch.Generator().manual_seed(21)
+        model = workloads.randomize_batchnorm(cls(), g).eval()
+        model, _ = convert.convert_to_shift(model, 1000, 'PS', convert_weights=True, use_kernel=True, **fmt)
+        model = model.to(DEV)
+        with torch.no_grad():
+            fused = fuse.fuse_conv_epilogues(model)
+            static_x = torch.randn(*shape, generator=g).to(DEV)
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(3):
+                    fused(static_x)  # warm-up: blobs, workspaces, attribute opt-ins
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                static_y = fused(static_x)
+            for i in range(3):
+                x = torch.randn(*shape, generator=g).to(DEV)
+                want = fused(x)           # eager work between the replays
+                torch.cuda.synchronize()
+                static_x.copy_(x)
+                graph.replay()
+                torch.cuda.synchronize()
+                assert torch.equal(static_y, want), (cls.__name__, i)
