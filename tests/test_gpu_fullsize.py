@@ -111,3 +111,41 @@ def test_config5_bottleneck_shapes_wb3_act35(oracle):
         want = oracle.conv2d(xp, shift.numpy().astype(np.int32), sign.numpy().astype(np.int32), None,
                              (stride, stride), nthreads=NTHREADS)
         np.testing.assert_array_equal(y.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("layer", [
+    # ResNet-50, batch 128 (configuration 5): Nb, C, H, O, F, stride, pad
+    (128, 64, 56, 256, 1, 1, 0),     # closes a stage-1 block: one tile per wave + cooperative tail
+    (128, 256, 56, 64, 1, 1, 0),     # K = 256: a single chunk only with the post-ReLU bound
+    (128, 128, 28, 128, 3, 1, 1),    # 3x3, K = 1152: cooperative, several chunks per wave
+    (128, 512, 7, 512, 3, 1, 1),     # few tiles, K = 4608: every tile shared between workgroups
+], ids=lambda v: "x".join(map(str, v)))
+def test_config5_int8_layers_full_size(oracle, layer):
+    """The int8 kernel at the real sizes of the 8-bit ResNet-50: against the int32 kernel on the same
+    values (an independent kernel, itself checked against the oracle here on the first image), with
+    and without the post-ReLU bound, plus a batch permutation."""
+    Nb, C, H, O, F, stride, pad = layer
+    g = torch.Generator().manual_seed(5)
+    x = torch.randint(0, 97, (Nb, C, H + 2 * pad, H + 2 * pad), generator=g, dtype=torch.int32)
+    if pad:
+        x[:, :, :pad] = 0; x[:, :, -pad:] = 0; x[:, :, :, :pad] = 0; x[:, :, :, -pad:] = 0
+    shift, sign = _codes(g, (O, C, F, F), lo=-3)
+    bias = torch.randint(-2 ** 10, 2 ** 10, (O,), generator=g, dtype=torch.int32).to(DEV)
+    cw = utils.compress_bits(shift, sign)
+    assert cw.bits == 2
+    fields = kernels.paired_fields(cw, O, 3, 5)
+    assert fields == (2, 2)
+    x32 = x.to(DEV)
+    x8 = x32.to(torch.int8)
+    want = kernels.conv2d_tiled(x32, kernels._tiled_of(cw, O, C, F, F), bias, O, (F, F), (stride, stride),
+                                kernels.kernel_bits(cw), cw.base)
+    first = oracle.conv2d(x[:1].numpy(), shift.numpy().astype(np.int32), sign.numpy().astype(np.int32),
+                          bias.cpu().numpy(), (stride, stride), nthreads=NTHREADS)
+    np.testing.assert_array_equal(want[:1].cpu().numpy(), first)
+    blob = kernels._paired_of(cw, fields, O, C, F, F)
+    for bound in (128, 96):
+        got = kernels.conv2d_paired(x8, blob, bias, O, (F, F), (stride, stride), 2, bound)
+        assert torch.equal(got, want), bound
+    perm = torch.randperm(Nb, generator=g).to(DEV)
+    assert torch.equal(kernels.conv2d_paired(x8[perm].contiguous(), blob, bias, O, (F, F), (stride, stride), 2, 96),
+                       want[perm])
