@@ -21,6 +21,13 @@
 // smaller bound on |x| -- post-ReLU activations of the 3.5 format stay below 97 -- and get longer
 // chunks).  The result is the int32 kernel's,
 // bit for bit.
+//
+// Fields of 3 and 4 bits leave no registers for negated planes; their loop (DS_PAIRX_ASM) applies the
+// sign as in the int32 kernel, acc = (plane[M0] ^ mask) + acc.  ~p = -p - 1 as a 32-bit number, so each
+// negative term takes one off the LOW half only: the per-channel count of negative codes (negcnt, kept
+// behind the codes in the blob) is added back to the pixels that live in low halves -- the even
+// 64-pixel blocks of a tile -- wherever the bias is added.  The highest field value means "no
+// contribution" (zero weights, indices past K); the caller vouches that no real code uses it.
 #include "ds_common.h"
 #include <cstdlib>
 
@@ -35,6 +42,7 @@ struct PairArgs {
     const int8_t *x;        // padded activations
     const uint32_t *codes;  // [N/64][comm*num][32] 16-bit plane indices, channel j | channel j+32 << 16
     const int32_t *bias;    // per channel or nullptr
+    const int32_t *negcnt;  // per channel count of negative codes (xor-mask forms) or nullptr
     int32_t *y;
     uint32_t x_bytes;
     int M, N, K, comm;
@@ -62,7 +70,11 @@ constexpr int kPairSlots = 2048;           // wave slots of the machine at 2 wav
 
 // K groups per call of the asm loop: as many reduction indices as keep a sum of terms of magnitude
 // <= x_bound within 16 bits (255 for x_bound = 128: 255 * 128 < 2^15)
-inline int pair_chunk(int bits, int x_bound) { return (32767 / x_bound) / codes_per_word(bits); }
+// (the xor-mask forms also take one off a low half per negative term: 32767 / (x_bound + 1))
+inline int pair_chunk(int bits, int x_bound)
+{
+    return (32767 / (bits >= 3 ? x_bound + 1 : x_bound)) / codes_per_word(bits);
+}
 
 #define DS_PAIRS_OPERANDS                                                                         \
     : "+{v[64:95]}"(a[0]), "+{v[96:127]}"(a[1]), "+{v[128:159]}"(a[2]), "+{v[160:191]}"(a[3]),    \
@@ -85,6 +97,19 @@ __device__ __forceinline__ void pairs_main_loop<2>(v32i (&a)[6], const uint32_t 
                                                    const uint32_t *wptr, int groups, const PairWalk &w)
 {
     asm volatile(DS_PAIRS_ASM_B2 DS_PAIRS_OPERANDS : DS_PAIRS_CLOBBERS_B2);
+}
+
+template <>
+__device__ __forceinline__ void pairs_main_loop<3>(v32i (&a)[6], const uint32_t (&xoff)[6], v4i rsrc,
+                                                   const uint32_t *wptr, int groups, const PairWalk &w)
+{
+    asm volatile(DS_PAIRX_ASM_B3 DS_PAIRS_OPERANDS : DS_PAIRX_CLOBBERS_B3);
+}
+template <>
+__device__ __forceinline__ void pairs_main_loop<4>(v32i (&a)[6], const uint32_t (&xoff)[6], v4i rsrc,
+                                                   const uint32_t *wptr, int groups, const PairWalk &w)
+{
+    asm volatile(DS_PAIRX_ASM_B4 DS_PAIRS_OPERANDS : DS_PAIRX_CLOBBERS_B4);
 }
 
 // K groups [g_begin, g_end) (at most PairArgs::chunk of them) of the tile made of the 64 channels of
@@ -168,6 +193,8 @@ __device__ __forceinline__ void pairs_segment(const PairArgs &p, int ntile, int 
     for (int j = 0; j < 64; ++j) {
         int32_t *yc = p.y + (size_t)(n0 + j) * p.y_ch_stride;
         const int32_t add = OUT == kAtomic ? 0 : (p.bias ? p.bias[n0 + j] : 0);
+        // pixels in low halves also get the negative-code count back (xor-mask forms)
+        const int32_t add_lo = add + ((OUT != kAtomic && p.negcnt) ? p.negcnt[n0 + j] : 0);
 #pragma unroll
         for (int r = 0; r < kPairRows; ++r) {
             const int32_t v = a[2 * r + j / 32][j % 32];
@@ -177,7 +204,7 @@ __device__ __forceinline__ void pairs_segment(const PairArgs &p, int ntile, int 
                 if (live[2 * r]) atomicAdd(dlo, lo);
                 if (live[2 * r + 1]) atomicAdd(dhi, hi);
             } else {
-                if (live[2 * r]) *dlo = lo + add;
+                if (live[2 * r]) *dlo = lo + add_lo;
                 if (live[2 * r + 1]) *dhi = hi + add;
             }
         }
@@ -270,6 +297,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int c = 0; c < 64 / kPairCuWaves; ++c) {
             const int j = wave * (64 / kPairCuWaves) + c, n = ntile * 64 + j;
             const int32_t add = whole && p.bias ? p.bias[n] : 0;
+            const int32_t neg = whole && p.negcnt ? p.negcnt[n] : 0;  // for the pixels of low halves
             for (int q = 0; q < 6; ++q) {
                 const int m = m0 + q * kWave + lane;
                 if (m >= p.M) break;
@@ -277,7 +305,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 int32_t *dst = p.y + (size_t)img * p.y_img_stride + (size_t)n * p.y_ch_stride +
                                (m - img * p.pix_per_img);
                 const int32_t v = tile_sums[j * kPairPixels + q * kWave + lane];
-                if (whole) *dst = v + add;
+                if (whole) *dst = v + add + ((q & 1) ? 0 : neg);
                 else atomicAdd(dst, v);
             }
         }
@@ -286,23 +314,25 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
-// y = bias[n] before an accumulating launch; y is [img][n][pix], dense.
+// y = bias[n] before an accumulating launch; y is [img][n][pix], dense.  With the xor-mask forms the
+// pixels that live in low halves (the even 64-pixel blocks of their tile) start at bias[n] + negcnt[n].
 __global__ void pairs_fill_kernel(const PairArgs p)
 {
     const uint32_t total = p.y_elems;
+    const uint32_t plane = (uint32_t)p.y_ch_stride, image = plane * (uint32_t)p.N;
     const bool vec = ((uintptr_t)p.y & 15) == 0 && p.y_ch_stride % 4 == 0;
-    if (vec) {
-        int4 *y4 = (int4 *)p.y;
-        for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < (total >> 2); i += gridDim.x * blockDim.x) {
-            const int n = (int)(((i << 2) / (uint32_t)p.y_ch_stride) % (uint32_t)p.N);
-            const int32_t b = p.bias ? p.bias[n] : 0;
-            y4[i] = make_int4(b, b, b, b);
+    const uint32_t step = vec ? 4 : 1;
+    for (uint32_t i = (blockIdx.x * blockDim.x + threadIdx.x) * step; i < total; i += gridDim.x * blockDim.x * step) {
+        const uint32_t img = i / image, rem = i - img * image;
+        const uint32_t n = rem / plane, pix = rem - n * plane;
+        int32_t b = p.bias ? p.bias[n] : 0;
+        if (p.negcnt) {
+            // four consecutive pixels of a plane whose size is a multiple of 4 share their 64-pixel block
+            const uint32_t m = img * plane + pix;
+            if ((((m % (uint32_t)kPairPixels) / kWave) & 1u) == 0u) b += p.negcnt[n];
         }
-    } else {
-        for (uint32_t i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
-            const int n = (int)((i / (uint32_t)p.y_ch_stride) % (uint32_t)p.N);
-            p.y[i] = p.bias ? p.bias[n] : 0;
-        }
+        if (vec) *(int4 *)(p.y + i) = make_int4(b, b, b, b);
+        else p.y[i] = b;
     }
 }
 
@@ -393,7 +423,7 @@ static int launch_pairs(PairArgs a, hipStream_t st)
 // one reduction index ahead).
 struct PairedGeom {
     int num, comm;
-    size_t rows, bytes;
+    size_t rows, negcnt_offset, bytes;
 };
 static PairedGeom paired_geom(int N, int K, int bits)
 {
@@ -401,7 +431,9 @@ static PairedGeom paired_geom(int N, int K, int bits)
     g.num = codes_per_word(bits);
     g.comm = ceil_div(K, g.num);
     g.rows = (size_t)(N / 64) * g.comm * g.num + 1;
-    g.bytes = align_up(g.rows * kTileWords * 4, 256);
+    g.negcnt_offset = align_up(g.rows * kTileWords * 4, 256);
+    // fields of 3 and 4 bits: followed by the per-channel counts of negative codes
+    g.bytes = g.negcnt_offset + (bits >= 3 ? align_up((size_t)N * 4, 256) : 0);
     return g;
 }
 
@@ -413,7 +445,8 @@ __global__ void tile_paired_kernel(const int32_t *__restrict__ w_ref, uint32_t *
 {
     const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= words) return;
-    const uint32_t P = 1u << bits, zero = 0x1000u | (2u * P);
+    const bool xor_mask = bits >= 3;  // field in 7:0, negative in bit 8; the highest field value = nothing
+    const uint32_t P = 1u << bits, zero = xor_mask ? (0x1000u | (P - 1u)) : (0x1000u | (2u * P));
     const int j = (int)(idx % kTileWords);
     const long rest = idx / kTileWords;
     const long rows = (long)comm * num;
@@ -430,11 +463,34 @@ __global__ void tile_paired_kernel(const int32_t *__restrict__ w_ref, uint32_t *
             const uint32_t field = code & ((1u << in_bits) - 1u);
             const uint32_t positive = (code >> in_bits) & 1u;
             uint32_t index = zero;                      // fields >= 32 (6-bit words): zero weight
-            if (field < 32u) index = 0x1000u | ((field & (P - 1u)) + (positive ? 0u : P));
+            if (field < 32u)
+                index = 0x1000u | (xor_mask ? ((field & (P - 1u)) | (positive ? 0u : 0x100u))
+                                            : ((field & (P - 1u)) + (positive ? 0u : P)));
             word |= index << (16 * c);
         }
     }
     out[idx] = word;
+}
+
+// negcnt[n] = number of negative, non-zero codes of channel n; one wave per channel.
+__global__ __launch_bounds__(256) void paired_negcount_kernel(const int32_t *__restrict__ w_ref,
+                                                              int32_t *__restrict__ negcnt, int N, int K,
+                                                              int in_bits, int in_comm)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int n = blockIdx.x * (blockDim.x / kWave) + (threadIdx.x / kWave);
+    if (n >= N) return;
+    const int in_cb = in_bits + 1, in_num = 32 / in_cb;
+    int count = 0;
+    for (int g = lane; g < in_comm; g += kWave) {
+        const uint32_t w = (uint32_t)w_ref[(long)n * in_comm + g];
+        for (int i = 0; i < in_num && g * in_num + i < K; ++i) {
+            const uint32_t code = w >> (i * in_cb);
+            if ((code & ((1u << in_bits) - 1u)) < 32u && ((code >> in_bits) & 1u) == 0u) ++count;
+        }
+    }
+    for (int off = kWave / 2; off > 0; off >>= 1) count += __shfl_down(count, off, kWave);
+    if (lane == 0) negcnt[n] = count;
 }
 
 }  // namespace ds
@@ -443,7 +499,7 @@ using namespace ds;
 
 static int check_paired(int N, int C, int FH, int FW, int bits)
 {
-    if (bits < 1 || bits > 2) return DS_EBITS;
+    if (bits < 1 || bits > 4) return DS_EBITS;
     if (N < 0 || C < 0 || FH < 1 || FW < 1 || N % 64 != 0) return DS_EINVAL;
     if (C >= (1 << 22) || FH > 31 || FW > 31 || (size_t)C * FH * FW >= (1u << 24)) return DS_ETOOLARGE;
     return DS_OK;
@@ -451,7 +507,7 @@ static int check_paired(int N, int C, int FH, int FW, int bits)
 
 DS_EXPORT size_t ds_paired_bytes(int N, int K, int field_bits)
 {
-    if (field_bits < 1 || field_bits > 2 || N < 0 || K < 0 || N % 64 != 0) return 0;
+    if (field_bits < 1 || field_bits > 4 || N < 0 || K < 0 || N % 64 != 0) return 0;
     return paired_geom(N, K, field_bits).bytes;
 }
 
@@ -463,14 +519,23 @@ DS_EXPORT int ds_tile_weights_paired_i32(const int32_t *w_ref, void *paired, int
     if (ref_bits != field_bits && ref_bits != 6) return DS_EBITS;
     if (N == 0) return DS_OK;
     if (!paired || (!w_ref && C > 0)) return DS_EINVAL;
-    rc = field_bits == 1 ? pairs_opt_in_lds<1>() : pairs_opt_in_lds<2>();
+    switch (field_bits) {
+    case 1: rc = pairs_opt_in_lds<1>(); break;
+    case 2: rc = pairs_opt_in_lds<2>(); break;
+    case 3: rc = pairs_opt_in_lds<3>(); break;
+    default: rc = pairs_opt_in_lds<4>(); break;
+    }
     if (rc) return rc;
     const int K = C * FH * FW;
     const PairedGeom g = paired_geom(N, K, field_bits);
     const long words = (long)g.rows * kTileWords;
+    const int in_comm = ceil_div(K, codes_per_word(ref_bits));
     hipLaunchKernelGGL(tile_paired_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, w_ref, (uint32_t *)paired, N, K, g.comm, field_bits, g.num, words,
-                       ref_bits, ceil_div(K, codes_per_word(ref_bits)));
+                       ref_bits, in_comm);
+    if (field_bits >= 3)
+        hipLaunchKernelGGL(paired_negcount_kernel, dim3(ceil_div(N, 4)), dim3(256), 0, (hipStream_t)stream, w_ref,
+                           (int32_t *)((char *)paired + g.negcnt_offset), N, K, ref_bits, in_comm);
     return launch_status();
 }
 
@@ -495,6 +560,7 @@ DS_EXPORT int ds_conv2d_paired_i8(const int8_t *x, const void *paired, const int
     a.x_bytes = (uint32_t)x_bytes;
     a.codes = (const uint32_t *)paired;
     a.bias = bias;
+    a.negcnt = field_bits >= 3 ? (const int32_t *)((const char *)paired + g.negcnt_offset) : nullptr;
     a.y = y;
     a.M = (int)M; a.N = O; a.K = (int)K; a.comm = g.comm;
     a.pix_per_img = OH * OW; a.OW = OW;
@@ -513,5 +579,10 @@ DS_EXPORT int ds_conv2d_paired_i8(const int8_t *x, const void *paired, const int
         hipLaunchKernelGGL(pairs_fill_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, a);
         return launch_status();
     }
-    return field_bits == 1 ? launch_pairs<1>(a, (hipStream_t)stream) : launch_pairs<2>(a, (hipStream_t)stream);
+    switch (field_bits) {
+    case 1: return launch_pairs<1>(a, (hipStream_t)stream);
+    case 2: return launch_pairs<2>(a, (hipStream_t)stream);
+    case 3: return launch_pairs<3>(a, (hipStream_t)stream);
+    default: return launch_pairs<4>(a, (hipStream_t)stream);
+    }
 }

@@ -45,6 +45,13 @@ terms of an int8 activation, so the caller runs at most that many reduction slot
 Its operands: %6..%11 per-pixel byte offsets, %12 descriptor, %13 word pointer, %14 groups,
 %15..%22 the walk.
 
+For 3- and 4-bit fields the int8 family has no room for negated planes; DS_PAIRX_ASM_B<n> keeps the
+xor-mask form of the int32 loops on the two-pixel planes instead: acc = (plane[M0] ^ mask) + acc with
+mask 0 or -1.  ~p = -p - 1 as a 32-bit number, so a negative term subtracts one from the LOW half only:
+the caller adds the count of negative codes back to the pixels that live in low halves.  The highest
+field value is reserved for "no contribution" (zero weights, reduction indices past K): its plane is
+held at 0.  One activation slot is prefetched (D = 1: 6 ring + 48 plane registers for 4-bit fields).
+
 Operands: %6..%8 per-row byte offsets (VGPR), %9 buffer descriptor, %10 word pointer, %11 number of
 K groups, %12..%14 initial walk state (offset, fw, fh), %15 FW, %16 FH, %17 offset step when fw wraps,
 %18 offset step when fh wraps, %19 largest valid offset (the walk runs D slots ahead and is clamped).
@@ -54,7 +61,7 @@ import os
 R = 3
 DEPTH = {1: 4, 2: 5, 3: 4, 4: 3}        # prefetch ring depth, 32-channel form
 DEPTH_WIDE = {1: 4, 2: 5, 3: 4, 4: 2}   # 64-channel form: 4-bit fields leave room for two slots only
-DEPTH_PAIRED = {1: 4, 2: 2}             # int8 form: six activation registers per slot
+DEPTH_PAIRED = {1: 4, 2: 2, 3: 1, 4: 1}  # int8 forms: six activation registers per slot
 
 
 class Form:
@@ -315,6 +322,74 @@ def body_paired(bits):
     return L
 
 
+def body_pairx(bits):
+    """The int8 form for 3- and 4-bit fields: two pixels per register, xor-mask signs."""
+    f = Form(bits, True, paired=True)
+    num = 32 // (bits + 1)
+    P = 1 << bits
+    S = P                                       # planes per row; plane P - 1 stays 0
+    D, ACC = 1, f.acc
+    PL = XP + 2 * R * D
+    assert PL + S * R <= ACC and ACC + R * f.J <= 256 and num % 2 == 0
+    SEL = IDX                                   # the relative-addressing switch takes a constant here
+    L = []
+    L += ["s_getreg_b32 s%d, hwreg(HW_REG_HW_ID, 0, 4)" % PRIO,
+          "s_mov_b32 s%d, %%%d" % (CNT, f.op_groups),
+          "s_mov_b64 s[%d:%d], %%%d" % (WP, WP + 1, f.op_wptr),
+          "s_mov_b32 s%d, %%%d" % (KOFF, f.op_walk), "s_mov_b32 s%d, %%%d" % (FWC, f.op_walk + 1),
+          "s_mov_b32 s%d, %%%d" % (FHC, f.op_walk + 2),
+          "s_mov_b32 s%d, 0x05040100" % SEL]    # v_perm_b32 selector: low halves of (src0, src1)
+    L += load_words(W)
+    L += ["s_memrealtime s[%d:%d]" % (TIME, TIME + 1)]
+    L += walk_and_load(0, f)
+    for r in range(R):
+        L += ["v_mov_b32 v%d, 0" % (PL + S * r + P - 1)]
+    L += ["1:"]
+    for i in range(num):
+        cur, nxt = (W, WS) if i % 2 == 0 else (WS, W)
+        L += ["s_add_u32 s%d, s%d, 128" % (WP, WP), "s_addc_u32 s%d, s%d, 0" % (WP + 1, WP + 1),
+              "s_waitcnt lgkmcnt(0)"]
+        if i % 2 == 0:
+            L += take_turn(i // 2, f.waves)
+        L += load_words(nxt)
+        if i % 2 == 1:
+            L += ["s_memrealtime s[%d:%d]" % (TIME, TIME + 1)]
+        L += ["s_waitcnt vmcnt(0)", "s_set_gpr_idx_off"]
+        for r in range(R):
+            lo, hi = XP + 2 * r, XP + 2 * r + 1
+            L += ["v_perm_b32 v%d, v%d, v%d, s%d" % (hi, hi, lo, SEL),      # both pixels as 16-bit fields
+                  "v_and_b32 v%d, 0x10000, v%d" % (lo, lo),                 # 65536 where pixel a < 0
+                  "v_sub_u32 v%d, v%d, v%d" % (PL + S * r, hi, lo)]         # plane 0 = hi * 65536 + lo
+        for s in range(1, P - 1):
+            for r in range(R):
+                L += ["v_pk_ashrrev_i16 v%d, %d, v%d op_sel_hi:[0,1]" % (PL + S * r + s, s, XP + 2 * r + 1)]
+        for s in range(1, P - 1):
+            for r in range(R):
+                L += ["v_sub_u32 v%d, v%d, v%d" % (PL + S * r + s, PL + S * r + s, XP + 2 * r)]
+        L += walk_and_load(0, f)                # the ring is free again: the next slot's activations
+        L += ["s_set_gpr_idx_on s%d, 0x1" % PRIO]
+        for half in (0, 1):
+            for j in range(32):
+                if half == 0:
+                    L += ["s_mov_b32 m0, s%d" % (cur + j)]
+                else:
+                    L += ["s_lshr_b32 m0, s%d, 16" % (cur + j)]
+                L += ["s_bfe_i32 s%d, s%d, 0x%x" % (MASK, cur + j, (1 << 16) | (16 * half + 8))]
+                for r in range(R):
+                    a = ACC + f.J * r + j + 32 * half
+                    L += ["v_xad_u32 v%d, v%d, s%d, v%d" % (a, PL + S * r, MASK, a)]
+    L += ["s_sub_u32 s%d, s%d, 1" % (CNT, CNT), "s_cmp_lg_u32 s%d, 0" % CNT, "s_cbranch_scc1 1b"]
+    L += ["s_set_gpr_idx_off", "s_setprio 0", "s_waitcnt vmcnt(0) lgkmcnt(0)"]
+    return L
+
+
+def clobbers_pairx(bits):
+    P = 1 << bits
+    v = ['"v%d"' % n for n in range(XP, XP + 2 * R + P * R)]
+    s = ['"s%d"' % n for n in list(range(4, 16)) + list(range(W, WS + 32)) + [TIME, TIME + 1]]
+    return ", ".join(v + s + ['"scc"', '"memory"'])
+
+
 def clobbers_paired(bits):
     f = Form(bits, True, paired=True)
     P = 1 << bits
@@ -340,6 +415,12 @@ def main():
         out.append(" \\\n".join('    "%s\\n"' % line for line in body_paired(bits)))
         out.append("")
         out.append("#define DS_PAIRS_CLOBBERS_B%d %s" % (bits, clobbers_paired(bits)))
+        out.append("")
+    for bits in (3, 4):
+        out.append("#define DS_PAIRX_ASM_B%d \\" % bits)
+        out.append(" \\\n".join('    "%s\\n"' % line for line in body_pairx(bits)))
+        out.append("")
+        out.append("#define DS_PAIRX_CLOBBERS_B%d %s" % (bits, clobbers_pairx(bits)))
         out.append("")
     with open(os.path.join(here, "ds_planes_asm.inc"), "w") as f:
         f.write("\n".join(out))

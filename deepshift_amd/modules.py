@@ -196,6 +196,22 @@ def _circular_pad(x, padding):
     return F.pad(x, expanded, mode='circular')
 
 
+def _small_for_int8(module, input_shape, field_bits):
+    """The int8 kernel works on tiles of 384 pixels x 64 channels; a layer with few of them and a short
+    reduction (the 1x1 shortcuts of a ResNet-18) is served better by the int32 kernels' smaller tiles.
+    Measured: below about 8000 (tile, K group) units the int32 path wins."""
+    Nb, _, H, W = input_shape
+    ph, pw = (0, 0) if module.padding_mode == 'circular' else module.padding
+    if module.padding_mode == 'circular':
+        H, W = H + module.padding[0], W + module.padding[1]
+    OH = (H + 2 * ph - module.kernel_size[0]) // module.stride[0] + 1
+    OW = (W + 2 * pw - module.kernel_size[1]) // module.stride[1] + 1
+    tiles = -(-Nb * OH * OW // 384) * (module.out_channels // 64)
+    K = module.in_channels * module.kernel_size[0] * module.kernel_size[1]
+    groups = -(-K // (32 // (field_bits + 1)))
+    return tiles * groups < 8192
+
+
 def conv_kernel_forward(module, input, conc_weight, scale=None, shift=None, residual=None, relu=False,
                         prequantized=False, emit=None, pool=None, input_nonneg=False):
     """Fixed-point shift convolution of a float NCHW input (modules.py:152-162,317-337).
@@ -222,6 +238,8 @@ def conv_kernel_forward(module, input, conc_weight, scale=None, shift=None, resi
     if prequantized:
         xq = input
     else:
+        if fields and _small_for_int8(module, input.shape, fields[1]):
+            fields = None
         padding = module.padding
         input = input.float()
         if module.padding_mode == 'circular':

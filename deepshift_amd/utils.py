@@ -71,10 +71,13 @@ class ConcWeight():
     reference's row-major word format, ``base`` (0 or the negative minimum of -shift) and ``bits``
     (width of the shift field; a code takes ``bits + 1`` bits)."""
 
-    def __init__(self, data=None, base=0, bits=8, zero_top_bits=0):
+    def __init__(self, data=None, base=0, bits=8, zero_top_bits=0, max_field=None):
         self.data = data
         self.base = base
         self.bits = bits
+        # Not in the reference: the largest shift field among the non-zero weights, when known (the
+        # int8 kernel for 3- and 4-bit fields needs the highest field value to be unused).
+        self.max_field = max_field
         # Not in the reference: for 6-bit words that only need them for the zero code (ternary
         # weights), the field width into which the non-zero shifts fit with one value to spare;
         # the kernels then run the layer from a narrower private blob (0: not applicable).
@@ -137,8 +140,9 @@ def compress_bits(shift, sign):
     row_length = int((shift.shape[1] * shift.shape[2] * shift.shape[3] + num - 1) / num)
     size = row_length * shift.shape[0]
 
+    real = s[s < ZERO_SHIFT]
+    conc_weight.max_field = (int(real.max()) if real.numel() else 0) - conc_weight.base
     if conc_weight.bits == 6 and conc_weight.base == 0:
-        real = s[s < ZERO_SHIFT]
         top = int(real.max()) if real.numel() else 0
         for width in (1, 2, 3, 4):
             if top <= 2 ** width - 2:

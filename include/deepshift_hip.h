@@ -85,17 +85,19 @@ int ds_tile_weights_zero_top_i32(const int32_t *w_ref, void *tiled, int N, int C
 
 /* Activation formats of at most 8 bits (act_integer_bits + act_fraction_bits <= 8, e.g. the 3.5 format
  * of the reference's 8-bit runs) can be held as int8.  |x >> s| <= 128 then, 255 terms fit a 16-bit
- * sum, and the vector ALU handles two pixels per register (packed 16-bit shifts and adds), widening
- * to the int32 output every 255 reduction indices: the int32 kernels' results, bit for bit, in about
- * half the vector instructions and a quarter of the activation bytes.  For layers with
- * O % 64 == 0 and shift fields of 1 or 2 bits (weight_bits <= 3).  No counterpart in the reference,
- * which always computes on int32 (modules.py:153).
+ * sum, and the vector ALU handles two pixels per register, widening to the int32 output every 255
+ * reduction indices: the int32 kernels' results, bit for bit, in about half the vector instructions
+ * and a quarter of the activation bytes.  For layers with O % 64 == 0 and shift fields of 1 to 4 bits
+ * (weight_bits <= 5).  No counterpart in the reference, which always computes on int32
+ * (modules.py:153).
  *
  * ds_tile_weights_paired_i32 lays reference-format words w_ref[N][ceil(K / (32 / (ref_bits + 1)))]
  * (ds_pack_i32's output, base 0) out for that kernel: ds_paired_bytes(N, K, field_bits) bytes.
  * ref_bits is the field width of the words: field_bits, or 6 for the words of a ternary layer whose
- * non-zero fields are all below 2^field_bits (zero weights, fields >= 32, then select a plane held
- * at 0). */
+ * non-zero fields fit field_bits (zero weights, fields >= 32, then contribute nothing).
+ * With field_bits 3 or 4 the kernel takes the highest field value (7 / 15) for "no contribution":
+ * the caller vouches that no non-zero weight uses it -- true of every layer whose shifts were clamped
+ * to the reference's range for its weight_bits, (-(2^(weight_bits-1) - 2), 0) (modules.py:88). */
 size_t ds_paired_bytes(int N, int K, int field_bits);
 int ds_tile_weights_paired_i32(const int32_t *w_ref, void *paired, int N, int C, int FH, int FW,
                                int ref_bits, int field_bits, ds_stream_t stream);
@@ -103,10 +105,10 @@ int ds_tile_weights_paired_i32(const int32_t *w_ref, void *paired, int N, int C,
 /* Conv2dShift forward on int8 activations: ds_conv2d_tiled_i32 (DEEP_SHIFT_CONV,
  * kernels/cuda/shift_cuda.cpp:41-53) with x int8 [Nb][C][Hp][Wp], already padded, and the blob of
  * ds_tile_weights_paired_i32.  y int32 [Nb][O][OH][OW].  DS_EINVAL when O % 64 != 0, DS_EBITS when
- * field_bits is not 1 or 2.
+ * field_bits is not 1..4.
  * x_bound (1..128): the caller vouches that every |x| <= x_bound.  128 is always true; a smaller
- * bound lets the kernel run 32767 / x_bound reduction indices between two widenings of its 16-bit
- * sums -- e.g. 96 for the output of a ReLU in the 3.5 format, whose round-to-fixed clamp
+ * bound lets the kernel run 32767 / x_bound (field_bits 3, 4: 32767 / (x_bound + 1)) reduction
+ * indices between two widenings of its 16-bit sums -- e.g. 96 for the output of a ReLU in the 3.5 format, whose round-to-fixed clamp
  * (utils.py:7-21) keeps the values in [0, 96]: a K = 256 layer is then a single chunk.  A value
  * beyond the bound makes the sums wrap: results are then wrong, nothing else. */
 int ds_conv2d_paired_i8(const int8_t *x, const void *paired, const int32_t *bias, int32_t *y, int Nb,

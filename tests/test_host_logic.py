@@ -190,8 +190,8 @@ def test_packed_export_rejects_foreign_files(tmp_path):
 
 def test_int8_kernel_eligibility():
     """kernels.paired_fields: activations of at most 8 bits (not the one-bit format), a multiple of 64
-    channels, base 0, shift fields of at most 2 bits (packed that narrow, or ternary 6-bit words whose
-    non-zero fields are)."""
+    channels, base 0, shift fields of at most 4 bits (packed that narrow, or ternary 6-bit words whose
+    non-zero fields are), the highest value of a 3- or 4-bit field unused."""
     from deepshift_amd import kernels
     from deepshift_amd.utils import ConcWeight
     narrow = ConcWeight(None, 0, 2)
@@ -202,8 +202,25 @@ def test_int8_kernel_eligibility():
     assert kernels.paired_fields(narrow, 64, 4, 5) is None        # 9 bits
     assert kernels.paired_fields(narrow, 96, 3, 5) is None        # channels
     assert kernels.paired_fields(ConcWeight(None, -1, 2), 64, 3, 5) is None
-    assert kernels.paired_fields(ConcWeight(None, 0, 3), 64, 3, 5) is None
+    assert kernels.paired_fields(ConcWeight(None, 0, 3), 64, 3, 5) is None            # top field unknown
+    assert kernels.paired_fields(ConcWeight(None, 0, 3, max_field=7), 64, 3, 5) is None
+    assert kernels.paired_fields(ConcWeight(None, 0, 3, max_field=6), 64, 3, 5) == (3, 3)
+    assert kernels.paired_fields(ConcWeight(None, 0, 4, max_field=14), 64, 3, 5) == (4, 4)
+    assert kernels.paired_fields(ConcWeight(None, 0, 4, max_field=15), 64, 3, 5) is None
+    assert kernels.paired_fields(ConcWeight(None, 0, 5, max_field=20), 64, 3, 5) is None
     assert kernels.paired_fields(None, 64, 3, 5) is None
     assert kernels.paired_fields(ConcWeight(None, 0, 6, 2), 64, 3, 5) == (6, 2)
-    assert kernels.paired_fields(ConcWeight(None, 0, 6, 3), 64, 3, 5) is None
+    assert kernels.paired_fields(ConcWeight(None, 0, 6, 4), 64, 3, 5) == (6, 4)
     assert kernels.paired_fields(ConcWeight(None, 0, 6, 0), 64, 3, 5) is None
+
+
+def test_small_layers_stay_on_the_int32_kernels():
+    """modules._small_for_int8: few 384-pixel x 64-channel tiles and a short reduction."""
+    from deepshift_amd import modules
+    shortcut = modules.Conv2dShift(64, 128, 1, stride=2, use_kernel=True)
+    assert modules._small_for_int8(shortcut, (64, 64, 56, 56), 4)          # ResNet-18 1x1/2 shortcut
+    body = modules.Conv2dShift(512, 512, 3, padding=1, use_kernel=True)
+    assert not modules._small_for_int8(body, (64, 512, 7, 7), 4)           # few tiles, K = 4608
+    assert modules._small_for_int8(body, (1, 512, 7, 7), 4)                # batch 1
+    wide = modules.Conv2dShift(64, 256, 1, use_kernel=True)
+    assert not modules._small_for_int8(wide, (128, 64, 56, 56), 2)         # ResNet-50 stage 1
