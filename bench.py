@@ -7,8 +7,8 @@ One step = one forward pass of ResNet-18 (every conv and the FC replaced by shif
 weight_bits 5, activations 16.16) over one synthetic batch of 64 x 3 x 224 x 224 that is already
 resident in HBM.  Prints ONE JSON line: images/s for the whole forward pass, the shift kernel's
 rate against the VALU roofline (timed live with HIP events on the launch stream), the 4096^3
-shift GEMM and the 3x3 conv of benchmark configuration 2, ResNet-50 with 8-bit activations
-(configuration 5), and the CPU restatement of the reference's shift kernel timed on this host's cores.
+shift GEMM and the 3x3 conv of benchmark configuration 2, ResNet-50 (configuration 5) and ResNet-18
+with 8-bit activations, and the CPU restatement of the reference's shift kernel timed on this host's cores.
 """
 import argparse
 import json
@@ -187,33 +187,51 @@ def config2(device, reps=10):
     return out
 
 
-def config5(device, steps=5):
-    """Benchmark configuration 5: ResNet-50, batch 128, weight_bits 3 (2-bit shift fields), activations
-    3.5 (8 bits).  Every convolution has a multiple of 64 channels, so the fused pipeline runs them on
-    the int8 kernel (two pixels per register); the FC stays on the int32 kernel."""
-    from deepshift_amd import convert, fuse, workloads
+def fused_model_timing(device, cls, batch, weight_bits, integer_bits, fraction_bits, workload, steps=5):
+    """Steps/s and shift-kernel rate of a converted, fused network on synthetic input."""
+    from deepshift_amd import convert, fuse
     g = torch.Generator().manual_seed(0)
-    model = workloads.ResNet50()
+    model = cls()
     for m in model.modules():
         if isinstance(m, (torch.nn.Conv2d, torch.nn.Linear)):
             torch.nn.init.kaiming_normal_(m.weight, generator=g)
+    from deepshift_amd import workloads
     workloads.randomize_batchnorm(model, g)
     model.eval()
     model, _ = convert.convert_to_shift(model, 1000, 'PS', convert_weights=True, use_kernel=True,
-                                        weight_bits=3, act_integer_bits=3, act_fraction_bits=5)
+                                        weight_bits=weight_bits, act_integer_bits=integer_bits,
+                                        act_fraction_bits=fraction_bits)
     model = model.to(device)
-    x = torch.randn(128, *CHW, generator=g).to(device)
+    convert.round_shift_weights(model)
+    x = torch.randn(batch, *CHW, generator=g).to(device)
     with torch.no_grad():
         fused = fuse.fuse_conv_epilogues(model)
     sec = time_steps(fused, x, steps, 2)
     layers = kernel_timings(fused, x, 3)
     pairs = sum(L["M"] * L["K"] * L["N"] for L in layers)
     kernel_s = sum(L["seconds"] for L in layers)
-    return dict(workload="ResNet-50, batch 128 x 3x224x224, weight_bits 3, activations 3.5",
-                ms_per_step=sec * 1e3, images_per_s=128 / sec, shift_layers=len(layers),
+    return dict(workload=workload, ms_per_step=sec * 1e3, images_per_s=batch / sec, shift_layers=len(layers),
                 pairs_per_step=pairs, shift_kernel_ms_per_step=kernel_s * 1e3,
                 shift_tpairs_per_s=pairs / kernel_s / 1e12,
                 frac_of_two_instruction_peak=pairs / kernel_s / PEAK_PAIRS)
+
+
+def config5(device, steps=5):
+    """Benchmark configuration 5: ResNet-50, batch 128, weight_bits 3 (2-bit shift fields), activations
+    3.5 (8 bits).  Every convolution has a multiple of 64 channels, so the fused pipeline runs them on
+    the int8 kernel (two pixels per register); the FC stays on the int32 kernel."""
+    from deepshift_amd import workloads
+    return fused_model_timing(device, workloads.ResNet50, 128, 3, 3, 5,
+                              "ResNet-50, batch 128 x 3x224x224, weight_bits 3, activations 3.5", steps)
+
+
+def config4_act8(device, steps=5):
+    """The headline network with the reference's 8-bit activation format (`-ab 3 5`, weight_bits 5):
+    the 3x3 layers and the stem run on the int8 kernel, the three 1x1 shortcuts and the FC on the
+    int32 kernels."""
+    from deepshift_amd import workloads
+    return fused_model_timing(device, workloads.ResNet18, BATCH, 5, 3, 5,
+                              "ResNet-18, batch 64 x 3x224x224, weight_bits 5, activations 3.5", steps)
 
 
 def pmc_target(device):
@@ -369,6 +387,7 @@ def main():
     peak_cal = None if args.resnet_only else calibrate_valu(device)
     cfg2 = None if args.resnet_only else config2(device)
     cfg5 = None if args.resnet_only else config5(device)
+    cfg4_act8 = None if args.resnet_only else config4_act8(device)
     result = {
         "metric": "resnet18_bs64_images_per_s",
         "value": BATCH / sec_per_step,
@@ -416,6 +435,7 @@ def main():
         },
         "config2": cfg2,
         "config5": cfg5,
+        "config4_act8": cfg4_act8,
         "shift_gemm_gops": cfg2["gemm_4096"]["gops"] if cfg2 else None,
     }
     if not args.no_cpu:
