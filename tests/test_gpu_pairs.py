@@ -247,3 +247,25 @@ def test_random_int8_convolutions(oracle, seed):
     blob = abi_tile_paired(w, O, C, FH, FW, bits, bits)
     got = abi_conv_paired(x8, blob, bias, O, FH, FW, (sh, sw), bits)
     np.testing.assert_array_equal(got, want, err_msg=str((bits, Nb, C, Hp, Wp, O, FH, FW, sh, sw)))
+
+
+def test_paired_degenerate_sizes(oracle):
+    """No input channels (the output is the bias), an empty batch, a single pixel."""
+    L = _lib.lib()
+    bias = np.arange(64, dtype=np.int32) - 7
+    blob = torch.zeros(max(1, L.ds_paired_bytes(64, 0, 2)), dtype=torch.uint8, device=DEV)
+    _lib.call("ds_tile_weights_paired_i32", None, _lib.ptr(blob), 64, 0, 1, 1, 2, 2, stream())
+    x8 = np.zeros((2, 0, 5, 5), np.int8)
+    got = abi_conv_paired(x8, blob, bias, 64, 1, 1, (1, 1), 2)
+    np.testing.assert_array_equal(got, np.broadcast_to(bias[None, :, None, None], (2, 64, 5, 5)))
+    # empty batch: nothing to do, no pointer is touched
+    _lib.call("ds_conv2d_paired_i8", None, _lib.ptr(blob), None, None, 0, 3, 5, 5, 64, 1, 1, 1, 1, 2, 128, stream())
+    # one output pixel, every field width
+    for bits in (1, 2, 3, 4):
+        rng = np.random.default_rng(bits)
+        x8 = random_int8(rng, (1, 5, 3, 3))
+        s, sign = random_codes(rng, (64, 5, 3, 3), max_s=top_field(bits))
+        w, _ = oracle.pack_words(s.reshape(64, -1), sign.reshape(64, -1), bits)
+        want = oracle.conv2d(x8.astype(np.int32), -s, sign, bias, (1, 1))
+        got = abi_conv_paired(x8, abi_tile_paired(w, 64, 5, 3, 3, bits, bits), bias, 64, 3, 3, (1, 1), bits)
+        np.testing.assert_array_equal(got, want)
