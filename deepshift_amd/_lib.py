@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libdeepshift_hip.so")
 DS_Q_ROUND_TO_FIXED = 0
 DS_Q_CAST = 1
 DS_BITS_ZERO_TOP = 0x100
+DS_BITS_TOP_UNUSED = 0x200
 
 _c_int = ctypes.c_int
 _c_i64 = ctypes.c_int64

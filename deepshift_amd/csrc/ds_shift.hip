@@ -57,6 +57,7 @@ struct ShiftArgs {
     int alt_ld;
     uint32_t y_elems;                     // elements the pre-fill covers
     int zero_top;                         // the highest field value is a zero weight (ternary blobs)
+    int top_unused;                       // no code carries the highest field value (the caller vouches)
 };
 
 // Redirects an atomic LinearShift launch to its channel-major scratch; returns the final y or nullptr.
@@ -827,6 +828,10 @@ static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
         if (planes) {
             int nsplit = plane_regime(a, wide) > 0 ? 1 : 0;
             if (const char *sp = getenv("DS_TUNE_SPLIT")) nsplit = atoi(sp);
+            // the highest field value unused: the form that holds its plane at 0 saves its shift
+            if (a.top_unused)
+                return wide ? launch_planes<BITS, true, true>(a, nsplit, st)
+                            : launch_planes<BITS, true, false>(a, nsplit, st);
             return wide ? launch_planes<BITS, false, true>(a, nsplit, st)
                         : launch_planes<BITS, false, false>(a, nsplit, st);
         }
@@ -861,6 +866,16 @@ static int dispatch_bits(const ShiftArgs &a, int bits, bool general, hipStream_t
     case 6: return dispatch_shape<6, true>(a, st);
     default: return DS_EBITS;
     }
+}
+
+// Splits the top-unused flag off `bits` (tiled entry points only); meaningful for fields of <= 4 bits
+// without a base, ignored otherwise.
+static int take_top_unused(int &bits, int base)
+{
+    if (!(bits & DS_BITS_TOP_UNUSED)) return 0;
+    bits &= ~DS_BITS_TOP_UNUSED;
+    return base == 0 && (bits & ~DS_BITS_ZERO_TOP) >= 1 && (bits & ~DS_BITS_ZERO_TOP) <= 4 &&
+           !(bits & DS_BITS_ZERO_TOP);
 }
 
 // Splits the zero-top flag off `bits` (tiled entry points only).
@@ -913,6 +928,7 @@ DS_EXPORT int ds_conv2d_tiled_i32(const int32_t *x, const void *tiled, const int
                                   size_t workspace_bytes, ds_stream_t stream)
 {
     (void)workspace; (void)workspace_bytes;
+    const int top_unused = take_top_unused(bits, base);
     const int zero_top = take_zero_top(bits, base);
     int rc = check_common(bits, base);
     if (rc) return rc;
@@ -947,6 +963,7 @@ DS_EXPORT int ds_conv2d_tiled_i32(const int32_t *x, const void *tiled, const int
     a.FH = FH; a.FW = FW;
     a.nbase = -base;
     a.zero_top = zero_top;
+    a.top_unused = top_unused;
     return dispatch_bits(a, bits, base != 0 || bits == 6, (hipStream_t)stream);
 }
 
@@ -984,7 +1001,7 @@ static size_t linear_scratch_bytes(int M, int N)
 DS_EXPORT size_t ds_linear_tiled_workspace_bytes(int M, int K, int N, int bits)
 {
     (void)K;
-    bits &= ~DS_BITS_ZERO_TOP;
+    bits &= ~(DS_BITS_ZERO_TOP | DS_BITS_TOP_UNUSED);
     if (bits < 1 || bits > 6 || M < 0 || N < 0) return 0;
     return linear_scratch_bytes(M, N);
 }
@@ -1001,6 +1018,7 @@ DS_EXPORT int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled,
                                   int32_t *y, int M, int K, int N, int bits, int base,
                                   void *workspace, size_t workspace_bytes, ds_stream_t stream)
 {
+    const int top_unused = take_top_unused(bits, base);
     const int zero_top = take_zero_top(bits, base);
     int rc = check_common(bits, base);
     if (rc) return rc;
@@ -1036,6 +1054,7 @@ DS_EXPORT int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled,
     a.FH = 1; a.FW = 1;
     a.nbase = -base;
     a.zero_top = zero_top;
+    a.top_unused = top_unused;
     return dispatch_bits(a, bits, base != 0 || bits == 6, (hipStream_t)stream);
 }
 

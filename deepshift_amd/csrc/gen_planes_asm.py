@@ -12,8 +12,9 @@ VGPR-relative addressing (s_set_gpr_idx_*), which needs a fixed register map:
                                             acc[r][j] = (plane[r][M0] ^ mask) + acc[r][j]   (v_xad_u32)
 
 so a shift-add term costs 1 + 2^BITS/32 vector instructions instead of 2.  Every width also comes in
-a "zero top" form (DS_PLANES_ASM_B<n>Z) for ternary weights: the highest field value stands for a
-zero weight and its plane is 0 instead of x >> (2^BITS - 1).
+a "zero top" form (DS_PLANES_ASM_B<n>Z) in which the plane of the highest field value is held at 0 and
+never computed: for ternary weights re-packed so that this value stands for a zero weight, and for
+layers that do not use it at all (one shift fewer per pixel row and reduction index).
 
 Register map (R = 3 pixels per lane, J = 32 channels, NUM = 32 // (BITS + 1) codes per word, D = depth
 of the activation prefetch ring in reduction slots, a divisor of NUM):
@@ -178,6 +179,9 @@ def body(bits, zero_top=False, wide=False):
     L += ["s_memrealtime s[%d:%d]" % (TIME, TIME + 1)]
     for i in range(D):
         L += walk_and_load(i, f)
+    if zero_top:
+        # the highest field value contributes nothing: its plane is 0, once and for all
+        L += ["v_mov_b32 v%d, 0" % (PL + P * r + P - 1) for r in range(R)]
     L += ["s_mov_b32 s%d, 0" % IDX, "s_set_gpr_idx_on s%d, 0x1" % IDX]  # src0 of vector ops is M0-relative
     # ---- one K group per iteration
     L += ["1:"]
@@ -214,8 +218,7 @@ def body(bits, zero_top=False, wide=False):
         for s in range(1, P):
             for r in range(R):
                 if zero_top and s == P - 1:
-                    # the highest field value encodes a zero weight: its plane is 0
-                    L += ["v_mov_b32 v%d, 0" % (PL + P * r + s)]
+                    continue  # held at 0 since the prologue
                 else:
                     L += ["v_ashrrev_i32 v%d, %d, v%d" % (PL + P * r + s, s, PL + P * r)]
         # the 16-bit code is a ready M0 value: plane index in 7:0, "src0 relative" in 15:12.  32-channel

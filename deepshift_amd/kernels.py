@@ -138,6 +138,9 @@ def kernel_bits(conc_weight):
     width = getattr(conc_weight, "zero_top_bits", 0)
     if width and conc_weight.bits == 6 and conc_weight.base == 0:
         return width | _lib.DS_BITS_ZERO_TOP
+    top = getattr(conc_weight, "max_field", None)
+    if conc_weight.bits <= 4 and conc_weight.base == 0 and top is not None and top <= 2 ** conc_weight.bits - 2:
+        return conc_weight.bits | _lib.DS_BITS_TOP_UNUSED  # the plane of the highest value is never needed
     return conc_weight.bits
 
 

@@ -78,6 +78,13 @@ int ds_tile_weights_i32(const int32_t *w_ref, void *tiled, int N, int C, int FH,
  * The caller vouches for the field range (deepshift_amd.utils.compress_bits checks it when it
  * packs).  No counterpart in the reference. */
 #define DS_BITS_ZERO_TOP 0x100
+/* For ordinary blobs (ds_tile_weights_i32) of 1..4-bit fields, base 0: bits | DS_BITS_TOP_UNUSED tells
+ * the tiled compute entry points that no code of the layer carries the highest field value -- true of
+ * every layer whose shifts were clamped to the reference's range for its weight_bits,
+ * (-(2^(weight_bits-1) - 2), 0) (modules.py:88).  The shift-plane kernel then skips that plane (one
+ * vector instruction fewer per pixel row and reduction index).  The caller vouches for it; a code
+ * with that value would contribute 0 instead of x >> value. */
+#define DS_BITS_TOP_UNUSED 0x200
 int ds_tile_weights_zero_top_i32(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW,
                                  int field_bits, ds_stream_t stream);
 

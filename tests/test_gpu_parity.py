@@ -475,3 +475,65 @@ def test_compress_bits_finds_the_zero_top_width(rng):
     s, sign = random_codes(rng, (8, 40), max_s=14)  # no zero weight: plain 4-bit fields
     cw = utils.compress_bits(torch.from_numpy(-s).float(), torch.from_numpy(sign).float())
     assert cw.bits == 4 and cw.zero_top_bits == 0
+    assert kernels.kernel_bits(cw) == 4 | _lib.DS_BITS_TOP_UNUSED  # 15 does not occur
+    s[0, 0] = 15
+    cw = utils.compress_bits(torch.from_numpy(-s).float(), torch.from_numpy(sign).float())
+    assert kernels.kernel_bits(cw) == 4
+
+
+@pytest.mark.parametrize("split", [None, 0, 1, 3])
+@pytest.mark.parametrize("bits", [1, 2, 3, 4])
+def test_top_unused_flag_matches_oracle(oracle, rng, bits, split):
+    """Ordinary blobs whose codes never carry the highest field value: with DS_BITS_TOP_UNUSED the tiled
+    entry points give the results they give without it, on every launch mode."""
+    from deepshift_amd import kernels
+    flag = bits | _lib.DS_BITS_TOP_UNUSED
+    top = 2 ** bits - 2
+    env = {"DS_TUNE_PLANES": 1} if split is None else {"DS_TUNE_PLANES": 1, "DS_TUNE_SPLIT": split}
+    for tune in ({}, env):
+        with _Tune(**tune):
+            for M, K, N, with_bias in [(200, 480, 64, False), (333, 517, 71, True), (2000, 1200, 128, True)]:
+                x = random_activations(rng, (M, K))
+                s, sign = random_codes(rng, (N, K), max_s=top)
+                bias = rng.integers(-2 ** 20, 2 ** 20, size=N).astype(np.int32) if with_bias else None
+                want = oracle.linear(x, -s, sign, bias, nthreads=NTHREADS)
+                blob = kernels.tile_weights(dev(so.np_pack_words(s, sign, bits)).reshape(-1), N, K, 1, 1, bits, 0)
+                xT = dev(np.ascontiguousarray(np.pad(x, ((0, (-M) % 64), (0, 0))).T))
+                for b in (flag, bits):
+                    got = kernels.linear_tiled(xT, M, blob, None if bias is None else dev(bias), N, b, 0)
+                    np.testing.assert_array_equal(got.cpu().numpy(), want)
+            Nb, C, Hp, Wp, O = 3, 24, 21, 17, 64
+            xp = random_activations(rng, (Nb, C, Hp, Wp))
+            s, sign = random_codes(rng, (O, C, 3, 3), max_s=top)
+            want = oracle.conv2d(xp, -s, sign, None, (1, 1), nthreads=NTHREADS)
+            w = dev(so.np_pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits))
+            blob = kernels.tile_weights(w.reshape(-1), O, C, 3, 3, bits, 0)
+            got = kernels.conv2d_tiled(dev(xp), blob, None, O, (3, 3), (1, 1), flag, 0)
+            np.testing.assert_array_equal(got.cpu().numpy(), want)
+
+
+def test_top_unused_flag_is_ignored_where_it_does_not_apply(oracle, rng):
+    """5- and 6-bit fields and blobs with a base have no plane to skip: the flag changes nothing; the
+    entry points that take reference words refuse it like any other unknown width."""
+    from deepshift_amd import kernels
+    L = _lib.lib()
+    M, K, N = 300, 640, 64
+    x = random_activations(rng, (M, K))
+    xT = dev(np.ascontiguousarray(np.pad(x, ((0, (-M) % 64), (0, 0))).T))
+    for bits in (5, 6):
+        s, sign = random_codes(rng, (N, K), max_s=31)
+        want = oracle.linear(x, -s, sign, None, nthreads=NTHREADS)
+        blob = kernels.tile_weights(dev(so.np_pack_words(s, sign, bits)).reshape(-1), N, K, 1, 1, bits, 0)
+        got = kernels.linear_tiled(xT, M, blob, None, N, bits | _lib.DS_BITS_TOP_UNUSED, 0)
+        np.testing.assert_array_equal(got.cpu().numpy(), want)
+    bits, base = 3, -3
+    sign = random_codes(rng, (N, K))[1]
+    s2 = rng.integers(base, base + 2 ** bits, size=(N, K)).astype(np.int32)  # the top field value occurs
+    w2, ovf = oracle.pack_words(s2, sign, bits, base)
+    assert ovf == 0
+    want = so.np_linear_planes(x, s2, sign, None, base)
+    blob = kernels.tile_weights(dev(w2).reshape(-1), N, K, 1, 1, bits, base)
+    got = kernels.linear_tiled(xT, M, blob, None, N, bits | _lib.DS_BITS_TOP_UNUSED, base)
+    np.testing.assert_array_equal(got.cpu().numpy(), want)
+    one = ctypes.c_void_p(16)
+    assert L.ds_linear_i32(one, one, None, one, 4, 4, 4, 4 | _lib.DS_BITS_TOP_UNUSED, 0, one, 1 << 20, None) == -2
