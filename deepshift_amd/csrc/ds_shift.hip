@@ -301,11 +301,12 @@ constexpr int kPlaneSlotsWide = 2048;  // the 64-channel form holds 246 register
 
 // Main loop of the 32-channel form (six 16-register accumulator vectors) and of the 64-channel form
 // (six of 32 registers).
-// ZT: the blob's highest field value stands for a zero weight (its plane is held at 0).
-template <int BITS, bool ZT>
+// ZT 1: the blob's highest field value stands for a zero weight (its plane is held at 0); 2: no code
+// carries the highest field value (its plane does not exist); 0: every field value is a shift.
+template <int BITS, int ZT>
 __device__ __forceinline__ void planes_main_loop(v16i (&a)[6], const uint32_t (&xoff)[3], v4i rsrc,
                                                  const uint32_t *wptr, int groups, const PlaneWalk &w);
-template <int BITS, bool ZT>
+template <int BITS, int ZT>
 __device__ __forceinline__ void planes_main_loop(v32i (&a)[6], const uint32_t (&xoff)[3], v4i rsrc,
                                                  const uint32_t *wptr, int groups, const PlaneWalk &w);
 #define DS_PLANES_ONE(B, ZT, VEC, ASM, OPERANDS, CLOBBERS)                                         \
@@ -317,10 +318,12 @@ __device__ __forceinline__ void planes_main_loop(v32i (&a)[6], const uint32_t (&
         asm volatile(ASM OPERANDS : CLOBBERS);                                                     \
     }
 #define DS_PLANES_SPECIALISE(B)                                                                    \
-    DS_PLANES_ONE(B, false, v16i, DS_PLANES_ASM_B##B, DS_PLANES_OPERANDS, DS_PLANES_CLOBBERS_B##B)   \
-    DS_PLANES_ONE(B, true, v16i, DS_PLANES_ASM_B##B##Z, DS_PLANES_OPERANDS, DS_PLANES_CLOBBERS_B##B) \
-    DS_PLANES_ONE(B, false, v32i, DS_PLANES_ASM_B##B##W, DS_PLANES_OPERANDS_WIDE, DS_PLANES_CLOBBERS_B##B##W) \
-    DS_PLANES_ONE(B, true, v32i, DS_PLANES_ASM_B##B##ZW, DS_PLANES_OPERANDS_WIDE, DS_PLANES_CLOBBERS_B##B##W)
+    DS_PLANES_ONE(B, 0, v16i, DS_PLANES_ASM_B##B, DS_PLANES_OPERANDS, DS_PLANES_CLOBBERS_B##B)      \
+    DS_PLANES_ONE(B, 1, v16i, DS_PLANES_ASM_B##B##Z, DS_PLANES_OPERANDS, DS_PLANES_CLOBBERS_B##B)   \
+    DS_PLANES_ONE(B, 2, v16i, DS_PLANES_ASM_B##B##U, DS_PLANES_OPERANDS, DS_PLANES_CLOBBERS_B##B##U) \
+    DS_PLANES_ONE(B, 0, v32i, DS_PLANES_ASM_B##B##W, DS_PLANES_OPERANDS_WIDE, DS_PLANES_CLOBBERS_B##B##W) \
+    DS_PLANES_ONE(B, 1, v32i, DS_PLANES_ASM_B##B##ZW, DS_PLANES_OPERANDS_WIDE, DS_PLANES_CLOBBERS_B##B##W) \
+    DS_PLANES_ONE(B, 2, v32i, DS_PLANES_ASM_B##B##UW, DS_PLANES_OPERANDS_WIDE, DS_PLANES_CLOBBERS_B##B##UW)
 DS_PLANES_SPECIALISE(1)
 DS_PLANES_SPECIALISE(2)
 DS_PLANES_SPECIALISE(3)
@@ -330,7 +333,7 @@ DS_PLANES_SPECIALISE(4)
 // channels of `ntile` and the R*64 pixels starting at m0.  `atomic` selects accumulation into a
 // pre-filled output (several segments share the tile) or a plain store of acc + bias.  WIDE: the
 // 64-channel form (layers with N % 64 == 0).
-template <int BITS, bool ZT, bool WIDE, bool TO_LDS = false>
+template <int BITS, int ZT, bool WIDE, bool TO_LDS = false>
 __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, int m0, int g_begin,
                                                int g_end, bool atomic, int32_t *lds = nullptr)
 {
@@ -406,7 +409,7 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
 #pragma unroll
             for (int i = 0; i < NUM; ++i) {
                 if (g * NUM + i >= p.K) break;  // the codes past K trail the word: nothing left to add
-                if (ZT) accumulate_code_zero_top<BITS, R, J>(acc, xt[i], w, i);
+                if (ZT == 1) accumulate_code_zero_top<BITS, R, J>(acc, xt[i], w, i);
                 else accumulate_code<BITS, false, R, J>(acc, xt[i], w, i, 0);
             }
         }
@@ -441,7 +444,7 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
 }
 
 // Tile-per-wave launch: gridDim.y K-slices per tile.
-template <int BITS, bool ZT, bool WIDE>
+template <int BITS, int ZT, bool WIDE>
 __device__ __forceinline__ void planes_tile_body(const ShiftArgs &p)
 {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -461,7 +464,7 @@ __device__ __forceinline__ void planes_tile_body(const ShiftArgs &p)
 // per wave, so every wave of the launch does the same number of group iterations whatever the tile
 // count (each wave touches at most a few tiles; tiles shared between waves are combined with
 // atomic adds onto the pre-filled output).  tiles_m4 holds the number of 192-pixel tiles here.
-template <int BITS, bool ZT, bool WIDE>
+template <int BITS, int ZT, bool WIDE>
 __device__ __forceinline__ void planes_balanced_body(const ShiftArgs &p)
 {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -486,25 +489,25 @@ __device__ __forceinline__ void planes_balanced_body(const ShiftArgs &p)
 }
 
 // 32-channel form: 168 registers, three waves per SIMD; 64-channel form: 256 registers, two.
-template <int BITS, bool ZT>
+template <int BITS, int ZT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void shift_planes_kernel(
     const ShiftArgs p)
 {
     planes_tile_body<BITS, ZT, false>(p);
 }
-template <int BITS, bool ZT>
+template <int BITS, int ZT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void shift_planes_balanced_kernel(
     const ShiftArgs p)
 {
     planes_balanced_body<BITS, ZT, false>(p);
 }
-template <int BITS, bool ZT>
+template <int BITS, int ZT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void shift_planes_wide_kernel(
     const ShiftArgs p)
 {
     planes_tile_body<BITS, ZT, true>(p);
 }
-template <int BITS, bool ZT>
+template <int BITS, int ZT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void shift_planes_wide_balanced_kernel(const ShiftArgs p)
 {
@@ -522,7 +525,7 @@ void shift_planes_wide_balanced_kernel(const ShiftArgs p)
 // WAVES = 8: one workgroup per compute unit, two tile buffers used alternately and one barrier per
 // tile.  WAVES = 4: two workgroups per compute unit, one buffer each and two barriers per tile; the two
 // waves of a SIMD then belong to different workgroups and are not held at the same barrier.
-template <int BITS, bool ZT, int WAVES>
+template <int BITS, int ZT, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void shift_planes_wide_cu_kernel(const ShiftArgs p)
 {
@@ -576,7 +579,7 @@ void shift_planes_wide_cu_kernel(const ShiftArgs p)
     }
 }
 
-template <int BITS, bool ZT, int WAVES>
+template <int BITS, int ZT, int WAVES>
 static int launch_planes_cu(const ShiftArgs &a, long iters, hipStream_t st)
 {
     constexpr int kLdsBytes = (WAVES == 8 ? 2 : 1) * 64 * kPlaneRows * kWave * 4;
@@ -710,7 +713,7 @@ static TileChoice choose_tile(const ShiftArgs &a)
     return c;
 }
 
-template <int BITS, bool ZT, bool WIDE>
+template <int BITS, int ZT, bool WIDE>
 static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
 {
     constexpr int R = kPlaneRows, J = WIDE ? 64 : 32;
@@ -804,7 +807,7 @@ static int dispatch_zero_top(const ShiftArgs &a, hipStream_t st)
     const int r = plane_regime(a, wide);
     int nsplit = (r >= 0 ? r : -1 - r) > 0 ? 1 : 0;
     if (const char *sp = getenv("DS_TUNE_SPLIT")) nsplit = atoi(sp);
-    return wide ? launch_planes<BITS, true, true>(a, nsplit, st) : launch_planes<BITS, true, false>(a, nsplit, st);
+    return wide ? launch_planes<BITS, 1, true>(a, nsplit, st) : launch_planes<BITS, 1, false>(a, nsplit, st);
 }
 
 template <int BITS, bool GENERAL>
@@ -828,12 +831,12 @@ static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
         if (planes) {
             int nsplit = plane_regime(a, wide) > 0 ? 1 : 0;
             if (const char *sp = getenv("DS_TUNE_SPLIT")) nsplit = atoi(sp);
-            // the highest field value unused: the form that holds its plane at 0 saves its shift
+            // the highest field value unused: the form without its plane
             if (a.top_unused)
-                return wide ? launch_planes<BITS, true, true>(a, nsplit, st)
-                            : launch_planes<BITS, true, false>(a, nsplit, st);
-            return wide ? launch_planes<BITS, false, true>(a, nsplit, st)
-                        : launch_planes<BITS, false, false>(a, nsplit, st);
+                return wide ? launch_planes<BITS, 2, true>(a, nsplit, st)
+                            : launch_planes<BITS, 2, false>(a, nsplit, st);
+            return wide ? launch_planes<BITS, 0, true>(a, nsplit, st)
+                        : launch_planes<BITS, 0, false>(a, nsplit, st);
         }
     }
     TileChoice c = choose_tile(a);

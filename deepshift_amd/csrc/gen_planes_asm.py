@@ -13,8 +13,10 @@ VGPR-relative addressing (s_set_gpr_idx_*), which needs a fixed register map:
 
 so a shift-add term costs 1 + 2^BITS/32 vector instructions instead of 2.  Every width also comes in
 a "zero top" form (DS_PLANES_ASM_B<n>Z) in which the plane of the highest field value is held at 0 and
-never computed: for ternary weights re-packed so that this value stands for a zero weight, and for
-layers that do not use it at all (one shift fewer per pixel row and reduction index).
+never computed, for ternary weights re-packed so that this value stands for a zero weight, and in a
+"top unused" form (DS_PLANES_ASM_B<n>U) for layers whose codes never carry that value: the plane does
+not exist (one shift fewer per pixel row and reduction index) and in the 64-channel form of 4-bit
+fields its three registers hold a third slot of the activation prefetch ring.
 
 Register map (R = 3 pixels per lane, J = 32 channels, NUM = 32 // (BITS + 1) codes per word, D = depth
 of the activation prefetch ring in reduction slots, a divisor of NUM):
@@ -62,6 +64,7 @@ import os
 R = 3
 DEPTH = {1: 4, 2: 5, 3: 4, 4: 3}        # prefetch ring depth, 32-channel form
 DEPTH_WIDE = {1: 4, 2: 5, 3: 4, 4: 2}   # 64-channel form: 4-bit fields leave room for two slots only
+DEPTH_WIDE_U = {1: 4, 2: 5, 3: 4, 4: 3}  # 64-channel form without the top plane: its registers buy a third slot
 DEPTH_PAIRED = {1: 4, 2: 2, 3: 1, 4: 1}  # int8 forms: six activation registers per slot
 
 
@@ -159,15 +162,22 @@ def take_turn(tag, waves):
             end + ":"]
 
 
-def body(bits, zero_top=False, wide=False):
+def body(bits, zero_top=False, wide=False, unused_top=False):
+    """zero_top: the plane of the highest field value is held at 0 (it stands for a zero weight).
+    unused_top: no code carries the highest field value, so its plane does not exist: PS planes per
+    row instead of P, and in the 64-channel form of 4-bit fields room for a third prefetch slot."""
+    assert not (zero_top and unused_top)
     f = Form(bits, wide)
+    if unused_top and wide:
+        f.depth = DEPTH_WIDE_U[bits]
     cb = bits + 1
     num = 32 // cb
     P = 1 << bits
+    PS = P - 1 if unused_top else P             # planes per row = register stride between rows
     D, ACC = f.depth, f.acc
     assert num % D == 0 and num % 2 == 0
     PL = XP + R * D
-    assert PL + P * R <= ACC and ACC + R * f.J <= 256
+    assert PL + PS * R <= ACC and ACC + R * f.J <= 256
     L = []
     # ---- prologue: mutable copies of the inputs, the first activation loads and code row
     L += ["s_getreg_b32 s%d, hwreg(HW_REG_HW_ID, 0, 4)" % PRIO,  # the wave's slot on its SIMD
@@ -181,7 +191,7 @@ def body(bits, zero_top=False, wide=False):
         L += walk_and_load(i, f)
     if zero_top:
         # the highest field value contributes nothing: its plane is 0, once and for all
-        L += ["v_mov_b32 v%d, 0" % (PL + P * r + P - 1) for r in range(R)]
+        L += ["v_mov_b32 v%d, 0" % (PL + PS * r + P - 1) for r in range(R)]
     L += ["s_mov_b32 s%d, 0" % IDX, "s_set_gpr_idx_on s%d, 0x1" % IDX]  # src0 of vector ops is M0-relative
     # ---- one K group per iteration
     L += ["1:"]
@@ -213,14 +223,14 @@ def body(bits, zero_top=False, wide=False):
         L += ["s_waitcnt vmcnt(%d)" % (R * (D - 1))]
         # plane 0 = the activation itself (a shift by 0 keeps src0 a constant: not M0-relative)
         for r in range(R):
-            L += ["v_ashrrev_i32 v%d, 0, v%d" % (PL + P * r, XP + R * slot + r)]
+            L += ["v_ashrrev_i32 v%d, 0, v%d" % (PL + PS * r, XP + R * slot + r)]
         L += walk_and_load(slot, f)  # the ring slot is free again: load reduction slot i + D into it
         for s in range(1, P):
             for r in range(R):
-                if zero_top and s == P - 1:
-                    continue  # held at 0 since the prologue
+                if (zero_top or unused_top) and s == P - 1:
+                    continue  # held at 0 since the prologue, or absent
                 else:
-                    L += ["v_ashrrev_i32 v%d, %d, v%d" % (PL + P * r + s, s, PL + P * r)]
+                    L += ["v_ashrrev_i32 v%d, %d, v%d" % (PL + PS * r + s, s, PL + PS * r)]
         # the 16-bit code is a ready M0 value: plane index in 7:0, "src0 relative" in 15:12.  32-channel
         # form: low / high half = even / odd slot of the row; 64-channel form: channel j / j + 32.
         halves = (0, 1) if wide else (i % 2,)
@@ -234,16 +244,18 @@ def body(bits, zero_top=False, wide=False):
                 ch = j + 32 * half if wide else j
                 for r in range(R):
                     a = ACC + f.J * r + ch
-                    L += ["v_xad_u32 v%d, v%d, s%d, v%d" % (a, PL + P * r, MASK, a)]
+                    L += ["v_xad_u32 v%d, v%d, s%d, v%d" % (a, PL + PS * r, MASK, a)]
     L += ["s_sub_u32 s%d, s%d, 1" % (CNT, CNT), "s_cmp_lg_u32 s%d, 0" % CNT, "s_cbranch_scc1 1b"]
     # ---- leave relative addressing, drain the loads that ran ahead of the last slot
     L += ["s_set_gpr_idx_off", "s_setprio 0", "s_waitcnt vmcnt(0) lgkmcnt(0)"]
     return L
 
 
-def clobbers(bits, wide=False):
+def clobbers(bits, wide=False, unused_top=False):
     f = Form(bits, wide)
-    P = 1 << bits
+    if unused_top and wide:
+        f.depth = DEPTH_WIDE_U[bits]
+    P = (1 << bits) - (1 if unused_top else 0)
     v = ['"v%d"' % n for n in range(XP, XP + R * f.depth + P * R)]
     s = ['"s%d"' % n for n in list(range(4, 16)) + list(range(W, WS + 32)) + [TIME, TIME + 1]]
     return ", ".join(v + s + ['"scc"', '"memory"'])
@@ -406,12 +418,13 @@ def main():
     out = ["// Generated by gen_planes_asm.py -- do not edit by hand.", ""]
     for wide, wtag in ((False, ""), (True, "W")):
         for bits in (1, 2, 3, 4):
-            for zero_top, tag in ((False, ""), (True, "Z")):
-                lines = body(bits, zero_top, wide)
+            for zero_top, tag in ((False, ""), (True, "Z"), (False, "U")):
+                lines = body(bits, zero_top, wide, unused_top=tag == "U")
                 out.append("#define DS_PLANES_ASM_B%d%s%s \\" % (bits, tag, wtag))
                 out.append(" \\\n".join('    "%s\\n"' % line for line in lines))
                 out.append("")
             out.append("#define DS_PLANES_CLOBBERS_B%d%s %s" % (bits, wtag, clobbers(bits, wide)))
+            out.append("#define DS_PLANES_CLOBBERS_B%dU%s %s" % (bits, wtag, clobbers(bits, wide, True)))
             out.append("")
     for bits in (1, 2):
         out.append("#define DS_PAIRS_ASM_B%d \\" % bits)
