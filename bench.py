@@ -419,10 +419,10 @@ def main():
             "unit": "Tpair/s",
             "frac": pairs / kernel_s / PEAK_PAIRS,
             # HBM bytes of one launch of the dominant shape (layer1 3x3 conv, 8 of the 21 launches are
-            # this size): 96.0 MB read + 81.1 MB written (tiles shared by two workgroups are combined
+            # this size): 100.4 MB read + 82.7 MB written (tiles shared by two workgroups are combined
             # with atomic adds), from the FETCH_SIZE / WRITE_SIZE runs summarised in
             # profiles/shift_kernel_layer1_conv_counters.md (106.6 MB algorithmic)
-            "traffic": 177.1e6,
+            "traffic": 183.1e6,
             # vector instructions the dominant kernel issues per pair (SQ_INSTS_VALU, same profile):
             # `peak` prices a pair at 2 instructions, so its fraction can exceed 1
             "valu_instr_per_pair": 1.29,
