@@ -426,6 +426,10 @@ def main():
             # vector instructions the dominant kernel issues per pair (SQ_INSTS_VALU, same profile):
             # `peak` prices a pair at 2 instructions, so its fraction can exceed 1
             "valu_instr_per_pair": 1.29,
+            # the same lanes x nominal clock priced at the kernel's own instruction count: the ceiling of
+            # this kernel design, below 1 by the vector-issue gaps (two scalar instructions per code)
+            "peak_at_kernel_mix": PEAK_PAIRS * VALU_INSTR_PER_PAIR / 1.29 / 1e12,
+            "frac_at_kernel_mix": pairs / kernel_s / (PEAK_PAIRS * VALU_INSTR_PER_PAIR / 1.29),
             "avg_launch_us": kernel_s / len(layers) * 1e6,
             "peak_calibrated": peak_cal / 1e12 if peak_cal else None,
             "frac_of_calibrated": pairs / kernel_s / peak_cal if peak_cal else None,
