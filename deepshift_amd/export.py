@@ -35,6 +35,8 @@ def packed_state(model):
         shape = list((m.shift if hasattr(m, "shift") else m.weight).shape)
         entry = {"words": cw.data.detach().cpu(), "bits": int(cw.bits), "base": int(cw.base), "shape": shape,
                  "zero_top_bits": int(getattr(cw, "zero_top_bits", 0))}
+        if getattr(cw, "max_field", None) is not None:
+            entry["max_field"] = int(cw.max_field)  # lets the loader pick the kernel form without the top plane
         if m.bias is not None:
             entry["bias"] = m.bias.detach().float().cpu()
         layers[name] = entry
@@ -72,7 +74,11 @@ def load_packed(model, path_or_state, device=None):
         words = entry["words"].to(dev, torch.int32).contiguous()
         if words.numel() != param.shape[0] * comm:
             raise ValueError("%s: %d packed words, expected %d" % (name, words.numel(), param.shape[0] * comm))
-        m.conc_weight = utils.ConcWeight(words, base, bits, int(entry.get("zero_top_bits", 0)))
+        top = entry.get("max_field")
+        if top is not None and not 0 <= int(top) < 2 ** bits:
+            raise ValueError("%s: max_field %s does not fit %d-bit fields" % (name, top, bits))
+        m.conc_weight = utils.ConcWeight(words, base, bits, int(entry.get("zero_top_bits", 0)),
+                                         None if top is None else int(top))
         m.use_kernel = True
         if "bias" in entry and m.bias is not None:
             with torch.no_grad():

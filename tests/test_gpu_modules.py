@@ -324,9 +324,18 @@ def test_packed_export_round_trip(tmp_path):
                         strict=False)  # BatchNorm statistics and biases; not the shift/sign parameters
     dst = dst.to(DEV)
     assert export.load_packed(dst, path) == n
+    tops = {name: m.conc_weight.max_field for name, m in src.named_modules() if getattr(m, "conc_weight", None)}
+    assert len(tops) == n and all(t is not None and t <= 14 for t in tops.values())
+    for name, m in dst.named_modules():
+        if name in tops:  # the loaded layers run the same kernel form as the ones that were saved
+            assert m.conc_weight.max_field == tops[name]
+            assert kernels.kernel_bits(m.conc_weight) == kernels.kernel_bits(dict(src.named_modules())[name].conc_weight)
     with torch.no_grad():
         got = dst(x)
     assert torch.equal(got, want)
+    blob["layers"][next(iter(blob["layers"]))]["max_field"] = 99
+    with pytest.raises(ValueError):
+        export.load_packed(dst, blob)
 
 
 def test_evaluate_cli_runs_the_three_modes(tmp_path, capsys):
