@@ -83,34 +83,25 @@ inline int pair_chunk(int bits, int x_bound)
       "s"(rsrc), "s"(wptr), "s"(groups), "s"(w.koff), "s"(w.fw), "s"(w.fh), "s"(w.FW), "s"(w.FH), \
       "s"(w.row_step), "s"(w.plane_step), "s"(w.koff_max)
 
-template <int BITS>
+// TU: no code carries the highest field value (index forms only: the blob's plane indices close up
+// over the planes that exist, see tile_paired_kernel).
+template <int BITS, bool TU>
 __device__ __forceinline__ void pairs_main_loop(v32i (&a)[6], const uint32_t (&xoff)[6], v4i rsrc,
                                                 const uint32_t *wptr, int groups, const PairWalk &w);
-template <>
-__device__ __forceinline__ void pairs_main_loop<1>(v32i (&a)[6], const uint32_t (&xoff)[6], v4i rsrc,
-                                                   const uint32_t *wptr, int groups, const PairWalk &w)
-{
-    asm volatile(DS_PAIRS_ASM_B1 DS_PAIRS_OPERANDS : DS_PAIRS_CLOBBERS_B1);
-}
-template <>
-__device__ __forceinline__ void pairs_main_loop<2>(v32i (&a)[6], const uint32_t (&xoff)[6], v4i rsrc,
-                                                   const uint32_t *wptr, int groups, const PairWalk &w)
-{
-    asm volatile(DS_PAIRS_ASM_B2 DS_PAIRS_OPERANDS : DS_PAIRS_CLOBBERS_B2);
-}
-
-template <>
-__device__ __forceinline__ void pairs_main_loop<3>(v32i (&a)[6], const uint32_t (&xoff)[6], v4i rsrc,
-                                                   const uint32_t *wptr, int groups, const PairWalk &w)
-{
-    asm volatile(DS_PAIRX_ASM_B3 DS_PAIRS_OPERANDS : DS_PAIRX_CLOBBERS_B3);
-}
-template <>
-__device__ __forceinline__ void pairs_main_loop<4>(v32i (&a)[6], const uint32_t (&xoff)[6], v4i rsrc,
-                                                   const uint32_t *wptr, int groups, const PairWalk &w)
-{
-    asm volatile(DS_PAIRX_ASM_B4 DS_PAIRS_OPERANDS : DS_PAIRX_CLOBBERS_B4);
-}
+#define DS_PAIRS_ONE(B, TU, ASM, CLOBBERS)                                                            \
+    template <>                                                                                       \
+    __device__ __forceinline__ void pairs_main_loop<B, TU>(v32i (&a)[6], const uint32_t (&xoff)[6],   \
+                                                           v4i rsrc, const uint32_t *wptr, int groups, \
+                                                           const PairWalk &w)                         \
+    {                                                                                                 \
+        asm volatile(ASM DS_PAIRS_OPERANDS : CLOBBERS);                                               \
+    }
+DS_PAIRS_ONE(1, false, DS_PAIRS_ASM_B1, DS_PAIRS_CLOBBERS_B1)
+DS_PAIRS_ONE(1, true, DS_PAIRS_ASM_B1U, DS_PAIRS_CLOBBERS_B1U)
+DS_PAIRS_ONE(2, false, DS_PAIRS_ASM_B2, DS_PAIRS_CLOBBERS_B2)
+DS_PAIRS_ONE(2, true, DS_PAIRS_ASM_B2U, DS_PAIRS_CLOBBERS_B2U)
+DS_PAIRS_ONE(3, false, DS_PAIRX_ASM_B3, DS_PAIRX_CLOBBERS_B3)
+DS_PAIRS_ONE(4, false, DS_PAIRX_ASM_B4, DS_PAIRX_CLOBBERS_B4)
 
 // K groups [g_begin, g_end) (at most PairArgs::chunk of them) of the tile made of the 64 channels of
 // `ntile` and the 384 pixels from m0.
@@ -118,7 +109,7 @@ __device__ __forceinline__ void pairs_main_loop<4>(v32i (&a)[6], const uint32_t 
 // pre-filled y) or kLds (add to the workgroup's tile buffer lds[channel][pixel of the tile]).
 enum { kStore, kAtomic, kLds };
 
-template <int BITS, int OUT>
+template <int BITS, int OUT, bool TU>
 __device__ __forceinline__ void pairs_segment(const PairArgs &p, int ntile, int m0, int g_begin, int g_end,
                                               int32_t *lds)
 {
@@ -159,7 +150,7 @@ __device__ __forceinline__ void pairs_segment(const PairArgs &p, int ntile, int 
         w.plane_step = p.x_plane - p.FH * p.x_row;
         // reduction indices past K (the codes there select the zero plane) read the last real one
         w.koff_max = (p.K / ff - 1) * p.x_plane + (p.FH - 1) * p.x_row + p.FW - 1;
-        pairs_main_loop<BITS>(a, xoff, rsrc,
+        pairs_main_loop<BITS, TU>(a, xoff, rsrc,
                               p.codes + ((size_t)ntile * p.comm + g_begin) * NUM * kTileWords,
                               __builtin_amdgcn_readfirstlane(g_end - g_begin), w);
     }
@@ -212,7 +203,7 @@ __device__ __forceinline__ void pairs_segment(const PairArgs &p, int ntile, int 
 }
 
 // One tile per wave, for reductions of a single chunk: plain stores of acc + bias.
-template <int BITS>
+template <int BITS, bool TU>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void shift_pairs_kernel(
     const PairArgs p)
 {
@@ -222,11 +213,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int tile = p.tile_begin + tile4 * 4 + wave;  // neighbouring channel tiles of a pixel range share a workgroup
     if (tile >= p.tile_end) return;
     const int mt = tile / p.tiles_n, ntile = tile - mt * p.tiles_n;
-    pairs_segment<BITS, kStore>(p, ntile, mt * kPairPixels, 0, p.comm, nullptr);
+    pairs_segment<BITS, kStore, TU>(p, ntile, mt * kPairPixels, 0, p.comm, nullptr);
 }
 
 // Equal shares of the (tile, K group) space, one per wave slot, as in the int32 kernel.
-template <int BITS>
+template <int BITS, bool TU>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void shift_pairs_balanced_kernel(
     const PairArgs p)
 {
@@ -244,7 +235,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         if (g_end > p.comm) g_end = p.comm;
         if (g_end > g_begin + p.chunk) g_end = g_begin + p.chunk;
         const int ntile = tile % p.tiles_n;
-        pairs_segment<BITS, kAtomic>(p, ntile, (tile / p.tiles_n) * kPairPixels, g_begin, g_end, nullptr);
+        pairs_segment<BITS, kAtomic, TU>(p, ntile, (tile / p.tiles_n) * kPairPixels, g_begin, g_end, nullptr);
         it += g_end - g_begin;
     }
 }
@@ -259,7 +250,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 constexpr int kPairCuWaves = 8;
 constexpr int kPairLdsBytes = 64 * kPairPixels * 4;
 
-template <int BITS>
+template <int BITS, bool TU>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void shift_pairs_cu_kernel(
     const PairArgs p)
 {
@@ -290,7 +281,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int wb = g0 + wave * len / kPairCuWaves, we = g0 + (wave + 1) * len / kPairCuWaves;
         for (int g = wb; g < we; g += p.chunk) {
             const int ge = g + p.chunk < we ? g + p.chunk : we;
-            pairs_segment<BITS, kLds>(p, ntile, m0, g, ge, tile_sums);
+            pairs_segment<BITS, kLds, TU>(p, ntile, m0, g, ge, tile_sums);
         }
         __syncthreads();
         const bool whole = len == p.comm;
@@ -339,14 +330,14 @@ __global__ void pairs_fill_kernel(const PairArgs p)
 // The tile buffer is above the default 64 KiB limit of a workgroup: opt in, once per device.  Also
 // called when a weight blob is laid out, so that the first convolution launch -- which may be under
 // stream capture -- finds it done.
-template <int BITS>
+template <int BITS, bool TU>
 static int pairs_opt_in_lds()
 {
     static bool opted_in[64] = {};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
     if (!opted_in[dev]) {
-        hipError_t e = hipFuncSetAttribute((const void *)shift_pairs_cu_kernel<BITS>,
+        hipError_t e = hipFuncSetAttribute((const void *)shift_pairs_cu_kernel<BITS, TU>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kPairLdsBytes);
         if (e != hipSuccess) return hip_status(e);
         opted_in[dev] = true;
@@ -354,15 +345,15 @@ static int pairs_opt_in_lds()
     return DS_OK;
 }
 
-template <int BITS>
+template <int BITS, bool TU>
 static int launch_pairs_cu(const PairArgs &a, int blocks, hipStream_t st)
 {
-    if (int rc = pairs_opt_in_lds<BITS>()) return rc;
-    hipLaunchKernelGGL((shift_pairs_cu_kernel<BITS>), dim3(blocks), dim3(512), kPairLdsBytes, st, a);
+    if (int rc = pairs_opt_in_lds<BITS, TU>()) return rc;
+    hipLaunchKernelGGL((shift_pairs_cu_kernel<BITS, TU>), dim3(blocks), dim3(512), kPairLdsBytes, st, a);
     return launch_status();
 }
 
-template <int BITS>
+template <int BITS, bool TU>
 static int launch_pairs(PairArgs a, hipStream_t st)
 {
     a.tiles_m = ceil_div(a.M, kPairPixels);
@@ -393,13 +384,13 @@ static int launch_pairs(PairArgs a, hipStream_t st)
         a.atomic_out = 0;
         a.tile_end = (int)head;
         a.blocks_per_xcd = ceil_div((int)ceil_div((int)head, 4), 8);
-        hipLaunchKernelGGL((shift_pairs_kernel<BITS>), dim3(a.blocks_per_xcd * 8), dim3(256), 0, st, a);
+        hipLaunchKernelGGL((shift_pairs_kernel<BITS, TU>), dim3(a.blocks_per_xcd * 8), dim3(256), 0, st, a);
         if (head == tiles) return launch_status();
         a.tile_begin = (int)head;
         a.tile_end = (int)tiles;
         a.whole_tiles = 1;
         const long rest_blocks = (rest + 7) / 8 * 8;
-        return launch_pairs_cu<BITS>(a, rest_blocks < 256 ? (int)rest_blocks : 256, st);
+        return launch_pairs_cu<BITS, TU>(a, rest_blocks < 256 ? (int)rest_blocks : 256, st);
     }
     a.atomic_out = 1;
     long fill_blocks = ((long)a.y_elems / 4 + 255) / 256;
@@ -410,12 +401,12 @@ static int launch_pairs(PairArgs a, hipStream_t st)
         int blocks = 256;
         const long fit = (iters / 64) / 8 * 8;  // small layers: at least 8 K groups per wave
         if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
-        return launch_pairs_cu<BITS>(a, blocks, st);
+        return launch_pairs_cu<BITS, TU>(a, blocks, st);
     }
     int blocks = kPairSlots / 4;
     const long fit = (iters / 16) / 8 * 8;  // small layers: at least 4 K groups per wave
     if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
-    hipLaunchKernelGGL((shift_pairs_balanced_kernel<BITS>), dim3(blocks), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((shift_pairs_balanced_kernel<BITS, TU>), dim3(blocks), dim3(256), 0, st, a);
     return launch_status();
 }
 
@@ -440,13 +431,18 @@ static PairedGeom paired_geom(int N, int K, int bits)
 // Reference-format words [N][in_comm] (fields of in_bits) -> plane indices of `bits`-wide fields:
 // word j of row (t, k) = index(k, channel 64t + j) | index(k, channel 64t + 32 + j) << 16, each with
 // "src0 is relative" (bit 12) set so that the half-word is a ready M0 value.
+// `shifts`: number of planes per sign of the index forms: 2^bits, or 2^bits - 1 for a blob whose codes
+// never carry the highest field value (a code that does would select the wrong plane; never a
+// register outside the planes).
 __global__ void tile_paired_kernel(const int32_t *__restrict__ w_ref, uint32_t *__restrict__ out, int N,
-                                   int K, int comm, int bits, int num, long words, int in_bits, int in_comm)
+                                   int K, int comm, int bits, int num, long words, int in_bits, int in_comm,
+                                   int shifts)
 {
     const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= words) return;
     const bool xor_mask = bits >= 3;  // field in 7:0, negative in bit 8; the highest field value = nothing
-    const uint32_t P = 1u << bits, zero = xor_mask ? (0x1000u | (P - 1u)) : (0x1000u | (2u * P));
+    const uint32_t P = 1u << bits, S = (uint32_t)shifts;
+    const uint32_t zero = xor_mask ? (0x1000u | (P - 1u)) : (0x1000u | (2u * S));
     const int j = (int)(idx % kTileWords);
     const long rest = idx / kTileWords;
     const long rows = (long)comm * num;
@@ -465,7 +461,7 @@ __global__ void tile_paired_kernel(const int32_t *__restrict__ w_ref, uint32_t *
             uint32_t index = zero;                      // fields >= 32 (6-bit words): zero weight
             if (field < 32u)
                 index = 0x1000u | (xor_mask ? ((field & (P - 1u)) | (positive ? 0u : 0x100u))
-                                            : ((field & (P - 1u)) + (positive ? 0u : P)));
+                                            : (min(field & (P - 1u), S - 1u) + (positive ? 0u : S)));
             word |= index << (16 * c);
         }
     }
@@ -497,6 +493,15 @@ __global__ __launch_bounds__(256) void paired_negcount_kernel(const int32_t *__r
 
 using namespace ds;
 
+// Splits DS_BITS_TOP_UNUSED off the field width; it applies to the index forms (1 and 2 bits) and is
+// ignored by the xor-mask forms, whose highest field value is reserved anyway.
+static bool take_paired_top_unused(int &bits)
+{
+    const bool flag = (bits & DS_BITS_TOP_UNUSED) != 0;
+    bits &= ~DS_BITS_TOP_UNUSED;
+    return flag && bits >= 1 && bits <= 2;
+}
+
 static int check_paired(int N, int C, int FH, int FW, int bits)
 {
     if (bits < 1 || bits > 4) return DS_EBITS;
@@ -507,6 +512,7 @@ static int check_paired(int N, int C, int FH, int FW, int bits)
 
 DS_EXPORT size_t ds_paired_bytes(int N, int K, int field_bits)
 {
+    field_bits &= ~DS_BITS_TOP_UNUSED;
     if (field_bits < 1 || field_bits > 4 || N < 0 || K < 0 || N % 64 != 0) return 0;
     return paired_geom(N, K, field_bits).bytes;
 }
@@ -514,16 +520,17 @@ DS_EXPORT size_t ds_paired_bytes(int N, int K, int field_bits)
 DS_EXPORT int ds_tile_weights_paired_i32(const int32_t *w_ref, void *paired, int N, int C, int FH, int FW,
                                          int ref_bits, int field_bits, ds_stream_t stream)
 {
+    const bool top_unused = take_paired_top_unused(field_bits);
     int rc = check_paired(N, C, FH, FW, field_bits);
     if (rc) return rc;
     if (ref_bits != field_bits && ref_bits != 6) return DS_EBITS;
     if (N == 0) return DS_OK;
     if (!paired || (!w_ref && C > 0)) return DS_EINVAL;
     switch (field_bits) {
-    case 1: rc = pairs_opt_in_lds<1>(); break;
-    case 2: rc = pairs_opt_in_lds<2>(); break;
-    case 3: rc = pairs_opt_in_lds<3>(); break;
-    default: rc = pairs_opt_in_lds<4>(); break;
+    case 1: rc = top_unused ? pairs_opt_in_lds<1, true>() : pairs_opt_in_lds<1, false>(); break;
+    case 2: rc = top_unused ? pairs_opt_in_lds<2, true>() : pairs_opt_in_lds<2, false>(); break;
+    case 3: rc = pairs_opt_in_lds<3, false>(); break;
+    default: rc = pairs_opt_in_lds<4, false>(); break;
     }
     if (rc) return rc;
     const int K = C * FH * FW;
@@ -532,7 +539,7 @@ DS_EXPORT int ds_tile_weights_paired_i32(const int32_t *w_ref, void *paired, int
     const int in_comm = ceil_div(K, codes_per_word(ref_bits));
     hipLaunchKernelGGL(tile_paired_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0,
                        (hipStream_t)stream, w_ref, (uint32_t *)paired, N, K, g.comm, field_bits, g.num, words,
-                       ref_bits, in_comm);
+                       ref_bits, in_comm, (1 << field_bits) - (top_unused ? 1 : 0));
     if (field_bits >= 3)
         hipLaunchKernelGGL(paired_negcount_kernel, dim3(ceil_div(N, 4)), dim3(256), 0, (hipStream_t)stream, w_ref,
                            (int32_t *)((char *)paired + g.negcnt_offset), N, K, ref_bits, in_comm);
@@ -543,6 +550,7 @@ DS_EXPORT int ds_conv2d_paired_i8(const int8_t *x, const void *paired, const int
                                   int Nb, int C, int Hp, int Wp, int O, int FH, int FW, int sh, int sw,
                                   int field_bits, int x_bound, ds_stream_t stream)
 {
+    const bool top_unused = take_paired_top_unused(field_bits);
     int rc = check_paired(O, C, FH, FW, field_bits);
     if (rc) return rc;
     if (Nb < 0 || sh < 1 || sw < 1 || Hp < FH || Wp < FW || x_bound < 1 || x_bound > 128) return DS_EINVAL;
@@ -580,9 +588,9 @@ DS_EXPORT int ds_conv2d_paired_i8(const int8_t *x, const void *paired, const int
         return launch_status();
     }
     switch (field_bits) {
-    case 1: return launch_pairs<1>(a, (hipStream_t)stream);
-    case 2: return launch_pairs<2>(a, (hipStream_t)stream);
-    case 3: return launch_pairs<3>(a, (hipStream_t)stream);
-    default: return launch_pairs<4>(a, (hipStream_t)stream);
+    case 1: return top_unused ? launch_pairs<1, true>(a, (hipStream_t)stream) : launch_pairs<1, false>(a, (hipStream_t)stream);
+    case 2: return top_unused ? launch_pairs<2, true>(a, (hipStream_t)stream) : launch_pairs<2, false>(a, (hipStream_t)stream);
+    case 3: return launch_pairs<3, false>(a, (hipStream_t)stream);
+    default: return launch_pairs<4, false>(a, (hipStream_t)stream);
     }
 }

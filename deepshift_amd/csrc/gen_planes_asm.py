@@ -66,6 +66,7 @@ DEPTH = {1: 4, 2: 5, 3: 4, 4: 3}        # prefetch ring depth, 32-channel form
 DEPTH_WIDE = {1: 4, 2: 5, 3: 4, 4: 2}   # 64-channel form: 4-bit fields leave room for two slots only
 DEPTH_WIDE_U = {1: 4, 2: 5, 3: 4, 4: 3}  # 64-channel form without the top plane: its registers buy a third slot
 DEPTH_PAIRED = {1: 4, 2: 2, 3: 1, 4: 1}  # int8 forms: six activation registers per slot
+DEPTH_PAIRED_U = {1: 4, 2: 5}            # index forms without the planes of the top field value
 
 
 class Form:
@@ -261,11 +262,15 @@ def clobbers(bits, wide=False, unused_top=False):
     return ", ".join(v + s + ['"scc"', '"memory"'])
 
 
-def body_paired(bits):
-    """The int8 form: 3 rows x 2 pixels x 64 channels per lane (see the module docstring)."""
+def body_paired(bits, unused_top=False):
+    """The int8 form: 3 rows x 2 pixels x 64 channels per lane (see the module docstring).
+    unused_top: no code carries the highest field value; P counts the shifts that exist, the plane
+    indices close up (field, P + field, 2P) and the registers saved deepen the prefetch ring."""
     f = Form(bits, True, paired=True)
+    if unused_top:
+        f.depth = DEPTH_PAIRED_U[bits]
     num = 32 // (bits + 1)
-    P = 1 << bits
+    P = (1 << bits) - (1 if unused_top else 0)
     S = 2 * P + 1                               # planes per row: shifts, negated shifts, zero
     D, ACC = f.depth, f.acc
     assert num % D == 0 and num % 2 == 0
@@ -405,9 +410,11 @@ def clobbers_pairx(bits):
     return ", ".join(v + s + ['"scc"', '"memory"'])
 
 
-def clobbers_paired(bits):
+def clobbers_paired(bits, unused_top=False):
     f = Form(bits, True, paired=True)
-    P = 1 << bits
+    if unused_top:
+        f.depth = DEPTH_PAIRED_U[bits]
+    P = (1 << bits) - (1 if unused_top else 0)
     v = ['"v%d"' % n for n in range(XP, XP + 2 * R * f.depth + (2 * P + 1) * R)]
     s = ['"s%d"' % n for n in list(range(4, 16)) + list(range(W, WS + 32)) + [TIME, TIME + 1]]
     return ", ".join(v + s + ['"scc"', '"memory"'])
@@ -431,6 +438,11 @@ def main():
         out.append(" \\\n".join('    "%s\\n"' % line for line in body_paired(bits)))
         out.append("")
         out.append("#define DS_PAIRS_CLOBBERS_B%d %s" % (bits, clobbers_paired(bits)))
+        out.append("")
+        out.append("#define DS_PAIRS_ASM_B%dU \\" % bits)
+        out.append(" \\\n".join('    "%s\\n"' % line for line in body_paired(bits, True)))
+        out.append("")
+        out.append("#define DS_PAIRS_CLOBBERS_B%dU %s" % (bits, clobbers_paired(bits, True)))
         out.append("")
     for bits in (3, 4):
         out.append("#define DS_PAIRX_ASM_B%d \\" % bits)

@@ -162,7 +162,8 @@ def _tiled_of(conc_weight, N, C, FH=1, FW=1):
 
 def paired_fields(conc_weight, out_channels, integer_bits, fraction_bits):
     """``(ref_bits, field_bits)`` when a layer can run on the int8 kernel (two pixels per register),
-    else ``None``: activations of at most 8 bits (and not the one-bit format), a channel count that is a
+    else ``None`` (``field_bits`` as the int8 entry points take it, i.e. with ``DS_BITS_TOP_UNUSED`` set
+    for 1- and 2-bit fields whose highest value does not occur): activations of at most 8 bits (and not the one-bit format), a channel count that is a
     multiple of 64, base 0, and shift fields of at most 4 bits -- either packed that narrow, or 6-bit
     ternary words whose non-zero fields are that narrow.  Fields of 3 and 4 bits must leave their
     highest value unused (weight_bits 5 clamps shifts to [-14, 0] for exactly this, modules.py:88): the
@@ -172,6 +173,10 @@ def paired_fields(conc_weight, out_channels, integer_bits, fraction_bits):
     if conc_weight is None or conc_weight.base != 0:
         return None
     if conc_weight.bits <= 2:
+        top = getattr(conc_weight, "max_field", None)
+        if top is not None and top <= 2 ** conc_weight.bits - 2:
+            # the highest field value does not occur: the kernel form without its planes
+            return (conc_weight.bits, conc_weight.bits | _lib.DS_BITS_TOP_UNUSED)
         return (conc_weight.bits, conc_weight.bits)
     if conc_weight.bits <= 4:
         top = getattr(conc_weight, "max_field", None)
@@ -180,7 +185,8 @@ def paired_fields(conc_weight, out_channels, integer_bits, fraction_bits):
         return None
     width = getattr(conc_weight, "zero_top_bits", 0)
     if conc_weight.bits == 6 and 1 <= width <= 4:
-        return (6, width)  # zero_top_bits: the non-zero fields are all <= 2**width - 2
+        # zero_top_bits: the non-zero fields are all <= 2**width - 2, so the top value is free here too
+        return (6, width | _lib.DS_BITS_TOP_UNUSED if width <= 2 else width)
     return None
 
 

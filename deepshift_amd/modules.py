@@ -208,7 +208,7 @@ def _small_for_int8(module, input_shape, field_bits):
     OW = (W + 2 * pw - module.kernel_size[1]) // module.stride[1] + 1
     tiles = -(-Nb * OH * OW // 384) * (module.out_channels // 64)
     K = module.in_channels * module.kernel_size[0] * module.kernel_size[1]
-    groups = -(-K // (32 // (field_bits + 1)))
+    groups = -(-K // (32 // ((field_bits & 0xff) + 1)))
     return tiles * groups < 8192
 
 

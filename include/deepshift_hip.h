@@ -104,7 +104,13 @@ int ds_tile_weights_zero_top_i32(const int32_t *w_ref, void *tiled, int N, int C
  * non-zero fields fit field_bits (zero weights, fields >= 32, then contribute nothing).
  * With field_bits 3 or 4 the kernel takes the highest field value (7 / 15) for "no contribution":
  * the caller vouches that no non-zero weight uses it -- true of every layer whose shifts were clamped
- * to the reference's range for its weight_bits, (-(2^(weight_bits-1) - 2), 0) (modules.py:88). */
+ * to the reference's range for its weight_bits, (-(2^(weight_bits-1) - 2), 0) (modules.py:88).
+ * With field_bits 1 or 2 the highest value (1 / 3) is an ordinary shift; a caller who knows that no
+ * non-zero weight uses it (the same clamp, weight_bits 2 and 3) may pass field_bits |
+ * DS_BITS_TOP_UNUSED to ds_tile_weights_paired_i32 AND to ds_conv2d_paired_i8 with that blob: the
+ * kernel then leaves the planes of that shift out (and prefetches activations deeper with their
+ * registers).  Same results; a weight that does carry the value is computed with the next lower
+ * shift.  The flag is ignored for field_bits 3 and 4. */
 size_t ds_paired_bytes(int N, int K, int field_bits);
 int ds_tile_weights_paired_i32(const int32_t *w_ref, void *paired, int N, int C, int FH, int FW,
                                int ref_bits, int field_bits, ds_stream_t stream);
@@ -112,7 +118,7 @@ int ds_tile_weights_paired_i32(const int32_t *w_ref, void *paired, int N, int C,
 /* Conv2dShift forward on int8 activations: ds_conv2d_tiled_i32 (DEEP_SHIFT_CONV,
  * kernels/cuda/shift_cuda.cpp:41-53) with x int8 [Nb][C][Hp][Wp], already padded, and the blob of
  * ds_tile_weights_paired_i32.  y int32 [Nb][O][OH][OW].  DS_EINVAL when O % 64 != 0, DS_EBITS when
- * field_bits is not 1..4.
+ * field_bits is not 1..4 (with or without DS_BITS_TOP_UNUSED, which must match the blob's).
  * x_bound (1..128): the caller vouches that every |x| <= x_bound.  128 is always true; a smaller
  * bound lets the kernel run 32767 / x_bound (field_bits 3, 4: 32767 / (x_bound + 1)) reduction
  * indices between two widenings of its 16-bit sums -- e.g. 96 for the output of a ReLU in the 3.5 format, whose round-to-fixed clamp

@@ -50,9 +50,20 @@ def random_int8(rng, shape):
     return x
 
 
-def top_field(bits):
-    """Largest shift field a real code may carry: the xor-mask forms (3, 4 bits) reserve the highest."""
-    return 2 ** bits - 1 if bits <= 2 else 2 ** bits - 2
+U = _lib.DS_BITS_TOP_UNUSED
+# kernel forms: the field width, for 1 and 2 bits also with "the highest field value does not occur"
+FORMS = [1, 2, 3, 4, 1 | U, 2 | U]
+
+
+def form_id(form):
+    return "%d%s" % (form & 0xff, "U" if form & U else "")
+
+
+def top_field(form):
+    """Largest shift field a real code may carry: the xor-mask forms (3, 4 bits) reserve the highest, and
+    so does the caller of a top-unused form."""
+    bits = form & 0xff
+    return 2 ** bits - 1 if form in (1, 2) else 2 ** bits - 2
 
 
 SHAPES = [
@@ -67,45 +78,48 @@ SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("bits", [1, 2, 3, 4])
+@pytest.mark.parametrize("form", FORMS, ids=form_id)
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s[:7])))
-def test_paired_convolution_matches_oracle(oracle, rng, bits, shape):
+def test_paired_convolution_matches_oracle(oracle, rng, form, shape):
     Nb, C, Hp, Wp, O, FH, FW, stride = shape
+    bits = form & 0xff
     x8 = random_int8(rng, (Nb, C, Hp, Wp))
-    s, sign = random_codes(rng, (O, C, FH, FW), max_s=top_field(bits))
+    s, sign = random_codes(rng, (O, C, FH, FW), max_s=top_field(form))
     bias = rng.integers(-2 ** 20, 2 ** 20, size=O).astype(np.int32)
     w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)
     want = oracle.conv2d(x8.astype(np.int32), -s, sign, bias, stride, nthreads=NTHREADS)
-    blob = abi_tile_paired(w, O, C, FH, FW, bits, bits)
-    got = abi_conv_paired(x8, blob, bias, O, FH, FW, stride, bits)
+    blob = abi_tile_paired(w, O, C, FH, FW, bits, form)
+    got = abi_conv_paired(x8, blob, bias, O, FH, FW, stride, form)
     np.testing.assert_array_equal(got, want)
 
 
-@pytest.mark.parametrize("bits", [1, 2, 3, 4])
-def test_paired_extreme_sums_do_not_overflow_the_halves(oracle, bits):
+@pytest.mark.parametrize("form", FORMS, ids=form_id)
+def test_paired_extreme_sums_do_not_overflow_the_halves(oracle, form):
     """Every activation -128 (or 127) and every code +(x >> 0): the 16-bit sums reach their bound."""
     Nb, C, Hp, Wp, O = 1, 600, 20, 20, 64
+    bits = form & 0xff
     for fill, sgn in ((-128, 1), (-128, -1), (127, 1), (127, -1)):
         x8 = np.full((Nb, C, Hp, Wp), fill, np.int8)
         s = np.zeros((O, C, 1, 1), np.int32)
         sign = np.full((O, C, 1, 1), sgn, np.int32)
         w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)
         want = oracle.conv2d(x8.astype(np.int32), -s, sign, None, (1, 1), nthreads=NTHREADS)
-        blob = abi_tile_paired(w, O, C, 1, 1, bits, bits)
-        np.testing.assert_array_equal(abi_conv_paired(x8, blob, None, O, 1, 1, (1, 1), bits), want)
+        blob = abi_tile_paired(w, O, C, 1, 1, bits, form)
+        np.testing.assert_array_equal(abi_conv_paired(x8, blob, None, O, 1, 1, (1, 1), form), want)
 
 
-@pytest.mark.parametrize("bits", [1, 2, 3, 4])
-def test_paired_ternary_words(oracle, rng, bits):
+@pytest.mark.parametrize("form", FORMS, ids=form_id)
+def test_paired_ternary_words(oracle, rng, form):
     """6-bit reference words of a ternary layer: zero weights select the zero plane."""
     Nb, C, Hp, Wp, O, FH, FW = 2, 40, 12, 12, 64, 3, 3
+    bits = form & 0xff
     x8 = random_int8(rng, (Nb, C, Hp, Wp))
-    s, sign = random_codes(rng, (O, C, FH, FW), max_s=top_field(bits), zero_frac=0.4)
+    s, sign = random_codes(rng, (O, C, FH, FW), max_s=top_field(form), zero_frac=0.4)
     s6 = np.where(sign == 0, 32, s).astype(np.int32)
     w, _ = oracle.pack_words(s6.reshape(O, -1), np.where(sign == 0, 1, sign).reshape(O, -1), 6)
     want = oracle.conv2d(x8.astype(np.int32), -s, sign, None, (1, 1), nthreads=NTHREADS)
-    blob = abi_tile_paired(w, O, C, FH, FW, 6, bits)
-    np.testing.assert_array_equal(abi_conv_paired(x8, blob, None, O, FH, FW, (1, 1), bits), want)
+    blob = abi_tile_paired(w, O, C, FH, FW, 6, form)
+    np.testing.assert_array_equal(abi_conv_paired(x8, blob, None, O, FH, FW, (1, 1), form), want)
 
 
 def test_paired_refusals():
@@ -121,12 +135,13 @@ def test_paired_refusals():
             _lib.call("ds_conv2d_paired_i8", None, None, None, None, 1, 1, 3, 3, 64, 1, 1, 1, 1, 2, bound, stream())
 
 
-@pytest.mark.parametrize("bits", [1, 2, 3, 4])
+@pytest.mark.parametrize("form", FORMS, ids=form_id)
 @pytest.mark.parametrize("bound", [96, 17, 1])
-def test_paired_vouched_bound_lengthens_the_chunks(oracle, rng, bits, bound):
+def test_paired_vouched_bound_lengthens_the_chunks(oracle, rng, form, bound):
     """Activations within [-bound, bound], every one at the bound with the same sign where it hurts
     most: 32767 // bound reduction indices per chunk must still not overflow a half."""
     O, FH, FW = 64, 1, 1
+    bits = form & 0xff
     for C in (256, 32767 // bound, 32767 // bound + 7, 1200):
         C = min(C, 4000)
         for fill, sgn in ((bound, 1), (bound, -1), (-bound, 1), (-bound, -1)):
@@ -135,15 +150,15 @@ def test_paired_vouched_bound_lengthens_the_chunks(oracle, rng, bits, bound):
             sign = np.full((O, C, 1, 1), sgn, np.int32)
             w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)
             want = oracle.conv2d(x8.astype(np.int32), -s, sign, None, (1, 1), nthreads=NTHREADS)
-            blob = abi_tile_paired(w, O, C, 1, 1, bits, bits)
-            got = abi_conv_paired(x8, blob, None, O, 1, 1, (1, 1), bits, bound)
+            blob = abi_tile_paired(w, O, C, 1, 1, bits, form)
+            got = abi_conv_paired(x8, blob, None, O, 1, 1, (1, 1), form, bound)
             np.testing.assert_array_equal(got, want, err_msg=str((C, fill, sgn)))
     x8 = rng.integers(-bound, bound + 1, size=(3, 300, 9, 9)).astype(np.int8)
-    s, sign = random_codes(rng, (128, 300, 3, 3), max_s=top_field(bits))
+    s, sign = random_codes(rng, (128, 300, 3, 3), max_s=top_field(form))
     w, _ = oracle.pack_words(s.reshape(128, -1), sign.reshape(128, -1), bits)
     want = oracle.conv2d(x8.astype(np.int32), -s, sign, None, (1, 1), nthreads=NTHREADS)
-    blob = abi_tile_paired(w, 128, 300, 3, 3, bits, bits)
-    np.testing.assert_array_equal(abi_conv_paired(x8, blob, None, 128, 3, 3, (1, 1), bits, bound), want)
+    blob = abi_tile_paired(w, 128, 300, 3, 3, bits, form)
+    np.testing.assert_array_equal(abi_conv_paired(x8, blob, None, 128, 3, 3, (1, 1), form, bound), want)
 
 
 # ----------------------------------------------------------------------------- conversion passes
@@ -229,10 +244,11 @@ def test_models_with_8_bit_activations_take_the_int8_kernel_and_keep_their_outpu
     assert torch.equal(unfused, want_unfused)
 
 
-@pytest.mark.parametrize("seed", range(16))
+@pytest.mark.parametrize("seed", range(24))
 def test_random_int8_convolutions(oracle, seed):
     rng = np.random.default_rng(4000 + seed)
-    bits = int(rng.integers(1, 5))
+    form = FORMS[int(rng.integers(0, len(FORMS)))] if seed >= 16 else int(rng.integers(1, 5))
+    bits = form & 0xff
     FH, FW = int(rng.integers(1, 6)), int(rng.integers(1, 6))
     sh, sw = int(rng.integers(1, 4)), int(rng.integers(1, 4))
     Nb = int(rng.integers(1, 9))
@@ -240,13 +256,13 @@ def test_random_int8_convolutions(oracle, seed):
     O = int(rng.choice([64, 128, 192]))
     Hp, Wp = FH + int(rng.integers(0, 30)), FW + int(rng.integers(0, 30))
     x8 = random_int8(rng, (Nb, C, Hp, Wp))
-    s, sign = random_codes(rng, (O, C, FH, FW), max_s=top_field(bits))
+    s, sign = random_codes(rng, (O, C, FH, FW), max_s=top_field(form))
     bias = rng.integers(-2 ** 20, 2 ** 20, size=O).astype(np.int32) if seed % 2 else None
     w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)
     want = oracle.conv2d(x8.astype(np.int32), -s, sign, bias, (sh, sw), nthreads=NTHREADS)
-    blob = abi_tile_paired(w, O, C, FH, FW, bits, bits)
-    got = abi_conv_paired(x8, blob, bias, O, FH, FW, (sh, sw), bits)
-    np.testing.assert_array_equal(got, want, err_msg=str((bits, Nb, C, Hp, Wp, O, FH, FW, sh, sw)))
+    blob = abi_tile_paired(w, O, C, FH, FW, bits, form)
+    got = abi_conv_paired(x8, blob, bias, O, FH, FW, (sh, sw), form)
+    np.testing.assert_array_equal(got, want, err_msg=str((form_id(form), Nb, C, Hp, Wp, O, FH, FW, sh, sw)))
 
 
 def test_paired_degenerate_sizes(oracle):
@@ -261,11 +277,28 @@ def test_paired_degenerate_sizes(oracle):
     # empty batch: nothing to do, no pointer is touched
     _lib.call("ds_conv2d_paired_i8", None, _lib.ptr(blob), None, None, 0, 3, 5, 5, 64, 1, 1, 1, 1, 2, 128, stream())
     # one output pixel, every field width
-    for bits in (1, 2, 3, 4):
+    for form in FORMS:
+        bits = form & 0xff
         rng = np.random.default_rng(bits)
         x8 = random_int8(rng, (1, 5, 3, 3))
-        s, sign = random_codes(rng, (64, 5, 3, 3), max_s=top_field(bits))
+        s, sign = random_codes(rng, (64, 5, 3, 3), max_s=top_field(form))
         w, _ = oracle.pack_words(s.reshape(64, -1), sign.reshape(64, -1), bits)
         want = oracle.conv2d(x8.astype(np.int32), -s, sign, bias, (1, 1))
-        got = abi_conv_paired(x8, abi_tile_paired(w, 64, 5, 3, 3, bits, bits), bias, 64, 3, 3, (1, 1), bits)
+        got = abi_conv_paired(x8, abi_tile_paired(w, 64, 5, 3, 3, bits, form), bias, 64, 3, 3, (1, 1), form)
         np.testing.assert_array_equal(got, want)
+
+
+def test_top_unused_flag_is_ignored_by_the_xor_mask_forms(oracle, rng):
+    """3- and 4-bit fields reserve their highest value anyway: the flag changes neither the blob nor the
+    results."""
+    Nb, C, Hp, Wp, O = 2, 50, 14, 14, 64  # K = 450: whole words of 8 and of 6 codes
+    x8 = random_int8(rng, (Nb, C, Hp, Wp))
+    for bits in (3, 4):
+        s, sign = random_codes(rng, (O, C, 3, 3), max_s=top_field(bits))
+        w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)
+        want = oracle.conv2d(x8.astype(np.int32), -s, sign, None, (1, 1), nthreads=NTHREADS)
+        plain, flagged = abi_tile_paired(w, O, C, 3, 3, bits, bits), abi_tile_paired(w, O, C, 3, 3, bits, bits | U)
+        used = C * 9 * (O // 64) * 32 * 4  # the code rows (what follows them is alignment padding and counts)
+        assert torch.equal(plain[:used], flagged[:used])
+        np.testing.assert_array_equal(abi_conv_paired(x8, flagged, None, O, 3, 3, (1, 1), bits | U), want)
+        np.testing.assert_array_equal(abi_conv_paired(x8, plain, None, O, 3, 3, (1, 1), bits | U), want)

@@ -209,7 +209,10 @@ def test_int8_kernel_eligibility():
     assert kernels.paired_fields(ConcWeight(None, 0, 4, max_field=15), 64, 3, 5) is None
     assert kernels.paired_fields(ConcWeight(None, 0, 5, max_field=20), 64, 3, 5) is None
     assert kernels.paired_fields(None, 64, 3, 5) is None
-    assert kernels.paired_fields(ConcWeight(None, 0, 6, 2), 64, 3, 5) == (6, 2)
+    assert kernels.paired_fields(ConcWeight(None, 0, 6, 2), 64, 3, 5) == (6, 2 | 0x200)  # fields <= 2: 3 is free
+    assert kernels.paired_fields(ConcWeight(None, 0, 2, max_field=2), 64, 3, 5) == (2, 2 | 0x200)
+    assert kernels.paired_fields(ConcWeight(None, 0, 2, max_field=3), 64, 3, 5) == (2, 2)
+    assert kernels.paired_fields(ConcWeight(None, 0, 1, max_field=0), 64, 3, 5) == (1, 1 | 0x200)
     assert kernels.paired_fields(ConcWeight(None, 0, 6, 4), 64, 3, 5) == (6, 4)
     assert kernels.paired_fields(ConcWeight(None, 0, 6, 0), 64, 3, 5) is None
 
