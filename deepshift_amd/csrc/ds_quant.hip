@@ -251,6 +251,72 @@ __global__ void requantize_affine_pad_kernel(const int32_t *__restrict__ y, floa
     }
 }
 
+// The same with padding for rows of a multiple of four elements: one thread per four consecutive
+// elements of a padded row's interior (16-byte loads of y and residual); the threads at the ends of a
+// row also write its left and right padding, the rows above and below the image are all zeros.
+// Needs W % 4 == 0 and 16-byte aligned y, out, residual.  Used when out is NULL.
+struct __attribute__((aligned(4))) QuadI32 {
+    int32_t v[4];
+};
+
+template <typename Q>
+__device__ __forceinline__ void store_quad(Q *dst, int32_t q0, int32_t q1, int32_t q2, int32_t q3)
+{
+    if (sizeof(Q) == 1) {
+        const uint32_t word = ((uint32_t)q0 & 0xffu) | (((uint32_t)q1 & 0xffu) << 8) |
+                              (((uint32_t)q2 & 0xffu) << 16) | ((uint32_t)q3 << 24);
+        __builtin_memcpy(dst, &word, 4);  // byte aligned: the row's interior starts pw elements in
+    } else {
+        QuadI32 quad{{q0, q1, q2, q3}};
+        *(QuadI32 *)dst = quad;           // 4-byte aligned
+    }
+}
+
+template <typename Q>
+__global__ void requantize_affine_pad4_kernel(const int32_t *__restrict__ y, float *__restrict__ out,
+                                              Q *__restrict__ q, const float *__restrict__ scale,
+                                              const float *__restrict__ shift,
+                                              const float *__restrict__ residual, uint32_t planes, int C,
+                                              int H, int W, int ph, int pw, float inv, int relu,
+                                              QuantSpec spec, FastDiv by_plane, FastDiv by_row,
+                                              FastDiv by_channels)
+{
+    const uint32_t Hp = H + 2 * ph, Wp = W + 2 * pw, quads = (uint32_t)W / 4;
+    const uint32_t total = planes * Hp * quads;
+    for (uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+        const uint32_t plane = div_by(idx, by_plane);   // by_plane divides by Hp * quads
+        const uint32_t rem = idx - plane * Hp * quads;
+        const uint32_t hp = div_by(rem, by_row);        // by_row divides by quads
+        const uint32_t qd = rem - hp * quads;
+        Q *row = q + ((size_t)plane * Hp + hp) * Wp;
+        int32_t q0 = 0, q1 = 0, q2 = 0, q3 = 0;
+        const int h = (int)hp - ph;
+        if ((unsigned)h < (unsigned)H) {
+            const uint32_t src4 = ((plane * H + h) * W) / 4 + qd;
+            const uint32_t c = plane - div_by(plane, by_channels) * (uint32_t)C;
+            const float a = scale ? scale[c] : 1.0f, b = shift ? shift[c] : 0.0f;
+            const int4 v = ((const int4 *)y)[src4];
+            float4 r = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (residual) r = ((const float4 *)residual)[src4];
+            float4 f;
+            f.x = affine_one(v.x, inv, a, b, residual ? &r.x : nullptr, relu);
+            f.y = affine_one(v.y, inv, a, b, residual ? &r.y : nullptr, relu);
+            f.z = affine_one(v.z, inv, a, b, residual ? &r.z : nullptr, relu);
+            f.w = affine_one(v.w, inv, a, b, residual ? &r.w : nullptr, relu);
+            if (out) ((float4 *)out)[src4] = f;
+            q0 = quantize_one(f.x, spec);
+            q1 = quantize_one(f.y, spec);
+            q2 = quantize_one(f.z, spec);
+            q3 = quantize_one(f.w, spec);
+        }
+        store_quad<Q>(row + pw + 4 * qd, q0, q1, q2, q3);
+        if (qd == 0)
+            for (int i = 0; i < pw; ++i) row[i] = (Q)0;
+        if (qd == quads - 1)
+            for (int i = 0; i < pw; ++i) row[pw + W + i] = (Q)0;
+    }
+}
+
 // The same without padding (ph = pw = 0: q has the layout of y), four consecutive elements of one
 // (image, channel) plane per thread: 16-byte loads and stores (4-byte for an int8 q).  Needs
 // HW % 4 == 0 and 16-byte aligned y, out, residual (q: 16 / 4-byte aligned).
@@ -516,6 +582,19 @@ static int requantize_affine_pad_any(const int32_t *y, float *out, Q *q, const f
         hipLaunchKernelGGL((requantize_affine_flat4_kernel<Q>), dim3(grid_for(total / 4)), dim3(256), 0,
                            (hipStream_t)stream, y, out, q, scale, shift, residual, (uint32_t)(total / 4), C,
                            ldexpf(1.0f, -F_in), relu, make_spec(I, F, mode), fast_div((uint32_t)(H * W / 4)),
+                           fast_div((uint32_t)C));
+        return launch_status();
+    }
+    // Four elements per thread when only q is written (a layer between two shift convolutions).  With
+    // the float result as a second output the element-per-thread pass below is the faster one: its
+    // stores of q are contiguous over a wave, the quads here start 16 bytes apart at an odd alignment.
+    const uintptr_t in16 = (uintptr_t)y | (uintptr_t)residual;
+    if (!out && W > 0 && W % 4 == 0 && (in16 & 15) == 0 && (sizeof(Q) == 1 || ((uintptr_t)q & 3) == 0)) {
+        const long items = (long)Nb * C * (H + 2 * ph) * (W / 4);
+        hipLaunchKernelGGL((requantize_affine_pad4_kernel<Q>), dim3(grid_for(items)), dim3(256), 0,
+                           (hipStream_t)stream, y, out, q, scale, shift, residual, (uint32_t)(Nb * C), C, H, W,
+                           ph, pw, ldexpf(1.0f, -F_in), relu, make_spec(I, F, mode),
+                           fast_div((uint32_t)((H + 2 * ph) * (W / 4))), fast_div((uint32_t)(W / 4)),
                            fast_div((uint32_t)C));
         return launch_status();
     }

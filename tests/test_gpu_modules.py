@@ -1,5 +1,6 @@
 """GPU: the Python-level API (kernels.*, utils.compress_bits, the shift modules, convert_to_shift)
 against the oracle (bit-exact on the int32 results) and against the float path (stated bound)."""
+import ctypes
 import os
 
 import numpy as np
@@ -254,7 +255,10 @@ def test_fixed_point_handoff_is_bit_identical():
 
 
 def test_requantize_affine_pad_matches_the_two_passes(rng):
-    for (Nb, C, H, W), pad in [((3, 5, 7, 4), (1, 1)), ((2, 3, 5, 9), (0, 2)), ((1, 4, 6, 6), (0, 0))]:
+    # rows of a multiple of four elements take the four-elements-per-thread pass
+    for (Nb, C, H, W), pad in [((3, 5, 7, 4), (1, 1)), ((2, 3, 5, 9), (0, 2)), ((1, 4, 6, 6), (0, 0)),
+                               ((2, 3, 5, 8), (1, 1)), ((1, 2, 3, 12), (2, 3)), ((2, 2, 4, 16), (0, 1)),
+                               ((1, 70, 28, 28), (1, 1))]:
         y = torch.from_numpy(rng.integers(-2 ** 27, 2 ** 27, size=(Nb, C, H, W)).astype(np.int32)).to(DEV)
         scale = torch.rand(C, device=DEV) + 0.5
         shift = torch.randn(C, device=DEV)
@@ -267,6 +271,38 @@ def test_requantize_affine_pad_matches_the_two_passes(rng):
             assert torch.equal(f, f_want) and torch.equal(q, q_want)
             f, q = kernels.requantize_affine_pad(y, 16, sc, sh, r, relu, pad, I, F, want_float=False)
             assert f is None and torch.equal(q, q_want)
+
+
+@pytest.mark.parametrize("dtype", [torch.int32, torch.int8])
+def test_requantize_affine_pad_stays_inside_its_output(rng, dtype):
+    """The padded conversion pass through the C ABI, output between guard bands: every element of the
+    padded tensor is written (padding included, over stale contents) and nothing outside it."""
+    from deepshift_amd import _lib
+    I, Fb = (3, 5) if dtype == torch.int8 else (16, 16)
+    name = "ds_requantize_affine_pad_i8" if dtype == torch.int8 else "ds_requantize_affine_pad_i32"
+    for (Nb, C, H, W), (ph, pw) in [((2, 3, 5, 8), (1, 1)), ((1, 2, 6, 4), (2, 3)), ((3, 1, 2, 12), (0, 2)),
+                                    ((1, 3, 4, 7), (1, 1))]:
+        y = torch.from_numpy(rng.integers(-2 ** 10, 2 ** 10, size=(Nb, C, H, W)).astype(np.int32)).to(DEV)
+        res = torch.randn(Nb, C, H, W, device=DEV)
+        f_want = kernels.dequantize_affine(y, Fb, None, None, res, True)
+        q_want = kernels.quantize_pad(f_want, (ph, pw), I, Fb, dtype=dtype)
+        total, guard = q_want.numel(), 64
+        buf = torch.full((total + 2 * guard,), 0x5A, dtype=dtype, device=DEV)
+        # an odd element offset: the int8 output is only byte aligned, the int32 one 4-byte aligned
+        off = guard + 1
+        q = buf[off:off + total]
+        for want_float in (True, False):  # without the float output: the four-elements-per-thread pass
+            buf.fill_(0x5A)
+            out = torch.empty(Nb, C, H, W, dtype=torch.float32, device=DEV) if want_float else None
+            args = [_lib.ptr(y), _lib.ptr(out), ctypes.c_void_p(q.data_ptr()), None, None, _lib.ptr(res), Nb, C,
+                    H, W, ph, pw, Fb, 1, I, Fb]
+            if dtype == torch.int32:
+                args.append(_lib.DS_Q_ROUND_TO_FIXED)
+            _lib.call(name, *args, _lib.current_stream(DEV))
+            torch.cuda.synchronize()
+            assert out is None or torch.equal(out, f_want)
+            assert torch.equal(q.view(q_want.shape), q_want)
+            assert (buf[:off] == 0x5A).all() and (buf[off + total:] == 0x5A).all()
 
 
 def test_requantize_affine_maxpool_matches_the_three_passes(rng):

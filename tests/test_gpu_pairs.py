@@ -183,6 +183,19 @@ def test_int8_conversion_passes_match_the_int32_ones(rng):
         assert torch.equal(f8, f32) and torch.equal(q8.to(torch.int32), q32)
         # unpadded, plane size a multiple of 4: the four-elements-per-thread pass, against the padded
         # one's interior and the two separate calls
+        # rows of a multiple of four elements, padded: the four-elements-per-thread padded pass
+        y8 = torch.from_numpy(rng.integers(-2 ** 12, 2 ** 12, size=(2, 5, 9, 8)).astype(np.int32)).to(DEV)
+        res8 = torch.randn(2, 5, 9, 8, generator=g).to(DEV)
+        for pad in [(1, 1), (2, 3), (0, 1)]:
+            f32, q32 = kernels.requantize_affine_pad(y8, Fb, scale, shift, res8, True, pad, I, Fb, True)
+            assert torch.equal(q32, kernels.quantize_pad(f32, pad, I, Fb))
+            f8, q8 = kernels.requantize_affine_pad(y8, Fb, scale, shift, res8, True, pad, I, Fb, True,
+                                                   dtype=torch.int8)
+            assert torch.equal(f8, f32) and torch.equal(q8.to(torch.int32), q32)
+            for dtype in (torch.int32, torch.int8):
+                f, q = kernels.requantize_affine_pad(y8, Fb, scale, shift, res8, True, pad, I, Fb, False,
+                                                     dtype=dtype)
+                assert f is None and torch.equal(q.to(torch.int32), q32)
         y4 = torch.from_numpy(rng.integers(-2 ** 12, 2 ** 12, size=(3, 5, 8, 6)).astype(np.int32)).to(DEV)
         res4 = torch.randn(3, 5, 8, 6, generator=g).to(DEV)
         for residual, relu, want_float in [(res4, True, True), (None, False, False), (res4, False, True)]:
