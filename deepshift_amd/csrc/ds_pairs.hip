@@ -105,9 +105,12 @@ DS_PAIRS_ONE(4, false, DS_PAIRX_ASM_B4, DS_PAIRX_CLOBBERS_B4)
 
 // K groups [g_begin, g_end) (at most PairArgs::chunk of them) of the tile made of the 64 channels of
 // `ntile` and the 384 pixels from m0.
-// OUT selects where the widened sums go: kStore (y = sum + bias), kAtomic (atomic add to a
-// pre-filled y) or kLds (add to the workgroup's tile buffer lds[channel][pixel of the tile]).
-enum { kStore, kAtomic, kLds };
+// OUT selects where the sums go: widened, kStore (y = sum + bias), kAtomic (atomic add to a
+// pre-filled y) or kLds (add to the workgroup's tile buffer lds[channel][pixel of the tile]); or as
+// they are, two pixels per word, kLdsPacked (add to lds[channel][row][lane]: the sum of such words is
+// the word of the sums as long as every 16-bit half stays in range, i.e. while the reduction indices
+// that all the waves of the workgroup add up for one tile fit one chunk).
+enum { kStore, kAtomic, kLds, kLdsPacked };
 
 template <int BITS, int OUT, bool TU>
 __device__ __forceinline__ void pairs_segment(const PairArgs &p, int ntile, int m0, int g_begin, int g_end,
@@ -155,6 +158,14 @@ __device__ __forceinline__ void pairs_segment(const PairArgs &p, int ntile, int 
                               __builtin_amdgcn_readfirstlane(g_end - g_begin), w);
     }
 
+    if (OUT == kLdsPacked) {
+#pragma unroll
+        for (int j = 0; j < 64; ++j)
+#pragma unroll
+            for (int r = 0; r < kPairRows; ++r)
+                atomicAdd(lds + j * (kPairRows * kWave) + r * kWave + lane, a[2 * r + j / 32][j % 32]);
+        return;
+    }
     // split the sums into their halves (v = hi * 65536 + lo) and add them to the output
     if (OUT == kLds) {
 #pragma unroll
@@ -305,6 +316,62 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
+// The same with workgroups of four waves for reductions of a single chunk: the tile buffer holds the
+// sums as the registers do, two pixels per word (48 KiB), so two workgroups share a CU, the two waves
+// of a SIMD belong to different workgroups and are never held at the same barrier, and a wave's share
+// of a short reduction is twice as long.
+constexpr int kPairCu4Waves = 4;
+
+template <int BITS, bool TU>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void shift_pairs_cu4_kernel(
+    const PairArgs p)
+{
+    __shared__ int32_t tile_pairs[64 * kPairRows * kWave];  // [64 channels][3 rows][64 lanes]
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int lane = threadIdx.x & (kWave - 1);
+    const int bid = blockIdx.x;
+    const int w = (bid & 7) * (int)(gridDim.x >> 3) + (bid >> 3);  // an XCD takes a contiguous range
+    const int ntiles = p.tile_end - p.tile_begin;
+    const long total = (long)ntiles * p.comm;
+    int it = (int)(w * total / (long)gridDim.x);
+    const int it_end = (int)((w + 1) * total / (long)gridDim.x);
+    while (it < it_end) {
+        const int tile = p.tile_begin + it / p.comm;
+        const int g0 = it - (tile - p.tile_begin) * p.comm;
+        int g1 = g0 + (it_end - it);
+        if (g1 > p.comm) g1 = p.comm;
+        const int ntile = tile % p.tiles_n, m0 = (tile / p.tiles_n) * kPairPixels;
+        for (int i = threadIdx.x; i < 64 * kPairRows * kWave; i += 256) tile_pairs[i] = 0;
+        __syncthreads();
+        const int len = g1 - g0;  // <= comm <= chunk: one call of the loop per wave
+        const int wb = g0 + wave * len / kPairCu4Waves, we = g0 + (wave + 1) * len / kPairCu4Waves;
+        if (wb < we) pairs_segment<BITS, kLdsPacked, TU>(p, ntile, m0, wb, we, tile_pairs);
+        __syncthreads();
+        const bool whole = len == p.comm;
+        for (int c = 0; c < 64 / kPairCu4Waves; ++c) {
+            const int j = wave * (64 / kPairCu4Waves) + c, n = ntile * 64 + j;
+            const int32_t add = whole && p.bias ? p.bias[n] : 0;
+            const int32_t neg = whole && p.negcnt ? p.negcnt[n] : 0;  // for the pixels of low halves
+            for (int r = 0; r < kPairRows; ++r) {
+                const int32_t v = tile_pairs[j * (kPairRows * kWave) + r * kWave + lane];
+                const int32_t lo = (int32_t)(int16_t)(v & 0xffff), hi = (v - lo) >> 16;
+                for (int h = 0; h < 2; ++h) {
+                    const int m = m0 + (2 * r + h) * kWave + lane;
+                    if (m >= p.M) break;
+                    const int img = m / p.pix_per_img;
+                    int32_t *dst = p.y + (size_t)img * p.y_img_stride + (size_t)n * p.y_ch_stride +
+                                   (m - img * p.pix_per_img);
+                    const int32_t sum = h ? hi : lo;
+                    if (whole) *dst = sum + add + (h ? 0 : neg);
+                    else atomicAdd(dst, sum);
+                }
+            }
+        }
+        __syncthreads();
+        it += len;
+    }
+}
+
 // y = bias[n] before an accumulating launch; y is [img][n][pix], dense.  With the xor-mask forms the
 // pixels that live in low halves (the even 64-pixel blocks of their tile) start at bias[n] + negcnt[n].
 __global__ void pairs_fill_kernel(const PairArgs p)
@@ -398,9 +465,16 @@ static int launch_pairs(PairArgs a, hipStream_t st)
     if (fill_blocks < 1) fill_blocks = 1;
     hipLaunchKernelGGL(pairs_fill_kernel, dim3((unsigned)fill_blocks), dim3(256), 0, st, a);
     if (regime == 2) {
-        int blocks = 256;
+        // reductions of a single chunk: four-wave workgroups on a tile buffer of packed pairs
+        bool four = a.comm <= a.chunk;
+        if (const char *t = getenv("DS_TUNE_CU")) four = four && atoi(t) == 4;
+        int blocks = four ? 512 : 256;
         const long fit = (iters / 64) / 8 * 8;  // small layers: at least 8 K groups per wave
         if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
+        if (four) {
+            hipLaunchKernelGGL((shift_pairs_cu4_kernel<BITS, TU>), dim3(blocks), dim3(256), 0, st, a);
+            return launch_status();
+        }
         return launch_pairs_cu<BITS, TU>(a, blocks, st);
     }
     int blocks = kPairSlots / 4;

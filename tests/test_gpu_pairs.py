@@ -8,7 +8,7 @@ import torch
 
 from deepshift_amd import _lib
 from tests.conftest import random_codes
-from tests.test_gpu_parity import DEV, dev, stream
+from tests.test_gpu_parity import DEV, _Tune, dev, stream
 
 pytestmark = pytest.mark.gpu
 
@@ -315,3 +315,26 @@ def test_top_unused_flag_is_ignored_by_the_xor_mask_forms(oracle, rng):
         assert torch.equal(plain[:used], flagged[:used])
         np.testing.assert_array_equal(abi_conv_paired(x8, flagged, None, O, 3, 3, (1, 1), bits | U), want)
         np.testing.assert_array_equal(abi_conv_paired(x8, plain, None, O, 3, 3, (1, 1), bits | U), want)
+
+
+@pytest.mark.parametrize("form", FORMS, ids=form_id)
+@pytest.mark.parametrize("regime", [(0, None), (1, None), (2, 4), (2, 8)], ids=lambda r: "split%s_cu%s" % r)
+def test_paired_launch_regimes(oracle, rng, form, regime):
+    """Every launch regime forced on reductions of a single chunk: wave-level shares, one tile per wave,
+    and the workgroup-cooperative kernels of four waves (tile buffer of packed pairs) and of eight."""
+    split, cu = regime
+    bits = form & 0xff
+    env = {"DS_TUNE_SPLIT": split}
+    if cu:
+        env["DS_TUNE_CU"] = cu
+    for Nb, C, Hp, Wp, O, FH, FW, stride in [(2, 64, 16, 16, 64, 1, 1, (1, 1)), (4, 128, 14, 14, 256, 1, 1, (2, 2)),
+                                             (3, 20, 21, 23, 128, 3, 3, (1, 1)), (9, 7, 40, 40, 64, 3, 3, (1, 1))]:
+        x8 = random_int8(rng, (Nb, C, Hp, Wp))
+        s, sign = random_codes(rng, (O, C, FH, FW), max_s=top_field(form))
+        bias = rng.integers(-2 ** 20, 2 ** 20, size=O).astype(np.int32)
+        w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)
+        want = oracle.conv2d(x8.astype(np.int32), -s, sign, bias, stride, nthreads=NTHREADS)
+        blob = abi_tile_paired(w, O, C, FH, FW, bits, form)
+        with _Tune(**env):
+            got = abi_conv_paired(x8, blob, bias, O, FH, FW, stride, form)
+        np.testing.assert_array_equal(got, want, err_msg=str((Nb, C, Hp, Wp, O, FH, FW)))
