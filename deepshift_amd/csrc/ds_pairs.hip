@@ -29,6 +29,7 @@
 // 64-pixel blocks of a tile -- wherever the bias is added.  The highest field value means "no
 // contribution" (zero weights, indices past K); the caller vouches that no real code uses it.
 #include "ds_common.h"
+#include <atomic>
 #include <cstdlib>
 
 #include "ds_planes_asm.inc"
@@ -400,14 +401,14 @@ __global__ void pairs_fill_kernel(const PairArgs p)
 template <int BITS, bool TU>
 static int pairs_opt_in_lds()
 {
-    static bool opted_in[64] = {};
+    static std::atomic<bool> opted_in[64];  // per device; setting the attribute twice is harmless
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
-    if (!opted_in[dev]) {
+    if (!opted_in[dev].load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute((const void *)shift_pairs_cu_kernel<BITS, TU>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, kPairLdsBytes);
         if (e != hipSuccess) return hip_status(e);
-        opted_in[dev] = true;
+        opted_in[dev].store(true, std::memory_order_release);
     }
     return DS_OK;
 }

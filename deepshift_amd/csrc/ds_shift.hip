@@ -24,6 +24,7 @@
 //     addition commutes, so the result stays bit-exact).
 #include "ds_common.h"
 #include <cstdio>
+#include <atomic>
 #include <cstdlib>
 #include <type_traits>
 
@@ -584,14 +585,14 @@ static int launch_planes_cu(const ShiftArgs &a, long iters, hipStream_t st)
 {
     constexpr int kLdsBytes = (WAVES == 8 ? 2 : 1) * 64 * kPlaneRows * kWave * 4;
     if (kLdsBytes > 64 * 1024) {  // above the default limit of a workgroup: opt in, once per device
-        static bool opted_in[64] = {};
+        static std::atomic<bool> opted_in[64];  // per device; setting the attribute twice is harmless
         int dev = 0;
         if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
-        if (!opted_in[dev]) {
+        if (!opted_in[dev].load(std::memory_order_acquire)) {
             hipError_t e = hipFuncSetAttribute((const void *)shift_planes_wide_cu_kernel<BITS, ZT, WAVES>,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
             if (e != hipSuccess) return hip_status(e);
-            opted_in[dev] = true;
+            opted_in[dev].store(true, std::memory_order_release);
         }
     }
     // one workgroup per 8 wave slots (2 waves per SIMD); small layers: >= 8 K groups per wave
