@@ -281,7 +281,10 @@ struct PlaneWalk {
     int koff, fw, fh, FW, FH, row_step, plane_step, koff_max;
 };
 
-constexpr int kPlaneRows = 3;      // pixels per lane (R of gen_planes_asm.py)
+constexpr int kPlaneRows = 3;      // pixels per lane of the 32-channel form (R of gen_planes_asm.py)
+constexpr int kPlaneRowsWide = 2;  // ... of the 64-channel form (ROWS_WIDE): two scalar and two vector
+                                   // instructions per code, which two waves interleave without gaps
+constexpr int plane_rows(bool wide) { return wide ? kPlaneRowsWide : kPlaneRows; }
 constexpr int kPlaneSlots = 3072;  // wave slots of the machine at 3 waves per SIMD (256 CUs x 4 SIMDs)
 
 constexpr int kPlaneSlotsWide = 2048;  // the 64-channel form holds 246 registers: 2 waves per SIMD
@@ -296,9 +299,10 @@ constexpr int kPlaneSlotsWide = 2048;  // the 64-channel form holds 246 register
     DS_PLANES_INPUTS
 // (six 32-register operands: an asm statement takes at most 30 operands, tied ones counted twice)
 #define DS_PLANES_OPERANDS_WIDE                                                                   \
-    : "+{v[64:95]}"(a[0]), "+{v[96:127]}"(a[1]), "+{v[128:159]}"(a[2]), "+{v[160:191]}"(a[3]),    \
-      "+{v[192:223]}"(a[4]), "+{v[224:255]}"(a[5])                                                \
-    DS_PLANES_INPUTS
+    : "+{v[64:95]}"(a[0]), "+{v[96:127]}"(a[1]), "+{v[128:159]}"(a[2]), "+{v[160:191]}"(a[3])     \
+    : "v"(xoff[0]), "v"(xoff[1]), "s"(rsrc), "s"(wptr), "s"(groups), "s"(w.koff),                 \
+      "s"(w.fw), "s"(w.fh), "s"(w.FW), "s"(w.FH), "s"(w.row_step), "s"(w.plane_step),             \
+      "s"(w.koff_max)
 
 // Main loop of the 32-channel form (six 16-register accumulator vectors) and of the 64-channel form
 // (six of 32 registers).
@@ -308,23 +312,24 @@ template <int BITS, int ZT>
 __device__ __forceinline__ void planes_main_loop(v16i (&a)[6], const uint32_t (&xoff)[3], v4i rsrc,
                                                  const uint32_t *wptr, int groups, const PlaneWalk &w);
 template <int BITS, int ZT>
-__device__ __forceinline__ void planes_main_loop(v32i (&a)[6], const uint32_t (&xoff)[3], v4i rsrc,
+__device__ __forceinline__ void planes_main_loop(v32i (&a)[2 * kPlaneRowsWide],
+                                                 const uint32_t (&xoff)[kPlaneRowsWide], v4i rsrc,
                                                  const uint32_t *wptr, int groups, const PlaneWalk &w);
-#define DS_PLANES_ONE(B, ZT, VEC, ASM, OPERANDS, CLOBBERS)                                         \
+#define DS_PLANES_ONE(B, ZT, VEC, ROWS, ASM, OPERANDS, CLOBBERS)                                   \
     template <>                                                                                    \
-    __device__ __forceinline__ void planes_main_loop<B, ZT>(VEC (&a)[6], const uint32_t (&xoff)[3], \
+    __device__ __forceinline__ void planes_main_loop<B, ZT>(VEC (&a)[2 * ROWS], const uint32_t (&xoff)[ROWS], \
                                                             v4i rsrc, const uint32_t *wptr, int groups, \
                                                             const PlaneWalk &w)                    \
     {                                                                                              \
         asm volatile(ASM OPERANDS : CLOBBERS);                                                     \
     }
 #define DS_PLANES_SPECIALISE(B)                                                                    \
-    DS_PLANES_ONE(B, 0, v16i, DS_PLANES_ASM_B##B, DS_PLANES_OPERANDS, DS_PLANES_CLOBBERS_B##B)      \
-    DS_PLANES_ONE(B, 1, v16i, DS_PLANES_ASM_B##B##Z, DS_PLANES_OPERANDS, DS_PLANES_CLOBBERS_B##B)   \
-    DS_PLANES_ONE(B, 2, v16i, DS_PLANES_ASM_B##B##U, DS_PLANES_OPERANDS, DS_PLANES_CLOBBERS_B##B##U) \
-    DS_PLANES_ONE(B, 0, v32i, DS_PLANES_ASM_B##B##W, DS_PLANES_OPERANDS_WIDE, DS_PLANES_CLOBBERS_B##B##W) \
-    DS_PLANES_ONE(B, 1, v32i, DS_PLANES_ASM_B##B##ZW, DS_PLANES_OPERANDS_WIDE, DS_PLANES_CLOBBERS_B##B##W) \
-    DS_PLANES_ONE(B, 2, v32i, DS_PLANES_ASM_B##B##UW, DS_PLANES_OPERANDS_WIDE, DS_PLANES_CLOBBERS_B##B##UW)
+    DS_PLANES_ONE(B, 0, v16i, kPlaneRows, DS_PLANES_ASM_B##B, DS_PLANES_OPERANDS, DS_PLANES_CLOBBERS_B##B) \
+    DS_PLANES_ONE(B, 1, v16i, kPlaneRows, DS_PLANES_ASM_B##B##Z, DS_PLANES_OPERANDS, DS_PLANES_CLOBBERS_B##B) \
+    DS_PLANES_ONE(B, 2, v16i, kPlaneRows, DS_PLANES_ASM_B##B##U, DS_PLANES_OPERANDS, DS_PLANES_CLOBBERS_B##B##U) \
+    DS_PLANES_ONE(B, 0, v32i, kPlaneRowsWide, DS_PLANES_ASM_B##B##W, DS_PLANES_OPERANDS_WIDE, DS_PLANES_CLOBBERS_B##B##W) \
+    DS_PLANES_ONE(B, 1, v32i, kPlaneRowsWide, DS_PLANES_ASM_B##B##ZW, DS_PLANES_OPERANDS_WIDE, DS_PLANES_CLOBBERS_B##B##W) \
+    DS_PLANES_ONE(B, 2, v32i, kPlaneRowsWide, DS_PLANES_ASM_B##B##UW, DS_PLANES_OPERANDS_WIDE, DS_PLANES_CLOBBERS_B##B##UW)
 DS_PLANES_SPECIALISE(1)
 DS_PLANES_SPECIALISE(2)
 DS_PLANES_SPECIALISE(3)
@@ -339,7 +344,7 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
                                                int g_end, bool atomic, int32_t *lds = nullptr)
 {
     constexpr int NUM = 32 / (BITS + 1);
-    constexpr int R = kPlaneRows, J = WIDE ? 64 : 32;
+    constexpr int R = plane_rows(WIDE), J = WIDE ? 64 : 32;
     constexpr int VEC = WIDE ? 32 : 16;  // registers per accumulator operand of the asm loop
     using acc_vec = typename std::conditional<WIDE, v32i, v16i>::type;
     const int lane = threadIdx.x & (kWave - 1);
@@ -361,9 +366,9 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
 
     const int full_groups = p.K / NUM;
     const int g_full_end = g_end < full_groups ? g_end : full_groups;
-    acc_vec a[6];
+    acc_vec a[2 * R];
 #pragma unroll
-    for (int i = 0; i < 6; ++i) a[i] = (acc_vec)(0);
+    for (int i = 0; i < 2 * R; ++i) a[i] = (acc_vec)(0);
     if (g_begin < g_full_end) {
         const uint64_t xaddr = (uint64_t)p.x;
         v4i rsrc;
@@ -453,7 +458,7 @@ __device__ __forceinline__ void planes_tile_body(const ShiftArgs &p)
     const int tile = (bid & 7) * p.blocks_per_xcd + (bid >> 3);
     if (tile >= p.tiles_m4 * p.tiles_n) return;
     const int ntile = tile % p.tiles_n;
-    const int m0 = ((tile / p.tiles_n) * 4 + wave) * (kPlaneRows * kWave);
+    const int m0 = ((tile / p.tiles_n) * 4 + wave) * (plane_rows(WIDE) * kWave);
     if (m0 >= p.M) return;
     const int g_begin = blockIdx.y * p.groups_per_split;
     int g_end = g_begin + p.groups_per_split;
@@ -483,7 +488,7 @@ __device__ __forceinline__ void planes_balanced_body(const ShiftArgs &p)
         int g_end = g_begin + (it_end - it);
         if (g_end > p.comm) g_end = p.comm;
         const int ntile = tile % p.tiles_n;
-        const int m0 = (tile / p.tiles_n) * (kPlaneRows * kWave);
+        const int m0 = (tile / p.tiles_n) * (plane_rows(WIDE) * kWave);
         planes_segment<BITS, ZT, WIDE>(p, ntile, m0, g_begin, g_end, true);
         it += g_end - g_begin;
     }
@@ -530,7 +535,7 @@ template <int BITS, int ZT, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void shift_planes_wide_cu_kernel(const ShiftArgs p)
 {
-    constexpr int PIX = kPlaneRows * kWave;
+    constexpr int PIX = kPlaneRowsWide * kWave;
     constexpr int BUFFERS = WAVES == 8 ? 2 : 1;
     // With two buffers: a wave adds its sums of tile t to buffer t % 2, waits for the others, writes
     // out and clears its channels of that buffer, and goes on to tile t + 1 in the other buffer;
@@ -561,7 +566,7 @@ void shift_planes_wide_cu_kernel(const ShiftArgs p)
         for (int c = 0; c < 64 / WAVES; ++c) {
             const int j = wave * (64 / WAVES) + c, n = ntile * 64 + j;
             const int32_t add = whole ? p.negcnt[n] + (p.bias ? p.bias[n] : 0) : 0;
-            for (int r = 0; r < kPlaneRows; ++r) {
+            for (int r = 0; r < kPlaneRowsWide; ++r) {
                 int32_t *cell = buf + j * PIX + r * kWave + lane;
                 const int32_t v = *cell;
                 *cell = 0;
@@ -583,7 +588,7 @@ void shift_planes_wide_cu_kernel(const ShiftArgs p)
 template <int BITS, int ZT, int WAVES>
 static int launch_planes_cu(const ShiftArgs &a, long iters, hipStream_t st)
 {
-    constexpr int kLdsBytes = (WAVES == 8 ? 2 : 1) * 64 * kPlaneRows * kWave * 4;
+    constexpr int kLdsBytes = (WAVES == 8 ? 2 : 1) * 64 * kPlaneRowsWide * kWave * 4;
     if (kLdsBytes > 64 * 1024) {  // above the default limit of a workgroup: opt in, once per device
         static std::atomic<bool> opted_in[64];  // per device; setting the attribute twice is harmless
         int dev = 0;
@@ -717,7 +722,7 @@ static TileChoice choose_tile(const ShiftArgs &a)
 template <int BITS, int ZT, bool WIDE>
 static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
 {
-    constexpr int R = kPlaneRows, J = WIDE ? 64 : 32;
+    constexpr int R = plane_rows(WIDE), J = WIDE ? 64 : 32;
     constexpr int kSlots = WIDE ? kPlaneSlotsWide : kPlaneSlots;
     a.tiles_n = ceil_div(a.N, J);
     if (nsplit <= 0 && a.comm > 0) {
@@ -781,7 +786,7 @@ static int plane_regime(const ShiftArgs &a, bool wide)
 {
     const long slots = wide ? kPlaneSlotsWide : kPlaneSlots;
     const int J = wide ? 64 : 32;
-    const long tiles = (long)ceil_div(a.M, kPlaneRows * kWave) * ceil_div(a.N, J);
+    const long tiles = (long)ceil_div(a.M, plane_rows(wide) * kWave) * ceil_div(a.N, J);
     const long iters = tiles * a.comm;
     const bool n_ok = a.N % 32 == 0 || a.N >= 256;
     const bool many_tiles = tiles * 10 >= slots * 13;

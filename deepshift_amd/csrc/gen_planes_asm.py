@@ -61,9 +61,10 @@ K groups, %12..%14 initial walk state (offset, fw, fh), %15 FW, %16 FH, %17 offs
 """
 import os
 
-R = 3
+R = 3                                    # pixel rows per lane (the int8 forms: rows of two pixels)
+ROWS_WIDE = 2                            # ... of the 64-channel int32 form
 DEPTH = {1: 4, 2: 5, 3: 4, 4: 3}        # prefetch ring depth, 32-channel form
-DEPTH_WIDE = {1: 4, 2: 5, 3: 4, 4: 2}   # 64-channel form: 4-bit fields leave room for two slots only
+DEPTH_WIDE = {1: 4, 2: 5, 3: 4, 4: 3}   # 64-channel form
 DEPTH_WIDE_U = {1: 4, 2: 5, 3: 4, 4: 3}  # 64-channel form without the top plane: its registers buy a third slot
 DEPTH_PAIRED = {1: 4, 2: 2, 3: 1, 4: 1}  # int8 forms: six activation registers per slot
 DEPTH_PAIRED_U = {1: 4, 2: 5}            # index forms without the planes of the top field value
@@ -78,8 +79,9 @@ class Form:
         self.acc = 64 if wide else 66
         self.depth = (DEPTH_WIDE if wide else DEPTH)[bits]
         self.waves = 2 if wide else 3
-        nacc = 2 * R                            # accumulator operands %0..%5, 16 or 32 registers each
-        nx = 2 * R if paired else R             # activation offsets: one per pixel held by a lane
+        self.R = ROWS_WIDE if wide and not paired else R
+        nacc = 2 * self.R                       # accumulator operands, 16 or 32 registers each
+        nx = 2 * R if paired else self.R        # activation offsets: one per pixel held by a lane
         if paired:
             self.depth = DEPTH_PAIRED[bits]
         self.op_xoff, self.op_rsrc, self.op_wptr, self.op_groups, self.op_walk = (
@@ -114,8 +116,8 @@ def walk_and_load(slot, f):
     else:
         L = ["s_min_u32 s%d, s%d, %%%d" % (T0, KOFF, koff_max),
              "s_lshl_b32 s%d, s%d, 2" % (KB, T0)]
-        L += ["buffer_load_dword v%d, %%%d, %%%d, s%d offen" % (XP + R * slot + r, OP_XOFF + r, OP_RSRC, KB)
-              for r in range(R)]
+        L += ["buffer_load_dword v%d, %%%d, %%%d, s%d offen" % (XP + f.R * slot + r, OP_XOFF + r, OP_RSRC, KB)
+              for r in range(f.R)]
     L += ["s_add_u32 s%d, s%d, 1" % (FWC, FWC),
           "s_add_u32 s%d, s%d, 1" % (KOFF, KOFF),
           "s_cmp_eq_u32 s%d, %%%d" % (FWC, fw_end),
@@ -171,6 +173,7 @@ def body(bits, zero_top=False, wide=False, unused_top=False):
     f = Form(bits, wide)
     if unused_top and wide:
         f.depth = DEPTH_WIDE_U[bits]
+    R = f.R
     cb = bits + 1
     num = 32 // cb
     P = 1 << bits
@@ -257,7 +260,7 @@ def clobbers(bits, wide=False, unused_top=False):
     if unused_top and wide:
         f.depth = DEPTH_WIDE_U[bits]
     P = (1 << bits) - (1 if unused_top else 0)
-    v = ['"v%d"' % n for n in range(XP, XP + R * f.depth + P * R)]
+    v = ['"v%d"' % n for n in range(XP, XP + f.R * f.depth + P * f.R)]
     s = ['"s%d"' % n for n in list(range(4, 16)) + list(range(W, WS + 32)) + [TIME, TIME + 1]]
     return ", ".join(v + s + ['"scc"', '"memory"'])
 
