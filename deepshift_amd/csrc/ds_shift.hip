@@ -381,12 +381,13 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
         const int ic = k0 / ff, rem = k0 - ic * ff;
         w.fh = rem / p.FW;
         w.fw = rem - w.fh * p.FW;
-        w.koff = ic * p.x_plane + w.fh * p.x_row + w.fw;
+        // byte offsets; row_step is the whole step of an fw wrap (the element step included)
+        w.koff = 4 * (ic * p.x_plane + w.fh * p.x_row + w.fw);
         w.FW = p.FW;
         w.FH = p.FH;
-        w.row_step = p.x_row - p.FW;
-        w.plane_step = p.x_plane - p.FH * p.x_row;
-        w.koff_max = (p.K / ff - 1) * p.x_plane + (p.FH - 1) * p.x_row + p.FW - 1;
+        w.row_step = 4 * (p.x_row - p.FW + 1);
+        w.plane_step = 4 * (p.x_plane - p.FH * p.x_row);
+        w.koff_max = 4 * ((p.K / ff - 1) * p.x_plane + (p.FH - 1) * p.x_row + p.FW - 1);
         // rows of 16-bit codes per K group: NUM/2 (two slots per row) or NUM (one slot, 64 channels)
         constexpr int ROWS = WIDE ? NUM : NUM / 2;
         planes_main_loop<BITS, ZT>(a, xoff, rsrc,

@@ -114,10 +114,22 @@ def walk_and_load(slot, f):
         L += ["buffer_load_sbyte v%d, %%%d, %%%d, s%d offen" % (XP + 2 * R * slot + q, OP_XOFF + q, OP_RSRC, KB)
               for q in range(2 * R)]
     else:
-        L = ["s_min_u32 s%d, s%d, %%%d" % (T0, KOFF, koff_max),
-             "s_lshl_b32 s%d, s%d, 2" % (KB, T0)]
+        # int32 activations: the walk keeps byte offsets (the caller passes its steps times four)
+        L = ["s_min_u32 s%d, s%d, %%%d" % (KB, KOFF, koff_max)]
         L += ["buffer_load_dword v%d, %%%d, %%%d, s%d offen" % (XP + f.R * slot + r, OP_XOFF + r, OP_RSRC, KB)
               for r in range(f.R)]
+        # fw += 1, wrapping into fh, wrapping into the next input channel; row_step already contains
+        # the ordinary step of one element, s_cmov / s_cselect leave the wrap flag in SCC for the add
+        return L + ["s_add_u32 s%d, s%d, 1" % (FWC, FWC),
+                    "s_cmp_eq_u32 s%d, %%%d" % (FWC, fw_end),
+                    "s_cmov_b32 s%d, 0" % FWC,
+                    "s_cselect_b32 s%d, %%%d, 4" % (T0, row_step),
+                    "s_addc_u32 s%d, s%d, 0" % (FHC, FHC),
+                    "s_add_u32 s%d, s%d, s%d" % (KOFF, KOFF, T0),
+                    "s_cmp_eq_u32 s%d, %%%d" % (FHC, fh_end),
+                    "s_cmov_b32 s%d, 0" % FHC,
+                    "s_cselect_b32 s%d, %%%d, 0" % (T0, plane_step),
+                    "s_add_u32 s%d, s%d, s%d" % (KOFF, KOFF, T0)]
     L += ["s_add_u32 s%d, s%d, 1" % (FWC, FWC),
           "s_add_u32 s%d, s%d, 1" % (KOFF, KOFF),
           "s_cmp_eq_u32 s%d, %%%d" % (FWC, fw_end),
@@ -207,10 +219,10 @@ def body(bits, zero_top=False, wide=False, unused_top=False):
             cur, nxt = (W, WS) if i % 2 == 0 else (WS, W)
             L += ["s_add_u32 s%d, s%d, 128" % (WP, WP), "s_addc_u32 s%d, s%d, 0" % (WP + 1, WP + 1),
                   "s_waitcnt lgkmcnt(0)"]
-            if i % 2 == 0:
-                L += take_turn(i // 2, f.waves)
+            if i == 0:
+                L += take_turn(0, f.waves)  # once per K group: a group is a few us, a turn 41
             L += load_words(nxt)
-            if i % 2 == 1:
+            if i == num - 1:
                 L += ["s_memrealtime s[%d:%d]" % (TIME, TIME + 1)]  # read at the next turn check
         elif i % 2 == 0:
             # one code row per two reduction slots: this row's codes leave the staging registers,
