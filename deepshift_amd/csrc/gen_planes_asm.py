@@ -98,9 +98,9 @@ PRIO = 13
 TIME = 34
 
 
-def load_words(dst=WS):
-    return ["s_load_dwordx16 s[%d:%d], s[%d:%d], 0x0" % (dst, dst + 15, WP, WP + 1),
-            "s_load_dwordx16 s[%d:%d], s[%d:%d], 0x40" % (dst + 16, dst + 31, WP, WP + 1)]
+def load_words(dst=WS, offset=0):
+    return ["s_load_dwordx16 s[%d:%d], s[%d:%d], 0x%x" % (dst, dst + 15, WP, WP + 1, offset),
+            "s_load_dwordx16 s[%d:%d], s[%d:%d], 0x%x" % (dst + 16, dst + 31, WP, WP + 1, offset + 0x40)]
 
 
 def walk_and_load(slot, f):
@@ -201,7 +201,12 @@ def body(bits, zero_top=False, wide=False, unused_top=False):
           "s_mov_b64 s[%d:%d], %%%d" % (WP, WP + 1, f.op_wptr),
           "s_mov_b32 s%d, %%%d" % (KOFF, f.op_walk), "s_mov_b32 s%d, %%%d" % (FWC, f.op_walk + 1),
           "s_mov_b32 s%d, %%%d" % (FHC, f.op_walk + 2)]
-    L += load_words(W if wide else WS)
+    if wide:
+        # the loop adds a group's 128 * num bytes before its first use of the pointer
+        L += ["s_sub_u32 s%d, s%d, %d" % (WP, WP, 128 * num), "s_subb_u32 s%d, s%d, 0" % (WP + 1, WP + 1)]
+        L += load_words(W, 128 * num)
+    else:
+        L += load_words(WS)
     L += ["s_memrealtime s[%d:%d]" % (TIME, TIME + 1)]
     for i in range(D):
         L += walk_and_load(i, f)
@@ -217,11 +222,13 @@ def body(bits, zero_top=False, wide=False, unused_top=False):
             # of slot 0 is the same in every group), the other set receives the next slot's row (one
             # row past the end reads the spare row that follows the codes in the weight blob)
             cur, nxt = (W, WS) if i % 2 == 0 else (WS, W)
-            L += ["s_add_u32 s%d, s%d, 128" % (WP, WP), "s_addc_u32 s%d, s%d, 0" % (WP + 1, WP + 1),
-                  "s_waitcnt lgkmcnt(0)"]
+            L += ["s_waitcnt lgkmcnt(0)"]
             if i == 0:
+                # the word pointer moves once per group (no load is in flight here); the rows of the
+                # group are at fixed offsets from it
+                L += ["s_add_u32 s%d, s%d, %d" % (WP, WP, 128 * num), "s_addc_u32 s%d, s%d, 0" % (WP + 1, WP + 1)]
                 L += take_turn(0, f.waves)  # once per K group: a group is a few us, a turn 41
-            L += load_words(nxt)
+            L += load_words(nxt, 128 * (i + 1))
             if i == num - 1:
                 L += ["s_memrealtime s[%d:%d]" % (TIME, TIME + 1)]  # read at the next turn check
         elif i % 2 == 0:
