@@ -419,17 +419,17 @@ def main():
             "unit": "Tpair/s",
             "frac": pairs / kernel_s / PEAK_PAIRS,
             # HBM bytes of one launch of the dominant shape (layer1 3x3 conv, 8 of the 21 launches are
-            # this size): 100.4 MB read + 82.7 MB written (tiles shared by two workgroups are combined
+            # this size): 109.4 MB read + 67.1 MB written (tiles shared by two workgroups are combined
             # with atomic adds), from the FETCH_SIZE / WRITE_SIZE runs summarised in
             # profiles/shift_kernel_layer1_conv_counters.md (106.6 MB algorithmic)
-            "traffic": 183.1e6,
+            "traffic": 176.5e6,
             # vector instructions the dominant kernel issues per pair (SQ_INSTS_VALU, same profile):
             # `peak` prices a pair at 2 instructions, so its fraction can exceed 1
-            "valu_instr_per_pair": 1.29,
+            "valu_instr_per_pair": 1.28,
             # the same lanes x nominal clock priced at the kernel's own instruction count: the ceiling of
             # this kernel design, below 1 by the vector-issue gaps (two scalar instructions per code)
-            "peak_at_kernel_mix": PEAK_PAIRS * VALU_INSTR_PER_PAIR / 1.29 / 1e12,
-            "frac_at_kernel_mix": pairs / kernel_s / (PEAK_PAIRS * VALU_INSTR_PER_PAIR / 1.29),
+            "peak_at_kernel_mix": PEAK_PAIRS * VALU_INSTR_PER_PAIR / 1.28 / 1e12,
+            "frac_at_kernel_mix": pairs / kernel_s / (PEAK_PAIRS * VALU_INSTR_PER_PAIR / 1.28),
             "avg_launch_us": kernel_s / len(layers) * 1e6,
             "peak_calibrated": peak_cal / 1e12 if peak_cal else None,
             "frac_of_calibrated": pairs / kernel_s / peak_cal if peak_cal else None,

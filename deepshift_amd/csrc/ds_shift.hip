@@ -287,7 +287,7 @@ constexpr int kPlaneRowsWide = 2;  // ... of the 64-channel form (ROWS_WIDE): tw
 constexpr int plane_rows(bool wide) { return wide ? kPlaneRowsWide : kPlaneRows; }
 constexpr int kPlaneSlots = 3072;  // wave slots of the machine at 3 waves per SIMD (256 CUs x 4 SIMDs)
 
-constexpr int kPlaneSlotsWide = 2048;  // the 64-channel form holds 246 registers: 2 waves per SIMD
+constexpr int kPlaneSlotsWide = 2048;  // the 64-channel form runs 2 waves per SIMD (they interleave best)
 
 #define DS_PLANES_INPUTS                                                                          \
     : "v"(xoff[0]), "v"(xoff[1]), "v"(xoff[2]), "s"(rsrc), "s"(wptr), "s"(groups), "s"(w.koff),   \
@@ -470,7 +470,7 @@ __device__ __forceinline__ void planes_tile_body(const ShiftArgs &p)
 // Work-balanced launch: the (tile, K group) iteration space is cut into one equal contiguous share
 // per wave, so every wave of the launch does the same number of group iterations whatever the tile
 // count (each wave touches at most a few tiles; tiles shared between waves are combined with
-// atomic adds onto the pre-filled output).  tiles_m4 holds the number of 192-pixel tiles here.
+// atomic adds onto the pre-filled output).  tiles_m4 holds the number of pixel tiles (192 or 128 pixels) here.
 template <int BITS, int ZT, bool WIDE>
 __device__ __forceinline__ void planes_balanced_body(const ShiftArgs &p)
 {
@@ -522,8 +522,8 @@ void shift_planes_wide_balanced_kernel(const ShiftArgs p)
 }
 
 // Workgroup-cooperative launch of the 64-channel form: the (tile, K group) space is cut into one
-// equal share per workgroup of eight waves; the waves split the K range of a tile among themselves
-// and combine their sums in a 48 KiB LDS tile (LDS atomics cost next to nothing), and the tile goes
+// equal share per workgroup of four (or eight) waves; the waves split the K range of a tile among
+// themselves and combine their sums in a 32 KiB LDS tile (LDS atomics cost next to nothing), and the tile goes
 // to the output once: a plain store of sum + bias when the workgroup ran the tile's whole reduction,
 // atomic adds onto the pre-filled output when it shares the tile with a neighbouring workgroup.
 // Global atomics retire one lane per clock and L2 channel and do not overlap the arithmetic of the
@@ -542,7 +542,7 @@ void shift_planes_wide_cu_kernel(const ShiftArgs p)
     // out and clears its channels of that buffer, and goes on to tile t + 1 in the other buffer;
     // nobody adds to buffer t % 2 again before the barrier of tile t + 1, which every wave reaches
     // after it has cleared its channels.  With one buffer a second barrier follows the clearing.
-    extern __shared__ int32_t tile_sums[];  // [BUFFERS][64 channels][192 pixels]
+    extern __shared__ int32_t tile_sums[];  // [BUFFERS][64 channels][128 pixels]
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lane = threadIdx.x & (kWave - 1);
     const int bid = blockIdx.x;

@@ -32,10 +32,12 @@ let three waves share a SIMD.
 
 Every loop also comes in a "wide" form (suffix W) for layers whose channel count is a multiple of 64:
 J = 64 channels per lane, so the planes are shared by twice as many terms (1 + 2^BITS/64 vector
-instructions per term).  It keeps 192 accumulators in v[64 + 64*r + j], needs 246 registers for 4-bit
-fields (two waves per SIMD), reads one code row per reduction slot -- word j holds the codes of
-channels j (low half) and j + 32 (high half) -- and alternates between the two SGPR sets instead of
-copying.
+instructions per term) and ROWS_WIDE = 2 pixel rows: a code then costs two scalar and two vector
+instructions, a pattern that the two waves of a SIMD interleave without gaps (with three rows the
+vector pipe idled 13 % of the time in a compute-only replica of the loop).  It keeps 128 accumulators
+in v[64 + 64*r + j], runs at two waves per SIMD, reads one code row per reduction slot -- word j holds
+the codes of channels j (low half) and j + 32 (high half) -- alternates between the two SGPR sets
+instead of copying, moves its code pointer and checks its priority turn once per K group.
 A third family (DS_PAIRS_ASM_B<n>, fields of 1 or 2 bits) serves int8 activations: a lane register
 holds TWO pixels, hi * 65536 + lo, the planes are built with packed 16-bit shifts, the sign of a code
 selects a negated plane instead of an xor mask (plane index = field, 2^BITS + field for a negative
