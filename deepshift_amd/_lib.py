@@ -27,6 +27,12 @@ SIGNATURES = {
     "ds_tiled_bytes": (_size, [_c_int, _c_int, _c_int]),
     "ds_tile_weights_i32": (_c_int, [_ptr, _ptr] + [_c_int] * 6 + [_ptr]),
     "ds_tile_weights_zero_top_i32": (_c_int, [_ptr, _ptr] + [_c_int] * 5 + [_ptr]),
+    "ds_convert_stats_f32": (_c_int, [_ptr, _c_i64, _c_int, _c_int, _ptr, _ptr]),
+    "ds_convert_weights_f32": (_c_int, [_ptr, _ptr] + [_c_int] * 6 + [_ptr]),
+    "ds_convert_codes_f32": (_c_int, [_ptr, _ptr, _ptr, _c_i64, _c_int, _c_int, _ptr]),
+    "ds_scan_words_i32": (_c_int, [_ptr, _c_int, _c_int, _c_int, _ptr, _ptr]),
+    "ds_check_words_i32": (_c_int, [_ptr] + [_c_int] * 5 + [_ptr, _ptr]),
+    "ds_check_bound_i8": (_c_int, [_ptr, _c_i64, _c_int, _ptr, _ptr]),
     "ds_paired_bytes": (_size, [_c_int, _c_int, _c_int]),
     "ds_tile_weights_paired_i32": (_c_int, [_ptr, _ptr] + [_c_int] * 6 + [_ptr]),
     "ds_conv2d_paired_i8": (_c_int, [_ptr] * 4 + [_c_int] * 11 + [_ptr]),
@@ -41,6 +47,8 @@ SIGNATURES = {
     "ds_conv2d_i32": (_c_int, [_ptr] * 4 + [_c_int] * 11 + [_ptr, _size, _ptr]),
     "ds_conv2d_tiled_workspace_bytes": (_size, [_c_int] * 10),
     "ds_conv2d_tiled_i32": (_c_int, [_ptr] * 4 + [_c_int] * 11 + [_ptr, _size, _ptr]),
+    "ds_cpu_linear_i32": (_c_int, [_ptr] * 5 + [_c_int] * 4),
+    "ds_cpu_conv2d_i32": (_c_int, [_ptr] * 5 + [_c_int] * 10),
     "ds_quantize_f32_i32": (_c_int, [_ptr, _ptr, _c_i64, _c_int, _c_int, _c_int, _ptr]),
     "ds_quantize_pad_f32_i32": (_c_int, [_ptr, _ptr] + [_c_int] * 9 + [_ptr]),
     "ds_quantize_transpose_f32_i32": (_c_int, [_ptr, _ptr] + [_c_int] * 6 + [_ptr]),
@@ -56,6 +64,7 @@ SIGNATURES = {
     "ds_mul_linear_f32": (_c_int, [_ptr, _c_int, _ptr, _ptr, _ptr] + [_c_int] * 3 + [_ptr]),
     "ds_valu_calibrate": (_c_int, [_ptr, _c_int, _c_int, _ptr]),
     "ds_copy_i32": (_c_int, [_ptr, _ptr, _c_i64, _ptr]),
+    "ds_test_tune": (_c_int, [ctypes.c_char_p, _c_int]),
 }
 
 _LIB = None

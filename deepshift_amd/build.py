@@ -2,6 +2,7 @@
 
     python -m deepshift_amd.build            # rebuild unconditionally
     python -m deepshift_amd.build --if-stale # only when a source is newer than the library
+    python -m deepshift_amd.build --incremental  # recompile only the units that changed
 """
 import glob
 import os
@@ -30,7 +31,8 @@ def hipcc():
 
 
 def sources():
-    return sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+    """The HIP translation units and the host-only ones (the CPU twins of the kernels)."""
+    return sorted(glob.glob(os.path.join(CSRC, "*.hip")) + glob.glob(os.path.join(CSRC, "*.cpp")))
 
 
 def is_stale():
@@ -42,8 +44,14 @@ def is_stale():
     return any(os.path.getmtime(p) > built for p in deps)
 
 
-def build(verbose=True):
-    """Compile every .hip translation unit (in parallel) and link the shared library."""
+def _deps(src):
+    return [src] + glob.glob(os.path.join(CSRC, "*.h")) + glob.glob(os.path.join(CSRC, "*.inc")) + \
+        glob.glob(os.path.join(_HERE, "..", "include", "*.h"))
+
+
+def build(verbose=True, incremental=False):
+    """Compile every translation unit (in parallel) and link the shared library.  ``incremental``
+    skips the units whose object file is newer than the source and every header."""
     os.makedirs(LIB_DIR, exist_ok=True)
     # the asm main loop of the shift-plane kernel is generated text (csrc/ds_planes_asm.inc)
     subprocess.check_call([sys.executable, os.path.join(CSRC, "gen_planes_asm.py")])
@@ -52,9 +60,16 @@ def build(verbose=True):
     procs = []
     objs = []
     for src in sources():
-        obj = os.path.join(obj_dir, os.path.basename(src)[:-4] + ".o")
+        obj = os.path.join(obj_dir, os.path.splitext(os.path.basename(src))[0] + ".o")
         objs.append(obj)
-        cmd = [hipcc()] + HIPCC_FLAGS + ["-c", src, "-o", obj]
+        if incremental and os.path.exists(obj) and \
+                all(os.path.getmtime(d) <= os.path.getmtime(obj) for d in _deps(src)):
+            continue
+        if src.endswith(".cpp"):
+            cmd = [hipcc(), "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-pthread", "-Wall",
+                   "-c", src, "-o", obj]
+        else:
+            cmd = [hipcc()] + HIPCC_FLAGS + ["-c", src, "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
@@ -70,7 +85,7 @@ def build(verbose=True):
             failed = True
     if failed:
         raise RuntimeError("hipcc failed")
-    cmd = [hipcc(), "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", LIB_PATH] + objs
+    cmd = [hipcc(), "--offload-arch=" + ARCH, "-shared", "-fPIC", "-pthread", "-o", LIB_PATH] + objs
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
@@ -81,4 +96,4 @@ if __name__ == "__main__":
     if "--if-stale" in sys.argv and not is_stale():
         print("up to date:", LIB_PATH)
     else:
-        print(build())
+        print(build(incremental="--incremental" in sys.argv))

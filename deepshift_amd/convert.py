@@ -40,7 +40,7 @@ def _convert_linear(linear, shift_type, convert_weights, freeze_sign, kw):
             layer.shift.data, layer.sign.data = utils.get_shift_and_sign(linear.weight)
             layer.bias = linear.bias
             if _kernel_on_gpu(kw['use_kernel'], kw['use_cuda']):
-                modules.pack_module_weights(layer)
+                modules.pack_from_float_weight(layer, linear.weight)
     else:
         raise ValueError('Unsupported shift_type argument: ', shift_type)
     return layer.to(linear.weight.device)
@@ -65,7 +65,10 @@ def _convert_conv2d(conv, shift_type, convert_weights, freeze_sign, kw):
             layer.bias = conv.bias
         layer = layer.to(conv.weight.device)
         if _kernel_on_gpu(kw['use_kernel'], kw['use_cuda']):
-            modules.pack_module_weights(layer)
+            if convert_weights == True:  # noqa: E712
+                modules.pack_from_float_weight(layer, conv.weight)
+            else:
+                modules.pack_module_weights(layer)
     else:
         raise ValueError('Unsupported shift_type argument: ', shift_type)
     return layer.to(conv.weight.device)

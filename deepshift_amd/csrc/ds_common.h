@@ -38,6 +38,21 @@ __device__ __forceinline__ uint32_t div_by(uint32_t n, const FastDiv &f)
     return (t + ((n - t) >> f.s1)) >> f.s2;
 }
 
+// Launch-variant overrides for the test-suite (ds_test_tune): kTuneUnset leaves the dispatch's own
+// choice in place.  Process-wide, set only between launches.
+constexpr int kTuneUnset = -2147483647 - 1;
+struct Tune {
+    int planes = kTuneUnset;  // 0 / 1: two-instruction kernel / shift-plane kernel
+    int split = kTuneUnset;   // K split (plane kernels: 0 = equal shares, 1 = one tile per wave, -r = r x shares)
+    int tile = kTuneUnset;    // R * 100 + J of the two-instruction kernel
+    int cu = kTuneUnset;      // 0 / 4 / 8: cooperative launch off / four / eight waves per workgroup
+    int notail = kTuneUnset;  // int8 kernel: keep the last round of tiles on the tile-per-wave launch
+};
+extern Tune g_tune;
+
+// Compute units of the current device (cached per device; 256 on an MI355X).
+int device_cus();
+
 inline int hip_status(hipError_t e) { return e == hipSuccess ? DS_OK : DS_EHIP - (int)e; }
 inline int launch_status() { return hip_status(hipGetLastError()); }
 

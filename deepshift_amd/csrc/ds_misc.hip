@@ -1,5 +1,7 @@
 // Version / status strings and the VALU calibration kernel.
 #include "ds_common.h"
+#include <atomic>
+#include <string>
 
 namespace ds {
 
@@ -36,9 +38,39 @@ __global__ __launch_bounds__(256) void valu_calibrate_kernel(int32_t *sink, int 
     sink[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = total;
 }
 
+Tune g_tune;
+
+int device_cus()
+{
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n > 0) return n;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) n = 256;
+    cached[dev].store(n, std::memory_order_relaxed);
+    return n;
+}
+
 }  // namespace ds
 
 using namespace ds;
+
+DS_EXPORT int ds_test_tune(const char *knob, int value)
+{
+    if (!knob) {
+        g_tune = Tune();
+        return DS_OK;
+    }
+    const std::string k(knob);
+    if (k == "planes") g_tune.planes = value;
+    else if (k == "split") g_tune.split = value;
+    else if (k == "tile") g_tune.tile = value;
+    else if (k == "cu") g_tune.cu = value;
+    else if (k == "notail") g_tune.notail = value;
+    else return DS_EINVAL;
+    return DS_OK;
+}
 
 DS_EXPORT int ds_version(void) { return 100; }
 

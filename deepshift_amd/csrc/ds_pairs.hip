@@ -67,7 +67,7 @@ struct PairWalk {
 
 constexpr int kPairRows = 3;               // accumulator rows per lane, two pixels each
 constexpr int kPairPixels = 6 * kWave;     // pixels of a tile
-constexpr int kPairSlots = 2048;           // wave slots of the machine at 2 waves per SIMD
+static int pair_slots() { return device_cus() * 8; }  // wave slots of the machine at 2 waves per SIMD
 
 // K groups per call of the asm loop: as many reduction indices as keep a sum of terms of magnitude
 // <= x_bound within 16 bits (255 for x_bound = 128: 255 * 128 < 2^15)
@@ -435,9 +435,10 @@ static int launch_pairs(PairArgs a, hipStream_t st)
     // A wave that has a SIMD to itself issues at well under half the rate of two that share one, so
     // with fewer tiles than wave slots only short reductions (where the cooperative split would leave
     // a wave a group or two) stay one tile per wave.
-    int regime = (a.comm <= a.chunk && (tiles >= kPairSlots || a.comm < 16)) ? 1 : 2;
-    if (const char *t = getenv("DS_TUNE_SPLIT")) {
-        regime = atoi(t);
+    const int slots = pair_slots();
+    int regime = (a.comm <= a.chunk && (tiles >= slots || a.comm < 16)) ? 1 : 2;
+    if (g_tune.split != kTuneUnset) {
+        regime = g_tune.split;
         if (regime == 1 && a.comm > a.chunk) regime = 0;
     }
     if (regime == 1) {
@@ -445,10 +446,10 @@ static int launch_pairs(PairArgs a, hipStream_t st)
         // 60 % of the slots goes to the workgroup-cooperative kernel instead, whole tiles per
         // workgroup (plain stores as well): its waves split each tile's reduction, so the tail of
         // the launch takes a fraction of a tile time instead of a whole one.
-        const long rounds = tiles / kPairSlots, rest = tiles % kPairSlots;
+        const long rounds = tiles / slots, rest = tiles % slots;
         long head = tiles;
-        if (rounds >= 1 && rest > 0 && rest * 10 <= (long)kPairSlots * 6) head = rounds * kPairSlots;
-        if (getenv("DS_TUNE_NOTAIL")) head = tiles;
+        if (rounds >= 1 && rest > 0 && rest * 10 <= (long)slots * 6) head = rounds * slots;
+        if (g_tune.notail != kTuneUnset && g_tune.notail) head = tiles;
         a.atomic_out = 0;
         a.tile_end = (int)head;
         a.blocks_per_xcd = ceil_div((int)ceil_div((int)head, 4), 8);
@@ -458,7 +459,7 @@ static int launch_pairs(PairArgs a, hipStream_t st)
         a.tile_end = (int)tiles;
         a.whole_tiles = 1;
         const long rest_blocks = (rest + 7) / 8 * 8;
-        return launch_pairs_cu<BITS, TU>(a, rest_blocks < 256 ? (int)rest_blocks : 256, st);
+        return launch_pairs_cu<BITS, TU>(a, rest_blocks < slots / 8 ? (int)rest_blocks : slots / 8, st);
     }
     a.atomic_out = 1;
     long fill_blocks = ((long)a.y_elems / 4 + 255) / 256;
@@ -468,8 +469,8 @@ static int launch_pairs(PairArgs a, hipStream_t st)
     if (regime == 2) {
         // reductions of a single chunk: four-wave workgroups on a tile buffer of packed pairs
         bool four = a.comm <= a.chunk;
-        if (const char *t = getenv("DS_TUNE_CU")) four = four && atoi(t) == 4;
-        int blocks = four ? 512 : 256;
+        if (g_tune.cu != kTuneUnset) four = four && g_tune.cu == 4;
+        int blocks = four ? slots / 4 : slots / 8;  // one or two workgroups per compute unit
         const long fit = (iters / 64) / 8 * 8;  // small layers: at least 8 K groups per wave
         if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
         if (four) {
@@ -478,7 +479,7 @@ static int launch_pairs(PairArgs a, hipStream_t st)
         }
         return launch_pairs_cu<BITS, TU>(a, blocks, st);
     }
-    int blocks = kPairSlots / 4;
+    int blocks = slots / 4;
     const long fit = (iters / 16) / 8 * 8;  // small layers: at least 4 K groups per wave
     if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
     hipLaunchKernelGGL((shift_pairs_balanced_kernel<BITS, TU>), dim3(blocks), dim3(256), 0, st, a);

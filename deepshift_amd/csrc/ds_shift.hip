@@ -285,9 +285,9 @@ constexpr int kPlaneRows = 3;      // pixels per lane of the 32-channel form (R 
 constexpr int kPlaneRowsWide = 2;  // ... of the 64-channel form (ROWS_WIDE): two scalar and two vector
                                    // instructions per code, which two waves interleave without gaps
 constexpr int plane_rows(bool wide) { return wide ? kPlaneRowsWide : kPlaneRows; }
-constexpr int kPlaneSlots = 3072;  // wave slots of the machine at 3 waves per SIMD (256 CUs x 4 SIMDs)
-
-constexpr int kPlaneSlotsWide = 2048;  // the 64-channel form runs 2 waves per SIMD (they interleave best)
+// Wave slots of the machine: the 32-channel form runs 3 waves per SIMD, the 64-channel form 2 (they
+// interleave best); 4 SIMDs per compute unit -- 3072 and 2048 on the 256 CUs of an MI355X.
+static int plane_slots(bool wide) { return device_cus() * 4 * (wide ? 2 : 3); }
 
 #define DS_PLANES_INPUTS                                                                          \
     : "v"(xoff[0]), "v"(xoff[1]), "v"(xoff[2]), "s"(rsrc), "s"(wptr), "s"(groups), "s"(w.koff),   \
@@ -602,7 +602,7 @@ static int launch_planes_cu(const ShiftArgs &a, long iters, hipStream_t st)
         }
     }
     // one workgroup per 8 wave slots (2 waves per SIMD); small layers: >= 8 K groups per wave
-    int blocks = kPlaneSlotsWide / WAVES;
+    int blocks = plane_slots(true) / WAVES;
     const long fit = (iters / (8 * WAVES)) / 8 * 8;
     if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
     hipLaunchKernelGGL((shift_planes_wide_cu_kernel<BITS, ZT, WAVES>), dim3(blocks), dim3(WAVES * 64), kLdsBytes,
@@ -687,7 +687,7 @@ static int launch_shift(ShiftArgs a, int nsplit, hipStream_t st)
 // tiles, i.e. 1..3.06 waves per SIMD, which caps it at ~77 %.  Splitting K multiplies the number of
 // (shorter) waves; measured on MI355X the best point is ~24k waves of >= 12 packed words each
 // (the atomic combine is hidden behind the VALU work), e.g. layer1 3x3x64: 60 % -> 80 % of peak.
-// DS_TUNE_TILE=RxJ and DS_TUNE_SPLIT=n (environment) override the choice for experiments.
+// The test hook ds_test_tune ("tile", "split") overrides the choice.
 struct TileChoice {
     int R, J, nsplit;
 };
@@ -699,7 +699,7 @@ static TileChoice choose_tile(const ShiftArgs &a)
     else if (a.M <= 64) { c.R = 1; c.J = a.N >= 256 ? 8 : 32; }  // a single wave of rows: many narrow tiles
     else if (a.comm <= 32 && a.N >= 64) { c.R = 4; c.J = 16; }  // short reduction (e.g. 7x7x3 stem)
     else if (a.x_col_stride > 1 && a.OW > 8) { c.R = 3; c.J = 16; }  // strided pixels: half-used lines
-    const long simds = 1024;
+    const long simds = 4L * device_cus();
     // short layers (the 1x1 shortcuts of small images): with fewer than two 128-pixel tiles per SIMD
     // the launch is set by its start-up and the fullest SIMD; single-row tiles double the waves
     if (c.R > 1 && a.N >= 32 && (long)ceil_div(a.M, 2 * kWave) * ceil_div(a.N, 32) < 2 * simds) {
@@ -724,7 +724,7 @@ template <int BITS, int ZT, bool WIDE>
 static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
 {
     constexpr int R = plane_rows(WIDE), J = WIDE ? 64 : 32;
-    constexpr int kSlots = WIDE ? kPlaneSlotsWide : kPlaneSlots;
+    const int kSlots = plane_slots(WIDE);
     a.tiles_n = ceil_div(a.N, J);
     if (nsplit <= 0 && a.comm > 0) {
         // balanced launch: one share of the iteration space per wave slot (3 waves per SIMD)
@@ -739,13 +739,13 @@ static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
         if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
         // Workgroup-cooperative (four waves per workgroup) when a wave's quarter of a tile's reduction
         // is long enough to carry the extra segment ends: from 64 K groups per tile.  Short reductions
-        // over many tiles (stems, 1x1 layers) keep the wave-level shares.  DS_TUNE_CU=0 / 4 / 8
-        // overrides (8: eight waves per workgroup).
+        // over many tiles (stems, 1x1 layers) keep the wave-level shares.  The test hook's "cu" knob
+        // (0 / 4 / 8) overrides (8: eight waves per workgroup).
         bool cooperative = WIDE && a.comm >= 64;
         int cu_waves = 4;
-        if (const char *t = getenv("DS_TUNE_CU")) {
-            cooperative = WIDE && atoi(t) > 0;
-            cu_waves = atoi(t) == 8 ? 8 : 4;
+        if (g_tune.cu != kTuneUnset) {
+            cooperative = WIDE && g_tune.cu > 0;
+            cu_waves = g_tune.cu == 8 ? 8 : 4;
         }
         if (cooperative) {
             if constexpr (WIDE) {
@@ -785,7 +785,7 @@ static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
 // -1 = the layer is better off on the two-instruction kernel.
 static int plane_regime(const ShiftArgs &a, bool wide)
 {
-    const long slots = wide ? kPlaneSlotsWide : kPlaneSlots;
+    const long slots = plane_slots(wide);
     const int J = wide ? 64 : 32;
     const long tiles = (long)ceil_div(a.M, plane_rows(wide) * kWave) * ceil_div(a.N, J);
     const long iters = tiles * a.comm;
@@ -813,7 +813,7 @@ static int dispatch_zero_top(const ShiftArgs &a, hipStream_t st)
     const bool wide = tiled_wide(a.N, a.K, BITS);
     const int r = plane_regime(a, wide);
     int nsplit = (r >= 0 ? r : -1 - r) > 0 ? 1 : 0;
-    if (const char *sp = getenv("DS_TUNE_SPLIT")) nsplit = atoi(sp);
+    if (g_tune.split != kTuneUnset) nsplit = g_tune.split;
     return wide ? launch_planes<BITS, 1, true>(a, nsplit, st) : launch_planes<BITS, 1, false>(a, nsplit, st);
 }
 
@@ -831,13 +831,12 @@ static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
         //    the pre-fill.  Tiles that already fill whole rounds of slots keep one tile per wave.
         // The 1x1 shortcuts of small images, single-wave batches and layers with few channels stay on
         // the two-instruction kernel.
-        const char *t = getenv("DS_TUNE_PLANES");
         const bool wide = tiled_wide(a.N, a.K, BITS);  // decided by the shape alone, as at tiling time
         bool planes = plane_regime(a, wide) >= 0;
-        if (t) planes = atoi(t) > 0;
+        if (g_tune.planes != kTuneUnset) planes = g_tune.planes > 0;
         if (planes) {
             int nsplit = plane_regime(a, wide) > 0 ? 1 : 0;
-            if (const char *sp = getenv("DS_TUNE_SPLIT")) nsplit = atoi(sp);
+            if (g_tune.split != kTuneUnset) nsplit = g_tune.split;
             // the highest field value unused: the form without its plane
             if (a.top_unused)
                 return wide ? launch_planes<BITS, 2, true>(a, nsplit, st)
@@ -847,8 +846,8 @@ static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
         }
     }
     TileChoice c = choose_tile(a);
-    if (const char *t = getenv("DS_TUNE_TILE")) sscanf(t, "%dx%d", &c.R, &c.J);
-    if (const char *t = getenv("DS_TUNE_SPLIT")) c.nsplit = atoi(t);
+    if (g_tune.tile != kTuneUnset) { c.R = g_tune.tile / 100; c.J = g_tune.tile % 100; }
+    if (g_tune.split != kTuneUnset) c.nsplit = g_tune.split;
     if (c.R == 4 && c.J == 16) return launch_shift<BITS, GENERAL, 4, 16>(a, c.nsplit, st);
     if (c.R == 3 && c.J == 16) return launch_shift<BITS, GENERAL, 3, 16>(a, c.nsplit, st);
     if (c.R == 1 && c.J == 32) return launch_shift<BITS, GENERAL, 1, 32>(a, c.nsplit, st);

@@ -18,12 +18,17 @@ def _shift_layers(model):
 
 
 def _pack(m):
-    if m.conc_weight is None:
-        if isinstance(m, (modules_q.LinearShiftQ, modules_q.Conv2dShiftQ)):
-            modules_q.pack_module_weights_q(m)
-        else:
-            modules.pack_module_weights(m)
-    return m.conc_weight
+    return m.packed_weights()
+
+
+def _scan_fields(words, N, K, bits):
+    """(largest field below 32 or -1, number of zero codes) of reference-format words, counted on the
+    device."""
+    from . import _lib
+    out = torch.empty(4, dtype=torch.int32, device=words.device)
+    _lib.call("ds_scan_words_i32", _lib.ptr(words), N, K, bits, _lib.ptr(out), _lib.current_stream(words.device))
+    top, zeros = out[:2].tolist()
+    return int(top), int(zeros)
 
 
 def packed_state(model):
@@ -74,11 +79,15 @@ def load_packed(model, path_or_state, device=None):
         words = entry["words"].to(dev, torch.int32).contiguous()
         if words.numel() != param.shape[0] * comm:
             raise ValueError("%s: %d packed words, expected %d" % (name, words.numel(), param.shape[0] * comm))
-        top = entry.get("max_field")
-        if top is not None and not 0 <= int(top) < 2 ** bits:
-            raise ValueError("%s: max_field %s does not fit %d-bit fields" % (name, top, bits))
-        m.conc_weight = utils.ConcWeight(words, base, bits, int(entry.get("zero_top_bits", 0)),
-                                         None if top is None else int(top))
+        # max_field and zero_top_bits select kernel forms that assume them: take them from the words,
+        # never from the file (an understated value would give wrong sums without any error)
+        top, _ = _scan_fields(words, param.shape[0], K, bits)
+        top = max(top, 0)
+        zero_top = utils._zero_top_width(top) if (bits == 6 and base == 0) else 0
+        for key, mine in (("max_field", top), ("zero_top_bits", zero_top)):
+            if key in entry and int(entry[key]) != mine:
+                raise ValueError("%s: the file says %s = %s, its words say %d" % (name, key, entry[key], mine))
+        m.conc_weight = utils.ConcWeight(words, base, bits, zero_top, top)
         m.use_kernel = True
         if "bias" in entry and m.bias is not None:
             with torch.no_grad():

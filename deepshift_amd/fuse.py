@@ -55,14 +55,23 @@ class FusedConv2dShift(nn.Module):
             self.scale = None
             self.shift = None
 
+    def _check_handoff_dtype(self, input, conc_weight):
+        """The producer's pass writes this layer's input in the dtype chosen when the model was fused;
+        weights repacked since (``load_state_dict``) may need the other kernel."""
+        if not self.prequantized:
+            return
+        conv = self.conv
+        paired = kernels.paired_fields(conc_weight, conv.out_channels, conv.act_integer_bits,
+                                       conv.act_fraction_bits)
+        if (input.dtype == torch.int8) != bool(paired):
+            raise RuntimeError("the weights of a fused shift convolution changed in a way that moves it "
+                               "between the int8 and int32 kernels; fuse the model again")
+
     def forward(self, input, residual=None):
         conv = self.conv
-        if isinstance(conv, modules_q.Conv2dShiftQ):
-            if conv.conc_weight is None:
-                modules_q.pack_module_weights_q(conv)
-        elif conv.conc_weight is None:
-            modules.pack_module_weights(conv)
-        return modules.conv_kernel_forward(conv, input, conv.conc_weight, self.scale, self.shift,
+        conc_weight = conv.packed_weights()
+        self._check_handoff_dtype(input, conc_weight)
+        return modules.conv_kernel_forward(conv, input, conc_weight, self.scale, self.shift,
                                            residual, self.relu, self.prequantized, self.emit, self.pool,
                                            self.input_nonneg)
 
@@ -187,12 +196,9 @@ def _input_key(conv):
     None if it pads by itself."""
     if conv.padding_mode != 'zeros' or not conv.use_kernel:
         return None
-    if conv.conc_weight is None and conv.shift.is_cuda:
-        if isinstance(conv, modules_q.Conv2dShiftQ):
-            modules_q.pack_module_weights_q(conv)
-        else:
-            modules.pack_module_weights(conv)
-    paired = kernels.paired_fields(conv.conc_weight, conv.out_channels, conv.act_integer_bits,
+    param = conv.weight if isinstance(conv, modules_q.Conv2dShiftQ) else conv.shift
+    conc_weight = conv.packed_weights() if param.is_cuda else conv.conc_weight
+    paired = kernels.paired_fields(conc_weight, conv.out_channels, conv.act_integer_bits,
                                    conv.act_fraction_bits)
     return (tuple(conv.padding), conv.act_integer_bits, conv.act_fraction_bits,
             torch.int8 if paired else torch.int32)

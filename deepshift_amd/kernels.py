@@ -7,7 +7,11 @@ the current HIP stream of the input's device; outputs are new int32 tensors.
 
 Differences from the reference, all deliberate:
 
-* ``use_cuda=False`` (the reference's CPU kernel) is not offered here: it raises.
+* ``use_cuda=False`` runs the library's host twins (``ds_cpu_linear_i32`` / ``ds_cpu_conv2d_i32``)
+  on CPU tensors and returns the int32 sums (the reference converts its result list with
+  ``torch.Tensor(out)``, i.e. to float32, which rounds sums above 2^24; kernels.py:23-24,59-63),
+  and its convolution pads H by ``ph`` and W by ``pw`` (the reference's CPU branch hands the
+  2-tuple to ``F.pad`` and so pads W only, kernels.py:58).
 * ``dilation != 1`` / ``groups != 1`` raise instead of being silently ignored (kernels.py:28).
 * padding ``(ph, pw)`` pads H by ph and W by pw (the reference's tuple order,
   kernels.py:32-33, swaps them; identical for square padding).
@@ -72,10 +76,82 @@ class _Timed:
         return False
 
 
-def _no_cpu_kernel():
-    raise NotImplementedError(
-        "use_cuda=False selects the reference's CPU shift kernel, which this GPU library does "
-        "not provide; run the layer with use_cuda=True on a ROCm device")
+def _host_i32(name, t):
+    if t.is_cuda:
+        raise ValueError("%s must be a CPU tensor when use_cuda=False" % name)
+    if t.dtype != torch.int32:
+        raise TypeError("%s must be int32, got %s" % (name, t.dtype))
+    return t.contiguous()
+
+
+def _host_codes(shift, sign):
+    """The unpacked codes as the reference's CPU kernel receives them (kernels.py:23,59): the signed
+    exponent truncated to int8 (pybind's cast of the float parameter; -inf, the log of a zero weight,
+    and anything below -128 saturate, and such a code contributes 0 or -1 like any shift >= 31) and
+    the sign as int32."""
+    sh = torch.nan_to_num(shift.detach().float().cpu(), nan=-128.0, posinf=127.0, neginf=-128.0)
+    sh = sh.clamp(-128, 127).trunc().to(torch.int8).contiguous()
+    sg = sign.detach().float().cpu().trunc().to(torch.int32).contiguous()
+    return sh, sg
+
+
+def cpu_threads():
+    """Threads the host twins use (``None``/0: every hardware thread, as ATen's intra-op pool)."""
+    return _CPU_THREADS
+
+
+def set_cpu_threads(n):
+    global _CPU_THREADS
+    _CPU_THREADS = int(n) if n else 0
+
+
+_CPU_THREADS = 0
+
+
+def linear_cpu(input, shift, sign, bias=None):
+    """``kernels.linear(..., use_cuda=False)``: the host twin of the shift GEMM on unpacked codes
+    (the reference's ``deepshift_cpu.linear_kernel``, kernels.py:22-24)."""
+    input = _host_i32("input", input)
+    if input.dim() != 2:
+        raise ValueError("input must be [M, K]")
+    M, K = input.shape
+    N = shift.size(0)
+    if shift.numel() != N * K or sign.numel() != N * K:
+        raise ValueError("shift/sign must be [N, K] with K = %d" % K)
+    sh, sg = _host_codes(shift, sign)
+    if bias is not None:
+        bias = _host_i32("bias", bias)
+    out = torch.empty([M, N], dtype=torch.int32)
+    _lib.call("ds_cpu_linear_i32", _lib.ptr(input), _lib.ptr(sh), _lib.ptr(sg), _lib.ptr(bias),
+              _lib.ptr(out), M, K, N, _CPU_THREADS)
+    return out
+
+
+def conv2d_cpu(input, shift, sign, bias=None, stride=1, padding=0):
+    """``kernels.conv2d(..., use_cuda=False)``: the host twin of the shift convolution
+    (the reference's ``deepshift_cpu.convolution_kernel``, kernels.py:57-63)."""
+    input = _host_i32("input", input)
+    if input.dim() != 4:
+        raise ValueError("input must be NCHW")
+    ph, pw = _pair(padding)
+    sh_, sw_ = _pair(stride)
+    Nb, C, H, W = input.shape
+    O, Cw, FH, FW = shift.shape
+    if Cw != C:
+        raise ValueError("filter has %d input channels, input has %d" % (Cw, C))
+    if ph or pw:
+        input = torch.nn.functional.pad(input, (pw, pw, ph, ph)).contiguous()
+    Hp, Wp = H + 2 * ph, W + 2 * pw
+    if Hp < FH or Wp < FW:
+        raise ValueError("padded input %dx%d is smaller than the %dx%d filter" % (Hp, Wp, FH, FW))
+    sh, sg = _host_codes(shift, sign)
+    if bias is not None:
+        bias = _host_i32("bias", bias)
+    OH, OW = (Hp - FH) // sh_ + 1, (Wp - FW) // sw_ + 1
+    out = torch.empty([Nb, O, OH, OW], dtype=torch.int32)
+    _lib.call("ds_cpu_conv2d_i32", _lib.ptr(input), _lib.ptr(sh), _lib.ptr(sg), _lib.ptr(bias),
+              _lib.ptr(out), Nb, C, Hp, Wp, O, FH, FW, sh_, sw_, _CPU_THREADS)
+    return out
 
 
 # ---------------------------------------------------------------------------------------------
@@ -391,7 +467,7 @@ def linear(input, shift, sign, bias=None, conc_weight=None, use_cuda=True):
     Returns int32 [M, N].
     """
     if not use_cuda:
-        _no_cpu_kernel()
+        return linear_cpu(input, shift, sign, bias)
     assert conc_weight is not None
     input = _require_device_i32("input", input)
     if input.dim() != 2:
@@ -458,11 +534,11 @@ def conv2d(input, shift, sign, bias=None, conc_weight=None, stride=1, padding=0,
     from ``conc_weight`` (K ordered (ic, fh, fw)), zero ``padding``, ``stride``; returns int32
     [Nb, O, OH, OW] with OH = (H + 2*ph - FH) // sh + 1.
     """
-    if not use_cuda:
-        _no_cpu_kernel()
-    assert conc_weight is not None
     if _pair(dilation) != (1, 1) or groups != 1:
         raise NotImplementedError("the shift kernel supports dilation=1 and groups=1 only")
+    if not use_cuda:
+        return conv2d_cpu(input, shift, sign, bias, stride, padding)
+    assert conc_weight is not None
     input = _require_device_i32("input", input)
     if input.dim() != 4:
         raise ValueError("input must be NCHW")

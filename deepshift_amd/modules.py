@@ -33,12 +33,59 @@ def _param_tensor(check_grad, *shape):
     return torch.empty(*shape, dtype=torch.float64 if check_grad else torch.float32)
 
 
-def pack_module_weights(module):
-    """Build ``module.conc_weight`` from its (shift, sign) parameters, clamped to ``shift_range``
-    and rounded the way the float path reads them (modules.py:125-128,313-316)."""
+def module_codes(module):
+    """The (shift, sign) a PS layer computes with: clamped to ``shift_range`` and rounded the way
+    the float path reads them (modules.py:125-128,313-316)."""
     shift = module.shift.detach().clamp(*module.shift_range).round()
     sign = module.sign.detach().round().sign()
+    return shift, sign
+
+
+def _params_key(*params):
+    """Identity and version of the parameters packed weights were built from."""
+    return tuple((p.data_ptr(), p._version, p.device) for p in params)
+
+
+class _PackedWeightsMixin:
+    """``conc_weight`` as the reference has it (an attribute that is None until the first kernel
+    forward, modules.py:25-27), plus what the reference lacks: packed words that were built from the
+    layer's own parameters are rebuilt when those parameters change (``load_state_dict``, fine-tuning
+    then evaluating, ``round_shift_weights``).  A ``conc_weight`` assigned from outside is used as
+    given.  Changes are seen through the parameters' storage address and version counter, i.e. every
+    in-place update of the parameter itself and every assignment to ``.data``; an in-place operation
+    on ``param.data`` bypasses the version counter -- set ``conc_weight = None`` after one."""
+
+    _conc_weight = None
+    _packed_from = None
+
+    @property
+    def conc_weight(self):
+        return self._conc_weight
+
+    @conc_weight.setter
+    def conc_weight(self, value):
+        object.__setattr__(self, "_conc_weight", value)
+        object.__setattr__(self, "_packed_from", None)
+
+    def _weight_params(self):
+        return (self.shift, self.sign)
+
+    def _pack(self):
+        return pack_module_weights(self)
+
+    def packed_weights(self):
+        """The layer's ConcWeight, (re)built if it is missing or older than the parameters."""
+        if self._conc_weight is None or (self._packed_from is not None and
+                                         self._packed_from != _params_key(*self._weight_params())):
+            self._pack()
+        return self._conc_weight
+
+
+def pack_module_weights(module):
+    """Build ``module.conc_weight`` from its (shift, sign) parameters (see :func:`module_codes`)."""
+    shift, sign = module_codes(module)
     module.conc_weight = utils.compress_bits(shift, sign)
+    object.__setattr__(module, "_packed_from", _params_key(module.shift, module.sign))
     return module.conc_weight
 
 
@@ -60,7 +107,18 @@ class _FixedBias:
         return self.value
 
 
-class LinearShift(nn.Module):
+def pack_from_float_weight(module, weight):
+    """Conversion of a trained float layer (convert.py:72-76): the packed words straight from the float
+    weights in device passes (``utils.convert_weights``), valid for the module's (shift, sign)
+    parameters when those were just derived from the same weights with ``get_shift_and_sign``."""
+    if not weight.is_cuda:
+        return pack_module_weights(module)
+    module.conc_weight = utils.convert_weights(weight, module.shift_range)
+    object.__setattr__(module, "_packed_from", _params_key(module.shift, module.sign))
+    return module.conc_weight
+
+
+class LinearShift(_PackedWeightsMixin, nn.Module):
     def __init__(self, in_features, out_features, bias=True, check_grad=False, freeze_sign=False,
                  use_kernel=False, use_cuda=True, rounding='deterministic', weight_bits=5,
                  act_integer_bits=16, act_fraction_bits=16):
@@ -70,7 +128,6 @@ class LinearShift(nn.Module):
         self.use_kernel = use_kernel
         self.check_grad = check_grad
         self.use_cuda = use_cuda
-        self.conc_weight = None
         self.rounding = rounding
         self.shift_range = _shift_range(weight_bits)
         self.act_integer_bits, self.act_fraction_bits = act_integer_bits, act_fraction_bits
@@ -95,19 +152,20 @@ class LinearShift(nn.Module):
 
     def _kernel_forward(self, input):
         # modules.py:24-31: the input is cast, NOT rounded/clamped first (truncation toward zero)
-        if not self.use_cuda:
-            kernels._no_cpu_kernel()
-        if self.conc_weight is None:
-            pack_module_weights(self)
         I, Fb = self.act_integer_bits, self.act_fraction_bits
         lead = input.shape[:-1]
         x2d = input.reshape(-1, self.in_features).float()
         M = x2d.shape[0]
+        if not self.use_cuda:
+            shift, sign = module_codes(self)
+            out = linear_cpu_forward(x2d, shift, sign, self.bias, I, Fb, round_to_fixed=False)
+            return out.reshape(*lead, self.out_features)
+        conc_weight = self.packed_weights()
         xT = kernels.quantize_transpose(x2d, I, Fb, round_to_fixed=False)
         bias = self._fixed_bias.get(self.bias, I, Fb, round_to_fixed=False)
-        tiled = kernels._tiled_of(self.conc_weight, self.out_features, self.in_features)
-        out = kernels.linear_tiled(xT, M, tiled, bias, self.out_features, kernels.kernel_bits(self.conc_weight),
-                                   self.conc_weight.base)
+        tiled = kernels._tiled_of(conc_weight, self.out_features, self.in_features)
+        out = kernels.linear_tiled(xT, M, tiled, bias, self.out_features, kernels.kernel_bits(conc_weight),
+                                   conc_weight.base)
         return kernels.dequantize(out, Fb).reshape(*lead, self.out_features)
 
     def forward(self, input):
@@ -126,7 +184,7 @@ class LinearShift(nn.Module):
             self.in_features, self.out_features, self.bias is not None)
 
 
-class _ConvNdShift(nn.Module):
+class _ConvNdShift(_PackedWeightsMixin, nn.Module):
     __constants__ = ['stride', 'padding', 'dilation', 'groups', 'bias', 'padding_mode']
 
     def __init__(self, in_channels, out_channels, kernel_size, stride, padding, dilation, transposed,
@@ -196,6 +254,44 @@ def _circular_pad(x, padding):
     return F.pad(x, expanded, mode='circular')
 
 
+def _host_fixed(x, integer_bits, fraction_bits, round_to_fixed):
+    """float CPU tensor -> int32 fixed point with the GPU passes' arithmetic: ``round_to_fixed`` then
+    ``* 2^F`` (utils.py:7-21, modules.py:153), or the saturating truncating cast alone
+    (modules.py:25)."""
+    x = x.detach().float().cpu()
+    if round_to_fixed:
+        x = utils.round_to_fixed(x, integer_bits, fraction_bits)
+    scaled = (x.double() * 2.0 ** fraction_bits).trunc()
+    scaled = torch.nan_to_num(scaled, nan=0.0).clamp(-2.0 ** 31, 2.0 ** 31 - 1)
+    return scaled.to(torch.int32)
+
+
+def linear_cpu_forward(x2d, shift, sign, bias, integer_bits, fraction_bits, round_to_fixed):
+    """LinearShift / LinearShiftQ with ``use_kernel=True, use_cuda=False``: the library's host kernel
+    on the unpacked codes (modules.py:24-31 with kernels.py:22-24)."""
+    xq = _host_fixed(x2d, integer_bits, fraction_bits, round_to_fixed)
+    bq = None if bias is None else _host_fixed(bias, integer_bits, fraction_bits, round_to_fixed)
+    out = kernels.linear(xq, shift, sign, bq, None, use_cuda=False)
+    return (out.float() / 2.0 ** fraction_bits).to(x2d.device)
+
+
+def conv_cpu_forward(module, input, shift, sign):
+    """Conv2dShift / Conv2dShiftQ with ``use_kernel=True, use_cuda=False`` (modules.py:152-162 with
+    kernels.py:57-63)."""
+    if module.dilation != (1, 1) or module.groups != 1:
+        raise NotImplementedError("the shift kernel supports dilation=1 and groups=1 only")
+    I, Fb = module.act_integer_bits, module.act_fraction_bits
+    padding = module.padding
+    x = input.float()
+    if module.padding_mode == 'circular':
+        x = _circular_pad(x, padding)
+        padding = (0, 0)
+    xq = _host_fixed(x, I, Fb, True)
+    bq = None if module.bias is None else _host_fixed(module.bias, I, Fb, True)
+    out = kernels.conv2d(xq, shift, sign, bq, None, module.stride, padding, use_cuda=False)
+    return (out.float() / 2.0 ** Fb).to(input.device)
+
+
 def _small_for_int8(module, input_shape, field_bits):
     """The int8 kernel works on tiles of 384 pixels x 64 channels; a layer with few of them and a short
     reduction (the 1x1 shortcuts of a ResNet-18) is served better by the int32 kernels' smaller tiles.
@@ -229,7 +325,7 @@ def conv_kernel_forward(module, input, conc_weight, scale=None, shift=None, resi
     producer of a prequantized input vouches that it is the output of a ReLU (the int8 kernel then
     knows a tighter bound on the activations and widens its 16-bit sums less often)."""
     if not module.use_cuda:
-        kernels._no_cpu_kernel()
+        raise ValueError("conv_kernel_forward is the GPU path; use_cuda=False layers run conv_cpu_forward")
     if module.dilation != (1, 1) or module.groups != 1:
         raise NotImplementedError("the shift kernel supports dilation=1 and groups=1 only")
     I, Fb = module.act_integer_bits, module.act_fraction_bits
@@ -297,7 +393,6 @@ class Conv2dShift(_ConvNdShift):
         dilation = _pair(dilation)
         self.use_kernel = use_kernel
         self.use_cuda = use_cuda
-        self.conc_weight = None
         super(Conv2dShift, self).__init__(
             in_channels, out_channels, kernel_size, stride, padding, dilation, False, _pair(0),
             groups, bias, padding_mode, check_grad, freeze_sign, rounding, weight_bits,
@@ -305,9 +400,9 @@ class Conv2dShift(_ConvNdShift):
 
     def forward(self, input):
         if self.use_kernel:
-            if self.conc_weight is None:
-                pack_module_weights(self)
-            return conv_kernel_forward(self, input, self.conc_weight)
+            if not self.use_cuda:
+                return conv_cpu_forward(self, input, *module_codes(self))
+            return conv_kernel_forward(self, input, self.packed_weights())
         self.shift.data = ste.clamp(self.shift.data, *self.shift_range)
 
         shift_rounded = ste.round(self.shift, self.rounding)

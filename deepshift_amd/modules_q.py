@@ -19,7 +19,8 @@ from torch.nn import init
 from torch.nn.modules.utils import _pair
 
 from . import kernels, ste, utils
-from .modules import _FixedBias, _param_tensor, _circular_pad, conv_kernel_forward
+from .modules import (_FixedBias, _PackedWeightsMixin, _param_tensor, _params_key, _circular_pad,
+                      conv_cpu_forward, conv_kernel_forward, linear_cpu_forward)
 
 __all__ = ["LinearShiftQ", "Conv2dShiftQ"]
 
@@ -29,16 +30,35 @@ def _shift_range_q(weight_bits):
     return (-1 * (2 ** (weight_bits - 1) - 1), 0)
 
 
-def pack_module_weights_q(module):
-    """Pack the power-of-two rounding of ``module.weight`` (clamped like the forward pass does)."""
+def module_codes_q(module):
+    """(shift, sign) of the power-of-two rounding of ``module.weight``, clamped like the forward pass
+    does (modules_q.py:116,21 / :284,147)."""
     w = module.weight.detach().clone()
     w = utils.clampabs(w, 2 ** module.shift_range[0], 2 ** module.shift_range[1])
-    shift, sign = utils.get_shift_and_sign(w, 'deterministic')
-    module.conc_weight = utils.compress_bits(shift, sign)
+    return utils.get_shift_and_sign(w, 'deterministic')
+
+
+def pack_module_weights_q(module):
+    """Pack the power-of-two rounding of ``module.weight``: on the GPU straight from the float weights
+    (clamping |w| to [2^lo, 2^hi] then rounding log2 equals rounding then clamping the shift to
+    [lo, hi]; exact zeros stay zero, utils.py:44-52), elsewhere through the float codes."""
+    if module.weight.is_cuda:
+        module.conc_weight = utils.convert_weights(module.weight, module.shift_range)
+    else:
+        module.conc_weight = utils.compress_bits(*module_codes_q(module))
+    object.__setattr__(module, "_packed_from", _params_key(module.weight))
     return module.conc_weight
 
 
-class LinearShiftQ(nn.Module):
+class _PackedQMixin(_PackedWeightsMixin):
+    def _weight_params(self):
+        return (self.weight,)
+
+    def _pack(self):
+        return pack_module_weights_q(self)
+
+
+class LinearShiftQ(_PackedQMixin, nn.Module):
     def __init__(self, in_features, out_features, bias=True, check_grad=False, use_kernel=False,
                  use_cuda=True, rounding='deterministic', weight_bits=5, act_integer_bits=16,
                  act_fraction_bits=16):
@@ -48,7 +68,6 @@ class LinearShiftQ(nn.Module):
         self.use_kernel = use_kernel
         self.check_grad = check_grad
         self.use_cuda = use_cuda
-        self.conc_weight = None
         self.rounding = rounding
         self.shift_range = _shift_range_q(weight_bits)
         self.act_integer_bits, self.act_fraction_bits = act_integer_bits, act_fraction_bits
@@ -68,19 +87,20 @@ class LinearShiftQ(nn.Module):
             init.uniform_(self.bias, -bound, bound)
 
     def _kernel_forward(self, input):
-        if not self.use_cuda:
-            kernels._no_cpu_kernel()
-        if self.conc_weight is None:
-            pack_module_weights_q(self)
         I, Fb = self.act_integer_bits, self.act_fraction_bits
         lead = input.shape[:-1]
         x2d = input.reshape(-1, self.in_features).float()
         M = x2d.shape[0]
+        if not self.use_cuda:
+            shift, sign = module_codes_q(self)
+            out = linear_cpu_forward(x2d, shift, sign, self.bias, I, Fb, round_to_fixed=True)
+            return out.reshape(*lead, self.out_features)
+        conc_weight = self.packed_weights()
         xT = kernels.quantize_transpose(x2d, I, Fb, round_to_fixed=True)
         bias = self._fixed_bias.get(self.bias, I, Fb, round_to_fixed=True)
-        tiled = kernels._tiled_of(self.conc_weight, self.out_features, self.in_features)
-        out = kernels.linear_tiled(xT, M, tiled, bias, self.out_features, kernels.kernel_bits(self.conc_weight),
-                                   self.conc_weight.base)
+        tiled = kernels._tiled_of(conc_weight, self.out_features, self.in_features)
+        out = kernels.linear_tiled(xT, M, tiled, bias, self.out_features, kernels.kernel_bits(conc_weight),
+                                   conc_weight.base)
         return kernels.dequantize(out, Fb).reshape(*lead, self.out_features)
 
     def forward(self, input):
@@ -103,7 +123,7 @@ class LinearShiftQ(nn.Module):
             self.in_features, self.out_features, self.bias is not None)
 
 
-class Conv2dShiftQ(nn.Module):
+class Conv2dShiftQ(_PackedQMixin, nn.Module):
     __constants__ = ['stride', 'padding', 'dilation', 'groups', 'bias', 'padding_mode']
 
     def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1,
@@ -127,7 +147,6 @@ class Conv2dShiftQ(nn.Module):
         self.padding_mode = padding_mode
         self.use_kernel = use_kernel
         self.use_cuda = use_cuda
-        self.conc_weight = None
         self.rounding = rounding
         self.shift_range = _shift_range_q(weight_bits)
         self.act_integer_bits, self.act_fraction_bits = act_integer_bits, act_fraction_bits
@@ -149,9 +168,9 @@ class Conv2dShiftQ(nn.Module):
 
     def forward(self, input):
         if self.use_kernel:
-            if self.conc_weight is None:
-                pack_module_weights_q(self)
-            return conv_kernel_forward(self, input, self.conc_weight)
+            if not self.use_cuda:
+                return conv_cpu_forward(self, input, *module_codes_q(self))
+            return conv_kernel_forward(self, input, self.packed_weights())
         self.weight.data = ste.clampabs(self.weight.data, 2 ** self.shift_range[0],
                                         2 ** self.shift_range[1])
         weight_q = ste.round_power_of_2(self.weight, self.rounding)

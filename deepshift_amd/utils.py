@@ -13,7 +13,7 @@ import torch
 from . import kernels
 
 __all__ = ["round_to_fixed", "get_shift_and_sign", "round_power_of_2", "round", "clampabs",
-           "ConcWeight", "compress_bits", "ZERO_SHIFT"]
+           "ConcWeight", "compress_bits", "convert_weights", "ZERO_SHIFT"]
 
 # the reference encodes "this weight is zero" as a right shift by 32 (utils.py:68-70)
 ZERO_SHIFT = 32
@@ -131,7 +131,8 @@ def compress_bits(shift, sign):
         conc_weight.bits = max(1, int(math.ceil(math.log2(int(torch.max(s)) - minimum + 1))))
     else:
         conc_weight.base = 0
-        conc_weight.bits = max(1, shift_field_bits(int(torch.min(shift))))
+        # the width of the largest ROUNDED field (a shift of -31.6 rounds to the zero code 32)
+        conc_weight.bits = max(1, shift_field_bits(-int(torch.max(s))))
     if conc_weight.bits > 6:
         raise ValueError("shift range needs %d bits per code; at most 6 are supported" %
                          conc_weight.bits)
@@ -143,12 +144,60 @@ def compress_bits(shift, sign):
     real = s[s < ZERO_SHIFT]
     conc_weight.max_field = (int(real.max()) if real.numel() else 0) - conc_weight.base
     if conc_weight.bits == 6 and conc_weight.base == 0:
-        top = int(real.max()) if real.numel() else 0
-        for width in (1, 2, 3, 4):
-            if top <= 2 ** width - 2:
-                conc_weight.zero_top_bits = width
-                break
+        conc_weight.zero_top_bits = _zero_top_width(int(real.max()) if real.numel() else 0)
 
     conc_weight.data = kernels.compress_sign_and_shift(
         s.int().cuda(), sign.int().cuda(), size, conc_weight.base, conc_weight.bits, row_length, num)
     return conc_weight
+
+
+def _zero_top_width(top):
+    for width in (1, 2, 3, 4):
+        if top <= 2 ** width - 2:
+            return width
+    return 0
+
+
+def convert_weights(weight, shift_range):
+    """Float weights -> :class:`ConcWeight` in device passes only: ``get_shift_and_sign`` (utils.py:23-29),
+    the clamp of the shift to ``shift_range`` (modules.py:88,125,313) and ``compress_bits`` (:61-88)
+    without materialising the float ``shift`` / ``sign`` tensors.  One reduction pass reads what
+    ``compress_bits`` takes from ``torch.min`` (the field range, whether zero weights exist) and one
+    pass writes the packed words.  Bit-identical to
+    ``compress_bits(clamp(round(log2|w|), *shift_range), sign(w))``."""
+    from . import _lib
+    w = weight.detach()
+    if not w.is_cuda:
+        raise ValueError("convert_weights runs on the GPU: move the weights there first")
+    w = w.float().contiguous()
+    if w.numel() == 0:
+        raise ValueError("cannot pack an empty weight tensor")
+    lo, hi = int(shift_range[0]), int(shift_range[1])
+    stats = torch.empty(4, dtype=torch.int32, device=w.device)
+    st = _lib.current_stream(w.device)
+    _lib.call("ds_convert_stats_f32", _lib.ptr(w), w.numel(), lo, hi, _lib.ptr(stats), st)
+    max_s, min_s, zeros = (int(v) for v in stats[:3].tolist())
+    if max_s < min_s:          # every weight is zero
+        max_s = min_s = 0
+    cw = ConcWeight()
+    if min_s < 0:
+        # left shifts: the fields are stored relative to the smallest one (utils.py:75-80)
+        cw.base = min_s
+        top = ZERO_SHIFT if zeros else max_s
+        cw.bits = max(1, int(math.ceil(math.log2(top - min_s + 1))))
+        cw.max_field = max_s - min_s
+    else:
+        cw.base = 0
+        cw.bits = max(1, shift_field_bits(-(ZERO_SHIFT if zeros else max_s)))
+        cw.max_field = max_s
+        if cw.bits == 6:
+            cw.zero_top_bits = _zero_top_width(max_s)
+    if cw.bits > 6:
+        raise ValueError("shift range needs %d bits per code; at most 6 are supported" % cw.bits)
+    O = w.shape[0]
+    K = w[0].numel()
+    num = 32 // (cw.bits + 1)
+    out = torch.empty([O * ((K + num - 1) // num)], dtype=torch.int32, device=w.device)
+    _lib.call("ds_convert_weights_f32", _lib.ptr(w), _lib.ptr(out), O, K, lo, hi, cw.bits, cw.base, st)
+    cw.data = out
+    return cw

@@ -88,6 +88,48 @@ int ds_tile_weights_i32(const int32_t *w_ref, void *tiled, int N, int C, int FH,
 int ds_tile_weights_zero_top_i32(const int32_t *w_ref, void *tiled, int N, int C, int FH, int FW,
                                  int field_bits, ds_stream_t stream);
 
+/* ---- weight conversion on the device ---------------------------------------------------- */
+
+/* Replace utils.get_shift_and_sign (utils.py:23-29) + the clamp to the layer's shift range
+ * (modules.py:88,125,313; utils.clampabs :44-52 for the Q layers) + utils.compress_bits /
+ * COMPRESS_SIGN_SHIFT (utils.py:61-88, shift.cu:27-55) for whole float weight tensors:
+ *   sign = sign(w), shift = clamp(round_half_even(log(|w|) / ln 2), shift_min, shift_max)
+ * with the logarithm and the division evaluated in float32 as torch does on the CPU; a zero weight
+ * becomes the reference's zero code (s = -shift = 32, sign +, utils.py:68-70).
+ * ds_convert_stats_f32: stats[0..2] (device) = max s, min s over the non-zero weights
+ *   (INT_MIN / INT_MAX if there are none) and the number of zero weights -- what compress_bits reads
+ *   with torch.min to choose `bits` and `base` (utils.py:72-80); stats holds 4 ints.
+ * ds_convert_weights_f32: w[O][K] -> out[O][comm] reference-format words in one pass (the layout of
+ *   ds_pack_i32); `bits` must be 6 when the tensor has zero weights.
+ * ds_convert_codes_f32: the unpacked codes, s[n] and sign[n] in {-1, 0, +1} (zero weights: s = 32,
+ *   sign = 0). */
+int ds_convert_stats_f32(const float *w, int64_t n, int shift_min, int shift_max, int32_t *stats,
+                         ds_stream_t stream);
+int ds_convert_weights_f32(const float *w, int32_t *out, int O, int K, int shift_min, int shift_max,
+                           int bits, int base, ds_stream_t stream);
+int ds_convert_codes_f32(const float *w, int32_t *s, int32_t *sign, int64_t n, int shift_min,
+                         int shift_max, ds_stream_t stream);
+
+/* ---- validation of what a caller vouches for -------------------------------------------- */
+
+/* The compute entry points trust three claims about their operands: DS_BITS_TOP_UNUSED (no code
+ * carries the highest field value), DS_BITS_ZERO_TOP / the int8 blobs of 3- and 4-bit fields (the
+ * non-zero fields leave the highest value free) and x_bound of ds_conv2d_paired_i8.  A violated
+ * claim gives wrong sums with status 0.  These calls check a claim on the data; they are
+ * SYNCHRONOUS (they wait for `stream`) and meant for conversion time or debug builds.  `scratch`:
+ * 16 bytes of device memory.  No counterpart in the reference.
+ * ds_scan_words_i32: asynchronous; out[0] (device) = the largest field among the codes of
+ *   w_ref[N][comm] whose field is below 32 (-1 if none), out[1] = number of zero codes (field >= 32).
+ * ds_check_words_i32: DS_OK if reference-format words of `ref_bits`-wide fields may be tiled and run
+ *   with `kernel_bits` (a width with or without DS_BITS_ZERO_TOP / DS_BITS_TOP_UNUSED) on the int32
+ *   kernels (int8_kernel = 0) or on ds_conv2d_paired_i8 (int8_kernel = 1); DS_EINVAL if a code
+ *   violates what the flags promise.
+ * ds_check_bound_i8: DS_OK if every |x[i]| <= x_bound, else DS_EINVAL. */
+int ds_scan_words_i32(const int32_t *w_ref, int N, int K, int bits, int32_t *out, ds_stream_t stream);
+int ds_check_words_i32(const int32_t *w_ref, int N, int K, int ref_bits, int kernel_bits, int int8_kernel,
+                       int32_t *scratch, ds_stream_t stream);
+int ds_check_bound_i8(const int8_t *x, int64_t n, int x_bound, int32_t *scratch, ds_stream_t stream);
+
 /* ---- int8 activations ------------------------------------------------------------------ */
 
 /* Activation formats of at most 8 bits (act_integer_bits + act_fraction_bits <= 8, e.g. the 3.5 format
@@ -188,6 +230,27 @@ int ds_conv2d_tiled_i32(const int32_t *x_padded, const void *tiled, const int32_
                         int sw, int bits, int base, void *workspace, size_t workspace_bytes,
                         ds_stream_t stream);
 
+/* ---- host (CPU) twins: use_cuda=False ---------------------------------------------------- */
+
+/* Replace the reference's CPU shift kernels, pybind module deepshift_cpu: linear_kernel
+ * (kernels/cpu/shift_cpu.cpp:109-113, loop nest :176-221) and convolution_kernel (:295-301, loop
+ * nest :317-367), called from kernels/kernels.py:22-24,57-63 when use_cuda is false.  All pointers
+ * are HOST memory; the calls are synchronous and touch no GPU.  As in the reference the codes come
+ * unpacked: shift[n][k] is the signed exponent of the weight (>= 0: x << shift, < 0: x >> -shift,
+ * arithmetic, applied before the sign), sign[n][k] < 0 / > 0 subtracts / adds the term and
+ * sign == 0 contributes nothing (shift_cpu.cpp:190-201; the convolution's final `else` at :351-353,
+ * which adds the term of a zero sign, is not reproduced).  Accumulation wraps modulo 2^32; bias may
+ * be NULL.  nthreads <= 0 uses every hardware thread (the reference splits the batch over ATen's
+ * intra-op pool, at::parallel_for :176,:326).
+ *   ds_cpu_linear_i32: x[M][K], shift/sign [N][K], y[M][N].
+ *   ds_cpu_conv2d_i32: x[Nb][C][Hp][Wp] already zero padded (kernels.py:58 pads before the call),
+ *                      shift/sign [O][C][FH][FW], y[Nb][O][OH][OW], OH = (Hp - FH) / sh + 1. */
+int ds_cpu_linear_i32(const int32_t *x, const int8_t *shift, const int32_t *sign, const int32_t *bias,
+                      int32_t *y, int M, int K, int N, int nthreads);
+int ds_cpu_conv2d_i32(const int32_t *x_padded, const int8_t *shift, const int32_t *sign,
+                      const int32_t *bias, int32_t *y, int Nb, int C, int Hp, int Wp, int O, int FH,
+                      int FW, int sh, int sw, int nthreads);
+
 /* ---- fixed-point conversion ------------------------------------------------------------ */
 
 /* Replaces utils.round_to_fixed (utils.py:7-21) + the (x * 2**F).int() cast (modules.py:25,153)
@@ -279,6 +342,14 @@ int ds_valu_calibrate(int32_t *sink, int blocks, int iters, ds_stream_t stream);
 
 /* Plain copy kernel of n int32 (used to scale HBM byte counters). */
 int ds_copy_i32(const int32_t *src, int32_t *dst, int64_t n, ds_stream_t stream);
+
+/* Test hook: forces a launch variant of the compute entry points, process-wide, so that the
+ * test-suite can run every kernel form on small shapes.  knob: "planes" (0 / 1: two-instruction /
+ * shift-plane kernel), "split" (K split; shift-plane kernels: 0 = equal shares, 1 = one tile per
+ * wave), "tile" (R * 100 + J of the two-instruction kernel), "cu" (0 / 4 / 8 waves per cooperative
+ * workgroup), "notail".  knob == NULL clears every override.  Not for production callers: the
+ * dispatch's own choice is the measured best. */
+int ds_test_tune(const char *knob, int value);
 
 #ifdef __cplusplus
 }

@@ -73,3 +73,30 @@ def random_activations(rng, shape, kind="mixed"):
     n = min(flat.size, extremes.size)
     flat[:n] = extremes[:n]
     return x.astype(np.int32)
+
+
+class Tune:
+    """Forces a launch variant of the compute entry points through the library's test hook
+    (``ds_test_tune``): ``Tune(planes=1, split=0)``, ``Tune(tile="4x16", split=4)``, ``Tune(cu=8)``."""
+
+    def __init__(self, **knobs):
+        self.knobs = {}
+        for name, value in knobs.items():
+            if value is None:
+                continue
+            if name == "tile":
+                r, j = str(value).split("x")
+                value = int(r) * 100 + int(j)
+            self.knobs[name] = int(value)
+
+    def __enter__(self):
+        from deepshift_amd import _lib
+        _lib.call("ds_test_tune", None, 0)
+        for name, value in self.knobs.items():
+            _lib.call("ds_test_tune", name.encode(), value)
+        return self
+
+    def __exit__(self, *exc):
+        from deepshift_amd import _lib
+        _lib.call("ds_test_tune", None, 0)
+        return False

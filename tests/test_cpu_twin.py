@@ -1,0 +1,180 @@
+"""The library's host kernels (use_cuda=False): ds_cpu_linear_i32 / ds_cpu_conv2d_i32 through the C ABI
+and through the Python mirror, bit for bit against the oracle and against the vectors the reference's
+own compiled CPU kernel produced (tests/golden/ref_cpu_vectors.npz).  No GPU needed."""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from deepshift_amd import _lib, kernels, modules, modules_q, utils
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def _p(a):
+    return ctypes.c_void_p(a.ctypes.data)
+
+
+def abi_cpu_linear(x, shift, sign, bias, nthreads):
+    M, K = x.shape
+    N = shift.shape[0]
+    y = np.full((M, N), 0x5A5A5A5A, np.int32)
+    _lib.call("ds_cpu_linear_i32", _p(x), _p(shift), _p(sign), None if bias is None else _p(bias), _p(y),
+              M, K, N, nthreads)
+    return y
+
+
+def abi_cpu_conv(xp, shift, sign, bias, stride, nthreads):
+    Nb, C, Hp, Wp = xp.shape
+    O, _, FH, FW = shift.shape
+    OH, OW = (Hp - FH) // stride[0] + 1, (Wp - FW) // stride[1] + 1
+    y = np.full((Nb, O, OH, OW), 0x5A5A5A5A, np.int32)
+    _lib.call("ds_cpu_conv2d_i32", _p(xp), _p(shift), _p(sign), None if bias is None else _p(bias), _p(y),
+              Nb, C, Hp, Wp, O, FH, FW, stride[0], stride[1], nthreads)
+    return y
+
+
+def _codes(rng, shape, lo=-40, hi=6):
+    """Signed exponents incl. left shifts and right shifts beyond 31, signs in {-1, 0, +1}."""
+    shift = rng.integers(lo, hi + 1, size=shape).astype(np.int8)
+    sign = rng.integers(-1, 2, size=shape).astype(np.int32)
+    return shift, sign
+
+
+def _acts(rng, shape):
+    x = rng.integers(-2 ** 31, 2 ** 31 - 1, size=shape, dtype=np.int64).astype(np.int32)
+    special = np.array([0, -1, 2 ** 31 - 1, -2 ** 31], np.int64).astype(np.int32)
+    n = min(4, x.size)
+    x.reshape(-1)[:n] = special[:n]
+    return x
+
+
+def test_reference_kernel_vectors():
+    z = np.load(os.path.join(HERE, "golden", "ref_cpu_vectors.npz"))
+    for threads in (1, 3):
+        got = abi_cpu_linear(z["lin_x"], z["lin_shift"], z["lin_sign"], z["lin_bias"], threads)
+        np.testing.assert_array_equal(got, z["lin_y"])
+        got = abi_cpu_conv(z["conv_x"], z["conv_shift"], z["conv_sign"], z["conv_bias"],
+                           tuple(int(v) for v in z["conv_stride"]), threads)
+        np.testing.assert_array_equal(got, z["conv_y"])
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1), (5, 7, 3), (37, 101, 19), (16, 64, 64), (70, 300, 129)])
+def test_linear_matches_oracle(oracle, rng, shape):
+    M, K, N = shape
+    x = _acts(rng, (M, K))
+    shift, sign = _codes(rng, (N, K))
+    bias = rng.integers(-2 ** 31, 2 ** 31 - 1, size=N, dtype=np.int64).astype(np.int32)
+    want = oracle.linear(x, shift, sign, bias)
+    for threads in (1, 4, 0):
+        np.testing.assert_array_equal(abi_cpu_linear(x, shift, sign, bias, threads), want)
+    np.testing.assert_array_equal(abi_cpu_linear(x, shift, sign, None, 2), oracle.linear(x, shift, sign, None))
+
+
+@pytest.mark.parametrize("geom", [
+    # Nb, C, Hp, Wp, O, FH, FW, stride
+    (1, 1, 3, 3, 1, 3, 3, (1, 1)),
+    (2, 5, 11, 12, 7, 3, 3, (1, 2)),
+    (3, 4, 9, 9, 6, 1, 1, (2, 2)),
+    (2, 3, 20, 17, 8, 7, 7, (2, 2)),
+    (1, 16, 10, 10, 33, 3, 2, (1, 1)),
+])
+def test_conv_matches_oracle(oracle, rng, geom):
+    Nb, C, Hp, Wp, O, FH, FW, stride = geom
+    xp = _acts(rng, (Nb, C, Hp, Wp))
+    shift, sign = _codes(rng, (O, C, FH, FW))
+    bias = rng.integers(-2 ** 20, 2 ** 20, size=O).astype(np.int32)
+    want = oracle.conv2d(xp, shift, sign, bias, stride)
+    for threads in (1, 5):
+        np.testing.assert_array_equal(abi_cpu_conv(xp, shift, sign, bias, stride, threads), want)
+
+
+def test_degenerate_sizes_and_errors():
+    L = _lib.lib()
+    one = ctypes.c_void_p(16)
+    assert L.ds_cpu_linear_i32(None, None, None, None, None, 0, 4, 4, 1) == 0
+    assert L.ds_cpu_linear_i32(one, one, one, None, one, -1, 4, 4, 1) == -1
+    assert L.ds_cpu_linear_i32(None, one, one, None, one, 2, 4, 4, 1) == -1
+    assert L.ds_cpu_conv2d_i32(one, one, one, None, one, 1, 1, 2, 2, 1, 3, 3, 1, 1, 1) == -1
+    assert L.ds_cpu_conv2d_i32(one, one, one, None, one, 1, 1, 4, 4, 1, 3, 3, 0, 1, 1) == -1
+    # K == 0: the bias alone
+    y = np.zeros((2, 3), np.int32)
+    bias = np.array([1, -2, 3], np.int32)
+    assert L.ds_cpu_linear_i32(None, None, None, _p(bias), _p(y), 2, 0, 3, 1) == 0
+    np.testing.assert_array_equal(y, [[1, -2, 3], [1, -2, 3]])
+
+
+def test_kernels_api_use_cuda_false(oracle, rng):
+    """kernels.linear / conv2d with use_cuda=False (kernels.py:22-24,57-63): CPU tensors in, the float
+    shift/sign parameters as the module holds them, int32 sums out."""
+    x = _acts(rng, (9, 40))
+    shift, sign = _codes(rng, (12, 40), lo=-14, hi=0)
+    bias = rng.integers(-2 ** 20, 2 ** 20, size=12).astype(np.int32)
+    got = kernels.linear(torch.from_numpy(x), torch.from_numpy(shift).float(), torch.from_numpy(sign).float(),
+                         torch.from_numpy(bias), None, use_cuda=False)
+    assert got.dtype == torch.int32 and not got.is_cuda
+    np.testing.assert_array_equal(got.numpy(), oracle.linear(x, shift, sign, bias))
+    xi = _acts(rng, (2, 3, 8, 9))
+    shift, sign = _codes(rng, (4, 3, 3, 3), lo=-14, hi=0)
+    got = kernels.conv2d(torch.from_numpy(xi), torch.from_numpy(shift).float(), torch.from_numpy(sign).float(),
+                         None, None, stride=(1, 2), padding=(1, 2), use_cuda=False)
+    xp = np.pad(xi, ((0, 0), (0, 0), (1, 1), (2, 2)))
+    np.testing.assert_array_equal(got.numpy(), oracle.conv2d(xp, shift, sign, None, (1, 2)))
+    with pytest.raises(NotImplementedError):
+        kernels.conv2d(torch.from_numpy(xi), torch.from_numpy(shift).float(), torch.from_numpy(sign).float(),
+                       None, None, dilation=2, use_cuda=False)
+
+
+def _oracle_module_linear(oracle, x, shift, sign, bias, I, F, round_input):
+    xq = oracle.quantize(x, I, F) if round_input else oracle.cast(x, F)
+    bq = None if bias is None else (oracle.quantize(bias, I, F) if round_input else oracle.cast(bias, F))
+    y = oracle.linear(xq, shift.astype(np.int8), sign.astype(np.int32), bq)
+    return y.astype(np.float32) / np.float32(2.0 ** F)
+
+
+def test_modules_use_kernel_on_cpu(oracle):
+    """LinearShift / Conv2dShift / their Q twins with use_kernel=True, use_cuda=False run the host
+    kernels (modules.py:24-31,152-162) and reproduce the oracle chain bit for bit."""
+    torch.manual_seed(0)
+    lin = modules.LinearShift(40, 12, use_kernel=True, use_cuda=False)
+    x = torch.randn(7, 40) * 3
+    got = lin(x)
+    shift, sign = modules.module_codes(lin)
+    want = _oracle_module_linear(oracle, x.numpy(), shift.numpy(), sign.numpy(), lin.bias.detach().numpy(),
+                                 16, 16, round_input=False)
+    np.testing.assert_array_equal(got.detach().numpy(), want)
+
+    conv = modules.Conv2dShift(3, 5, 3, stride=2, padding=1, use_kernel=True, use_cuda=False)
+    xi = torch.randn(2, 3, 9, 10)
+    got = conv(xi)
+    shift, sign = modules.module_codes(conv)
+    xq = oracle.quantize(np.pad(xi.numpy(), ((0, 0), (0, 0), (1, 1), (1, 1))), 16, 16)
+    bq = oracle.quantize(conv.bias.detach().numpy(), 16, 16)
+    want = oracle.conv2d(xq, shift.numpy().astype(np.int8), sign.numpy().astype(np.int32), bq, (2, 2))
+    np.testing.assert_array_equal(got.detach().numpy(), want.astype(np.float32) / np.float32(65536.0))
+
+    lq = modules_q.LinearShiftQ(40, 12, use_kernel=True, use_cuda=False, act_integer_bits=3, act_fraction_bits=5)
+    got = lq(x)
+    shift, sign = modules_q.module_codes_q(lq)
+    want = _oracle_module_linear(oracle, x.numpy(), shift.numpy(), sign.numpy(), lq.bias.detach().numpy(),
+                                 3, 5, round_input=True)
+    np.testing.assert_array_equal(got.detach().numpy(), want)
+
+    cq = modules_q.Conv2dShiftQ(3, 5, 3, padding=1, use_kernel=True, use_cuda=False)
+    got = cq(xi)
+    shift, sign = modules_q.module_codes_q(cq)
+    bq = oracle.quantize(cq.bias.detach().numpy(), 16, 16)
+    want = oracle.conv2d(xq, shift.numpy().astype(np.int8), sign.numpy().astype(np.int32), bq, (1, 1))
+    np.testing.assert_array_equal(got.detach().numpy(), want.astype(np.float32) / np.float32(65536.0))
+    # the float path on the same layer stays within the fixed-point bound
+    cq.use_kernel = False
+    assert (got - cq(xi)).abs().max().item() < 27 * 2.0 ** -16 + 1e-4
+
+
+def test_host_codes_saturate_like_int8():
+    shift = torch.tensor([[-1000.0, float("-inf"), 3.7, -3.7, 200.0]])
+    sign = torch.tensor([[1.0, 0.0, -1.0, 1.0, 1.0]])
+    sh, sg = kernels._host_codes(shift, sign)
+    assert sh.tolist() == [[-128, -128, 3, -3, 127]] and sg.tolist() == [[1, 0, -1, 1, 1]]

@@ -324,9 +324,9 @@ def test_paired_launch_regimes(oracle, rng, form, regime):
     and the workgroup-cooperative kernels of four waves (tile buffer of packed pairs) and of eight."""
     split, cu = regime
     bits = form & 0xff
-    env = {"DS_TUNE_SPLIT": split}
+    env = {"split": split}
     if cu:
-        env["DS_TUNE_CU"] = cu
+        env["cu"] = cu
     for Nb, C, Hp, Wp, O, FH, FW, stride in [(2, 64, 16, 16, 64, 1, 1, (1, 1)), (4, 128, 14, 14, 256, 1, 1, (2, 2)),
                                              (3, 20, 21, 23, 128, 3, 3, (1, 1)), (9, 7, 40, 40, 64, 3, 3, (1, 1))]:
         x8 = random_int8(rng, (Nb, C, Hp, Wp))

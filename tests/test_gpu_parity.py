@@ -9,7 +9,7 @@ import torch
 
 from deepshift_amd import _lib
 from oracle import shift_oracle as so
-from tests.conftest import random_activations, random_codes
+from tests.conftest import Tune, random_activations, random_codes
 
 pytestmark = pytest.mark.gpu
 
@@ -248,22 +248,7 @@ def test_conv_split_k_path(oracle, rng):
 
 # ----------------------------------------------------------------------------- kernel variants
 
-class _Tune:
-    """Forces a kernel variant through the library's DS_TUNE_* environment overrides."""
-
-    def __init__(self, **kv):
-        self.kv = {k: str(v) for k, v in kv.items()}
-
-    def __enter__(self):
-        self.old = {k: os.environ.get(k) for k in self.kv}
-        os.environ.update(self.kv)
-
-    def __exit__(self, *exc):
-        for k, v in self.old.items():
-            if v is None:
-                os.environ.pop(k, None)
-            else:
-                os.environ[k] = v
+_Tune = Tune
 
 
 # split 0: equal shares of the (tile, K group) space; 1: one tile per wave; 3: tiles with K cut in 3
@@ -272,7 +257,7 @@ class _Tune:
 def test_shift_plane_kernel_every_field_width_and_launch(oracle, rng, bits, split):
     """The shift-plane kernel is normally chosen for large layers only; force it on shapes with ragged
     pixel counts, channel counts that do not fill a tile and reductions with a partial last word."""
-    with _Tune(DS_TUNE_PLANES=1, DS_TUNE_SPLIT=split):
+    with _Tune(planes=1, split=split):
         # convolution, stride 2, 40 channels (a 32-channel tile and a quarter), K = 5*3*3 = 45
         Nb, C, Hp, Wp, O = 3, 5, 21, 17, 40
         xp = random_activations(rng, (Nb, C, Hp, Wp))
@@ -316,7 +301,7 @@ def test_shift_plane_kernel_every_field_width_and_launch(oracle, rng, bits, spli
 @pytest.mark.parametrize("tile", ["2x32", "4x16", "3x16", "1x32", "1x8"])
 @pytest.mark.parametrize("split", [1, 4])
 def test_two_instruction_kernel_every_tile_shape(oracle, rng, tile, split):
-    with _Tune(DS_TUNE_PLANES=0, DS_TUNE_TILE=tile, DS_TUNE_SPLIT=split):
+    with _Tune(planes=0, tile=tile, split=split):
         Nb, C, Hp, Wp, O = 2, 11, 19, 22, 45
         xp = random_activations(rng, (Nb, C, Hp, Wp))
         s, sign = random_codes(rng, (O, C, 3, 3), max_s=15)
@@ -425,7 +410,7 @@ def test_zero_top_blob_matches_oracle(oracle, rng, width, split):
     from deepshift_amd import kernels
     L = _lib.lib()
     flag = width | _lib.DS_BITS_ZERO_TOP
-    env = {} if split is None else {"DS_TUNE_SPLIT": split}
+    env = {} if split is None else {"split": split}
     with _Tune(**env):
         # 64-channel form (N % 64 == 0, K a whole number of words of every width)
         M, K, N = 200, 480, 64
@@ -489,7 +474,7 @@ def test_top_unused_flag_matches_oracle(oracle, rng, bits, split):
     from deepshift_amd import kernels
     flag = bits | _lib.DS_BITS_TOP_UNUSED
     top = 2 ** bits - 2
-    env = {"DS_TUNE_PLANES": 1} if split is None else {"DS_TUNE_PLANES": 1, "DS_TUNE_SPLIT": split}
+    env = {"planes": 1} if split is None else {"planes": 1, "split": split}
     for tune in ({}, env):
         with _Tune(**tune):
             for M, K, N, with_bias in [(200, 480, 64, False), (333, 517, 71, True), (2000, 1200, 128, True)]:

@@ -120,16 +120,31 @@ def test_round_shift_weights():
     assert not torch.equal(model[0].shift.data, out[0].shift.data)  # clone left the original alone
 
 
-def test_kernel_path_has_no_cpu_fallback():
-    lin = modules.LinearShift(4, 3, use_kernel=True, use_cuda=False)
-    with pytest.raises(NotImplementedError):
-        lin(torch.randn(2, 4))
-    with pytest.raises(NotImplementedError):
-        kernels.linear(torch.zeros(1, 1, dtype=torch.int32), torch.zeros(1, 1), torch.zeros(1, 1),
-                       conc_weight=utils.ConcWeight(), use_cuda=False)
+def test_gpu_kernel_path_never_falls_back_to_the_host():
+    """use_cuda=True with CPU tensors is an error, not a silent host computation (use_cuda=False is
+    the explicit way to the host kernels, tests/test_cpu_twin.py)."""
     with pytest.raises((ValueError, RuntimeError, AssertionError)):
         kernels.linear(torch.zeros(1, 1, dtype=torch.int32), torch.zeros(1, 1), torch.zeros(1, 1),
                        conc_weight=utils.ConcWeight(torch.zeros(1, dtype=torch.int32), 0, 4))
+    lin = modules.LinearShift(4, 3, use_kernel=True, use_cuda=True)
+    with pytest.raises((ValueError, RuntimeError, TypeError, AssertionError)):
+        lin(torch.randn(2, 4))
+
+
+def test_packed_weights_follow_the_parameters():
+    """conc_weight assigned from outside is kept; one built from the layer's parameters carries the
+    key of those parameters so that a later change repacks."""
+    lin = modules.LinearShift(4, 3, use_kernel=True)
+    assert lin.conc_weight is None and lin._packed_from is None
+    given = utils.ConcWeight(torch.zeros(3, dtype=torch.int32), 0, 4)
+    lin.conc_weight = given
+    assert lin.packed_weights() is given       # nothing to compare against: used as given
+    key = modules._params_key(lin.shift, lin.sign)
+    with torch.no_grad():
+        lin.shift.add_(1.0)                    # what an optimizer step or load_state_dict does
+    assert modules._params_key(lin.shift, lin.sign) != key
+    lin.load_state_dict(lin.state_dict())
+    assert "conc_weight" not in lin.state_dict() and "_conc_weight" not in lin.state_dict()
 
 
 def test_workload_pair_counts():
