@@ -325,6 +325,48 @@ def np_round_to_fixed(x, I=16, F=16):
     return np.clip(r, np.float32(-bound), np.float32(bound - 1)).astype(np.float32)
 
 
+def np_dequantize_affine(y, F_in, scale=None, shift=None, residual=None, relu=False):
+    """What follows a shift layer at inference time, in float32 with one rounding per operation:
+    ``out = y.float() / 2**F`` (modules.py:30-31,161-162), a per-channel affine ``* scale[c] + shift[c]``
+    (an eval-mode BatchNorm folded to one multiply and one add), ``+ residual``, ``max(., 0)``.
+    y [Nb, C, ...] int32.  The int32 -> float32 conversion rounds to nearest even, the division by a
+    power of two is exact."""
+    y = np.asarray(y, np.int32)
+    v = y.astype(np.float32) / np.float32(2.0 ** F_in)
+    bshape = (1, -1) + (1,) * (y.ndim - 2)
+    if scale is not None:
+        v = v * np.asarray(scale, np.float32).reshape(bshape)
+    if shift is not None:
+        v = v + np.asarray(shift, np.float32).reshape(bshape)
+    if residual is not None:
+        v = v + np.asarray(residual, np.float32)
+    if relu:
+        v = np.maximum(v, np.float32(0))
+    return v.astype(np.float32)
+
+
+def np_max_pool2d(v, kernel, stride, padding):
+    """nn.MaxPool2d(kernel, stride, padding) in floor mode: windows padded with -inf."""
+    v = np.asarray(v, np.float32)
+    Nb, C, H, W = v.shape
+    OH, OW = (H + 2 * padding - kernel) // stride + 1, (W + 2 * padding - kernel) // stride + 1
+    vp = np.full((Nb, C, H + 2 * padding, W + 2 * padding), -np.inf, np.float32)
+    vp[:, :, padding:padding + H, padding:padding + W] = v
+    out = np.full((Nb, C, OH, OW), -np.inf, np.float32)
+    for i in range(kernel):
+        for j in range(kernel):
+            out = np.maximum(out, vp[:, :, i:i + stride * OH:stride, j:j + stride * OW:stride])
+    return out
+
+
+def np_requantize(v, I=16, F=16, padding=(0, 0)):
+    """The next shift convolution's input from a float tensor: ``round_to_fixed`` (utils.py:7-21),
+    ``(x * 2**F).int()`` (modules.py:153) and the zero padding of kernels.py:32-36."""
+    q = (np_round_to_fixed(v, I, F).astype(np.float64) * 2.0 ** F).astype(np.int64).astype(np.int32)
+    ph, pw = padding
+    return np.pad(q, ((0, 0), (0, 0), (ph, ph), (pw, pw)))
+
+
 def bits_from_min_shift(min_shift):
     """utils.py:72: ceil(log(1 - min(shift)) / ln 2) evaluated in float32 like torch.log."""
     v = np.float32(-min_shift + 1)

@@ -149,3 +149,93 @@ def test_config5_int8_layers_full_size(oracle, layer):
     perm = torch.randperm(Nb, generator=g).to(DEV)
     assert torch.equal(kernels.conv2d_paired(x8[perm].contiguous(), blob, bias, O, (F, F), (stride, stride), 2, 96),
                        want[perm])
+
+
+def _default_init_codes(g, shape, weight_bits=5):
+    """Codes as a converted model has them: PyTorch's default (Kaiming-uniform) weights through
+    get_shift_and_sign and the clamp of weight_bits (modules.py:88) -- fields 0..14, so kernel_bits()
+    selects the kernel form without the plane of the highest value."""
+    fan_in = int(np.prod(shape[1:]))
+    bound = 1.0 / np.sqrt(fan_in)
+    w = (torch.rand(shape, generator=g) * 2 - 1) * bound
+    shift, sign = utils.get_shift_and_sign(w)
+    lo = -(2 ** (weight_bits - 1) - 2)
+    return shift.clamp(lo, 0), sign
+
+
+def _run_layer_full(oracle, g, L, images, lo_hi=(-2 ** 18, 2 ** 20)):
+    """One shift layer at its full benchmark size through kernel_bits(); the oracle on `images`."""
+    if L["kind"] == "linear":
+        x = torch.randint(lo_hi[0], lo_hi[1], (L["M"], L["K"]), generator=g, dtype=torch.int32)
+        shift, sign = _default_init_codes(g, (L["N"], L["K"]))
+        bias = torch.randint(-2 ** 20, 2 ** 20, (L["N"],), generator=g, dtype=torch.int32)
+        cw = utils.compress_bits(shift, sign)
+        y = kernels.linear(x.to(DEV), shift, sign, bias.to(DEV), cw)
+        rows = sorted(set(images) | {L["M"] - 1})
+        want = oracle.linear(x[rows].numpy(), shift.numpy().astype(np.int32), sign.numpy().astype(np.int32),
+                             bias.numpy(), NTHREADS)
+        np.testing.assert_array_equal(y[rows].cpu().numpy(), want, err_msg=L["name"])
+        return cw
+    x = torch.randint(lo_hi[0], lo_hi[1], (L["Nb"], L["C"], L["H"], L["W"]), generator=g, dtype=torch.int32)
+    shift, sign = _default_init_codes(g, (L["O"], L["C"], L["FH"], L["FW"]))
+    bias = torch.randint(-2 ** 20, 2 ** 20, (L["O"],), generator=g, dtype=torch.int32)
+    cw = utils.compress_bits(shift, sign)
+    assert kernels.kernel_bits(cw) == 4 | 0x200, "the clamped range leaves the top field value unused"
+    xd = x.to(DEV)
+    y = kernels.conv2d(xd, shift, sign, bias.to(DEV), cw, L["stride"], L["padding"])
+    ph, pw = L["padding"]
+    s_np, sg_np = shift.numpy().astype(np.int32), sign.numpy().astype(np.int32)
+    for img in images:
+        xp = np.pad(x[img:img + 1].numpy(), ((0, 0), (0, 0), (ph, ph), (pw, pw)))
+        want = oracle.conv2d(xp, s_np, sg_np, bias.numpy(), L["stride"], nthreads=NTHREADS)
+        np.testing.assert_array_equal(y[img:img + 1].cpu().numpy(), want, err_msg="%s image %d" % (L["name"], img))
+    # size-independent properties on the whole batch: a batch permutation permutes the output; flipping
+    # every sign negates y - bias
+    perm = torch.randperm(L["Nb"], generator=g).to(DEV)
+    assert torch.equal(kernels.conv2d(xd[perm].contiguous(), shift, sign, bias.to(DEV), cw, L["stride"],
+                                      L["padding"]), y[perm]), L["name"]
+    b4 = bias.to(DEV).view(1, -1, 1, 1)
+    y_flip = kernels.conv2d(xd, shift, -sign, bias.to(DEV), utils.compress_bits(shift, -sign), L["stride"],
+                            L["padding"])
+    assert torch.equal(y - b4, -(y_flip - b4)), L["name"]
+    return cw
+
+
+def _distinct_shapes(model, chw, batch):
+    from deepshift_amd import workloads
+    seen, out = set(), []
+    for L in workloads.shift_layer_shapes(model, chw, batch):
+        key = tuple(sorted((k, v) for k, v in L.items() if k != "name"))
+        if key not in seen:
+            seen.add(key)
+            out.append(L)
+    return out
+
+
+def test_config3_resnet20_batch256_every_layer_shape(oracle):
+    """Benchmark configuration 3 at its real size: every distinct shift-layer shape of ResNet-20 at batch
+    256 (cifar10_models/resnet.py:23-55,85-140: 3x3 convolutions of 16/32/64 channels on 32/16/8 pixel
+    images, FC 64 -> 10), codes from default-init weights clamped for weight_bits 5, the WHOLE output of
+    every layer against the oracle."""
+    from deepshift_amd import workloads
+    g = torch.Generator().manual_seed(33)
+    shapes = _distinct_shapes(workloads.ResNet20(), (3, 32, 32), 256)
+    assert len(shapes) == 7
+    for L in shapes:
+        if L["kind"] == "linear":
+            _run_layer_full(oracle, g, L, list(range(L["M"])))
+        else:
+            _run_layer_full(oracle, g, L, list(range(L["Nb"])))
+
+
+def test_config4_resnet18_batch64_every_layer_shape(oracle):
+    """The headline configuration at its real size: every distinct shift-layer shape of ResNet-18 at batch
+    64 through kernel_bits() -- the launches bench.py times (top-unused cooperative kernel for the 3x3
+    layers, wave-level shares for the stem, the shortcut and FC kernels) -- against the oracle on the first
+    and last image, plus the permutation and negation properties on the whole batch."""
+    from deepshift_amd import workloads
+    g = torch.Generator().manual_seed(44)
+    shapes = _distinct_shapes(workloads.ResNet18(), (3, 224, 224), 64)
+    assert len(shapes) == 12
+    for L in shapes:
+        _run_layer_full(oracle, g, L, [0, 63])

@@ -152,6 +152,38 @@ def test_q_modules_and_circular_padding():
         modules.Conv2dShift(4, 4, 3, dilation=2, use_kernel=True).to(DEV)(torch.randn(1, 4, 9, 9, device=DEV))
 
 
+def test_q_modules_match_the_oracle(oracle):
+    """LinearShiftQ / Conv2dShiftQ on the kernel path (modules_q.py:20-43,146-170): the int32 sums are the
+    oracle's on the codes derived from the clamped, power-of-two-rounded weight, bit for bit (the
+    reference's LinearShiftQ never reached its kernel: argument slots, modules_q.py:125)."""
+    torch.manual_seed(12)
+    for I, Fb, wb in [(16, 16, 5), (3, 5, 3)]:
+        lq = modules_q.LinearShiftQ(300, 70, use_kernel=True, weight_bits=wb, act_integer_bits=I,
+                                    act_fraction_bits=Fb).to(DEV)
+        x = torch.randn(33, 300) * 2
+        with torch.no_grad():
+            got = lq(x.to(DEV))
+        shift, sign = modules_q.module_codes_q(lq)
+        assert int(shift.min()) >= lq.shift_range[0] and set(sign.unique().tolist()) <= {-1.0, 1.0}
+        y = oracle.linear(oracle.quantize(x.numpy(), I, Fb), shift.cpu().numpy().astype(np.int32),
+                          sign.cpu().numpy().astype(np.int32), oracle.quantize(lq.bias.detach().cpu().numpy(), I, Fb))
+        np.testing.assert_array_equal(got.cpu().numpy(), y.astype(np.float32) / np.float32(2.0 ** Fb))
+        cq = modules_q.Conv2dShiftQ(12, 64, 3, stride=2, padding=1, use_kernel=True, weight_bits=wb,
+                                    act_integer_bits=I, act_fraction_bits=Fb).to(DEV)
+        with torch.no_grad():
+            cq.weight[0, 0, 0, 0] = 0.0          # an exact zero stays a zero weight (utils.py:44-52)
+        xi = torch.randn(3, 12, 15, 13)
+        with torch.no_grad():
+            got = cq(xi.to(DEV))
+        shift, sign = modules_q.module_codes_q(cq)
+        assert float(sign[0, 0, 0, 0]) == 0.0
+        xq = oracle.quantize(np.pad(xi.numpy(), ((0, 0), (0, 0), (1, 1), (1, 1))), I, Fb)
+        sh = torch.nan_to_num(shift, neginf=-32.0).cpu().numpy().astype(np.int32)
+        y = oracle.conv2d(xq, sh, sign.cpu().numpy().astype(np.int32),
+                          oracle.quantize(cq.bias.detach().cpu().numpy(), I, Fb), (2, 2))
+        np.testing.assert_array_equal(got.cpu().numpy(), y.astype(np.float32) / np.float32(2.0 ** Fb))
+
+
 def test_mlp_config1_end_to_end(oracle):
     """Benchmark configuration 1 (MLP): 784-512-512-10, batch 64, ternary sign, shift in [-15, 0], 16.16."""
     g = torch.Generator().manual_seed(0)
@@ -321,6 +353,40 @@ def test_requantize_affine_maxpool_matches_the_three_passes(rng):
             assert f is None and torch.equal(q, q_want)
             f, q = kernels.requantize_affine_maxpool(y, 16, sc, sh, relu, pool)
             assert q is None and torch.equal(f, f_want)
+
+
+def test_inter_layer_passes_match_the_oracle_chain(rng):
+    """The fused conversion passes against the oracle's restatement of what runs between two shift layers
+    (modules.py:161-162 -> per-channel affine -> residual -> ReLU [-> max pooling] -> round_to_fixed and the
+    cast of the next layer, :317,:153 -> zero padding, kernels.py:32-36), float and fixed-point outputs
+    bit for bit."""
+    for (Nb, C, H, W), pad, (I, Fb), dtype in [((3, 5, 7, 4), (1, 1), (16, 16), torch.int32),
+                                                ((2, 3, 5, 9), (0, 2), (8, 8), torch.int32),
+                                                ((1, 70, 28, 28), (1, 1), (16, 16), torch.int32),
+                                                ((2, 6, 9, 8), (1, 1), (3, 5), torch.int8),
+                                                ((2, 64, 7, 7), (0, 0), (3, 5), torch.int8)]:
+        hi = 2 ** 27 if Fb == 16 else 2 ** 12
+        y = rng.integers(-hi, hi, size=(Nb, C, H, W)).astype(np.int32)
+        scale = (rng.random(C) + 0.5).astype(np.float32)
+        shift = rng.standard_normal(C).astype(np.float32)
+        res = (rng.standard_normal((Nb, C, H, W)) * 3).astype(np.float32)
+        yd = torch.from_numpy(y).to(DEV)
+        for sc, sh, r, relu in [(scale, shift, res, True), (scale, None, None, False), (None, None, res, True),
+                                (None, None, None, False)]:
+            t = [None if a is None else torch.from_numpy(a).to(DEV) for a in (sc, sh, r)]
+            v = so.np_dequantize_affine(y, Fb, sc, sh, r, relu)
+            np.testing.assert_array_equal(kernels.dequantize_affine(yd, Fb, t[0], t[1], t[2], relu).cpu().numpy(), v)
+            f, q = kernels.requantize_affine_pad(yd, Fb, t[0], t[1], t[2], relu, pad, I, Fb, True, dtype)
+            np.testing.assert_array_equal(f.cpu().numpy(), v)
+            np.testing.assert_array_equal(q.cpu().numpy().astype(np.int32), so.np_requantize(v, I, Fb, pad))
+            f, q = kernels.requantize_affine_pad(yd, Fb, t[0], t[1], t[2], relu, pad, I, Fb, False, dtype)
+            np.testing.assert_array_equal(q.cpu().numpy().astype(np.int32), so.np_requantize(v, I, Fb, pad))
+        for pool in [(3, 2, 1), (2, 2, 0)]:
+            t = [torch.from_numpy(a).to(DEV) for a in (scale - 0.8, shift)]   # some channels flip the order
+            v = so.np_max_pool2d(so.np_dequantize_affine(y, Fb, scale - 0.8, shift, None, True), *pool)
+            f, q = kernels.requantize_affine_maxpool(yd, Fb, t[0], t[1], True, pool, pad, I, Fb, True, dtype)
+            np.testing.assert_array_equal(f.cpu().numpy(), v)
+            np.testing.assert_array_equal(q.cpu().numpy().astype(np.int32), so.np_requantize(v, I, Fb, pad))
 
 
 def test_dequantize_affine_matches_torch(rng):

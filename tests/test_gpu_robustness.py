@@ -52,8 +52,12 @@ def test_cpu_tensors_and_unsupported_geometry_are_refused():
     m = _conv()
     with pytest.raises((TypeError, RuntimeError, ValueError)):
         m(torch.randn(1, 8, 12, 10))                      # CPU input to a GPU layer
-    with pytest.raises(NotImplementedError):
-        modules.Conv2dShift(8, 16, 3, use_kernel=True, use_cuda=False)(torch.randn(1, 8, 12, 10))
+    # use_cuda=False is the host kernel: same sums as the GPU layer with the same parameters
+    host = modules.Conv2dShift(8, 16, 3, padding=1, use_kernel=True, use_cuda=False)
+    host.load_state_dict(m.state_dict())
+    xc = torch.randn(1, 8, 12, 10)
+    with torch.no_grad():
+        assert torch.equal(host(xc), m(xc.to(DEV)).cpu())
     g = modules.Conv2dShift(8, 16, 3, groups=2, use_kernel=True).to(DEV)
     with pytest.raises(NotImplementedError):
         g(torch.randn(1, 8, 12, 10, device=DEV))

@@ -315,3 +315,66 @@ def test_reference_vectors_fixture(oracle):
     np.testing.assert_array_equal(
         oracle.conv2d(z["conv_x"], z["conv_shift"], z["conv_sign"], z["conv_bias"],
                       tuple(int(v) for v in z["conv_stride"])), z["conv_y"])
+
+
+# ----------------------------------------------------------------------------- inter-layer chain
+
+def test_dequantize_affine_known_answers():
+    """Hand-derived: y = 98304 (1.5 in 16.16), scale 2, shift -0.25 -> 2.75; + residual -3 -> -0.25;
+    ReLU -> 0.  y = -65536 (-1.0): * 0.5 + 1 = 0.5.  int32 extremes convert with round-to-nearest-even:
+    2^31 - 1 -> 2^31 -> / 2^16 = 32768.0."""
+    y = np.array([[[98304, -65536, 2 ** 31 - 1]]], np.int32).reshape(1, 1, 3)
+    np.testing.assert_array_equal(so.np_dequantize_affine(y, 16), [[[1.5, -1.0, 32768.0]]])
+    y2 = np.array([98304, -65536], np.int32).reshape(1, 2, 1)
+    out = so.np_dequantize_affine(y2, 16, scale=[2.0, 0.5], shift=[-0.25, 1.0])
+    np.testing.assert_array_equal(out.reshape(-1), [2.75, 0.5])
+    res = np.array([-3.0, 0.0], np.float32).reshape(1, 2, 1)
+    out = so.np_dequantize_affine(y2, 16, [2.0, 0.5], [-0.25, 1.0], res, relu=True)
+    np.testing.assert_array_equal(out.reshape(-1), [0.0, 0.5])
+
+
+def test_inter_layer_chain_against_torch_cpu(rng):
+    """The numpy chain against the same steps spelled with torch CPU ops (a different library's float32
+    arithmetic, F.max_pool2d, F.pad) and against the C oracle's quantize."""
+    import torch
+    import torch.nn.functional as F
+    y = rng.integers(-2 ** 31, 2 ** 31 - 1, size=(2, 5, 9, 11), dtype=np.int64).astype(np.int32)
+    y[0, 0, 0, :4] = [0, -1, 2 ** 31 - 1, -2 ** 31]
+    scale = (rng.standard_normal(5) * 2).astype(np.float32)
+    shift = rng.standard_normal(5).astype(np.float32)
+    res = (rng.standard_normal(y.shape) * 100).astype(np.float32)
+    for relu in (False, True):
+        got = so.np_dequantize_affine(y, 16, scale, shift, res, relu)
+        t = torch.from_numpy(y).float() / 65536.0
+        t = t * torch.from_numpy(scale).view(1, -1, 1, 1) + torch.from_numpy(shift).view(1, -1, 1, 1)
+        t = t + torch.from_numpy(res)
+        if relu:
+            t = torch.relu(t)
+        np.testing.assert_array_equal(got, t.numpy())
+    v = so.np_dequantize_affine(y, 16, scale, shift, None, True)
+    for (k, st, pd) in [(3, 2, 1), (2, 2, 0), (3, 1, 1)]:
+        np.testing.assert_array_equal(so.np_max_pool2d(v, k, st, pd),
+                                      F.max_pool2d(torch.from_numpy(v), k, st, pd).numpy())
+    oracle_c = so.get()
+    for (I, Fb) in [(16, 16), (3, 5), (8, 8)]:
+        vv = (v / np.float32(64.0)).astype(np.float32)
+        want = np.pad(oracle_c.quantize(vv, I, Fb), ((0, 0), (0, 0), (1, 1), (2, 2)))
+        np.testing.assert_array_equal(so.np_requantize(vv, I, Fb, (1, 2)), want)
+        tt = torch.from_numpy(vv)
+        rt = torch.clamp(torch.floor(tt / 2.0 ** -Fb) * 2.0 ** -Fb, -2.0 ** (I - 1), 2.0 ** (I - 1) - 1)
+        np.testing.assert_array_equal(so.np_requantize(vv, I, Fb), (rt * 2 ** Fb).int().numpy())
+
+
+def test_get_shift_and_sign_fixture():
+    """The package's get_shift_and_sign (the reference's three torch ops, utils.py:23-29) on the committed
+    torch-CPU fixture: the weights whose log2 lands on or next to a half-way point."""
+    import torch
+    from deepshift_amd import utils
+    z = np.load(os.path.join(HERE, "golden", "codegen_vectors.npz"))
+    shift, sign = utils.get_shift_and_sign(torch.from_numpy(z["w"]))
+    np.testing.assert_array_equal(shift.numpy(), z["shift"])
+    np.testing.assert_array_equal(sign.numpy(), z["sign"])
+    # known answers (log2 0.75 = -0.415, 0.7 -> -0.515, 0.35 -> -1.515, 0.1 -> -3.32)
+    s, g = utils.get_shift_and_sign(torch.tensor([0.75, 0.7, 0.35, -0.1, 4.0, -0.125, 0.0]))
+    assert s.tolist() == [0.0, -1.0, -2.0, -3.0, 2.0, -3.0, float("-inf")]
+    assert g.tolist() == [1.0, 1.0, 1.0, -1.0, 1.0, -1.0, 0.0]
