@@ -83,6 +83,7 @@ DS_EXPORT const char *ds_status_string(int status)
     case DS_EBASE: return "unsupported base (must be in -31..0)";
     case DS_EWORKSPACE: return "workspace missing or too small";
     case DS_ETOOLARGE: return "tensor too large for 32-bit offsets";
+    case DS_ESCRATCH: return "problem needs more than the built-in scratch of the allocation-free entry point";
     default: break;
     }
     if (status <= DS_EHIP) return hipGetErrorString((hipError_t)(DS_EHIP - status));

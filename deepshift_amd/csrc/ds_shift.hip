@@ -1067,6 +1067,49 @@ DS_EXPORT int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled,
     return dispatch_bits(a, bits, base != 0 || bits == 6, (hipStream_t)stream);
 }
 
+// Scratch of the allocation-free entry point: device memory that belongs to the library's code object
+// (one copy per GPU, held until the process ends).  The array's name is a host-side stand-in; the
+// device address comes from hipGetSymbolAddress, once per device, with that device current.
+constexpr size_t kBuiltinScratchBytes = (size_t)16 << 20;
+static __device__ __align__(256) unsigned char scratch[kBuiltinScratchBytes];
+
+static int builtin_scratch(void **out)
+{
+    static std::atomic<void *> per_device[64];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_status(e);
+    if (dev < 0 || dev >= 64) return DS_EINVAL;
+    void *p = per_device[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_status(e);
+        if (!p) return DS_EHIP;
+        per_device[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return DS_OK;
+}
+
+DS_EXPORT size_t ds_linear_tiled_noalloc_max_bytes(void) { return kBuiltinScratchBytes; }
+
+DS_EXPORT int ds_linear_tiled_noalloc_i32(const int32_t *xT, int ldx, const void *tiled, const int32_t *bias,
+                                          int32_t *y, int M, int K, int N, int bits, int base,
+                                          ds_stream_t stream)
+{
+    if (M < 0 || K < 0 || N < 0) return DS_EINVAL;
+    const size_t need = linear_scratch_bytes(M, N);
+    if (need > kBuiltinScratchBytes) return DS_ESCRATCH;
+    void *ws = nullptr;
+    if (need) {
+        const int rc = builtin_scratch(&ws);
+        if (rc) return rc;
+    }
+    // every cell of the scratch that the kernels read is written first (the pre-fill pass covers the
+    // [N][ld] range a launch accumulates into), so nothing has to be cleared between calls
+    return ds_linear_tiled_i32(xT, ldx, tiled, bias, y, M, K, N, bits, base, ws, need, stream);
+}
+
 DS_EXPORT int ds_linear_i32(const int32_t *x, const int32_t *w_ref, const int32_t *bias, int32_t *y,
                             int M, int K, int N, int bits, int base, void *workspace,
                             size_t workspace_bytes, ds_stream_t stream)

@@ -29,6 +29,7 @@ enum {
     DS_EBASE = -3,       /* base > 0 (base is min(-shift) when that is negative, else 0: utils.py:75-80) */
     DS_EWORKSPACE = -4,  /* workspace missing or smaller than ds_*_workspace_bytes() */
     DS_ETOOLARGE = -5,   /* a tensor exceeds the 32-bit offsets the kernels use (>= 2^31 bytes) */
+    DS_ESCRATCH = -6,    /* the problem needs more scratch than ds_linear_tiled_noalloc_max_bytes() */
     DS_EHIP = -100       /* DS_EHIP - hipError_t for a failed launch */
 };
 
@@ -206,6 +207,17 @@ size_t ds_linear_tiled_workspace_bytes(int M, int K, int N, int bits);
 int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled, const int32_t *bias,
                         int32_t *y, int M, int K, int N, int bits, int base, void *workspace,
                         size_t workspace_bytes, ds_stream_t stream);
+
+/* ds_linear_tiled_i32 for callers that cannot allocate (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): no workspace argument; the partial-sum scratch lives in a
+ * device array inside the library (ds_linear_tiled_noalloc_max_bytes() = 16 MiB per GPU, held until
+ * the process ends).  The call allocates nothing.  DS_ESCRATCH when
+ * ds_linear_tiled_workspace_bytes(M, K, N, bits) exceeds that size (4 * N * round_up(M, 64) bytes,
+ * e.g. 2048 x 2048).  All calls on one GPU share the array: calls that overlap in time on one GPU
+ * (different streams) race.  No counterpart in the reference. */
+size_t ds_linear_tiled_noalloc_max_bytes(void);
+int ds_linear_tiled_noalloc_i32(const int32_t *xT, int ldx, const void *tiled, const int32_t *bias,
+                                int32_t *y, int M, int K, int N, int bits, int base, ds_stream_t stream);
 
 /* ---- Conv2dShift ----------------------------------------------------------------------- */
 

@@ -1,0 +1,76 @@
+"""GPU: the allocation-free entry point ds_linear_tiled_noalloc_i32 against ds_linear_tiled_i32, through the
+C ABI, bit for bit: two calls in a row on launches that combine partial sums through the scratch (the second
+with a smaller input, so stale contents of the shared array would show), a launch that needs no scratch, and
+the size limit."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from deepshift_amd import _lib, kernels
+from oracle import shift_oracle as so
+from tests.conftest import Tune, random_activations, random_codes
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def _case(rng, M, K, N, bits=4):
+    x = random_activations(rng, (M, K))
+    s, sign = random_codes(rng, (N, K), max_s=2 ** bits - 1)
+    bias = rng.integers(-2 ** 20, 2 ** 20, size=N).astype(np.int32)
+    blob = kernels.tile_weights(_dev(so.np_pack_words(s, sign, bits)).reshape(-1), N, K, 1, 1, bits, 0)
+    xT = _dev(np.ascontiguousarray(np.pad(x, ((0, (-M) % 64), (0, 0))).T))
+    return x, s, sign, bias, blob, xT
+
+
+def _both(xT, blob, bias, M, K, N, bits):
+    """(ds_linear_tiled_i32 with a caller workspace, ds_linear_tiled_noalloc_i32) on the same operands."""
+    st = _lib.current_stream(torch.device(DEV))
+    bd = _dev(bias)
+    want = kernels.linear_tiled(xT, M, blob, bd, N, bits, 0)
+    guard = 64
+    ybuf = torch.full((M * N + 2 * guard,), 0x5A5A5A5A, dtype=torch.int32, device=DEV)
+    y = ybuf[guard:guard + M * N]
+    before = torch.cuda.memory_allocated()
+    _lib.call("ds_linear_tiled_noalloc_i32", _lib.ptr(xT), xT.shape[1], _lib.ptr(blob), _lib.ptr(bd),
+              ctypes.c_void_p(y.data_ptr()), M, K, N, bits, 0, st)
+    assert torch.cuda.memory_allocated() == before
+    torch.cuda.synchronize()
+    host = ybuf.cpu().numpy()
+    assert (host[:guard] == 0x5A5A5A5A).all() and (host[guard + M * N:] == 0x5A5A5A5A).all()
+    return want.cpu().numpy(), host[guard:guard + M * N].reshape(M, N)
+
+
+@pytest.mark.parametrize("split", [0, 3, None], ids=lambda s: "split%s" % s)
+def test_noalloc_matches_workspace_entry_point_twice(oracle, rng, split):
+    """split 0 (equal shares) and 3 (K cut in three) accumulate into the scratch; None is the dispatch's own
+    choice.  The second call is smaller than the first."""
+    tune = {"planes": 1} if split is None else {"planes": 1, "split": split}
+    with Tune(**tune):
+        for (M, K, N) in [(333, 517, 128), (130, 240, 64)]:
+            x, s, sign, bias, blob, xT = _case(rng, M, K, N)
+            want, got = _both(xT, blob, bias, M, K, N, 4)
+            np.testing.assert_array_equal(got, want)
+            np.testing.assert_array_equal(got, oracle.linear(x, -s, sign, bias, nthreads=8))
+
+
+def test_noalloc_two_instruction_kernel_and_limit(oracle, rng):
+    with Tune(planes=0, tile="2x32", split=4):
+        for (M, K, N) in [(200, 600, 77), (64, 300, 40)]:
+            x, s, sign, bias, blob, xT = _case(rng, M, K, N)
+            want, got = _both(xT, blob, bias, M, K, N, 4)
+            np.testing.assert_array_equal(got, want)
+    L = _lib.lib()
+    limit = L.ds_linear_tiled_noalloc_max_bytes()
+    assert limit == 16 << 20
+    one = ctypes.c_void_p(256)
+    # 4 * N * round_up(M, 64) beyond the built-in scratch: rejected before anything is launched
+    assert L.ds_linear_tiled_noalloc_i32(one, 4096, one, None, one, 4096, 64, 2048, 4, 0, None) == -6
+    assert b"scratch" in L.ds_status_string(-6)
+    assert L.ds_linear_tiled_workspace_bytes(2048, 64, 2048, 4) == limit
