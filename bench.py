@@ -27,12 +27,22 @@ if ROOT not in sys.path:
 CU_COUNT = 256
 LANES_PER_CU = 64
 CLOCK_HZ = 2.4e9
-VALU_INSTR_PER_PAIR = 2  # v_ashrrev_i32 + v_xad_u32
-PEAK_PAIRS = CU_COUNT * LANES_PER_CU * CLOCK_HZ / VALU_INSTR_PER_PAIR  # 19.66e12 pairs/s
+LANE_OPS = CU_COUNT * LANES_PER_CU * CLOCK_HZ  # 39.3e12 int32 lane-operations per second
+# The bound: a shift-add pair needs at least ONE vector instruction per lane (the accumulate; the shifted
+# operand can be shared between output channels, which is what the shift-plane kernels do), so no int32
+# kernel can exceed 39.3 Tpair/s; the int8 kernels hold two pixels per lane register: 0.5 per pair.
+PEAK_PAIRS = LANE_OPS / 1.0
+PEAK_PAIRS_INT8 = LANE_OPS / 0.5
+# secondary figure: a kernel that shifts and accumulates every pair separately (v_ashrrev_i32 + v_xad_u32)
+PEAK_PAIRS_TWO_INSTR = LANE_OPS / 2.0
 HBM_PEAK = 8.0e12
 
 BATCH = 64
 CHW = (3, 224, 224)
+
+# the kernel behind the 3x3 convolutions of the headline network, as rocprofv3 names it
+DOMINANT_KERNEL = "ds::shift_planes_wide_cu_kernel<4, 2, 4>"
+TRAFFIC_LAYER1_BYTES = 176.5e6
 
 
 def log(*a):
@@ -56,29 +66,53 @@ def build_model(device):
     return model, x, n
 
 
+def host_threads():
+    """Threads for the CPU legs: every core this process may use (os.cpu_count(), capped by the
+    OMP_NUM_THREADS the box exports for its CPU share)."""
+    n = os.cpu_count() or 1
+    try:
+        n = min(n, int(os.environ.get("OMP_NUM_THREADS", n)))
+    except ValueError:
+        pass
+    return max(1, n)
+
+
 def parity_gate(model, x):
-    """Before any timing: the first 3x3 shift conv of the network on a one-image slice of its real
-    input, GPU int32 output against the oracle, bit for bit."""
+    """Before any timing: the launches that are about to be timed -- the stem, the first 3x3 convolution
+    (the dominant kernel) and the first strided 3x3 / 1x1 pair, each on its real batch-64 input and
+    through kernels.kernel_bits() -- against the oracle on the first and the last image, bit for bit."""
     from deepshift_amd import kernels, modules
     from oracle import shift_oracle
     oracle = shift_oracle.get()
-    layer = [m for m in model.modules() if isinstance(m, modules.Conv2dShift)][1]
+    convs = [m for m in model.modules() if isinstance(m, modules.Conv2dShift)]
+    strided = [i for i, m in enumerate(convs) if m.stride == (2, 2) and i > 0][:2]
+    picked = {i: convs[i] for i in [0, 1] + strided}
     captured = {}
-    h = layer.register_forward_hook(lambda mod, inp, out: captured.setdefault("x", inp[0]))
+
+    def keep(k):
+        def hook(mod, inp, out):
+            captured[k] = inp[0]   # (a hook's return value would replace the layer's output)
+        return hook
+
+    hooks = [m.register_forward_hook(keep(i)) for i, m in picked.items()]
     with torch.no_grad():
-        model(x[:2])
-    h.remove()
-    xin = captured["x"][:1].contiguous()
-    xq = kernels.quantize_pad(xin, layer.padding, 16, 16)
-    tiled = kernels._tiled_of(layer.conc_weight, layer.out_channels, layer.in_channels, *layer.kernel_size)
-    y = kernels.conv2d_tiled(xq, tiled, None, layer.out_channels, layer.kernel_size, layer.stride,
-                             layer.conc_weight.bits, layer.conc_weight.base)
-    shift = layer.shift.detach().clamp(*layer.shift_range).round().cpu().numpy().astype(np.int32)
-    sign = layer.sign.detach().round().sign().cpu().numpy().astype(np.int32)
-    want = oracle.conv2d(xq.cpu().numpy(), shift, sign, None, layer.stride,
-                         nthreads=min(16, os.cpu_count() or 1))
-    if not np.array_equal(y.cpu().numpy(), want):
-        raise SystemExit("parity gate failed: GPU shift conv differs from the oracle")
+        model(x)
+    for h in hooks:
+        h.remove()
+    for i, layer in picked.items():
+        xq = kernels.quantize_pad(captured[i].contiguous(), layer.padding, 16, 16)
+        cw = layer.packed_weights()
+        tiled = kernels._tiled_of(cw, layer.out_channels, layer.in_channels, *layer.kernel_size)
+        y = kernels.conv2d_tiled(xq, tiled, None, layer.out_channels, layer.kernel_size, layer.stride,
+                                 kernels.kernel_bits(cw), cw.base)
+        shift = layer.shift.detach().clamp(*layer.shift_range).round().cpu().numpy().astype(np.int32)
+        sign = layer.sign.detach().round().sign().cpu().numpy().astype(np.int32)
+        for img in (0, x.shape[0] - 1):
+            want = oracle.conv2d(xq[img:img + 1].cpu().numpy(), shift, sign, None, layer.stride,
+                                 nthreads=host_threads())
+            if not np.array_equal(y[img:img + 1].cpu().numpy(), want):
+                raise SystemExit("parity gate failed: shift conv %d, image %d differs from the oracle" % (i, img))
+    return len(picked)
 
 
 def time_steps(model, x, steps, warmup):
@@ -187,7 +221,8 @@ def config2(device, reps=10):
     return out
 
 
-def fused_model_timing(device, cls, batch, weight_bits, integer_bits, fraction_bits, workload, steps=5):
+def fused_model_timing(device, cls, batch, weight_bits, integer_bits, fraction_bits, workload, steps=5,
+                       chw=CHW, peak=PEAK_PAIRS):
     """Steps/s and shift-kernel rate of a converted, fused network on synthetic input."""
     from deepshift_amd import convert, fuse
     g = torch.Generator().manual_seed(0)
@@ -203,7 +238,7 @@ def fused_model_timing(device, cls, batch, weight_bits, integer_bits, fraction_b
                                         act_fraction_bits=fraction_bits)
     model = model.to(device)
     convert.round_shift_weights(model)
-    x = torch.randn(batch, *CHW, generator=g).to(device)
+    x = torch.randn(batch, *chw, generator=g).to(device)
     with torch.no_grad():
         fused = fuse.fuse_conv_epilogues(model)
     sec = time_steps(fused, x, steps, 2)
@@ -213,7 +248,8 @@ def fused_model_timing(device, cls, batch, weight_bits, integer_bits, fraction_b
     return dict(workload=workload, ms_per_step=sec * 1e3, images_per_s=batch / sec, shift_layers=len(layers),
                 pairs_per_step=pairs, shift_kernel_ms_per_step=kernel_s * 1e3,
                 shift_tpairs_per_s=pairs / kernel_s / 1e12,
-                frac_of_two_instruction_peak=pairs / kernel_s / PEAK_PAIRS)
+                valu_bound_tpairs_per_s=peak / 1e12, valu_frac=pairs / kernel_s / peak,
+                frac_of_two_instruction_peak=pairs / kernel_s / PEAK_PAIRS_TWO_INSTR)
 
 
 def config5(device, steps=5):
@@ -222,7 +258,8 @@ def config5(device, steps=5):
     the int8 kernel (two pixels per register); the FC stays on the int32 kernel."""
     from deepshift_amd import workloads
     return fused_model_timing(device, workloads.ResNet50, 128, 3, 3, 5,
-                              "ResNet-50, batch 128 x 3x224x224, weight_bits 3, activations 3.5", steps)
+                              "ResNet-50, batch 128 x 3x224x224, weight_bits 3, activations 3.5", steps,
+                              peak=PEAK_PAIRS_INT8)
 
 
 def config4_act8(device, steps=5):
@@ -231,7 +268,92 @@ def config4_act8(device, steps=5):
     int32 kernels."""
     from deepshift_amd import workloads
     return fused_model_timing(device, workloads.ResNet18, BATCH, 5, 3, 5,
-                              "ResNet-18, batch 64 x 3x224x224, weight_bits 5, activations 3.5", steps)
+                              "ResNet-18, batch 64 x 3x224x224, weight_bits 5, activations 3.5", steps,
+                              peak=PEAK_PAIRS_INT8)
+
+
+def config3(device, steps=10):
+    """Benchmark configuration 3: ResNet-20 (CIFAR topology, 19 convolutions + FC), batch 256 x 3x32x32,
+    weight_bits 5, activations 16.16."""
+    from deepshift_amd import workloads
+    return fused_model_timing(device, workloads.ResNet20, 256, 5, 16, 16,
+                              "ResNet-20, batch 256 x 3x32x32, weight_bits 5, activations 16.16", steps,
+                              chw=(3, 32, 32))
+
+
+def config1(device, with_cpu=True, reps=50):
+    """Benchmark configuration 1: the 784-512-512-10 LinearShift MLP at batch 64, ternary signs, shifts in
+    [-15, 0], 16.16 -- microseconds per forward on the GPU, and the same network on this host through the
+    oracle's restatement of the reference's CPU kernel (the path the reference runs this model on,
+    mnist.py:213 with --no-cuda) and through the library's own host kernel (use_cuda=False)."""
+    from deepshift_amd import convert, modules, workloads
+    g = torch.Generator().manual_seed(0)
+    x = torch.rand(64, 784, generator=g)
+
+    def build(use_cuda):
+        gg = torch.Generator().manual_seed(1)
+        model, _ = convert.convert_to_shift(workloads.MLP(), 0, 'PS', convert_weights=False, use_kernel=True,
+                                            use_cuda=use_cuda, weight_bits=6)
+        for layer in model.layers:
+            layer.sign.data = torch.randint(-1, 2, layer.sign.shape, generator=gg).float()
+            layer.shift.data = torch.randint(-15, 1, layer.shift.shape, generator=gg).float()
+            layer.bias.data = torch.randn(layer.bias.shape, generator=gg) * 0.01
+        return model.eval()
+
+    gpu_model = build(True).to(device)
+    xd = x.to(device)
+    with torch.no_grad():
+        for _ in range(5):
+            y_gpu = gpu_model(xd)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            gpu_model(xd)
+        torch.cuda.synchronize()
+        gpu_s = (time.perf_counter() - t0) / reps
+    layers = kernel_timings(gpu_model, xd, 5)
+    out = {"workload": "MLP 784-512-512-10, batch 64, ternary signs, shifts [-15, 0], activations 16.16",
+           "us_per_forward": gpu_s * 1e6, "shift_kernel_us_per_forward": sum(L["seconds"] for L in layers) * 1e6,
+           "pairs_per_forward": sum(L["M"] * L["K"] * L["N"] for L in layers)}
+    if with_cpu:
+        from oracle import shift_oracle
+        oracle = shift_oracle.get()
+        threads = host_threads()
+        cpu_model = build(False)
+        codes = [(modules.module_codes(l), l.bias.detach().numpy()) for l in cpu_model.layers]
+
+        def oracle_forward(nthreads):
+            h = x.numpy()
+            for i, ((shift, sign), bias) in enumerate(codes):
+                y = oracle.linear(oracle.cast(h, 16), shift.numpy().astype(np.int8), sign.numpy().astype(np.int32),
+                                  oracle.cast(bias, 16), nthreads)
+                h = y.astype(np.float32) / np.float32(65536.0)
+                if i < 2:
+                    h = np.maximum(h, 0)
+            return h
+
+        want = oracle_forward(threads)
+        identical = bool(np.array_equal(y_gpu.cpu().numpy(), want))
+        t0 = time.perf_counter()
+        for _ in range(5):
+            oracle_forward(threads)
+        t_multi = (time.perf_counter() - t0) / 5
+        t0 = time.perf_counter()
+        oracle_forward(1)
+        t_single = time.perf_counter() - t0
+        with torch.no_grad():
+            host = cpu_model(x)
+            t0 = time.perf_counter()
+            for _ in range(5):
+                cpu_model(x)
+            t_twin = (time.perf_counter() - t0) / 5
+        out["cpu"] = {"kind": "port", "cores": threads, "us_per_forward": t_multi * 1e6,
+                      "single_thread_us_per_forward": t_single * 1e6, "gpu_equals_cpu_bit_for_bit": identical,
+                      "host_twin_us_per_forward": t_twin * 1e6,
+                      "host_twin_equals_gpu": bool(torch.equal(host, y_gpu.cpu()))}
+        if not identical:
+            raise SystemExit("configuration 1: the GPU forward differs from the oracle chain")
+    return out
 
 
 def pmc_target(device):
@@ -259,7 +381,7 @@ def cpu_baseline(shapes):
     images split over threads) on every shift layer of ResNet-18 at a reduced batch."""
     from oracle import shift_oracle
     oracle = shift_oracle.get()
-    threads = min(16, os.cpu_count() or 1)
+    threads = host_threads()
     batch = threads
     rng = np.random.default_rng(0)
 
@@ -306,7 +428,8 @@ def cpu_baseline(shapes):
                  "identical": bool(np.array_equal(np.array(y_ref, np.int64).astype(np.int32), y_port))}
     return {
         "reference_kernel_check": check,
-        "value": batch / t_multi, "unit": "images/s", "cores": threads, "kind": "port",
+        "value": batch / t_multi, "unit": "images/s", "cores": threads, "host_cpu_count": os.cpu_count(),
+        "kind": "port",
         "sample": "all 21 shift layers of ResNet-18 at batch %d (one image per thread), kernel time "
                   "only, int32 inputs resident in host memory; single thread on 1 image: %.3f images/s"
                   % (batch, 1.0 / t_single),
@@ -345,8 +468,8 @@ def main():
 
     from deepshift_amd import workloads
     model, x, n_conv = build_model(device)
-    parity_gate(model, x)
-    log("parity gate passed; %d conv + 1 fc shift layers" % n_conv)
+    checked = parity_gate(model, x)
+    log("parity gate passed on %d timed launches; %d conv + 1 fc shift layers" % (checked, n_conv))
 
     # The measured pipeline: the converted model with the fp32 glue after every shift conv
     # (BatchNorm, residual add, ReLU) folded into that conv's dequantisation pass.  The shift
@@ -384,8 +507,17 @@ def main():
                 L["name"], L["M"], L["K"], L["N"], L["seconds"] * 1e6, p / L["seconds"] / 1e12,
                 100 * p / L["seconds"] / PEAK_PAIRS, 100 * L["bytes"] / L["seconds"] / HBM_PEAK))
 
+    # The dominant kernel: the launches of the 3x3 convolutions (16 of the 21, 92 % of the pairs) all run
+    # the same kernel; its roofline figures come from their HIP-event durations.
+    dominant = [L for L in layers if L["K"] % 9 == 0 and L["K"] >= 576]
+    dom_pairs = sum(L["M"] * L["K"] * L["N"] for L in dominant)
+    dom_s = sum(L["seconds"] for L in dominant)
+    dom_bytes = sum(L["bytes"] for L in dominant)
+
     peak_cal = None if args.resnet_only else calibrate_valu(device)
+    cfg1 = None if args.resnet_only else config1(device, with_cpu=not args.no_cpu)
     cfg2 = None if args.resnet_only else config2(device)
+    cfg3 = None if args.resnet_only else config3(device)
     cfg5 = None if args.resnet_only else config5(device)
     cfg4_act8 = None if args.resnet_only else config4_act8(device)
     result = {
@@ -411,33 +543,37 @@ def main():
         "shift_gops": 2 * pairs / kernel_s / 1e9,
         "shift_layers_images_per_s": BATCH / kernel_s,
         "roofline": {
+            # Bound: vector ALU.  peak = 256 CUs x 64 lanes x 2.4 GHz / 1 vector instruction per pair (the
+            # accumulate; no int32 kernel can need fewer) = 39.3 Tpair/s.  achieved = the pairs of the
+            # dominant kernel's launches / their HIP-event durations in this run.
             "bound": "valu",
-            "kernel": "ds::shift_planes_wide_cu_kernel<4> (16 launches) + ds::shift_planes_wide_balanced_kernel<4> "
-                      "(1 launch) + ds::shift_kernel (4 launches) per step",
-            "achieved": pairs / kernel_s / 1e12,
+            "kernel": DOMINANT_KERNEL,
+            "launches_per_step": len(dominant),
+            "achieved": dom_pairs / dom_s / 1e12,
             "peak": PEAK_PAIRS / 1e12,
             "unit": "Tpair/s",
-            "frac": pairs / kernel_s / PEAK_PAIRS,
-            # HBM bytes of one launch of the dominant shape (layer1 3x3 conv, 8 of the 21 launches are
-            # this size): 109.4 MB read + 67.1 MB written (tiles shared by two workgroups are combined
-            # with atomic adds), from the FETCH_SIZE / WRITE_SIZE runs summarised in
-            # profiles/shift_kernel_layer1_conv_counters.md (106.6 MB algorithmic)
-            "traffic": 176.5e6,
-            # vector instructions the dominant kernel issues per pair (SQ_INSTS_VALU, same profile):
-            # `peak` prices a pair at 2 instructions, so its fraction can exceed 1
-            "valu_instr_per_pair": 1.28,
-            # the same lanes x nominal clock priced at the kernel's own instruction count: the ceiling of
-            # this kernel design, below 1 by the vector-issue gaps (two scalar instructions per code)
-            "peak_at_kernel_mix": PEAK_PAIRS * VALU_INSTR_PER_PAIR / 1.28 / 1e12,
-            "frac_at_kernel_mix": pairs / kernel_s / (PEAK_PAIRS * VALU_INSTR_PER_PAIR / 1.28),
-            "avg_launch_us": kernel_s / len(layers) * 1e6,
-            "peak_calibrated": peak_cal / 1e12 if peak_cal else None,
-            "frac_of_calibrated": pairs / kernel_s / peak_cal if peak_cal else None,
-            "hbm_achieved_GBps": alg_bytes / kernel_s / 1e9,
-            "hbm_frac": alg_bytes / kernel_s / HBM_PEAK,
+            "frac": dom_pairs / dom_s / PEAK_PAIRS,
+            "avg_launch_us": dom_s / len(dominant) * 1e6,
+            "pairs_per_launch": dom_pairs / len(dominant),
+            # HBM bytes of one launch of the dominant kernel on the layer1 shape (M = 200704, K = 576,
+            # N = 64; 106.6 MB algorithmic), a constant copied from the FETCH_SIZE / WRITE_SIZE runs in
+            # profiles/shift_kernel_layer1_conv_counters.md -- not measured in this run
+            "traffic": TRAFFIC_LAYER1_BYTES,
+            "traffic_source": "profiles/shift_kernel_layer1_conv_counters.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)",
+            # the whole step (all 21 launches, pre-fill passes included) against the same bound
+            "step_achieved": pairs / kernel_s / 1e12,
+            "step_frac": pairs / kernel_s / PEAK_PAIRS,
+            # secondary: against a kernel that spends two vector instructions on every pair
+            "peak_two_instruction": PEAK_PAIRS_TWO_INSTR / 1e12,
+            "frac_of_two_instruction_peak": dom_pairs / dom_s / PEAK_PAIRS_TWO_INSTR,
+            "peak_two_instruction_calibrated": peak_cal / 1e12 if peak_cal else None,
+            "hbm_achieved_GBps": dom_bytes / dom_s / 1e9,
+            "hbm_frac": dom_bytes / dom_s / HBM_PEAK,
             "algorithmic_bytes_per_step": alg_bytes,
         },
+        "config1": cfg1,
         "config2": cfg2,
+        "config3": cfg3,
         "config5": cfg5,
         "config4_act8": cfg4_act8,
         "shift_gemm_gops": cfg2["gemm_4096"]["gops"] if cfg2 else None,
