@@ -13,6 +13,7 @@ DS_Q_ROUND_TO_FIXED = 0
 DS_Q_CAST = 1
 DS_BITS_ZERO_TOP = 0x100
 DS_BITS_TOP_UNUSED = 0x200
+DS_Q_BORDER_KEPT = 0x100
 
 _c_int = ctypes.c_int
 _c_i64 = ctypes.c_int64
@@ -51,6 +52,8 @@ SIGNATURES = {
     "ds_conv2d_tiled_i32": (_c_int, [_ptr] * 4 + [_c_int] * 11 + [_ptr, _size, _ptr]),
     "ds_cpu_linear_i32": (_c_int, [_ptr] * 5 + [_c_int] * 4),
     "ds_cpu_conv2d_i32": (_c_int, [_ptr] * 5 + [_c_int] * 10),
+    "ds_conv2d_tiled_fusable": (_c_int, [_c_int] * 11),
+    "ds_conv2d_tiled_fused_i32": (_c_int, [_ptr] * 8 + [_c_int] * 18 + [_ptr, _size, _ptr]),
     "ds_quantize_f32_i32": (_c_int, [_ptr, _ptr, _c_i64, _c_int, _c_int, _c_int, _ptr]),
     "ds_quantize_pad_f32_i32": (_c_int, [_ptr, _ptr] + [_c_int] * 9 + [_ptr]),
     "ds_quantize_transpose_f32_i32": (_c_int, [_ptr, _ptr] + [_c_int] * 6 + [_ptr]),

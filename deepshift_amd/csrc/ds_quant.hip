@@ -1,58 +1,9 @@
 // Fixed-point conversion passes around the shift kernels (HBM-bound, one read + one write each).
 #include "ds_common.h"
+#include "ds_epilogue.h"
 
 namespace ds {
 
-// float -> int32 on the 2^-F grid.
-//   ROUND_TO_FIXED: utils.round_to_fixed (utils.py:7-21) followed by (x * 2**F).int()
-//   (modules.py:153).  floor(x / 2^-F) * 2^-F is clamped to [-2^(I-1), 2^(I-1) - 1] and scaled back
-//   by 2^F; all three scalings are by powers of two, hence exact, so the clamp can be applied to
-//   floor(x * 2^F) directly with bounds scaled by 2^F.  I == 1 is the reference's special case
-//   sign(x) - 1.
-//   CAST: (x * 2**F).int() alone (modules.py:25): truncation toward zero; the hardware conversion
-//   saturates and maps NaN to 0.
-struct QuantSpec {
-    float scale, lo, hi;
-    int mode, I;
-};
-
-// float -> int32 toward zero, saturating, NaN -> 0 (what v_cvt_i32_f32 returns; spelled out because
-// an out-of-range C++ conversion is undefined).
-__device__ __forceinline__ int32_t f2i_sat(float v)
-{
-    if (v != v) return 0;
-    if (v >= 2147483648.0f) return 2147483647;
-    if (v <= -2147483648.0f) return (int32_t)0x80000000;
-    return (int32_t)v;
-}
-
-__device__ __forceinline__ int32_t quantize_one(float v, const QuantSpec &q)
-{
-    if (q.mode == DS_Q_CAST) return f2i_sat(v * q.scale);
-    float r;
-    if (q.I == 1) {
-        r = ((v > 0.0f) ? 1.0f : ((v < 0.0f) ? -1.0f : 0.0f)) - 1.0f;
-        if (v != v) r = v;
-        r *= q.scale;
-    } else {
-        r = floorf(v * q.scale);
-        // torch.clamp semantics: NaN propagates
-        r = (r < q.lo) ? q.lo : r;
-        r = (r > q.hi) ? q.hi : r;
-    }
-    return f2i_sat(r);
-}
-
-static QuantSpec make_spec(int I, int F, int mode)
-{
-    QuantSpec q;
-    q.scale = ldexpf(1.0f, F);
-    q.lo = -ldexpf(1.0f, I - 1 + F);
-    q.hi = (ldexpf(1.0f, I - 1) - 1.0f) * q.scale;
-    q.mode = mode;
-    q.I = I;
-    return q;
-}
 
 __global__ void quantize_kernel(const float *__restrict__ x, int32_t *__restrict__ q, long n,
                                 QuantSpec spec)
@@ -185,18 +136,6 @@ __global__ void dequantize_kernel(const int32_t *__restrict__ y, float *__restri
 // out = act(float(y) / 2^F * scale[c] + shift[c] (+ residual)): the dequantisation of a shift layer
 // fused with an inference-mode per-channel affine (a folded BatchNorm), a residual add and ReLU.
 // One thread per 4 consecutive pixels of one (image, channel) plane when HW % 4 == 0.
-// The float value that follows a shift layer: act(float(y) / 2^F * a + b (+ r)).  One definition, with
-// contraction off, so that every kernel that needs it rounds the same way.
-__device__ __forceinline__ float affine_one(int32_t y, float inv, float a, float b, const float *r,
-                                            int relu)
-{
-#pragma clang fp contract(off)
-    float v = ((float)y * inv) * a + b;
-    if (r) v += *r;
-    if (relu) v = v > 0.0f ? v : 0.0f;
-    return v;
-}
-
 template <int VEC>
 __global__ void dequantize_affine_kernel(const int32_t *__restrict__ y, float *__restrict__ out,
                                          const float *__restrict__ scale, const float *__restrict__ shift,

@@ -23,6 +23,7 @@
 //   * layers with few pixels split K over gridDim.y and combine with integer atomics (wrap-around
 //     addition commutes, so the result stays bit-exact).
 #include "ds_common.h"
+#include "ds_epilogue.h"
 #include <cstdio>
 #include <atomic>
 #include <cstdlib>
@@ -59,6 +60,21 @@ struct ShiftArgs {
     uint32_t y_elems;                     // elements the pre-fill covers
     int zero_top;                         // the highest field value is a zero weight (ternary blobs)
     int top_unused;                       // no code carries the highest field value (the caller vouches)
+    // Workgroup-cooperative launch: per-workgroup arrival counters and partial-tile slots in the
+    // caller's workspace (nullptr: no room, the launch falls back to wave-level shares).
+    int32_t *coop_counters;
+    int32_t *coop_slots;
+    // Fused epilogue of the cooperative launch (convolutions only): instead of the int32 sums the
+    // finished tile goes through act(sum / 2^F * scale[c] + shift[c] + residual) and is stored as float
+    // (out) and / or as the next shift convolution's round-to-fixed, zero padded input (q).
+    int fused;
+    float *ep_out;
+    void *ep_q;
+    const float *ep_scale, *ep_shift, *ep_residual;
+    float ep_inv;                         // 2^-F of the sums
+    int ep_relu, ep_ph, ep_pw, ep_q_bytes;
+    int ep_border_kept;                   // the padding of q already holds zeros: write the interior only
+    QuantSpec ep_spec;
 };
 
 // Redirects an atomic LinearShift launch to its channel-major scratch; returns the final y or nullptr.
@@ -522,91 +538,343 @@ void shift_planes_wide_balanced_kernel(const ShiftArgs p)
 }
 
 // Workgroup-cooperative launch of the 64-channel form: the (tile, K group) space is cut into one
-// equal share per workgroup of four (or eight) waves; the waves split the K range of a tile among
-// themselves and combine their sums in a 32 KiB LDS tile (LDS atomics cost next to nothing), and the tile goes
-// to the output once: a plain store of sum + bias when the workgroup ran the tile's whole reduction,
-// atomic adds onto the pre-filled output when it shares the tile with a neighbouring workgroup.
-// Global atomics retire one lane per clock and L2 channel and do not overlap the arithmetic of the
-// waves that wait on them; the wave-level shares above issue one per output and share, this launch
-// one per output and workgroup boundary.
-// WAVES = 8: one workgroup per compute unit, two tile buffers used alternately and one barrier per
-// tile.  WAVES = 4: two workgroups per compute unit, one buffer each and two barriers per tile; the two
-// waves of a SIMD then belong to different workgroups and are not held at the same barrier.
-template <int BITS, int ZT, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void shift_planes_wide_cu_kernel(const ShiftArgs p)
+// equal share per workgroup of four waves; the waves split the K range of a tile among themselves
+// and combine their sums in a 32 KiB LDS tile (LDS atomics cost next to nothing).  A tile whose whole
+// reduction ran in this workgroup goes to the output from there.  A tile that straddles a workgroup
+// boundary is finished by whichever of its workgroups arrives last: every contributor stores its
+// partial tile in its own slot of the workspace, releases it and bumps the tile's arrival counter;
+// the one that sees the count complete acquires, sums the slots and writes the tile -- no pre-filled
+// output, no global atomics on it, nobody waits for anybody.  Two workgroups per compute unit, so the
+// two waves of a SIMD belong to different workgroups and are never held at the same barrier.
+//
+// The finished tile is still in LDS as [channel][pixel], so what follows the layer can run right
+// there (FUSED): dequantise, per-channel affine (a folded BatchNorm), residual add, ReLU, and the next
+// shift convolution's round-to-fixed + zero padding, written as float and / or fixed point instead of
+// the int32 sums (modules.py:161-162 then :317,:153 of the next layer).
+constexpr int kCoopWaves = 4;
+constexpr int kCoopPix = kPlaneRowsWide * kWave;       // pixels of a tile
+constexpr int kCoopTileElems = 64 * kCoopPix;          // int32 sums of a tile
+constexpr int kCoopLdsBytes = kCoopTileElems * 4;
+
+static size_t coop_counter_bytes(int blocks) { return align_up((size_t)blocks * 4, 256); }
+static size_t coop_workspace_bytes(int blocks)
 {
-    constexpr int PIX = kPlaneRowsWide * kWave;
-    constexpr int BUFFERS = WAVES == 8 ? 2 : 1;
-    // With two buffers: a wave adds its sums of tile t to buffer t % 2, waits for the others, writes
-    // out and clears its channels of that buffer, and goes on to tile t + 1 in the other buffer;
-    // nobody adds to buffer t % 2 again before the barrier of tile t + 1, which every wave reaches
-    // after it has cleared its channels.  With one buffer a second barrier follows the clearing.
-    extern __shared__ int32_t tile_sums[];  // [BUFFERS][64 channels][128 pixels]
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int lane = threadIdx.x & (kWave - 1);
-    const int bid = blockIdx.x;
-    const int w = (bid & 7) * (int)(gridDim.x >> 3) + (bid >> 3);  // an XCD takes a contiguous range
-    const long total = (long)p.tiles_m4 * p.tiles_n * p.comm;
-    int it = (int)(w * total / (long)gridDim.x);
-    const int it_end = (int)((w + 1) * total / (long)gridDim.x);
-    for (int i = threadIdx.x; i < BUFFERS * 64 * PIX; i += WAVES * 64) tile_sums[i] = 0;
+    // a workgroup has at most two partial tiles: the one its share starts in and the one it ends in
+    return coop_counter_bytes(blocks) + (size_t)2 * blocks * kCoopTileElems * 4;
+}
+// one workgroup per 8 wave slots (2 waves per SIMD); small layers: >= 8 K groups per wave
+static int coop_blocks(long iters)
+{
+    int blocks = plane_slots(true) / kCoopWaves;
+    const long fit = (iters / (8 * kCoopWaves)) / 8 * 8;
+    if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
+    // every workgroup must own at least one iteration: a tile is finished by the LAST of the
+    // workgroups that its range of iterations names, and an empty share would never arrive
+    if (blocks > iters) blocks = iters < 1 ? 1 : (int)iters;
+    return blocks;
+}
+
+// Partial tiles travel between workgroups that may sit on different XCDs, whose L2 caches are not
+// coherent with each other.  Fences at agent scope would write back and invalidate a whole L2 per
+// exchange (measured: +45 % on a ResNet 3x3 layer, the other workgroups lose their cached activations);
+// instead the slots are written and read with agent-scope (relaxed atomic) accesses, which go through to
+// the level all XCDs share, like the atomic adds of the per-wave launches do.
+__device__ __forceinline__ void store_agent(int32_t *p, int32_t v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ int32_t load_agent(const int32_t *p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The workgroup whose share [w * total / G, (w + 1) * total / G) holds iteration i.
+__device__ __forceinline__ int coop_owner(long i, long G, long total) { return (int)(((i + 1) * G - 1) / total); }
+
+// What the tail of a tile needs (write-out, partial-tile exchange), copied once per workgroup from
+// the kernel arguments into LDS: the tail runs as a function of its own (coop_finish_tile, not inlined),
+// so that its registers are allocated apart from the main loop's fixed map and scalar clobbers -- inlined,
+// the compiler kept its dozens of wave-uniform values in spilled scalar registers and branched per element.
+struct TileTail {
+    const int32_t *negcnt, *bias;
+    int32_t *y;
+    int32_t *slots, *counters;
+    float *out;
+    void *q;
+    const float *scale, *shift, *residual;
+    long y_img_stride, y_pix_stride, y_ch_stride;
+    long G, total;
+    int M, N, comm, pix_per_img, OW;
+    float inv;
+    int relu, ph, pw, q_bytes, border_kept;
+    QuantSpec spec;
+};
+typedef __attribute__((address_space(3))) int32_t lds_i32;
+typedef __attribute__((address_space(3))) const TileTail lds_tail;
+
+// round_to_fixed + cast of the fused epilogue without branches: the clamp keeps the value inside int32,
+// so only NaN (propagated by the clamp, as torch.clamp does) needs the conversion's "NaN -> 0".
+__device__ __forceinline__ int32_t quantize_fixed(float v, float scale, float lo, float hi, bool one_bit)
+{
+    float r = floorf(v * scale);
+    r = (r < lo) ? lo : r;
+    r = (r > hi) ? hi : r;
+    if (one_bit) {  // integer_bits == 1: sign(x) - 1 (utils.py:12-13)
+        float s = ((v > 0.0f) ? 1.0f : ((v < 0.0f) ? -1.0f : 0.0f)) - 1.0f;
+        s = (v != v) ? v : s;
+        r = s * scale;
+    }
+    return (int32_t)((r == r) ? r : 0.0f);
+}
+
+// The zero padding of the next layer's input around this tile's pixels: the pixels on an image edge
+// write their row's margins, those of the first / last row also the rows above / below.
+template <typename Q>
+__device__ __forceinline__ void write_padding(Q *q, size_t plane_base, int oh, int ow, int OH, int OW, int ph,
+                                              int pw, int Wq)
+{
+    const bool left = ow == 0, right = ow == OW - 1, top = oh == 0, bottom = oh == OH - 1;
+    if (!(left || right || top || bottom)) return;
+    const size_t qrow = plane_base + (size_t)(oh + ph) * Wq;
+    if (left) for (int dx = 0; dx < pw; ++dx) q[qrow + dx] = 0;
+    if (right) for (int dx = 0; dx < pw; ++dx) q[qrow + pw + OW + dx] = 0;
+    if (!(top || bottom)) return;
+    for (int dy = 0; dy < ph; ++dy) {
+        if (top) {
+            const size_t row = plane_base + (size_t)dy * Wq;
+            q[row + ow + pw] = 0;
+            if (left) for (int dx = 0; dx < pw; ++dx) q[row + dx] = 0;
+            if (right) for (int dx = 0; dx < pw; ++dx) q[row + pw + OW + dx] = 0;
+        }
+        if (bottom) {
+            const size_t row = plane_base + (size_t)(ph + OH + dy) * Wq;
+            q[row + ow + pw] = 0;
+            if (left) for (int dx = 0; dx < pw; ++dx) q[row + dx] = 0;
+            if (right) for (int dx = 0; dx < pw; ++dx) q[row + pw + OW + dx] = 0;
+        }
+    }
+}
+
+// The finished tile leaves the workgroup's LDS buffer: wave w takes channels 16w .. 16w + 15, its lanes
+// the 128 pixels.  Everything that comes from memory is requested up front -- the per-channel constants
+// by the lanes (lane c holds those of the wave's channel c and hands them out with v_readlane), the
+// residuals of all 32 outputs of a lane before the first is used -- so that the tile pays the memory
+// latency once, not once per channel.
+template <bool FUSED, typename Q>
+__device__ __forceinline__ void write_tile(lds_tail *t, lds_i32 *buf, int ntile, int m0, int wave, int lane)
+{
+    constexpr int CH = 64 / kCoopWaves, R = kPlaneRowsWide;
+    const int M = t->M, N = t->N, pix_per_img = t->pix_per_img, OW = t->OW;
+    const int n0 = ntile * 64 + wave * CH;
+    const int mine = n0 + (lane & (CH - 1));
+    const int32_t *bias = t->bias;
+    const int32_t add_l = t->negcnt[mine] + (bias ? bias[mine] : 0);
+    float sa_l = 1.0f, sb_l = 0.0f;
+    const float *residual = nullptr;
+    float *out = nullptr;
+    Q *q = nullptr;
+    if (FUSED) {
+        const float *scale = t->scale, *shift = t->shift;
+        if (scale) sa_l = scale[mine];
+        if (shift) sb_l = shift[mine];
+        residual = t->residual;
+        out = t->out;
+        q = (Q *)t->q;
+    }
+    const int ph = FUSED ? t->ph : 0, pw = FUSED ? t->pw : 0;
+    const int OH = pix_per_img / OW;
+    const int Hq = OH + 2 * ph, Wq = OW + 2 * pw;
+    const size_t qplane = (size_t)Hq * Wq;
+    bool live[R];
+    size_t pix[R], qpix[R], qimg[R];
+    int oh[R], ow[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int m = m0 + r * kWave + lane;
+        live[r] = m < M;
+        const int mm = live[r] ? m : 0;
+        const int img = mm / pix_per_img, rem = mm - img * pix_per_img;
+        oh[r] = rem / OW;
+        ow[r] = rem - oh[r] * OW;
+        if (FUSED) {
+            pix[r] = ((size_t)img * N + n0) * pix_per_img + rem;
+            qimg[r] = ((size_t)img * N + n0) * qplane;
+            qpix[r] = qimg[r] + (size_t)(oh[r] + ph) * Wq + ow[r] + pw;
+        } else {
+            pix[r] = (size_t)img * t->y_img_stride + (size_t)rem * t->y_pix_stride + (size_t)n0 * t->y_ch_stride;
+        }
+    }
+    float res[CH][R];
+    if (FUSED && residual) {
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+#pragma unroll
+            for (int r = 0; r < R; ++r) res[c][r] = live[r] ? residual[pix[r] + (size_t)c * pix_per_img] : 0.0f;
+    }
+    int32_t sums[CH][R];
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            lds_i32 *cell = buf + (wave * CH + c) * kCoopPix + r * kWave + lane;
+            sums[c][r] = *cell;
+            *cell = 0;
+        }
+    if (!FUSED) {
+        int32_t *y = t->y;
+        const size_t ch = (size_t)t->y_ch_stride;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int32_t add = __builtin_amdgcn_readlane(add_l, c);
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                if (live[r]) y[pix[r] + c * ch] = sums[c][r] + add;
+        }
+        return;
+    }
+    const float inv = t->inv, qs = t->spec.scale, qlo = t->spec.lo, qhi = t->spec.hi;
+    const bool relu = t->relu != 0, one_bit = t->spec.I == 1, has_res = residual != nullptr;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int32_t add = __builtin_amdgcn_readlane(add_l, c);
+        const float sa = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sa_l), c));
+        const float sb = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sb_l), c));
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            float f;
+            {
+#pragma clang fp contract(off)
+                f = ((float)(sums[c][r] + add) * inv) * sa + sb;
+                if (has_res) f += res[c][r];
+                if (relu) f = f > 0.0f ? f : 0.0f;
+            }
+            if (!live[r]) continue;
+            if (out) out[pix[r] + (size_t)c * pix_per_img] = f;
+            if (q) q[qpix[r] + c * qplane] = (Q)quantize_fixed(f, qs, qlo, qhi, one_bit);
+        }
+    }
+    if (q && (ph | pw) && !t->border_kept) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (!live[r]) continue;
+            if (!(ow[r] == 0 || ow[r] == OW - 1 || oh[r] == 0 || oh[r] == OH - 1)) continue;
+            for (int c = 0; c < CH; ++c) write_padding(q, qimg[r] + c * qplane, oh[r], ow[r], OH, OW, ph, pw, Wq);
+        }
+    }
+}
+
+// The tail of one tile segment, after the workgroup's waves have added their sums into `buf` and met
+// at a barrier.  A whole tile (len == comm) is written out.  A partial one is published to this
+// workgroup's slot, its arrival counted, and whichever workgroup arrives last gathers the slots of all
+// contributors and writes the tile.  Ends with the buffer cleared and a barrier.
+template <bool FUSED>
+__device__ __attribute__((noinline)) void coop_finish_tile(lds_tail *t, lds_i32 *buf, lds_i32 *flag, int w, int tile,
+                                                           int g0, int len, int ntile, int m0)
+{
+    constexpr int THREADS = kCoopWaves * 64, PER = kCoopTileElems / THREADS;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
+    const int comm = t->comm;
+    bool finish = len == comm;
+    if (!finish) {
+        // slot 0 of a workgroup holds the tile its share starts in (g0 > 0), slot 1 the tile it ends in
+        int32_t *slot = t->slots + ((size_t)2 * w + (g0 > 0 ? 0 : 1)) * kCoopTileElems + threadIdx.x;
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+            store_agent(slot + k * THREADS, buf[threadIdx.x + k * THREADS]);
+            buf[threadIdx.x + k * THREADS] = 0;
+        }
+        // the slot is complete (every store acknowledged) before the arrival is counted
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        const long G = t->G, total = t->total;
+        const int first = coop_owner((long)tile * comm, G, total);
+        const int last = coop_owner((long)(tile + 1) * comm - 1, G, total);
+        if (threadIdx.x == 0)
+            *flag = __hip_atomic_fetch_add(t->counters + first, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
+                    last - first;
+        __syncthreads();
+        if (*flag) {
+            for (int c = first; c <= last; ++c) {
+                const int32_t *src = t->slots + ((size_t)2 * c + (c == first ? 1 : 0)) * kCoopTileElems + threadIdx.x;
+                int32_t v[PER];
+#pragma unroll
+                for (int k = 0; k < PER; ++k) v[k] = load_agent(src + k * THREADS);
+#pragma unroll
+                for (int k = 0; k < PER; ++k) buf[threadIdx.x + k * THREADS] += v[k];
+            }
+            finish = true;
+        }
+        __syncthreads();
+    }
+    if (finish) {
+        if (FUSED && t->q_bytes == 1) write_tile<FUSED, int8_t>(t, buf, ntile, m0, wave, lane);
+        else write_tile<FUSED, int32_t>(t, buf, ntile, m0, wave, lane);
+    }
     __syncthreads();
-    int32_t *buf = tile_sums;
+}
+
+template <int BITS, int ZT, bool FUSED>
+__global__ __launch_bounds__(kCoopWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void shift_planes_wide_coop_kernel(const ShiftArgs p)
+{
+    extern __shared__ int32_t tile_sums[];  // [64 channels][128 pixels]
+    __shared__ TileTail tail;
+    __shared__ int32_t last_arrival;
+    constexpr int THREADS = kCoopWaves * 64;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int bid = blockIdx.x;
+    const long G = gridDim.x;
+    // an XCD (workgroup ids congruent modulo 8) takes a contiguous range of shares
+    const int w = (gridDim.x & 7) ? bid : (bid & 7) * (int)(gridDim.x >> 3) + (bid >> 3);
+    const long total = (long)p.tiles_m4 * p.tiles_n * p.comm;
+    int it = (int)(w * total / G);
+    const int it_end = (int)((w + 1) * total / G);
+    if (threadIdx.x == 0) {
+        tail.negcnt = p.negcnt; tail.bias = p.bias; tail.y = p.y;
+        tail.slots = p.coop_slots; tail.counters = p.coop_counters;
+        tail.out = p.ep_out; tail.q = p.ep_q;
+        tail.scale = p.ep_scale; tail.shift = p.ep_shift; tail.residual = p.ep_residual;
+        tail.y_img_stride = p.y_img_stride; tail.y_pix_stride = p.y_pix_stride; tail.y_ch_stride = p.y_ch_stride;
+        tail.G = G; tail.total = total;
+        tail.M = p.M; tail.N = p.N; tail.comm = p.comm; tail.pix_per_img = p.pix_per_img; tail.OW = p.OW;
+        tail.inv = p.ep_inv; tail.relu = p.ep_relu; tail.ph = p.ep_ph; tail.pw = p.ep_pw;
+        tail.q_bytes = p.ep_q_bytes; tail.border_kept = p.ep_border_kept; tail.spec = p.ep_spec;
+    }
+    for (int i = threadIdx.x; i < kCoopTileElems; i += THREADS) tile_sums[i] = 0;
+    __syncthreads();
     while (it < it_end) {
         const int tile = it / p.comm;
         const int g0 = it - tile * p.comm;
         int g1 = g0 + (it_end - it);
         if (g1 > p.comm) g1 = p.comm;
-        const int ntile = tile % p.tiles_n, m0 = (tile / p.tiles_n) * PIX;
+        const int ntile = tile % p.tiles_n, m0 = (tile / p.tiles_n) * kCoopPix;
         const int len = g1 - g0;
-        const int wb = g0 + wave * len / WAVES, we = g0 + (wave + 1) * len / WAVES;
-        if (wb < we) planes_segment<BITS, ZT, true, true>(p, ntile, m0, wb, we, true, buf);
+        const int wb = g0 + wave * len / kCoopWaves, we = g0 + (wave + 1) * len / kCoopWaves;
+        if (wb < we) planes_segment<BITS, ZT, true, true>(p, ntile, m0, wb, we, true, tile_sums);
         __syncthreads();
-        const bool whole = len == p.comm;
-        for (int c = 0; c < 64 / WAVES; ++c) {
-            const int j = wave * (64 / WAVES) + c, n = ntile * 64 + j;
-            const int32_t add = whole ? p.negcnt[n] + (p.bias ? p.bias[n] : 0) : 0;
-            for (int r = 0; r < kPlaneRowsWide; ++r) {
-                int32_t *cell = buf + j * PIX + r * kWave + lane;
-                const int32_t v = *cell;
-                *cell = 0;
-                const int m = m0 + r * kWave + lane;
-                if (m >= p.M) continue;
-                const int img = m / p.pix_per_img;
-                int32_t *dst = p.y + (size_t)n * p.y_ch_stride + (size_t)img * p.y_img_stride +
-                               (size_t)(m - img * p.pix_per_img) * p.y_pix_stride;
-                if (whole) *dst = v + add;
-                else atomicAdd(dst, v);
-            }
-        }
-        if (BUFFERS == 2) buf = buf == tile_sums ? tile_sums + 64 * PIX : tile_sums;
-        else __syncthreads();
+        coop_finish_tile<FUSED>((lds_tail *)&tail, (lds_i32 *)tile_sums, (lds_i32 *)&last_arrival, w, tile, g0, len,
+                                ntile, m0);
         it += len;
     }
 }
 
-template <int BITS, int ZT, int WAVES>
-static int launch_planes_cu(const ShiftArgs &a, long iters, hipStream_t st)
+__global__ void zero_i32_kernel(int32_t *dst, int n)
 {
-    constexpr int kLdsBytes = (WAVES == 8 ? 2 : 1) * 64 * kPlaneRowsWide * kWave * 4;
-    if (kLdsBytes > 64 * 1024) {  // above the default limit of a workgroup: opt in, once per device
-        static std::atomic<bool> opted_in[64];  // per device; setting the attribute twice is harmless
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
-        if (!opted_in[dev].load(std::memory_order_acquire)) {
-            hipError_t e = hipFuncSetAttribute((const void *)shift_planes_wide_cu_kernel<BITS, ZT, WAVES>,
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-            if (e != hipSuccess) return hip_status(e);
-            opted_in[dev].store(true, std::memory_order_release);
-        }
-    }
-    // one workgroup per 8 wave slots (2 waves per SIMD); small layers: >= 8 K groups per wave
-    int blocks = plane_slots(true) / WAVES;
-    const long fit = (iters / (8 * WAVES)) / 8 * 8;
-    if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
-    hipLaunchKernelGGL((shift_planes_wide_cu_kernel<BITS, ZT, WAVES>), dim3(blocks), dim3(WAVES * 64), kLdsBytes,
-                       st, a);
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) dst[i] = 0;
+}
+
+template <int BITS, int ZT>
+static int launch_planes_coop(const ShiftArgs &a, long iters, hipStream_t st)
+{
+    const int blocks = coop_blocks(iters);
+    // the arrival counters start at zero (a fill kernel, not a memset node: callers may capture this)
+    hipLaunchKernelGGL(zero_i32_kernel, dim3(1), dim3(256), 0, st, a.coop_counters, blocks);
+    if (a.fused)
+        hipLaunchKernelGGL((shift_planes_wide_coop_kernel<BITS, ZT, true>), dim3(blocks), dim3(kCoopWaves * 64),
+                           kCoopLdsBytes, st, a);
+    else
+        hipLaunchKernelGGL((shift_planes_wide_coop_kernel<BITS, ZT, false>), dim3(blocks), dim3(kCoopWaves * 64),
+                           kCoopLdsBytes, st, a);
     return launch_status();
 }
 
@@ -727,39 +995,41 @@ static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
     const int kSlots = plane_slots(WIDE);
     a.tiles_n = ceil_div(a.N, J);
     if (nsplit <= 0 && a.comm > 0) {
-        // balanced launch: one share of the iteration space per wave slot (3 waves per SIMD)
+        // balanced launch: one share of the iteration space per wave slot
         a.tiles_m4 = ceil_div(a.M, R * kWave);
+        const long iters = (long)a.tiles_m4 * a.tiles_n * a.comm;
+        // Workgroup-cooperative (four waves per workgroup) when a wave's quarter of a tile's reduction
+        // is long enough to carry the extra segment ends: from 64 K groups per tile.  Short reductions
+        // over many tiles (stems, 1x1 layers) keep the wave-level shares.  A fused epilogue exists only
+        // there.  The test hook's "cu" knob (0 / 4) overrides.
+        bool cooperative = WIDE && (a.comm >= 64 || a.fused);
+        if (g_tune.cu != kTuneUnset) cooperative = WIDE && (g_tune.cu > 0 || a.fused);
+        if (!a.coop_slots) cooperative = false;  // no workspace for the partial tiles
+        if (a.fused && !cooperative) return DS_EWORKSPACE;
+        if (cooperative) {
+            if constexpr (WIDE) {
+                int32_t *final_y = a.fused ? nullptr : redirect_to_scratch(a);
+                const int rc = launch_planes_coop<BITS, ZT>(a, iters, st);
+                if (rc) return rc;
+                if (final_y) return launch_transpose_strided(a.y, a.alt_ld, final_y, a.N, a.M, a.N, st);
+                return DS_OK;
+            }
+        }
         a.atomic_out = 1;
         int32_t *final_y = redirect_to_scratch(a);
         launch_fill(a, st);
         int blocks = (kSlots / 4) * (nsplit < 0 ? -nsplit : 1);
         // small layers: at least 8 K groups per wave (the workgroup count stays a multiple of 8)
-        const long iters = (long)a.tiles_m4 * a.tiles_n * a.comm;
         const long fit = (iters / 32) / 8 * 8;
         if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
-        // Workgroup-cooperative (four waves per workgroup) when a wave's quarter of a tile's reduction
-        // is long enough to carry the extra segment ends: from 64 K groups per tile.  Short reductions
-        // over many tiles (stems, 1x1 layers) keep the wave-level shares.  The test hook's "cu" knob
-        // (0 / 4 / 8) overrides (8: eight waves per workgroup).
-        bool cooperative = WIDE && a.comm >= 64;
-        int cu_waves = 4;
-        if (g_tune.cu != kTuneUnset) {
-            cooperative = WIDE && g_tune.cu > 0;
-            cu_waves = g_tune.cu == 8 ? 8 : 4;
-        }
-        if (cooperative) {
-            if constexpr (WIDE) {
-                const int rc = cu_waves == 4 ? launch_planes_cu<BITS, ZT, 4>(a, iters, st)
-                                             : launch_planes_cu<BITS, ZT, 8>(a, iters, st);
-                if (rc) return rc;
-            }
-        } else if (WIDE)
+        if (WIDE)
             hipLaunchKernelGGL((shift_planes_wide_balanced_kernel<BITS, ZT>), dim3(blocks), dim3(256), 0, st, a);
         else
             hipLaunchKernelGGL((shift_planes_balanced_kernel<BITS, ZT>), dim3(blocks), dim3(256), 0, st, a);
         if (final_y) return launch_transpose_strided(a.y, a.alt_ld, final_y, a.N, a.M, a.N, st);
         return launch_status();
     }
+    if (a.fused) return DS_EINVAL;  // the fused epilogue exists in the cooperative launch only
     a.tiles_m4 = ceil_div(ceil_div(a.M, R * kWave), 4);
     const int tiles = a.tiles_m4 * a.tiles_n;
     a.blocks_per_xcd = ceil_div(tiles, 8);
@@ -814,6 +1084,10 @@ static int dispatch_zero_top(const ShiftArgs &a, hipStream_t st)
     const int r = plane_regime(a, wide);
     int nsplit = (r >= 0 ? r : -1 - r) > 0 ? 1 : 0;
     if (g_tune.split != kTuneUnset) nsplit = g_tune.split;
+    if (a.fused) {
+        if (!wide) return DS_EINVAL;
+        nsplit = 0;
+    }
     return wide ? launch_planes<BITS, 1, true>(a, nsplit, st) : launch_planes<BITS, 1, false>(a, nsplit, st);
 }
 
@@ -834,9 +1108,14 @@ static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
         const bool wide = tiled_wide(a.N, a.K, BITS);  // decided by the shape alone, as at tiling time
         bool planes = plane_regime(a, wide) >= 0;
         if (g_tune.planes != kTuneUnset) planes = g_tune.planes > 0;
+        if (a.fused) {
+            if (!wide) return DS_EINVAL;
+            planes = true;
+        }
         if (planes) {
             int nsplit = plane_regime(a, wide) > 0 ? 1 : 0;
             if (g_tune.split != kTuneUnset) nsplit = g_tune.split;
+            if (a.fused) nsplit = 0;
             // the highest field value unused: the form without its plane
             if (a.top_unused)
                 return wide ? launch_planes<BITS, 2, true>(a, nsplit, st)
@@ -845,6 +1124,7 @@ static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
                         : launch_planes<BITS, 0, false>(a, nsplit, st);
         }
     }
+    if (a.fused) return DS_EINVAL;  // general codes and 5-bit fields have no fused form
     TileChoice c = choose_tile(a);
     if (g_tune.tile != kTuneUnset) { c.R = g_tune.tile / 100; c.J = g_tune.tile % 100; }
     if (g_tune.split != kTuneUnset) c.nsplit = g_tune.split;
@@ -915,28 +1195,57 @@ using namespace ds;
 // Conv2dShift
 // ---------------------------------------------------------------------------------------------
 
+// Workspace of the cooperative launch for a layer of M pixels, K reduction indices, N channels (0
+// when the layer cannot run there: its channel count is not a multiple of 64 or its fields are wider
+// than 4 bits).
+static size_t coop_bytes_for(size_t M, int K, int N, int bits)
+{
+    bits &= ~(DS_BITS_ZERO_TOP | DS_BITS_TOP_UNUSED);
+    if (bits < 1 || bits > 4 || !tiled_wide(N, K, bits) || M == 0 || K <= 0) return 0;
+    const long tiles = (long)((M + kCoopPix - 1) / kCoopPix) * (N / 64);
+    return coop_workspace_bytes(coop_blocks(tiles * ceil_div(K, codes_per_word(bits))));
+}
+
+static void take_coop_workspace(ShiftArgs &a, void *workspace, size_t workspace_bytes, int bits)
+{
+    const size_t need = coop_bytes_for((size_t)a.M, a.K, a.N, bits);
+    if (!need || !workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return;
+    const long tiles = (long)ceil_div(a.M, kCoopPix) * (a.N / 64);
+    a.coop_counters = (int32_t *)workspace;
+    a.coop_slots = (int32_t *)((char *)workspace + coop_counter_bytes(coop_blocks(tiles * a.comm)));
+}
+
 DS_EXPORT size_t ds_conv2d_tiled_workspace_bytes(int Nb, int C, int Hp, int Wp, int O, int FH,
                                                  int FW, int sh, int sw, int bits)
 {
-    (void)Nb; (void)C; (void)Hp; (void)Wp; (void)O; (void)FH; (void)FW; (void)sh; (void)sw; (void)bits;
-    return 0;  // the tiled entry point needs no scratch memory
+    if (Nb <= 0 || C <= 0 || O <= 0 || FH < 1 || FW < 1 || sh < 1 || sw < 1 || Hp < FH || Wp < FW) return 0;
+    const size_t M = (size_t)Nb * ((Hp - FH) / sh + 1) * ((Wp - FW) / sw + 1);
+    return coop_bytes_for(M, C * FH * FW, O, bits);
 }
 
 DS_EXPORT size_t ds_conv2d_workspace_bytes(int Nb, int C, int Hp, int Wp, int O, int FH, int FW,
                                            int sh, int sw, int bits)
 {
-    (void)Nb; (void)Hp; (void)Wp; (void)sh; (void)sw;
     if (bits < 1 || bits > 6 || C < 0 || O < 0 || FH < 1 || FW < 1) return 0;
     if ((size_t)C * FH * FW >= (1u << 24)) return 0;
-    return align_up(tiled_geom(O, C * FH * FW, bits).bytes, 256);
+    return align_up(tiled_geom(O, C * FH * FW, bits).bytes, 256) +
+           ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits);
 }
 
-DS_EXPORT int ds_conv2d_tiled_i32(const int32_t *x, const void *tiled, const int32_t *bias,
-                                  int32_t *y, int Nb, int C, int Hp, int Wp, int O, int FH, int FW,
-                                  int sh, int sw, int bits, int base, void *workspace,
-                                  size_t workspace_bytes, ds_stream_t stream)
+// Epilogue of a fused call (all fields zero: plain int32 output).
+struct FusedSpec {
+    float *out;
+    void *q;
+    const float *scale, *shift, *residual;
+    int F_in, relu, I, F, ph, pw, q_bytes, border_kept;
+};
+
+static int conv2d_tiled_any(const int32_t *x, const void *tiled, const int32_t *bias, int32_t *y,
+                            const FusedSpec *fs, int Nb, int C, int Hp, int Wp, int O, int FH, int FW,
+                            int sh, int sw, int bits, int base, void *workspace, size_t workspace_bytes,
+                            ds_stream_t stream)
 {
-    (void)workspace; (void)workspace_bytes;
+    const int bits_in = bits;
     const int top_unused = take_top_unused(bits, base);
     const int zero_top = take_zero_top(bits, base);
     int rc = check_common(bits, base);
@@ -946,7 +1255,7 @@ DS_EXPORT int ds_conv2d_tiled_i32(const int32_t *x, const void *tiled, const int
     const int OH = (Hp - FH) / sh + 1, OW = (Wp - FW) / sw + 1;
     const size_t M = (size_t)Nb * OH * OW;
     if (M == 0 || O == 0) return DS_OK;
-    if (!tiled || !y || (!x && C > 0)) return DS_EINVAL;
+    if (!tiled || (!y && !fs) || (!x && C > 0)) return DS_EINVAL;
     const size_t K = (size_t)C * FH * FW;
     const size_t x_bytes = (size_t)Nb * C * Hp * Wp * 4;
     if (x_bytes >= kMaxBytes || M * O * 4 >= kMaxBytes || K >= (1u << 24) || C >= (1 << 22) ||
@@ -973,7 +1282,73 @@ DS_EXPORT int ds_conv2d_tiled_i32(const int32_t *x, const void *tiled, const int
     a.nbase = -base;
     a.zero_top = zero_top;
     a.top_unused = top_unused;
+    take_coop_workspace(a, workspace, workspace_bytes, bits_in);
+    if (fs) {
+        if (!a.coop_slots) return coop_bytes_for(M, (int)K, O, bits_in) ? DS_EWORKSPACE : DS_EINVAL;
+        if ((size_t)Nb * O * (OH + 2 * fs->ph) * (OW + 2 * fs->pw) * (size_t)fs->q_bytes >= kMaxBytes)
+            return DS_ETOOLARGE;
+        a.fused = 1;
+        a.ep_out = fs->out;
+        a.ep_q = fs->q;
+        a.ep_scale = fs->scale;
+        a.ep_shift = fs->shift;
+        a.ep_residual = fs->residual;
+        a.ep_inv = ldexpf(1.0f, -fs->F_in);
+        a.ep_relu = fs->relu;
+        a.ep_ph = fs->q ? fs->ph : 0;
+        a.ep_pw = fs->q ? fs->pw : 0;
+        a.ep_q_bytes = fs->q_bytes;
+        a.ep_border_kept = fs->border_kept;
+        a.ep_spec = make_spec(fs->I, fs->F, DS_Q_ROUND_TO_FIXED);
+    }
     return dispatch_bits(a, bits, base != 0 || bits == 6, (hipStream_t)stream);
+}
+
+DS_EXPORT int ds_conv2d_tiled_i32(const int32_t *x, const void *tiled, const int32_t *bias,
+                                  int32_t *y, int Nb, int C, int Hp, int Wp, int O, int FH, int FW,
+                                  int sh, int sw, int bits, int base, void *workspace,
+                                  size_t workspace_bytes, ds_stream_t stream)
+{
+    return conv2d_tiled_any(x, tiled, bias, y, nullptr, Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits, base, workspace,
+                            workspace_bytes, stream);
+}
+
+DS_EXPORT int ds_conv2d_tiled_fusable(int Nb, int C, int Hp, int Wp, int O, int FH, int FW, int sh, int sw,
+                                      int bits, int base)
+{
+    const int width = bits & ~(DS_BITS_ZERO_TOP | DS_BITS_TOP_UNUSED);
+    if (base != 0 || width < 1 || width > 4) return 0;
+    if (ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits) == 0) return 0;
+    // where the dispatch would launch cooperatively anyway: long reductions on few tiles
+    ShiftArgs a{};
+    a.M = Nb * ((Hp - FH) / sh + 1) * ((Wp - FW) / sw + 1);
+    a.N = O;
+    a.K = C * FH * FW;
+    a.comm = ceil_div(a.K, codes_per_word(width));
+    return a.comm >= 64 && plane_regime(a, true) == 0;
+}
+
+DS_EXPORT int ds_conv2d_tiled_fused_i32(const int32_t *x, const void *tiled, const int32_t *bias, float *out,
+                                        void *q, const float *scale, const float *shift, const float *residual,
+                                        int Nb, int C, int Hp, int Wp, int O, int FH, int FW, int sh, int sw,
+                                        int bits, int base, int F_in, int relu, int I, int F, int ph, int pw,
+                                        int q_bytes, void *workspace, size_t workspace_bytes, ds_stream_t stream)
+{
+    if (!out && !q) return DS_EINVAL;
+    if (F_in < 0 || F_in > 31 || ph < 0 || pw < 0) return DS_EINVAL;
+    const int border_kept = (q_bytes & DS_Q_BORDER_KEPT) != 0;
+    q_bytes &= ~DS_Q_BORDER_KEPT;
+    if (q) {
+        if (q_bytes != 4 && q_bytes != 1) return DS_EINVAL;
+        if (I < 1 || F < 0 || I + F > 32) return DS_EINVAL;
+        if (q_bytes == 1 && (I < 2 || I + F > 8)) return DS_EINVAL;
+    } else {
+        I = 16; F = 16; q_bytes = 4; ph = pw = 0;
+    }
+    if (!ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits) || base != 0) return DS_EINVAL;
+    FusedSpec fs{out, q, scale, shift, residual, F_in, relu, I, F, ph, pw, q_bytes, border_kept};
+    return conv2d_tiled_any(x, tiled, bias, nullptr, &fs, Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits, base, workspace,
+                            workspace_bytes, stream);
 }
 
 DS_EXPORT int ds_conv2d_i32(const int32_t *x, const int32_t *w_ref, const int32_t *bias, int32_t *y,
@@ -992,8 +1367,9 @@ DS_EXPORT int ds_conv2d_i32(const int32_t *x, const int32_t *w_ref, const int32_
     if (!w_ref && C > 0) return DS_EINVAL;
     rc = launch_tile(w_ref, workspace, O, C, FH, FW, bits, (hipStream_t)stream);
     if (rc) return rc;
+    const size_t blob = align_up(tiled_geom(O, C * FH * FW, bits).bytes, 256);
     return ds_conv2d_tiled_i32(x, workspace, bias, y, Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits, base,
-                               nullptr, 0, stream);
+                               (char *)workspace + blob, need - blob, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1009,10 +1385,10 @@ static size_t linear_scratch_bytes(int M, int N)
 
 DS_EXPORT size_t ds_linear_tiled_workspace_bytes(int M, int K, int N, int bits)
 {
-    (void)K;
-    bits &= ~(DS_BITS_ZERO_TOP | DS_BITS_TOP_UNUSED);
-    if (bits < 1 || bits > 6 || M < 0 || N < 0) return 0;
-    return linear_scratch_bytes(M, N);
+    const int width = bits & ~(DS_BITS_ZERO_TOP | DS_BITS_TOP_UNUSED);
+    if (width < 1 || width > 6 || M < 0 || N < 0) return 0;
+    // the channel-major scratch, then the partial tiles of the cooperative launch
+    return linear_scratch_bytes(M, N) + coop_bytes_for((size_t)M, K, N, bits);
 }
 
 DS_EXPORT size_t ds_linear_workspace_bytes(int M, int K, int N, int bits)
@@ -1020,13 +1396,14 @@ DS_EXPORT size_t ds_linear_workspace_bytes(int M, int K, int N, int bits)
     if (bits < 1 || bits > 6 || M < 0 || K < 0 || N < 0) return 0;
     const size_t ldx = align_up((size_t)M, 64);
     return align_up(tiled_geom(N, K, bits).bytes, 256) + align_up(ldx * K * 4, 256) +
-           linear_scratch_bytes(M, N);
+           ds_linear_tiled_workspace_bytes(M, K, N, bits);
 }
 
 DS_EXPORT int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled, const int32_t *bias,
                                   int32_t *y, int M, int K, int N, int bits, int base,
                                   void *workspace, size_t workspace_bytes, ds_stream_t stream)
 {
+    const int bits_in = bits;
     const int top_unused = take_top_unused(bits, base);
     const int zero_top = take_zero_top(bits, base);
     int rc = check_common(bits, base);
@@ -1064,6 +1441,10 @@ DS_EXPORT int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled,
     a.nbase = -base;
     a.zero_top = zero_top;
     a.top_unused = top_unused;
+    // what the workspace holds beyond the scratch serves the cooperative launch (without it the
+    // launches that combine partial sums fall back to wave-level shares)
+    if (workspace && workspace_bytes > scratch)
+        take_coop_workspace(a, (char *)workspace + scratch, workspace_bytes - scratch, bits_in);
     return dispatch_bits(a, bits, base != 0 || bits == 6, (hipStream_t)stream);
 }
 
@@ -1134,8 +1515,8 @@ DS_EXPORT int ds_linear_i32(const int32_t *x, const int32_t *w_ref, const int32_
         rc = launch_transpose(x, xT, M, K, ldx, st);
         if (rc) return rc;
     }
-    const size_t scratch = linear_scratch_bytes(M, N);
+    const size_t rest = ds_linear_tiled_workspace_bytes(M, K, N, bits);
     return ds_linear_tiled_i32(xT, ldx, tiled, bias, y, M, K, N, bits, base,
-                               scratch ? (char *)xT + align_up((size_t)ldx * K * 4, 256) : nullptr, scratch,
+                               rest ? (char *)xT + align_up((size_t)ldx * K * 4, 256) : nullptr, rest,
                                stream);
 }

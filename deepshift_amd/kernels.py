@@ -23,7 +23,8 @@ import torch
 from . import _lib
 
 __all__ = ["linear", "conv2d", "compress_sign_and_shift", "quantize", "quantize_pad",
-           "quantize_transpose", "dequantize", "tile_weights", "linear_tiled", "conv2d_tiled"]
+           "quantize_transpose", "dequantize", "tile_weights", "linear_tiled", "conv2d_tiled",
+           "conv2d_tiled_fused", "conv2d_fusable"]
 
 
 def _pair(v):
@@ -502,6 +503,68 @@ def conv2d_tiled(x_padded, tiled, bias, O, kernel_size, stride, bits, base=0):
                   _lib.ptr(out), Nb, C, Hp, Wp, O, FH, FW, sh, sw, int(bits), int(base),
                   _lib.ptr(ws), ws_bytes, _lib.current_stream(x_padded.device))
     return out
+
+
+def conv2d_fusable(x_padded_shape, O, kernel_size, stride, bits, base=0):
+    """Whether :func:`conv2d_tiled_fused` serves this layer and is the faster choice for it (long
+    reductions on a multiple of 64 channels, fields of at most 4 bits, base 0)."""
+    Nb, C, Hp, Wp = x_padded_shape
+    FH, FW = _pair(kernel_size)
+    sh, sw = _pair(stride)
+    if Hp < FH or Wp < FW or Nb == 0:
+        return False
+    return bool(_lib.lib().ds_conv2d_tiled_fusable(Nb, C, Hp, Wp, O, FH, FW, sh, sw, int(bits), int(base)))
+
+
+def conv2d_tiled_fused(x_padded, tiled, bias, O, kernel_size, stride, bits, fraction_bits_in, scale=None,
+                       shift=None, residual=None, relu=False, emit=None, want_float=True, q_cache=None):
+    """:func:`conv2d_tiled` with what follows the layer done in the kernel's epilogue: returns
+    ``(out, q)`` = the float result ``act(y / 2**F * scale[c] + shift[c] + residual)`` (``None`` unless
+    ``want_float``) and, with ``emit = (padding, integer_bits, fraction_bits, dtype)``, the next shift
+    convolution's round-to-fixed, zero padded input.  Bit-identical to :func:`conv2d_tiled` followed by
+    :func:`requantize_affine_pad` / :func:`dequantize_affine`; the int32 sums are never stored.
+    ``q_cache``: a dict in which the padded buffer is kept between calls (zeroed once, so the kernel
+    writes the interior only); the returned ``q`` is then that buffer, overwritten by the next call."""
+    x_padded = _require_device_i32("x_padded", x_padded)
+    Nb, C, Hp, Wp = x_padded.shape
+    FH, FW = _pair(kernel_size)
+    sh, sw = _pair(stride)
+    OH, OW = (Hp - FH) // sh + 1, (Wp - FW) // sw + 1
+    dev = x_padded.device
+    for name, t in (("scale", scale), ("shift", shift)):
+        if t is not None and (t.dtype != torch.float32 or t.numel() != O or not t.is_contiguous()):
+            raise ValueError("%s must be a contiguous float32 tensor of %d elements" % (name, O))
+    if residual is not None:
+        if tuple(residual.shape) != (Nb, O, OH, OW) or residual.dtype != torch.float32:
+            raise ValueError("residual must be float32 with the shape of the output")
+        residual = residual.contiguous()
+    if emit is None and not want_float:
+        raise ValueError("nothing to produce")
+    out = torch.empty([Nb, O, OH, OW], dtype=torch.float32, device=dev) if want_float else None
+    q, ph, pw, I, Fq, qb = None, 0, 0, 16, 16, 4
+    if emit is not None:
+        padding, I, Fq, dtype = emit
+        ph, pw = _pair(padding)
+        qb = 1 if dtype == torch.int8 else 4
+        shape = (Nb, O, OH + 2 * ph, OW + 2 * pw)
+        if q_cache is not None and (ph or pw):
+            key = (shape, dtype, dev)
+            q = q_cache.get(key)
+            if q is None:
+                q_cache.clear()            # one geometry at a time: a new batch size replaces the buffer
+                q = q_cache[key] = torch.zeros(shape, dtype=dtype, device=dev)
+            qb |= _lib.DS_Q_BORDER_KEPT
+        else:
+            q = torch.empty(shape, dtype=dtype, device=dev)
+    L = _lib.lib()
+    ws_bytes = L.ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, int(bits))
+    ws = _workspace(ws_bytes, dev)
+    with _Timed("conv", Nb * OH * OW, C * FH * FW, O, dev):
+        _lib.call("ds_conv2d_tiled_fused_i32", _lib.ptr(x_padded), _lib.ptr(tiled), _lib.ptr(bias), _lib.ptr(out),
+                  _lib.ptr(q), _lib.ptr(scale), _lib.ptr(shift), _lib.ptr(residual), Nb, C, Hp, Wp, O, FH, FW,
+                  sh, sw, int(bits), 0, int(fraction_bits_in), int(bool(relu)), int(I), int(Fq), ph, pw, qb,
+                  _lib.ptr(ws), ws_bytes, _lib.current_stream(dev))
+    return out, q
 
 
 def conv2d_paired(x_padded, paired, bias, O, kernel_size, stride, field_bits, x_bound=128):

@@ -292,6 +292,11 @@ def conv_cpu_forward(module, input, shift, sign):
     return (out.float() / 2.0 ** Fb).to(input.device)
 
 
+# Switch for the fused convolution epilogue (kernels.conv2d_tiled_fused); off = always the separate
+# conversion pass, which the tests compare it with.
+_FUSE_EPILOGUE = True
+
+
 def _small_for_int8(module, input_shape, field_bits):
     """The int8 kernel works on tiles of 384 pixels x 64 channels; a layer with few of them and a short
     reduction (the 1x1 shortcuts of a ResNet-18) is served better by the int32 kernels' smaller tiles.
@@ -358,8 +363,26 @@ def conv_kernel_forward(module, input, conc_weight, scale=None, shift=None, resi
     else:
         tiled = kernels._tiled_of(conc_weight, module.out_channels, module.in_channels,
                                   module.kernel_size[0], module.kernel_size[1])
+        kbits = kernels.kernel_bits(conc_weight)
+        if pool is None and _FUSE_EPILOGUE and kernels.conv2d_fusable(
+                xq.shape, module.out_channels, module.kernel_size, module.stride, kbits, conc_weight.base):
+            # the layer's epilogue does the dequantisation, the affine / residual / ReLU and the next
+            # layer's conversion while the tile is still on chip: the int32 sums are never stored
+            want_float, spec = True, None
+            if emit is not None:
+                next_padding, next_I, next_F, want_float = emit[:4]
+                spec = (next_padding, next_I, next_F, emit[4] if len(emit) == 5 else torch.int32)
+            # the consumers' padded input lives in a buffer of this layer that is zeroed once: the kernel
+            # then writes the interior only (the next forward pass overwrites it, in stream order)
+            cache = module.__dict__.setdefault("_handoff_buffers", {})
+            f, q = kernels.conv2d_tiled_fused(xq, tiled, bias, module.out_channels, module.kernel_size,
+                                              module.stride, kbits, Fb, scale, shift, residual, relu, spec,
+                                              want_float, cache)
+            if emit is None:
+                return f
+            return (f, q) if want_float else q
         out = kernels.conv2d_tiled(xq, tiled, bias, module.out_channels, module.kernel_size,
-                                   module.stride, kernels.kernel_bits(conc_weight), conc_weight.base)
+                                   module.stride, kbits, conc_weight.base)
     emit_dtype = torch.int32
     if emit is not None and len(emit) == 5:
         emit, emit_dtype = emit[:4], emit[4]

@@ -202,7 +202,9 @@ int ds_linear_i32(const int32_t *x, const int32_t *w_ref, const int32_t *bias, i
 
 /* Same computation on pre-tiled weights and pre-transposed activations xT[K][ldx]
  * (ldx >= M, a multiple of 64 -- what ds_quantize_transpose_f32_i32 writes).  Workspace:
- * ds_linear_tiled_workspace_bytes(). */
+ * ds_linear_tiled_workspace_bytes(): a channel-major scratch of 4 * N * round_up(M, 64) bytes, which
+ * is required, followed by the partial tiles of the cooperative launch, which are optional (a
+ * workspace that holds the scratch only selects per-wave shares with atomic adds instead). */
 size_t ds_linear_tiled_workspace_bytes(int M, int K, int N, int bits);
 int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled, const int32_t *bias,
                         int32_t *y, int M, int K, int N, int bits, int base, void *workspace,
@@ -211,9 +213,9 @@ int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled, const int
 /* ds_linear_tiled_i32 for callers that cannot allocate (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc): no workspace argument; the partial-sum scratch lives in a
  * device array inside the library (ds_linear_tiled_noalloc_max_bytes() = 16 MiB per GPU, held until
- * the process ends).  The call allocates nothing.  DS_ESCRATCH when
- * ds_linear_tiled_workspace_bytes(M, K, N, bits) exceeds that size (4 * N * round_up(M, 64) bytes,
- * e.g. 2048 x 2048).  All calls on one GPU share the array: calls that overlap in time on one GPU
+ * the process ends).  The call allocates nothing.  DS_ESCRATCH when the channel-major scratch,
+ * 4 * N * round_up(M, 64) bytes, exceeds that size (e.g. beyond 2048 x 2048).  The array holds the
+ * scratch only, so launches that combine partial sums take per-wave shares here.  All calls on one GPU share the array: calls that overlap in time on one GPU
  * (different streams) race.  No counterpart in the reference. */
 size_t ds_linear_tiled_noalloc_max_bytes(void);
 int ds_linear_tiled_noalloc_i32(const int32_t *xT, int ldx, const void *tiled, const int32_t *bias,
@@ -234,7 +236,11 @@ int ds_conv2d_i32(const int32_t *x_padded, const int32_t *w_ref, const int32_t *
                   int Nb, int C, int Hp, int Wp, int O, int FH, int FW, int sh, int sw, int bits,
                   int base, void *workspace, size_t workspace_bytes, ds_stream_t stream);
 
-/* Same computation on pre-tiled weights. */
+/* Same computation on pre-tiled weights.  The workspace is optional: with
+ * ds_conv2d_tiled_workspace_bytes() bytes (256-byte aligned; 0 for layers that need none) the long
+ * reductions on few tiles -- the 3x3 layers of a ResNet -- run workgroup-cooperatively and finish the
+ * tiles that two workgroups share through partial tiles in the workspace; without it they fall back
+ * to per-wave shares combined with atomic adds on a pre-filled output (same results, slower). */
 size_t ds_conv2d_tiled_workspace_bytes(int Nb, int C, int Hp, int Wp, int O, int FH, int FW,
                                        int sh, int sw, int bits);
 int ds_conv2d_tiled_i32(const int32_t *x_padded, const void *tiled, const int32_t *bias,
@@ -262,6 +268,30 @@ int ds_cpu_linear_i32(const int32_t *x, const int8_t *shift, const int32_t *sign
 int ds_cpu_conv2d_i32(const int32_t *x_padded, const int8_t *shift, const int32_t *sign,
                       const int32_t *bias, int32_t *y, int Nb, int C, int Hp, int Wp, int O, int FH,
                       int FW, int sh, int sw, int nthreads);
+
+/* ds_conv2d_tiled_i32 with what follows the layer at inference time done in the kernel's epilogue,
+ * while the finished tile is still on chip: the int32 sums are never stored.
+ *   v = act(float(sum) / 2^F_in * scale[c] + shift[c] + residual)       (ds_dequantize_affine_i32_f32)
+ *   out [Nb][O][OH][OW] float = v                                        (or NULL)
+ *   q   [Nb][O][OH+2ph][OW+2pw] = round_to_fixed(v, I, F) * 2^F, zero padded   (or NULL)
+ * i.e. Conv2dShiftFunction's out.float() / 2**F (modules.py:161-162), the ops between two shift
+ * layers, and the next layer's round_to_fixed + cast + padding (modules.py:317,:153, kernels.py:32-36):
+ * bit-identical to ds_conv2d_tiled_i32 followed by ds_requantize_affine_pad_i32 / _i8.  q_bytes 4:
+ * q is int32; 1: int8 (2 <= I, I + F <= 8); | DS_Q_BORDER_KEPT: the caller vouches that the padding of
+ * q already holds zeros (a buffer it zeroed once and reuses), and the kernel writes the interior only.  scale, shift, residual may be NULL.  base must be 0.
+ * Needs the workspace of ds_conv2d_tiled_workspace_bytes() (DS_EWORKSPACE without it) and a layer
+ * the cooperative launch serves: O a multiple of 64, fields of at most 4 bits (DS_EINVAL otherwise);
+ * ds_conv2d_tiled_fusable() says whether the fused call is also the faster choice for a shape (long
+ * reductions; short ones lose more in the launch form than the separate pass costs).
+ * No counterpart in the reference. */
+#define DS_Q_BORDER_KEPT 0x100
+int ds_conv2d_tiled_fusable(int Nb, int C, int Hp, int Wp, int O, int FH, int FW, int sh, int sw,
+                            int bits, int base);
+int ds_conv2d_tiled_fused_i32(const int32_t *x_padded, const void *tiled, const int32_t *bias, float *out,
+                              void *q, const float *scale, const float *shift, const float *residual,
+                              int Nb, int C, int Hp, int Wp, int O, int FH, int FW, int sh, int sw,
+                              int bits, int base, int F_in, int relu, int I, int F, int ph, int pw,
+                              int q_bytes, void *workspace, size_t workspace_bytes, ds_stream_t stream);
 
 /* ---- fixed-point conversion ------------------------------------------------------------ */
 

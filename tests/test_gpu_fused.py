@@ -1,0 +1,240 @@
+"""GPU: the cooperative launch of the shift convolution -- tiles shared between workgroups finished by
+the last arrival through partial tiles in the workspace -- and its fused epilogue
+(ds_conv2d_tiled_fused_i32), through the C ABI, bit for bit against the oracle chain."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from deepshift_amd import _lib, kernels
+from oracle import shift_oracle as so
+from tests.conftest import Tune, random_activations, random_codes
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+NTHREADS = 8
+U = _lib.DS_BITS_TOP_UNUSED
+
+
+def _dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def _stream():
+    return _lib.current_stream(torch.device(DEV))
+
+
+def abi_conv_tiled(xp, blob, bias, O, FH, FW, stride, bits, with_workspace=True):
+    Nb, C, Hp, Wp = xp.shape
+    sh, sw = stride
+    OH, OW = (Hp - FH) // sh + 1, (Wp - FW) // sw + 1
+    L = _lib.lib()
+    ws_bytes = L.ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits) if with_workspace else 0
+    ws = torch.full((max(ws_bytes, 1),), 0x77, dtype=torch.uint8, device=DEV)   # stale contents on purpose
+    total, guard = Nb * O * OH * OW, 64
+    ybuf = torch.full((total + 2 * guard,), 0x5A5A5A5A, dtype=torch.int32, device=DEV)
+    y = ybuf[guard:guard + total]
+    xd = _dev(xp)
+    bd = None if bias is None else _dev(bias)
+    _lib.call("ds_conv2d_tiled_i32", _lib.ptr(xd), _lib.ptr(blob), _lib.ptr(bd), ctypes.c_void_p(y.data_ptr()),
+              Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits, 0, _lib.ptr(ws) if ws_bytes else None, ws_bytes, _stream())
+    torch.cuda.synchronize()
+    host = ybuf.cpu().numpy()
+    assert (host[:guard] == 0x5A5A5A5A).all() and (host[guard + total:] == 0x5A5A5A5A).all()
+    return host[guard:guard + total].reshape(Nb, O, OH, OW)
+
+
+def abi_conv_fused(xp, blob, bias, O, FH, FW, stride, bits, F_in, scale, shift, res, relu, want_float, emit):
+    """emit = (ph, pw, I, F, torch dtype) or None; returns (out or None, q or None), guard bands checked."""
+    Nb, C, Hp, Wp = xp.shape
+    sh, sw = stride
+    OH, OW = (Hp - FH) // sh + 1, (Wp - FW) // sw + 1
+    L = _lib.lib()
+    ws_bytes = L.ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits)
+    assert ws_bytes > 0
+    ws = torch.full((ws_bytes,), 0x77, dtype=torch.uint8, device=DEV)
+    guard = 64
+    n_out = Nb * O * OH * OW
+    obuf = torch.full((n_out + 2 * guard,), 12345.0, dtype=torch.float32, device=DEV)
+    out = obuf[guard:guard + n_out] if want_float else None
+    q = qbuf = None
+    ph = pw = 0
+    I, Fq, qb = 16, 16, 4
+    if emit is not None:
+        ph, pw, I, Fq, dtype = emit
+        n_q = Nb * O * (OH + 2 * ph) * (OW + 2 * pw)
+        qbuf = torch.full((n_q + 2 * guard,), 0x5A, dtype=dtype, device=DEV)
+        q = qbuf[guard:guard + n_q]
+        qb = 1 if dtype == torch.int8 else 4
+    xd = _dev(xp)
+    t = [None if a is None else _dev(a) for a in (bias, scale, shift, res)]
+    _lib.call("ds_conv2d_tiled_fused_i32", _lib.ptr(xd), _lib.ptr(blob), _lib.ptr(t[0]),
+              None if out is None else ctypes.c_void_p(out.data_ptr()),
+              None if q is None else ctypes.c_void_p(q.data_ptr()), _lib.ptr(t[1]), _lib.ptr(t[2]), _lib.ptr(t[3]),
+              Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits, 0, F_in, int(relu), I, Fq, ph, pw, qb, _lib.ptr(ws), ws_bytes,
+              _stream())
+    torch.cuda.synchronize()
+    oh = obuf.cpu().numpy()
+    assert (oh[:guard] == 12345.0).all() and (oh[guard + n_out:] == 12345.0).all(), "write outside out"
+    got_out = oh[guard:guard + n_out].reshape(Nb, O, OH, OW) if want_float else None
+    if not want_float:
+        assert (oh == 12345.0).all()
+    got_q = None
+    if q is not None:
+        qh = qbuf.cpu().numpy()
+        assert (qh[:guard] == 0x5A).all() and (qh[guard + n_q:] == 0x5A).all(), "write outside q"
+        got_q = qh[guard:guard + n_q].reshape(Nb, O, OH + 2 * ph, OW + 2 * pw).astype(np.int32)
+    return got_out, got_q
+
+
+# geometries: many tiles per workgroup, tiles shared by several workgroups (few pixels, long reduction),
+# ragged pixel counts, strides, 1x1 and 3x3, several channel tiles
+GEOMS = [
+    # Nb, C, Hp, Wp, O, FH, FW, stride
+    (2, 64, 30, 30, 64, 3, 3, (1, 1)),       # 1568 pixels: 13 tiles, K = 576
+    (1, 256, 9, 9, 128, 3, 3, (1, 1)),       # 49 pixels: one ragged pixel tile, every tile cut many times
+    (3, 128, 16, 15, 192, 3, 3, (2, 2)),     # strided, three channel tiles
+    (5, 384, 12, 12, 64, 1, 1, (1, 1)),      # 1x1 with a long reduction (64 K groups)
+    (2, 40, 21, 19, 64, 5, 3, (1, 2)),       # 5x3 filter, K = 600
+]
+
+
+@pytest.mark.parametrize("geom", GEOMS, ids=lambda g: "x".join(str(v) for v in g[:7]))
+@pytest.mark.parametrize("bits", [4, 2])
+def test_cooperative_launch_matches_oracle(oracle, rng, geom, bits):
+    """ds_conv2d_tiled_i32 with its workspace (cooperative launch, forced where the dispatch would pick
+    another one) and without it (per-wave shares), both flag forms, over stale workspace contents."""
+    Nb, C, Hp, Wp, O, FH, FW, stride = geom
+    xp = random_activations(rng, (Nb, C, Hp, Wp))
+    top = 2 ** bits - 2
+    s, sign = random_codes(rng, (O, C, FH, FW), max_s=top)
+    bias = rng.integers(-2 ** 20, 2 ** 20, size=O).astype(np.int32)
+    want = oracle.conv2d(xp, -s, sign, bias, stride, nthreads=NTHREADS)
+    blob = kernels.tile_weights(_dev(so.np_pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)).reshape(-1),
+                                O, C, FH, FW, bits, 0)
+    with Tune(planes=1, split=0, cu=4):
+        for b in (bits, bits | U):
+            np.testing.assert_array_equal(abi_conv_tiled(xp, blob, bias, O, FH, FW, stride, b), want)
+        np.testing.assert_array_equal(abi_conv_tiled(xp, blob, None, O, FH, FW, stride, bits),
+                                      oracle.conv2d(xp, -s, sign, None, stride, nthreads=NTHREADS))
+        np.testing.assert_array_equal(abi_conv_tiled(xp, blob, bias, O, FH, FW, stride, bits, False), want)
+
+
+@pytest.mark.parametrize("geom", GEOMS, ids=lambda g: "x".join(str(v) for v in g[:7]))
+def test_fused_epilogue_matches_oracle_chain(oracle, rng, geom):
+    """Float and fixed-point outputs of the fused call against oracle.conv2d -> np_dequantize_affine ->
+    np_requantize, for every combination of what may follow the layer."""
+    Nb, C, Hp, Wp, O, FH, FW, stride = geom
+    OH, OW = (Hp - FH) // stride[0] + 1, (Wp - FW) // stride[1] + 1
+    xp = rng.integers(-2 ** 17, 2 ** 19, size=(Nb, C, Hp, Wp)).astype(np.int32)
+    s, sign = random_codes(rng, (O, C, FH, FW), max_s=14)
+    bias = rng.integers(-2 ** 16, 2 ** 16, size=O).astype(np.int32)
+    y = oracle.conv2d(xp, -s, sign, bias, stride, nthreads=NTHREADS)
+    blob = kernels.tile_weights(_dev(so.np_pack_words(s.reshape(O, -1), sign.reshape(O, -1), 4)).reshape(-1),
+                                O, C, FH, FW, 4, 0)
+    scale = ((rng.random(O) + 0.5) * 2.0 ** -6).astype(np.float32)
+    shift = rng.standard_normal(O).astype(np.float32)
+    res = (rng.standard_normal((Nb, O, OH, OW)) * 2).astype(np.float32)
+    cases = [
+        (scale, shift, res, True, True, (1, 1, 16, 16, torch.int32)),     # block end: float + q
+        (scale, shift, None, True, False, (1, 1, 16, 16, torch.int32)),   # between two convolutions: q only
+        (scale, None, None, False, True, None),                           # float only
+        (None, None, None, False, True, (0, 0, 16, 16, torch.int32)),     # plain dequantisation, no padding
+        (scale, shift, res, True, True, (2, 3, 12, 4, torch.int32)),      # wider padding, another format
+        (scale, shift, None, True, False, (1, 1, 3, 5, torch.int8)),      # int8 consumer
+    ]
+    for sc, sh, r, relu, want_float, emit in cases:
+        v = so.np_dequantize_affine(y, 16, sc, sh, r, relu)
+        out, q = abi_conv_fused(xp, blob, bias, O, FH, FW, stride, 4 | U, 16, sc, sh, r, relu, want_float, emit)
+        if want_float:
+            np.testing.assert_array_equal(out, v)
+        if emit is not None:
+            np.testing.assert_array_equal(q, so.np_requantize(v, emit[2], emit[3], emit[:2]))
+
+
+def test_border_kept_writes_the_interior_only(oracle, rng):
+    """q_bytes | DS_Q_BORDER_KEPT: the caller's buffer keeps its padding (zeroed once by the caller), the
+    kernel overwrites the interior; with the flag off the kernel writes the padding itself."""
+    Nb, C, Hp, Wp, O, FH, FW, stride = GEOMS[0]
+    OH, OW = Hp - 2, Wp - 2
+    xp = rng.integers(-2 ** 17, 2 ** 19, size=(Nb, C, Hp, Wp)).astype(np.int32)
+    s, sign = random_codes(rng, (O, C, FH, FW), max_s=14)
+    y = oracle.conv2d(xp, -s, sign, None, stride, nthreads=NTHREADS)
+    want = so.np_requantize(so.np_dequantize_affine(y, 16, None, None, None, True), 16, 16, (1, 2))
+    blob = kernels.tile_weights(_dev(so.np_pack_words(s.reshape(O, -1), sign.reshape(O, -1), 4)).reshape(-1),
+                                O, C, FH, FW, 4, 0)
+    L = _lib.lib()
+    ws_bytes = L.ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, 1, 1, 4)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=DEV)
+    xd = _dev(xp)
+    for kept in (True, False):
+        q = torch.full((Nb, O, OH + 2, OW + 4), 7, dtype=torch.int32, device=DEV)
+        _lib.call("ds_conv2d_tiled_fused_i32", _lib.ptr(xd), _lib.ptr(blob), None, None, _lib.ptr(q), None, None,
+                  None, Nb, C, Hp, Wp, O, FH, FW, 1, 1, 4, 0, 16, 1, 16, 16, 1, 2,
+                  4 | (_lib.DS_Q_BORDER_KEPT if kept else 0), _lib.ptr(ws), ws_bytes, _stream())
+        got = q.cpu().numpy()
+        np.testing.assert_array_equal(got[:, :, 1:-1, 2:-2], want[:, :, 1:-1, 2:-2])
+        border = np.ones_like(got, bool)
+        border[:, :, 1:-1, 2:-2] = False
+        assert (got[border] == (7 if kept else 0)).all()
+
+
+def test_fused_entry_point_refuses_what_it_cannot_do(rng):
+    L = _lib.lib()
+    one = ctypes.c_void_p(256)
+    args = lambda O, bits, base, ws: (one, one, None, one, None, None, None, None, 2, 64, 30, 30, O, 3, 3, 1, 1,
+                                      bits, base, 16, 0, 16, 16, 0, 0, 4, one if ws else None, 1 << 30 if ws else 0,
+                                      None)
+    assert L.ds_conv2d_tiled_fused_i32(*args(48, 4, 0, True)) == -1     # not a multiple of 64 channels
+    assert L.ds_conv2d_tiled_fused_i32(*args(64, 5, 0, True)) == -1     # 5-bit fields
+    assert L.ds_conv2d_tiled_fused_i32(*args(64, 4, -1, True)) == -1    # left shifts
+    assert L.ds_conv2d_tiled_fused_i32(*args(64, 4, 0, False)) == -4    # no workspace
+    assert L.ds_conv2d_tiled_fusable(64, 64, 58, 58, 64, 3, 3, 1, 1, 4 | U, 0) == 1
+    assert L.ds_conv2d_tiled_fusable(64, 64, 58, 58, 64, 3, 3, 1, 1, 5, 0) == 0
+    assert L.ds_conv2d_tiled_fusable(64, 64, 58, 58, 48, 3, 3, 1, 1, 4, 0) == 0
+    assert L.ds_conv2d_tiled_fusable(64, 64, 56, 56, 128, 1, 1, 2, 2, 4, 0) == 0   # short reduction
+
+
+def test_fused_module_path_equals_the_separate_passes():
+    """conv_kernel_forward with the fused epilogue against the same call with it switched off (int32 sums,
+    then the conversion pass): every output bit-identical."""
+    from deepshift_amd import modules
+    torch.manual_seed(3)
+    conv = modules.Conv2dShift(64, 128, 3, stride=1, padding=1, use_kernel=True).to(DEV)
+    conv.sign.data = torch.where(conv.sign.data >= 0, torch.ones_like(conv.sign), -torch.ones_like(conv.sign))
+    x = torch.randn(16, 64, 40, 40, device=DEV)
+    scale = torch.rand(128, device=DEV) + 0.5
+    shift = torch.randn(128, device=DEV)
+    res = torch.randn(16, 128, 40, 40, device=DEV)
+    cw = conv.packed_weights()
+    assert kernels.conv2d_fusable((16, 64, 42, 42), 128, (3, 3), (1, 1), kernels.kernel_bits(cw), 0)
+    results = {}
+
+    def keep(r):  # the hand-off buffer is reused by the next call: copy what a call returned
+        return tuple(t.clone() for t in (r if isinstance(r, tuple) else (r,)))
+
+    for fused in (True, False):
+        modules._FUSE_EPILOGUE = fused
+        try:
+            with torch.no_grad():
+                results[fused] = [
+                    keep(modules.conv_kernel_forward(conv, x, cw)),
+                    keep(modules.conv_kernel_forward(conv, x, cw, scale, shift, res, True)),
+                    keep(modules.conv_kernel_forward(conv, x, cw, scale, shift, res, True,
+                                                     emit=((1, 1), 16, 16, True))),
+                    keep(modules.conv_kernel_forward(conv, x, cw, scale, shift, None, True,
+                                                     emit=((1, 1), 16, 16, False))),
+                    # a second geometry replaces the cached buffer, a return to the first re-zeroes one
+                    keep(modules.conv_kernel_forward(conv, x[:8], cw, scale, shift, None, True,
+                                                     emit=((1, 1), 16, 16, False))),
+                    keep(modules.conv_kernel_forward(conv, x, cw, scale, shift, None, True,
+                                                     emit=((1, 1), 16, 16, False))),
+                ]
+        finally:
+            modules._FUSE_EPILOGUE = True
+    for a, b in zip(results[True], results[False]):
+        a = a if isinstance(a, tuple) else (a,)
+        b = b if isinstance(b, tuple) else (b,)
+        for t, u in zip(a, b):
+            assert torch.equal(t, u)

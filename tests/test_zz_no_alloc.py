@@ -73,4 +73,5 @@ def test_noalloc_two_instruction_kernel_and_limit(oracle, rng):
     # 4 * N * round_up(M, 64) beyond the built-in scratch: rejected before anything is launched
     assert L.ds_linear_tiled_noalloc_i32(one, 4096, one, None, one, 4096, 64, 2048, 4, 0, None) == -6
     assert b"scratch" in L.ds_status_string(-6)
-    assert L.ds_linear_tiled_workspace_bytes(2048, 64, 2048, 4) == limit
+    assert 4 * 2048 * 2048 == limit      # the channel-major scratch of a 2048 x 2048 output just fits
+    assert L.ds_linear_tiled_noalloc_i32(one, 2048, one, None, one, 2048, 0, 2048, 9, 0, None) == -2   # bits
