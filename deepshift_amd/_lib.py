@@ -20,6 +20,16 @@ _c_i64 = ctypes.c_int64
 _ptr = ctypes.c_void_p
 _size = ctypes.c_size_t
 
+class FusedConv(ctypes.Structure):
+    """``ds_fused_conv`` of the header: one convolution of a two-convolution launch."""
+    _fields_ = [("tiled", _ptr), ("bias", _ptr), ("out", _ptr), ("q", _ptr), ("scale", _ptr), ("shift", _ptr),
+                ("residual", _ptr)] + [(name, _c_int) for name in
+                                       ("O", "FH", "FW", "crop_h", "crop_w", "bits", "relu", "I", "F", "ph", "pw",
+                                        "q_bytes")]
+
+
+_fcp = ctypes.POINTER(FusedConv)
+
 # name -> (restype, argtypes); mirrors include/deepshift_hip.h one to one
 SIGNATURES = {
     "ds_version": (_c_int, []),
@@ -54,6 +64,8 @@ SIGNATURES = {
     "ds_cpu_conv2d_i32": (_c_int, [_ptr] * 5 + [_c_int] * 10),
     "ds_conv2d_tiled_fusable": (_c_int, [_c_int] * 11),
     "ds_conv2d_tiled_fused_i32": (_c_int, [_ptr] * 8 + [_c_int] * 18 + [_ptr, _size, _ptr]),
+    "ds_conv2d_tiled_fused_pair_workspace_bytes": (_size, [_c_int] * 6 + [_fcp, _fcp]),
+    "ds_conv2d_tiled_fused_pair_i32": (_c_int, [_ptr] + [_c_int] * 7 + [_fcp, _fcp, _ptr, _size, _ptr]),
     "ds_quantize_f32_i32": (_c_int, [_ptr, _ptr, _c_i64, _c_int, _c_int, _c_int, _ptr]),
     "ds_quantize_pad_f32_i32": (_c_int, [_ptr, _ptr] + [_c_int] * 9 + [_ptr]),
     "ds_quantize_transpose_f32_i32": (_c_int, [_ptr, _ptr] + [_c_int] * 6 + [_ptr]),

@@ -768,8 +768,8 @@ __device__ __forceinline__ void write_tile(lds_tail *t, lds_i32 *buf, int ntile,
 // workgroup's slot, its arrival counted, and whichever workgroup arrives last gathers the slots of all
 // contributors and writes the tile.  Ends with the buffer cleared and a barrier.
 template <bool FUSED>
-__device__ __attribute__((noinline)) void coop_finish_tile(lds_tail *t, lds_i32 *buf, lds_i32 *flag, int w, int tile,
-                                                           int g0, int len, int ntile, int m0)
+__device__ __attribute__((noinline)) void coop_finish_tile(lds_tail *t, lds_i32 *buf, lds_i32 *flag, int w,
+                                                           long tile_start, int g0, int len, int ntile, int m0)
 {
     constexpr int THREADS = kCoopWaves * 64, PER = kCoopTileElems / THREADS;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
@@ -787,8 +787,9 @@ __device__ __attribute__((noinline)) void coop_finish_tile(lds_tail *t, lds_i32 
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         const long G = t->G, total = t->total;
-        const int first = coop_owner((long)tile * comm, G, total);
-        const int last = coop_owner((long)(tile + 1) * comm - 1, G, total);
+        // tile_start: the tile's first iteration in the launch's (tile, K group) space
+        const int first = coop_owner(tile_start, G, total);
+        const int last = coop_owner(tile_start + comm - 1, G, total);
         if (threadIdx.x == 0)
             *flag = __hip_atomic_fetch_add(t->counters + first, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
                     last - first;
@@ -813,12 +814,30 @@ __device__ __attribute__((noinline)) void coop_finish_tile(lds_tail *t, lds_i32 
     __syncthreads();
 }
 
-template <int BITS, int ZT, bool FUSED>
+__device__ __forceinline__ void fill_tail(TileTail &tail, const ShiftArgs &p, long G, long total)
+{
+    tail.negcnt = p.negcnt; tail.bias = p.bias; tail.y = p.y;
+    tail.slots = p.coop_slots; tail.counters = p.coop_counters;
+    tail.out = p.ep_out; tail.q = p.ep_q;
+    tail.scale = p.ep_scale; tail.shift = p.ep_shift; tail.residual = p.ep_residual;
+    tail.y_img_stride = p.y_img_stride; tail.y_pix_stride = p.y_pix_stride; tail.y_ch_stride = p.y_ch_stride;
+    tail.G = G; tail.total = total;
+    tail.M = p.M; tail.N = p.N; tail.comm = p.comm; tail.pix_per_img = p.pix_per_img; tail.OW = p.OW;
+    tail.inv = p.ep_inv; tail.relu = p.ep_relu; tail.ph = p.ep_ph; tail.pw = p.ep_pw;
+    tail.q_bytes = p.ep_q_bytes; tail.border_kept = p.ep_border_kept; tail.spec = p.ep_spec;
+}
+
+// PAIR: the launch serves two convolutions over the same input -- a residual block's first 3x3 stride-s
+// convolution and its 1x1 stride-s shortcut, whose pixels are the centre taps of the former -- as one
+// (tile, K group) space: the tiles of p, then those of p2 (p.pair_total = the iterations of p2, which
+// shares the workspace, the counters and the slots).  The shortcut alone is a launch of a few
+// microseconds of work that cannot fill the machine; here its tiles ride along in the shares.
+template <int BITS, int ZT, bool FUSED, bool PAIR>
 __global__ __launch_bounds__(kCoopWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void shift_planes_wide_coop_kernel(const ShiftArgs p)
+void shift_planes_wide_coop_kernel(const ShiftArgs p, const ShiftArgs p2)
 {
     extern __shared__ int32_t tile_sums[];  // [64 channels][128 pixels]
-    __shared__ TileTail tail;
+    __shared__ TileTail tail[PAIR ? 2 : 1];
     __shared__ int32_t last_arrival;
     constexpr int THREADS = kCoopWaves * 64;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -826,34 +845,41 @@ void shift_planes_wide_coop_kernel(const ShiftArgs p)
     const long G = gridDim.x;
     // an XCD (workgroup ids congruent modulo 8) takes a contiguous range of shares
     const int w = (gridDim.x & 7) ? bid : (bid & 7) * (int)(gridDim.x >> 3) + (bid >> 3);
-    const long total = (long)p.tiles_m4 * p.tiles_n * p.comm;
-    int it = (int)(w * total / G);
-    const int it_end = (int)((w + 1) * total / G);
+    // The iteration space: pixel tiles outermost; inside one, the channel tiles of p (each p.comm K groups),
+    // then -- PAIR -- those of p2.  The tiles of the small second convolution are thereby spread evenly
+    // over the workgroups (each tile costs a fixed tail besides its K groups), and the two convolutions
+    // read a pixel range's activations at about the same time.
+    const int span1 = p.tiles_n * p.comm;
+    const int span = span1 + (PAIR ? p2.tiles_n * p2.comm : 0);
+    const long total = (long)p.tiles_m4 * span;
+    long it = w * total / G;
+    const long it_end = (w + 1) * total / G;
     if (threadIdx.x == 0) {
-        tail.negcnt = p.negcnt; tail.bias = p.bias; tail.y = p.y;
-        tail.slots = p.coop_slots; tail.counters = p.coop_counters;
-        tail.out = p.ep_out; tail.q = p.ep_q;
-        tail.scale = p.ep_scale; tail.shift = p.ep_shift; tail.residual = p.ep_residual;
-        tail.y_img_stride = p.y_img_stride; tail.y_pix_stride = p.y_pix_stride; tail.y_ch_stride = p.y_ch_stride;
-        tail.G = G; tail.total = total;
-        tail.M = p.M; tail.N = p.N; tail.comm = p.comm; tail.pix_per_img = p.pix_per_img; tail.OW = p.OW;
-        tail.inv = p.ep_inv; tail.relu = p.ep_relu; tail.ph = p.ep_ph; tail.pw = p.ep_pw;
-        tail.q_bytes = p.ep_q_bytes; tail.border_kept = p.ep_border_kept; tail.spec = p.ep_spec;
+        fill_tail(tail[0], p, G, total);
+        if (PAIR) fill_tail(tail[1], p2, G, total);
     }
     for (int i = threadIdx.x; i < kCoopTileElems; i += THREADS) tile_sums[i] = 0;
     __syncthreads();
     while (it < it_end) {
-        const int tile = it / p.comm;
-        const int g0 = it - tile * p.comm;
-        int g1 = g0 + (it_end - it);
-        if (g1 > p.comm) g1 = p.comm;
-        const int ntile = tile % p.tiles_n, m0 = (tile / p.tiles_n) * kCoopPix;
-        const int len = g1 - g0;
+        const int mtile = (int)(it / span);
+        const int within = (int)(it - (long)mtile * span);
+        const bool second = PAIR && within >= span1;
+        const int comm = second ? p2.comm : p.comm;
+        const int ntile = (second ? within - span1 : within) / comm;
+        const long tile_start = (long)mtile * span + (second ? span1 : 0) + (long)ntile * comm;
+        const int g0 = (int)(it - tile_start);
+        long g1 = g0 + (it_end - it);
+        if (g1 > comm) g1 = comm;
+        const int m0 = mtile * kCoopPix;
+        const int len = (int)g1 - g0;
         const int wb = g0 + wave * len / kCoopWaves, we = g0 + (wave + 1) * len / kCoopWaves;
-        if (wb < we) planes_segment<BITS, ZT, true, true>(p, ntile, m0, wb, we, true, tile_sums);
+        if (wb < we) {
+            if (second) planes_segment<BITS, ZT, true, true>(p2, ntile, m0, wb, we, true, tile_sums);
+            else planes_segment<BITS, ZT, true, true>(p, ntile, m0, wb, we, true, tile_sums);
+        }
         __syncthreads();
-        coop_finish_tile<FUSED>((lds_tail *)&tail, (lds_i32 *)tile_sums, (lds_i32 *)&last_arrival, w, tile, g0, len,
-                                ntile, m0);
+        coop_finish_tile<FUSED>((lds_tail *)&tail[second ? 1 : 0], (lds_i32 *)tile_sums, (lds_i32 *)&last_arrival, w,
+                                tile_start, g0, len, ntile, m0);
         it += len;
     }
 }
@@ -864,17 +890,22 @@ __global__ void zero_i32_kernel(int32_t *dst, int n)
 }
 
 template <int BITS, int ZT>
-static int launch_planes_coop(const ShiftArgs &a, long iters, hipStream_t st)
+static int launch_planes_coop(const ShiftArgs &a, long iters, hipStream_t st, const ShiftArgs *second = nullptr)
 {
     const int blocks = coop_blocks(iters);
     // the arrival counters start at zero (a fill kernel, not a memset node: callers may capture this)
     hipLaunchKernelGGL(zero_i32_kernel, dim3(1), dim3(256), 0, st, a.coop_counters, blocks);
-    if (a.fused)
-        hipLaunchKernelGGL((shift_planes_wide_coop_kernel<BITS, ZT, true>), dim3(blocks), dim3(kCoopWaves * 64),
-                           kCoopLdsBytes, st, a);
+    const dim3 grid(blocks), block(kCoopWaves * 64);
+    if (second) {
+        if constexpr (ZT != 1)
+            hipLaunchKernelGGL((shift_planes_wide_coop_kernel<BITS, ZT, true, true>), grid, block, kCoopLdsBytes, st, a,
+                               *second);
+        else
+            return DS_EINVAL;
+    } else if (a.fused)
+        hipLaunchKernelGGL((shift_planes_wide_coop_kernel<BITS, ZT, true, false>), grid, block, kCoopLdsBytes, st, a, a);
     else
-        hipLaunchKernelGGL((shift_planes_wide_coop_kernel<BITS, ZT, false>), dim3(blocks), dim3(kCoopWaves * 64),
-                           kCoopLdsBytes, st, a);
+        hipLaunchKernelGGL((shift_planes_wide_coop_kernel<BITS, ZT, false, false>), grid, block, kCoopLdsBytes, st, a, a);
     return launch_status();
 }
 
@@ -1349,6 +1380,132 @@ DS_EXPORT int ds_conv2d_tiled_fused_i32(const int32_t *x, const void *tiled, con
     FusedSpec fs{out, q, scale, shift, residual, F_in, relu, I, F, ph, pw, q_bytes, border_kept};
     return conv2d_tiled_any(x, tiled, bias, nullptr, &fs, Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits, base, workspace,
                             workspace_bytes, stream);
+}
+
+// ---- two convolutions over one input in one launch ------------------------------------------------
+
+static int fused_conv_shape(const ds_fused_conv *f, int Hp, int Wp, int sh, int sw, int *OH, int *OW)
+{
+    if (!f || f->O < 1 || f->FH < 1 || f->FW < 1 || f->crop_h < 0 || f->crop_w < 0) return DS_EINVAL;
+    const int He = Hp - 2 * f->crop_h, We = Wp - 2 * f->crop_w;
+    if (He < f->FH || We < f->FW) return DS_EINVAL;
+    *OH = (He - f->FH) / sh + 1;
+    *OW = (We - f->FW) / sw + 1;
+    return DS_OK;
+}
+
+static int pair_check(int Nb, int C, int Hp, int Wp, int sh, int sw, const ds_fused_conv *a, const ds_fused_conv *b,
+                      int *OH, int *OW)
+{
+    if (Nb < 1 || C < 1 || sh < 1 || sw < 1 || !a || !b) return DS_EINVAL;
+    int OHb = 0, OWb = 0;
+    int rc = fused_conv_shape(a, Hp, Wp, sh, sw, OH, OW);
+    if (rc) return rc;
+    rc = fused_conv_shape(b, Hp, Wp, sh, sw, &OHb, &OWb);
+    if (rc) return rc;
+    if (OHb != *OH || OWb != *OW) return DS_EINVAL;        // the two outputs cover the same pixels
+    const int wa = a->bits & 0xff, wb = b->bits & 0xff;
+    if (wa < 1 || wa > 4 || wa != wb) return DS_EBITS;     // one kernel form serves both
+    if ((a->bits | b->bits) & DS_BITS_ZERO_TOP) return DS_EBITS;
+    if ((a->bits & DS_BITS_TOP_UNUSED) != (b->bits & DS_BITS_TOP_UNUSED)) return DS_EBITS;
+    if (a->O % 64 || b->O % 64) return DS_EINVAL;
+    return DS_OK;
+}
+
+static long pair_iters(int Nb, int C, int OH, int OW, const ds_fused_conv *a, const ds_fused_conv *b)
+{
+    const long tiles_m = ((long)Nb * OH * OW + kCoopPix - 1) / kCoopPix;
+    const int num = codes_per_word(a->bits & 0xff);
+    return tiles_m * (a->O / 64) * ceil_div(C * a->FH * a->FW, num) +
+           tiles_m * (b->O / 64) * ceil_div(C * b->FH * b->FW, num);
+}
+
+DS_EXPORT size_t ds_conv2d_tiled_fused_pair_workspace_bytes(int Nb, int C, int Hp, int Wp, int sh, int sw,
+                                                            const ds_fused_conv *a, const ds_fused_conv *b)
+{
+    int OH = 0, OW = 0;
+    if (pair_check(Nb, C, Hp, Wp, sh, sw, a, b, &OH, &OW)) return 0;
+    return coop_workspace_bytes(coop_blocks(pair_iters(Nb, C, OH, OW, a, b)));
+}
+
+static int pair_args(ShiftArgs &s, const int32_t *x, const ds_fused_conv *f, int Nb, int C, int Hp, int Wp, int sh,
+                     int sw, int OH, int OW, int F_in)
+{
+    const int width = f->bits & 0xff;
+    const size_t K = (size_t)C * f->FH * f->FW, M = (size_t)Nb * OH * OW;
+    const size_t x_bytes = (size_t)Nb * C * Hp * Wp * 4, skip = ((size_t)f->crop_h * Wp + f->crop_w) * 4;
+    if (!f->tiled || (!f->out && !f->q)) return DS_EINVAL;
+    if (x_bytes >= kMaxBytes || M * f->O * 4 >= kMaxBytes || K >= (1u << 24) || C >= (1 << 22) || f->FH > 31 ||
+        f->FW > 31)
+        return DS_ETOOLARGE;
+    int I = f->I, Fq = f->F, qb = f->q_bytes & ~DS_Q_BORDER_KEPT, ph = f->ph, pw = f->pw;
+    if (f->q) {
+        if ((qb != 4 && qb != 1) || I < 1 || Fq < 0 || I + Fq > 32 || ph < 0 || pw < 0) return DS_EINVAL;
+        if (qb == 1 && (I < 2 || I + Fq > 8)) return DS_EINVAL;
+        if ((size_t)Nb * f->O * (OH + 2 * ph) * (OW + 2 * pw) * (size_t)qb >= kMaxBytes) return DS_ETOOLARGE;
+    } else {
+        I = 16; Fq = 16; qb = 4; ph = pw = 0;
+    }
+    const TiledGeom g = tiled_geom(f->O, (int)K, width);
+    s = ShiftArgs{};
+    s.x = (const int32_t *)((const char *)x + skip);   // the window starts crop rows / columns in
+    s.x_bytes = (uint32_t)(x_bytes - skip);
+    s.wt = (const uint32_t *)f->tiled;
+    s.wt16 = tiled_words16(f->tiled, g);
+    s.negcnt = tiled_negcount(f->tiled, g);
+    s.bias = f->bias;
+    s.M = (int)M; s.N = f->O; s.K = (int)K; s.comm = g.comm;
+    s.pix_per_img = OH * OW; s.OW = OW;
+    s.x_img_stride = C * Hp * Wp; s.x_row_stride = sh * Wp; s.x_col_stride = sw;
+    s.y_img_stride = f->O * OH * OW; s.y_pix_stride = 1; s.y_ch_stride = OH * OW;
+    s.ktab = tiled_ktab(f->tiled, g);
+    s.x_plane = Hp * Wp; s.x_row = Wp;
+    s.FH = f->FH; s.FW = f->FW;
+    s.top_unused = (f->bits & DS_BITS_TOP_UNUSED) != 0;
+    s.tiles_m4 = ceil_div((int)M, kCoopPix);
+    s.tiles_n = f->O / 64;
+    s.fused = 1;
+    s.ep_out = f->out; s.ep_q = f->q;
+    s.ep_scale = f->scale; s.ep_shift = f->shift; s.ep_residual = f->residual;
+    s.ep_inv = ldexpf(1.0f, -F_in);
+    s.ep_relu = f->relu;
+    s.ep_ph = ph; s.ep_pw = pw; s.ep_q_bytes = qb;
+    s.ep_border_kept = (f->q_bytes & DS_Q_BORDER_KEPT) != 0;
+    s.ep_spec = make_spec(I, Fq, DS_Q_ROUND_TO_FIXED);
+    return DS_OK;
+}
+
+template <int BITS>
+static int launch_pair(const ShiftArgs &a, const ShiftArgs &b, long iters, hipStream_t st)
+{
+    return a.top_unused ? launch_planes_coop<BITS, 2>(a, iters, st, &b) : launch_planes_coop<BITS, 0>(a, iters, st, &b);
+}
+
+DS_EXPORT int ds_conv2d_tiled_fused_pair_i32(const int32_t *x, int Nb, int C, int Hp, int Wp, int sh, int sw, int F_in,
+                                             const ds_fused_conv *a, const ds_fused_conv *b, void *workspace,
+                                             size_t workspace_bytes, ds_stream_t stream)
+{
+    int OH = 0, OW = 0;
+    int rc = pair_check(Nb, C, Hp, Wp, sh, sw, a, b, &OH, &OW);
+    if (rc) return rc;
+    if (!x || F_in < 0 || F_in > 31) return DS_EINVAL;
+    const long iters = pair_iters(Nb, C, OH, OW, a, b);
+    const int blocks = coop_blocks(iters);
+    if (!workspace || workspace_bytes < coop_workspace_bytes(blocks) || ((uintptr_t)workspace & 255)) return DS_EWORKSPACE;
+    ShiftArgs sa, sb;
+    rc = pair_args(sa, x, a, Nb, C, Hp, Wp, sh, sw, OH, OW, F_in);
+    if (rc) return rc;
+    rc = pair_args(sb, x, b, Nb, C, Hp, Wp, sh, sw, OH, OW, F_in);
+    if (rc) return rc;
+    sa.coop_counters = sb.coop_counters = (int32_t *)workspace;
+    sa.coop_slots = sb.coop_slots = (int32_t *)((char *)workspace + coop_counter_bytes(blocks));
+    hipStream_t st = (hipStream_t)stream;
+    switch (a->bits & 0xff) {
+    case 1: return launch_pair<1>(sa, sb, iters, st);
+    case 2: return launch_pair<2>(sa, sb, iters, st);
+    case 3: return launch_pair<3>(sa, sb, iters, st);
+    default: return launch_pair<4>(sa, sb, iters, st);
+    }
 }
 
 DS_EXPORT int ds_conv2d_i32(const int32_t *x, const int32_t *w_ref, const int32_t *bias, int32_t *y,

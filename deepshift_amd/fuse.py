@@ -76,6 +76,64 @@ class FusedConv2dShift(nn.Module):
                                            self.input_nonneg)
 
 
+class FusedShortcutPair(nn.Module):
+    """A residual block's first convolution and its 1 x 1 shortcut, both fused convolutions over the same
+    tensor with the same stride, run as ONE launch (``kernels.conv2d_tiled_fused_pair``): the shortcut
+    reads the centre taps of the padded fixed-point input that was made for the first convolution, so
+    it needs neither a conversion pass of its own nor the float form of the block's input.  Returns
+    ``(result of the first, result of the shortcut)``, each what the module by itself would return."""
+
+    def __init__(self, first, shortcut):
+        super().__init__()
+        self.first = first
+        self.shortcut = shortcut
+
+    @staticmethod
+    def _spec(fused, conc_weight, crop, residual):
+        conv = fused.conv
+        spec = dict(tiled=kernels._tiled_of(conc_weight, conv.out_channels, conv.in_channels, *conv.kernel_size),
+                    bias=conv._fixed_bias.get(conv.bias, conv.act_integer_bits, conv.act_fraction_bits,
+                                              round_to_fixed=True),
+                    O=conv.out_channels, kernel_size=conv.kernel_size, crop=crop,
+                    bits=kernels.kernel_bits(conc_weight), scale=fused.scale, shift=fused.shift,
+                    residual=residual, relu=fused.relu, want_float=True,
+                    q_cache=conv.__dict__.setdefault("_handoff_buffers", {}))
+        if fused.emit is not None:
+            padding, I, Fq, want_float = fused.emit[:4]
+            spec["emit"] = (padding, I, Fq, fused.emit[4] if len(fused.emit) == 5 else torch.int32)
+            spec["want_float"] = want_float
+        return spec
+
+    @staticmethod
+    def _result(fused, out, q):
+        if fused.emit is None:
+            return out
+        return (out, q) if fused.emit[3] else q
+
+    def forward(self, xq, residual_first=None, residual_shortcut=None):
+        a, b = self.first, self.shortcut
+        cwa, cwb = a.conv.packed_weights(), b.conv.packed_weights()
+        if not _pairable_weights(cwa, cwb) or xq.dtype != torch.int32:
+            raise RuntimeError("the weights of a paired shortcut changed in a way that needs another kernel; "
+                               "fuse the model again")
+        (oa, qa), (ob, qb) = kernels.conv2d_tiled_fused_pair(
+            xq, a.conv.stride, a.conv.act_fraction_bits,
+            self._spec(a, cwa, (0, 0), residual_first), self._spec(b, cwb, tuple(a.conv.padding), residual_shortcut))
+        return self._result(a, oa, qa), self._result(b, ob, qb)
+
+
+def _pairable_weights(cwa, cwb):
+    """Both layers run the same form of the shift-plane kernel: fields of the same width (at most 4
+    bits), no base, no ternary blob, the same "top value unused" flag."""
+    if cwa is None or cwb is None or cwa.base != 0 or cwb.base != 0:
+        return False
+    ka, kb = kernels.kernel_bits(cwa), kernels.kernel_bits(cwb)
+    from . import _lib
+    if (ka | kb) & _lib.DS_BITS_ZERO_TOP:
+        return False
+    return ka == kb and (ka & 0xff) <= 4
+
+
 class _Tracer(fx.Tracer):
     def is_leaf_module(self, m, qualname):
         return isinstance(m, _SHIFT_LEAVES) or super().is_leaf_module(m, qualname)
@@ -186,6 +244,7 @@ def fuse_conv_epilogues(model, handoff=True):
             gm.graph.erase_node(old)
     if handoff:
         _hand_off_fixed_point(gm)
+        _pair_shortcuts(gm)
     gm.graph.lint()
     gm.recompile()
     return gm
@@ -243,3 +302,85 @@ def _hand_off_fixed_point(gm):
             user.args = (q,) + tuple(user.args[1:])
             fused(user).prequantized = True
             fused(user).input_nonneg = bool(producer.relu)
+
+
+def _pair_shortcuts(gm):
+    """Third pass: where a fused k x k convolution A reads the fixed-point tensor its producer P made for
+    it, and a fused 1 x 1 convolution B with the same stride and no padding reads P's float result -- the
+    two branches of a down-sampling residual block -- run A and B as one launch on P's fixed-point tensor
+    (B reads the centre taps: the padded tensor cropped by A's padding).  If nothing else reads P's
+    float result it is no longer written."""
+    mods = dict(gm.named_modules())
+
+    def fused(n):
+        m = mods.get(n.target) if n.op == "call_module" else None
+        return m if isinstance(m, FusedConv2dShift) else None
+
+    count = 0
+    for node in list(gm.graph.nodes):
+        A = fused(node)
+        if A is None or not A.prequantized or A.pool is not None:
+            continue
+        q_node = node.args[0]
+        if q_node.op == "call_function" and q_node.target is operator.getitem and q_node.args[1] == 1:
+            producer, f_nodes = q_node.args[0], [u for u in q_node.args[0].users
+                                                 if u.op == "call_function" and u.target is operator.getitem
+                                                 and u.args[1] == 0]
+        else:
+            continue   # the producer writes no float result: nobody reads the block input as float
+        ca = A.conv
+        for f_node in f_nodes:
+            for user in list(f_node.users):
+                B = fused(user)
+                if B is None or user.args[0] is not f_node or B.prequantized or B.pool is not None:
+                    continue
+                cb = B.conv
+                if (tuple(cb.kernel_size) != (1, 1) or tuple(cb.padding) != (0, 0) or cb.padding_mode != 'zeros'
+                        or tuple(cb.stride) != tuple(ca.stride) or cb.in_channels != ca.in_channels
+                        or ca.padding_mode != 'zeros'
+                        or (cb.act_integer_bits, cb.act_fraction_bits) != (ca.act_integer_bits, ca.act_fraction_bits)
+                        or ca.out_channels % 64 or cb.out_channels % 64
+                        or tuple(ca.kernel_size) != (2 * ca.padding[0] + 1, 2 * ca.padding[1] + 1)):
+                    continue
+                param = ca.shift if hasattr(ca, "shift") else ca.weight
+                if not param.is_cuda or not _pairable_weights(ca.packed_weights(), cb.packed_weights()):
+                    continue
+                if kernels.paired_fields(ca.packed_weights(), ca.out_channels, ca.act_integer_bits,
+                                         ca.act_fraction_bits):
+                    continue   # int8 activations: another kernel
+                # the pair runs where the earlier of the two stands (the users of both come later), so
+                # every operand must exist by then
+                order = {n: i for i, n in enumerate(gm.graph.nodes)}
+                earlier = node if order[node] < order[user] else user
+                operands = [q_node] + [a for a in list(node.args[1:]) + list(user.args[1:]) if isinstance(a, fx.Node)]
+                if any(order[a] > order[earlier] for a in operands):
+                    continue
+                name = "pair_%d" % count
+                count += 1
+                gm.add_module(name, FusedShortcutPair(A, B))
+                res_a = node.args[1] if len(node.args) > 1 else None
+                res_b = user.args[1] if len(user.args) > 1 else None
+                with gm.graph.inserting_before(earlier):
+                    both = gm.graph.call_module(name, (q_node, res_a, res_b))
+                with gm.graph.inserting_after(both):
+                    out_b = gm.graph.call_function(operator.getitem, (both, 1))
+                    out_a = gm.graph.call_function(operator.getitem, (both, 0))
+                node.replace_all_uses_with(out_a)
+                user.replace_all_uses_with(out_b)
+                gm.graph.erase_node(node)
+                gm.graph.erase_node(user)
+                # P's float result: still written only if something else reads it
+                if not f_node.users:
+                    P = fused(producer)
+                    gm.graph.erase_node(f_node)
+                    if P is not None and P.emit is not None and not any(
+                            u.op == "call_function" and u.target is operator.getitem and u.args[1] == 0
+                            for u in producer.users):
+                        P.emit = P.emit[:3] + (False,) + P.emit[4:]
+                        q_node.replace_all_uses_with(producer)
+                        gm.graph.erase_node(q_node)
+                break
+            else:
+                continue
+            break
+    return count

@@ -18,6 +18,8 @@ Differences from the reference, all deliberate:
 * weights that have to stay zero contribute exactly 0 (see ``utils.compress_bits``).
 """
 
+import ctypes
+
 import torch
 
 from . import _lib
@@ -565,6 +567,84 @@ def conv2d_tiled_fused(x_padded, tiled, bias, O, kernel_size, stride, bits, frac
                   sh, sw, int(bits), 0, int(fraction_bits_in), int(bool(relu)), int(I), int(Fq), ph, pw, qb,
                   _lib.ptr(ws), ws_bytes, _lib.current_stream(dev))
     return out, q
+
+
+def _fused_conv_struct(x_shape, stride, spec, keep):
+    """One ``ds_fused_conv`` of a two-convolution launch from ``spec`` (see :func:`conv2d_tiled_fused_pair`);
+    allocates its outputs.  ``keep`` collects the tensors that must stay alive until the launch is issued."""
+    Nb, C, Hp, Wp = x_shape
+    sh, sw = stride
+    O = int(spec["O"])
+    FH, FW = _pair(spec["kernel_size"])
+    ch, cw_ = _pair(spec.get("crop", 0))
+    OH, OW = (Hp - 2 * ch - FH) // sh + 1, (Wp - 2 * cw_ - FW) // sw + 1
+    dev = spec["tiled"].device
+    want_float = spec.get("want_float", True)
+    emit = spec.get("emit")
+    if emit is None and not want_float:
+        raise ValueError("nothing to produce")
+    out = torch.empty([Nb, O, OH, OW], dtype=torch.float32, device=dev) if want_float else None
+    q, ph, pw, I, Fq, qb = None, 0, 0, 16, 16, 4
+    if emit is not None:
+        padding, I, Fq, dtype = emit
+        ph, pw = _pair(padding)
+        qb = 1 if dtype == torch.int8 else 4
+        shape = (Nb, O, OH + 2 * ph, OW + 2 * pw)
+        cache = spec.get("q_cache")
+        if cache is not None and (ph or pw):
+            key = (shape, dtype, dev)
+            q = cache.get(key)
+            if q is None:
+                cache.clear()
+                q = cache[key] = torch.zeros(shape, dtype=dtype, device=dev)
+            qb |= _lib.DS_Q_BORDER_KEPT
+        else:
+            q = torch.empty(shape, dtype=dtype, device=dev)
+    residual = spec.get("residual")
+    if residual is not None:
+        if tuple(residual.shape) != (Nb, O, OH, OW) or residual.dtype != torch.float32:
+            raise ValueError("residual must be float32 with the shape of the output")
+        residual = residual.contiguous()
+    for name in ("scale", "shift"):
+        t = spec.get(name)
+        if t is not None and (t.dtype != torch.float32 or t.numel() != O or not t.is_contiguous()):
+            raise ValueError("%s must be a contiguous float32 tensor of %d elements" % (name, O))
+    keep.extend([residual, out, q])
+
+    def p(t):
+        return None if t is None else t.data_ptr()
+
+    c = _lib.FusedConv(p(spec["tiled"]), p(spec.get("bias")), p(out), p(q), p(spec.get("scale")),
+                       p(spec.get("shift")), p(residual), O, FH, FW, ch, cw_, int(spec["bits"]),
+                       int(bool(spec.get("relu", False))), int(I), int(Fq), ph, pw, qb)
+    return c, out, q, (Nb * OH * OW, C * FH * FW, O)
+
+
+def conv2d_tiled_fused_pair(x_padded, stride, fraction_bits_in, first, second):
+    """Two fused shift convolutions over one padded int32 input in ONE launch (a residual block's first
+    k x k convolution and its 1 x 1 shortcut).  ``first`` / ``second``: dicts with ``tiled``, ``bias``, ``O``,
+    ``kernel_size``, ``bits``, ``crop`` (rows / columns of the padded tensor outside the convolution's
+    own window: 0 for the convolution the padding was made for, its padding for the shortcut) and what
+    :func:`conv2d_tiled_fused` takes: ``scale``, ``shift``, ``residual``, ``relu``, ``emit``,
+    ``want_float``, ``q_cache``.  Returns ``[(out, q), (out, q)]``."""
+    x_padded = _require_device_i32("x_padded", x_padded)
+    Nb, C, Hp, Wp = x_padded.shape
+    sh, sw = _pair(stride)
+    keep = []
+    ca, out_a, q_a, dims_a = _fused_conv_struct(x_padded.shape, (sh, sw), first, keep)
+    cb, out_b, q_b, dims_b = _fused_conv_struct(x_padded.shape, (sh, sw), second, keep)
+    L = _lib.lib()
+    ws_bytes = L.ds_conv2d_tiled_fused_pair_workspace_bytes(Nb, C, Hp, Wp, sh, sw, ca, cb)
+    if not ws_bytes:
+        raise ValueError("these two convolutions cannot share a launch")
+    ws = _workspace(ws_bytes, x_padded.device)
+    dev = x_padded.device
+    # one launch: the timing sink sees it as the larger convolution, with the pairs of both
+    with _Timed("conv", dims_a[0], dims_a[1] + dims_b[1] * dims_b[2] // dims_a[2], dims_a[2], dev):
+        _lib.call("ds_conv2d_tiled_fused_pair_i32", _lib.ptr(x_padded), Nb, C, Hp, Wp, sh, sw,
+                  int(fraction_bits_in), ctypes.byref(ca), ctypes.byref(cb), _lib.ptr(ws), ws_bytes,
+                  _lib.current_stream(dev))
+    return [(out_a, q_a), (out_b, q_b)]
 
 
 def conv2d_paired(x_padded, paired, bias, O, kernel_size, stride, field_bits, x_bound=128):

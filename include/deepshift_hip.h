@@ -293,6 +293,29 @@ int ds_conv2d_tiled_fused_i32(const int32_t *x_padded, const void *tiled, const 
                               int bits, int base, int F_in, int relu, int I, int F, int ph, int pw,
                               int q_bytes, void *workspace, size_t workspace_bytes, ds_stream_t stream);
 
+/* Two convolutions over ONE padded input in one launch: a residual block's first k x k stride-s
+ * convolution and its 1 x 1 stride-s shortcut (whose pixels are the centre taps of the former's
+ * windows), each with its own weights, epilogue and outputs as in ds_conv2d_tiled_fused_i32.  A
+ * convolution reads the window that starts crop_h rows and crop_w columns inside the padded tensor
+ * (0 for the k x k convolution that the padding was made for, its padding for the 1 x 1 shortcut):
+ * OH = (Hp - 2 * crop_h - FH) / sh + 1, and both must give the same OH x OW.  Both need O % 64 == 0,
+ * the same field width (<= 4 bits) and the same DS_BITS_TOP_UNUSED flag in `bits`, base 0.  The
+ * shortcut alone is too small a launch to fill the machine; here its tiles share the launch of the
+ * large convolution.  No counterpart in the reference (modules.py:312-340 runs every layer by itself). */
+typedef struct ds_fused_conv {
+    const void *tiled;      /* ds_tile_weights_i32 blob of an [O][C][FH][FW] layer */
+    const int32_t *bias;    /* or NULL */
+    float *out;             /* [Nb][O][OH][OW] or NULL */
+    void *q;                /* [Nb][O][OH + 2 ph][OW + 2 pw] or NULL */
+    const float *scale, *shift, *residual; /* or NULL */
+    int O, FH, FW, crop_h, crop_w, bits, relu, I, F, ph, pw, q_bytes;
+} ds_fused_conv;
+size_t ds_conv2d_tiled_fused_pair_workspace_bytes(int Nb, int C, int Hp, int Wp, int sh, int sw,
+                                                  const ds_fused_conv *a, const ds_fused_conv *b);
+int ds_conv2d_tiled_fused_pair_i32(const int32_t *x_padded, int Nb, int C, int Hp, int Wp, int sh, int sw,
+                                   int F_in, const ds_fused_conv *a, const ds_fused_conv *b, void *workspace,
+                                   size_t workspace_bytes, ds_stream_t stream);
+
 /* ---- fixed-point conversion ------------------------------------------------------------ */
 
 /* Replaces utils.round_to_fixed (utils.py:7-21) + the (x * 2**F).int() cast (modules.py:25,153)

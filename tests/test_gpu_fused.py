@@ -238,3 +238,83 @@ def test_fused_module_path_equals_the_separate_passes():
         b = b if isinstance(b, tuple) else (b,)
         for t, u in zip(a, b):
             assert torch.equal(t, u)
+
+
+@pytest.mark.parametrize("geom", [
+    # Nb, C, H, W, O_first, k, O_shortcut, stride
+    (4, 64, 28, 28, 128, 3, 128, 2),     # a ResNet-18 down-sampling block in small
+    (2, 128, 15, 13, 64, 3, 192, 2),     # odd sizes, different channel counts
+    (3, 64, 12, 12, 64, 5, 64, 1),       # 5 x 5 first convolution (padding 2), stride 1
+], ids=lambda g: "x".join(map(str, g)))
+def test_pair_launch_matches_oracle_chain(oracle, rng, geom):
+    """ds_conv2d_tiled_fused_pair_i32: a k x k convolution and a 1 x 1 shortcut over one padded input in one
+    launch, each output against oracle.conv2d -> np_dequantize_affine -> np_requantize of the layer alone."""
+    Nb, C, H, W, Oa, k, Ob, st = geom
+    p = (k - 1) // 2
+    x = rng.integers(-2 ** 17, 2 ** 19, size=(Nb, C, H, W)).astype(np.int32)
+    xp = np.pad(x, ((0, 0), (0, 0), (p, p), (p, p)))
+    sa, ga = random_codes(rng, (Oa, C, k, k), max_s=14)
+    sb, gb = random_codes(rng, (Ob, C, 1, 1), max_s=14)
+    ba = rng.integers(-2 ** 16, 2 ** 16, size=Oa).astype(np.int32)
+    bb = rng.integers(-2 ** 16, 2 ** 16, size=Ob).astype(np.int32)
+    ya = oracle.conv2d(xp, -sa, ga, ba, (st, st), nthreads=NTHREADS)
+    yb = oracle.conv2d(x, -sb, gb, bb, (st, st), nthreads=NTHREADS)      # the shortcut sees the unpadded input
+    assert ya.shape[2:] == yb.shape[2:]
+    scale_a = ((rng.random(Oa) + 0.5) * 2.0 ** -6).astype(np.float32)
+    shift_a = rng.standard_normal(Oa).astype(np.float32)
+    scale_b = ((rng.random(Ob) + 0.5) * 2.0 ** -4).astype(np.float32)
+    shift_b = rng.standard_normal(Ob).astype(np.float32)
+    res_b = rng.standard_normal(yb.shape).astype(np.float32)
+    blob_a = kernels.tile_weights(_dev(so.np_pack_words(sa.reshape(Oa, -1), ga.reshape(Oa, -1), 4)).reshape(-1),
+                                  Oa, C, k, k, 4, 0)
+    blob_b = kernels.tile_weights(_dev(so.np_pack_words(sb.reshape(Ob, -1), gb.reshape(Ob, -1), 4)).reshape(-1),
+                                  Ob, C, 1, 1, 4, 0)
+    first = dict(tiled=blob_a, bias=_dev(ba), O=Oa, kernel_size=(k, k), crop=(0, 0), bits=4 | U,
+                 scale=_dev(scale_a), shift=_dev(shift_a), relu=True, emit=((1, 1), 16, 16, torch.int32),
+                 want_float=False)
+    second = dict(tiled=blob_b, bias=_dev(bb), O=Ob, kernel_size=(1, 1), crop=(p, p), bits=4 | U,
+                  scale=_dev(scale_b), shift=_dev(shift_b), residual=_dev(res_b), relu=False, want_float=True)
+    (oa, qa), (ob, qb) = kernels.conv2d_tiled_fused_pair(_dev(xp), (st, st), 16, first, second)
+    va = so.np_dequantize_affine(ya, 16, scale_a, shift_a, None, True)
+    vb = so.np_dequantize_affine(yb, 16, scale_b, shift_b, res_b, False)
+    assert oa is None and qb is None
+    np.testing.assert_array_equal(qa.cpu().numpy(), so.np_requantize(va, 16, 16, (1, 1)))
+    np.testing.assert_array_equal(ob.cpu().numpy(), vb)
+    # the other way round: float from the first, fixed point (int8 format) from the shortcut
+    first.update(want_float=True, emit=None)
+    second.update(want_float=False, emit=((0, 0), 3, 5, torch.int8), residual=None)
+    (oa, qa), (ob, qb) = kernels.conv2d_tiled_fused_pair(_dev(xp), (st, st), 16, first, second)
+    np.testing.assert_array_equal(oa.cpu().numpy(), va)
+    vb2 = so.np_dequantize_affine(yb, 16, scale_b, shift_b, None, False)
+    np.testing.assert_array_equal(qb.cpu().numpy().astype(np.int32), so.np_requantize(vb2, 3, 5, (0, 0)))
+    # what cannot share a launch is refused
+    bad = dict(second, bits=3)
+    with pytest.raises(ValueError):
+        kernels.conv2d_tiled_fused_pair(_dev(xp), (st, st), 16, first, bad)
+    with pytest.raises(ValueError):
+        kernels.conv2d_tiled_fused_pair(_dev(xp), (st, st), 16, first, dict(second, crop=(0, 0)))
+
+
+def test_fused_resnet18_pairs_its_shortcuts():
+    """fuse_conv_epilogues on a ResNet-18: the three down-sampling blocks run their first convolution and
+    their shortcut as one launch, and the network output equals the pipeline without the in-kernel
+    epilogue (int32 sums + separate conversion passes, separate shortcut launches) bit for bit."""
+    from deepshift_amd import convert, fuse, modules, workloads
+    g = torch.Generator().manual_seed(7)
+    model = workloads.randomize_batchnorm(workloads.ResNet18(), g).eval()
+    model, _ = convert.convert_to_shift(model, 1000, 'PS', convert_weights=True, use_kernel=True)
+    model = model.to(DEV)
+    convert.round_shift_weights(model)
+    x = torch.randn(4, 3, 96, 96, generator=g).to(DEV)
+    with torch.no_grad():
+        fused = fuse.fuse_conv_epilogues(model)
+        pairs = [m for m in fused.modules() if isinstance(m, fuse.FusedShortcutPair)]
+        assert len(pairs) == 3
+        got = fused(x).clone()
+        modules._FUSE_EPILOGUE = False
+        try:
+            plain = fuse.fuse_conv_epilogues(model, handoff=False)
+            want = plain(x)
+        finally:
+            modules._FUSE_EPILOGUE = True
+    assert torch.equal(got, want)
