@@ -357,30 +357,59 @@ def config1(device, with_cpu=True, reps=50):
 
 
 def pmc_target(device):
-    """Counter targets for `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`: a plain copy of 64 MiB (reads
-    64 MiB, writes 64 MiB: the scale of the counters) and the dominant shift-kernel launch."""
+    """Counter targets for `rocprofv3 --pmc`: a plain copy of 64 MiB (reads 64 MiB, writes 64 MiB: the scale
+    of the byte counters), then one launch each of the kernels of the headline step, three times over:
+      * the dominant kernel on the layer1 shape (3x3, 64 -> 64, batch 64, 56x56), with the fused epilogue
+        (shift_planes_wide_coop_kernel<4, 2, true, false>) and with the plain int32 output (<.., false, false>);
+      * the stem (7x7 stride 2, 3 -> 64, 224x224): shift_planes_wide_balanced_kernel + its pre-fill;
+      * a down-sampling block's first 3x3 stride-2 convolution with its 1x1 shortcut as one launch
+        (<4, 2, true, true>), 64 -> 128 channels at 56x56;
+      * the int8 kernel (shift_pairs_cu_kernel) on a ResNet-50 3x3 layer, 128 -> 128 at 28x28, batch 128,
+        weight_bits 3."""
     from deepshift_amd import _lib, kernels, utils
     g = torch.Generator().manual_seed(0)
     n = 16 * 1024 * 1024
     src = torch.randint(0, 2 ** 20, (n,), generator=g, dtype=torch.int32).to(device)
     dst = torch.empty_like(src)
-    x = torch.randint(0, 2 ** 20, (BATCH, 64, 58, 58), generator=g, dtype=torch.int32).to(device)
-    shift = torch.randint(-14, 1, (64, 64, 3, 3), generator=g).float()  # the range of weight_bits 5
-    sign = (torch.randint(0, 2, (64, 64, 3, 3), generator=g) * 2 - 1).float()
-    cw = utils.compress_bits(shift, sign)
-    tiled = kernels._tiled_of(cw, 64, 64, 3, 3)
+
+    def layer(O, C, F, lo=-14):
+        shift = torch.randint(lo, 1, (O, C, F, F), generator=g).float()  # the range the weight_bits clamp leaves
+        sign = (torch.randint(0, 2, (O, C, F, F), generator=g) * 2 - 1).float()
+        cw = utils.compress_bits(shift, sign)
+        return cw, kernels._tiled_of(cw, O, C, F, F), kernels.kernel_bits(cw)
+
+    x1 = torch.randint(0, 2 ** 20, (BATCH, 64, 58, 58), generator=g, dtype=torch.int32).to(device)
+    cw1, tiled1, kb1 = layer(64, 64, 3)
     scale = torch.rand(64, generator=g).to(device) * 2.0 ** -6
     offs = torch.randn(64, generator=g).to(device)
-    cache = {}
+    xs = torch.randint(-2 ** 17, 2 ** 17, (BATCH, 3, 230, 230), generator=g, dtype=torch.int32).to(device)
+    cws, tileds, kbs = layer(64, 3, 7)
+    cwa, tileda, kba = layer(128, 64, 3)
+    cwb, tiledb, kbb = layer(128, 64, 1)
+    scale2 = torch.rand(128, generator=g).to(device) * 2.0 ** -6
+    offs2 = torch.randn(128, generator=g).to(device)
+    x8 = torch.randint(0, 97, (128, 128, 30, 30), generator=g, dtype=torch.int32).to(torch.int8).to(device)
+    cw8, _, _ = layer(128, 128, 3, lo=-2)
+    fields = kernels.paired_fields(cw8, 128, 3, 5)
+    blob8 = kernels._paired_of(cw8, fields, 128, 128, 3, 3)
+    cache, cache2 = {}, {}
     torch.cuda.synchronize()
     for _ in range(3):
         _lib.call("ds_copy_i32", _lib.ptr(src), _lib.ptr(dst), n, _lib.current_stream(device))
-        # the launch as the fused pipeline issues it between two convolutions of a block: BatchNorm affine,
-        # ReLU and the next layer's padded fixed-point input from the kernel's epilogue ...
-        kernels.conv2d_tiled_fused(x, tiled, None, 64, (3, 3), (1, 1), kernels.kernel_bits(cw), 16, scale, offs,
-                                   None, True, ((1, 1), 16, 16, torch.int32), False, cache)
+        # as the fused pipeline issues it between two convolutions of a block: BatchNorm affine, ReLU and
+        # the next layer's padded fixed-point input from the kernel's epilogue ...
+        kernels.conv2d_tiled_fused(x1, tiled1, None, 64, (3, 3), (1, 1), kb1, 16, scale, offs, None, True,
+                                   ((1, 1), 16, 16, torch.int32), False, cache)
         # ... and with the plain int32 output of ds_conv2d_tiled_i32
-        kernels.conv2d_tiled(x, tiled, None, 64, (3, 3), (1, 1), kernels.kernel_bits(cw), cw.base)
+        kernels.conv2d_tiled(x1, tiled1, None, 64, (3, 3), (1, 1), kb1, cw1.base)
+        kernels.conv2d_tiled(xs, tileds, None, 64, (7, 7), (2, 2), kbs, cws.base)
+        kernels.conv2d_tiled_fused_pair(
+            x1, (2, 2), 16,
+            dict(tiled=tileda, O=128, kernel_size=(3, 3), crop=(0, 0), bits=kba, scale=scale2, shift=offs2, relu=True,
+                 emit=((1, 1), 16, 16, torch.int32), want_float=False, q_cache=cache2),
+            dict(tiled=tiledb, O=128, kernel_size=(1, 1), crop=(1, 1), bits=kbb, scale=scale2, shift=offs2,
+                 want_float=True))
+        kernels.conv2d_paired(x8, blob8, None, 128, (3, 3), (1, 1), fields[1], 96)
     torch.cuda.synchronize()
 
 

@@ -163,14 +163,19 @@ __global__ void tile16_kernel(const int32_t *__restrict__ w_ref, uint32_t *__res
     const int t = (int)(rest / rows);
     const int g = row / half, h = row - g * half;
     const int n = t * kTileWords + j;
-    uint32_t out = 0x10001000u;
-    if (n < N) {
-        for (int c = 0; c < 2; ++c) {
-            const int k = g * num + 2 * h + c;
-            if (k >= K) continue;
+    // Codes past K (and padding channels) carry the HIGHEST field value, positive: the kernel forms that
+    // hold that value's plane at zero run the padded last K group like any other; the other forms never
+    // execute these codes (they finish the partial group from the packed words).
+    const uint32_t pad = 0x1000u | ((1u << bits) - 1u);
+    uint32_t out = 0;
+    for (int c = 0; c < 2; ++c) {
+        const int k = g * num + 2 * h + c;
+        uint32_t code = pad;
+        if (n < N && k < K) {
             const OwnCode o = own_code(ref_code(w_ref, n, k, in_comm, in_bits), bits, zero_top);
-            out |= (o.field | (o.neg << 8)) << (16 * c);
+            code = 0x1000u | o.field | (o.neg << 8);
         }
+        out |= code << (16 * c);
     }
     w16[idx] = out;
 }
@@ -188,14 +193,16 @@ __global__ void tile16_wide_kernel(const int32_t *__restrict__ w_ref, uint32_t *
     const long rows = (long)comm * num;  // one row per reduction slot, K rounded up to whole groups
     const int k = (int)(rest % rows);
     const int t = (int)(rest / rows);
-    uint32_t out = 0x10001000u;
-    if (k < K) {
-        for (int c = 0; c < 2; ++c) {
-            const int n = t * 64 + 32 * c + j;
-            if (n >= N) continue;
+    const uint32_t pad = 0x1000u | ((1u << bits) - 1u);  // see tile16_kernel
+    uint32_t out = 0;
+    for (int c = 0; c < 2; ++c) {
+        const int n = t * 64 + 32 * c + j;
+        uint32_t code = pad;
+        if (k < K && n < N) {
             const OwnCode o = own_code(ref_code(w_ref, n, k, in_comm, in_bits), bits, zero_top);
-            out |= (o.field | (o.neg << 8)) << (16 * c);
+            code = 0x1000u | o.field | (o.neg << 8);
         }
+        out |= code << (16 * c);
     }
     w16[idx] = out;
 }

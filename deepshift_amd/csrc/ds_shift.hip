@@ -26,6 +26,7 @@
 #include "ds_epilogue.h"
 #include <cstdio>
 #include <atomic>
+#include <chrono>
 #include <cstdlib>
 #include <type_traits>
 
@@ -62,7 +63,8 @@ struct ShiftArgs {
     int top_unused;                       // no code carries the highest field value (the caller vouches)
     // Workgroup-cooperative launch: per-workgroup arrival counters and partial-tile slots in the
     // caller's workspace (nullptr: no room, the launch falls back to wave-level shares).
-    int32_t *coop_counters;
+    unsigned long long *coop_counters;
+    unsigned long long coop_token;        // this launch's tag in the counters (never 0)
     int32_t *coop_slots;
     // Fused epilogue of the cooperative launch (convolutions only): instead of the int32 sums the
     // finished tile goes through act(sum / 2^F * scale[c] + shift[c] + residual) and is stored as float
@@ -74,6 +76,7 @@ struct ShiftArgs {
     float ep_inv;                         // 2^-F of the sums
     int ep_relu, ep_ph, ep_pw, ep_q_bytes;
     int ep_border_kept;                   // the padding of q already holds zeros: write the interior only
+    int whole_tile_shares;                // cooperative launch: shares end on tile boundaries, tiles go one per wave
     QuantSpec ep_spec;
 };
 
@@ -98,6 +101,8 @@ __device__ __forceinline__ int32_t xor_add(int32_t t, int32_t mask, int32_t acc)
     asm("v_xad_u32 %0, %1, %2, %3" : "=v"(out) : "v"(t), "s"(mask), "v"(acc));
     return out;
 }
+
+__device__ __forceinline__ int32_t uniform(int32_t v) { return __builtin_amdgcn_readfirstlane(v); }
 
 __device__ __forceinline__ int32_t *at_lane(int32_t *uniform_base, uint32_t lane_bytes)
 {
@@ -380,35 +385,41 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
         yoff[r] = 4u * (uint32_t)(img * p.y_img_stride + rem * p.y_pix_stride);
     }
 
-    const int full_groups = p.K / NUM;
+    // The form that holds the highest field value's plane at zero (ZT 1) runs the padded last group in
+    // the main loop too: the blob codes reduction indices past K with that value.
+    const int full_groups = ZT == 1 ? p.comm : p.K / NUM;
     const int g_full_end = g_end < full_groups ? g_end : full_groups;
     acc_vec a[2 * R];
 #pragma unroll
     for (int i = 0; i < 2 * R; ++i) a[i] = (acc_vec)(0);
     if (g_begin < g_full_end) {
+        // Every scalar operand of the loop goes through v_readfirstlane: all of them are wave-uniform,
+        // but where this code runs inside a function of its own the compiler no longer knows that.
         const uint64_t xaddr = (uint64_t)p.x;
         v4i rsrc;
-        rsrc.x = (int32_t)(uint32_t)xaddr;
-        rsrc.y = (int32_t)(uint32_t)(xaddr >> 32);  // stride 0: raw buffer
-        rsrc.z = (int32_t)p.x_bytes;
+        rsrc.x = uniform((int32_t)(uint32_t)xaddr);
+        rsrc.y = uniform((int32_t)(uint32_t)(xaddr >> 32));  // stride 0: raw buffer
+        rsrc.z = uniform((int32_t)p.x_bytes);
         rsrc.w = 0x00020000;
         PlaneWalk w;
-        const int k0 = g_begin * NUM, ff = p.FH * p.FW;
+        const int FH = uniform(p.FH), FW = uniform(p.FW), x_plane = uniform(p.x_plane), x_row = uniform(p.x_row);
+        const int k0 = uniform(g_begin) * NUM, ff = FH * FW;
         const int ic = k0 / ff, rem = k0 - ic * ff;
-        w.fh = rem / p.FW;
-        w.fw = rem - w.fh * p.FW;
+        w.fh = uniform(rem / FW);
+        w.fw = uniform(rem - w.fh * FW);
         // byte offsets; row_step is the whole step of an fw wrap (the element step included)
-        w.koff = 4 * (ic * p.x_plane + w.fh * p.x_row + w.fw);
-        w.FW = p.FW;
-        w.FH = p.FH;
-        w.row_step = 4 * (p.x_row - p.FW + 1);
-        w.plane_step = 4 * (p.x_plane - p.FH * p.x_row);
-        w.koff_max = 4 * ((p.K / ff - 1) * p.x_plane + (p.FH - 1) * p.x_row + p.FW - 1);
+        w.koff = uniform(4 * (ic * x_plane + w.fh * x_row + w.fw));
+        w.FW = FW;
+        w.FH = FH;
+        w.row_step = 4 * (x_row - FW + 1);
+        w.plane_step = 4 * (x_plane - FH * x_row);
+        w.koff_max = uniform(4 * ((uniform(p.K) / ff - 1) * x_plane + (FH - 1) * x_row + FW - 1));
         // rows of 16-bit codes per K group: NUM/2 (two slots per row) or NUM (one slot, 64 channels)
         constexpr int ROWS = WIDE ? NUM : NUM / 2;
-        planes_main_loop<BITS, ZT>(a, xoff, rsrc,
-                                   p.wt16 + ((size_t)ntile * p.comm + g_begin) * ROWS * kTileWords,
-                                   __builtin_amdgcn_readfirstlane(g_full_end - g_begin), w);
+        const uint64_t waddr = (uint64_t)(p.wt16 + ((size_t)ntile * p.comm + g_begin) * ROWS * kTileWords);
+        const uint64_t wuni = (uint64_t)(uint32_t)uniform((int32_t)(uint32_t)waddr) |
+                              ((uint64_t)(uint32_t)uniform((int32_t)(uint32_t)(waddr >> 32)) << 32);
+        planes_main_loop<BITS, ZT>(a, xoff, rsrc, (const uint32_t *)wuni, uniform(g_full_end - g_begin), w);
     }
 
     int32_t acc[R][J];
@@ -448,6 +459,13 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
         return;
     }
     const int n0 = ntile * J;
+    // bias + negative-code count of the tile's channels: lane j fetches channel n0 + j, so the tile pays
+    // the memory latency once instead of once per channel (the stores below take them with v_readlane)
+    int32_t add_l = 0;
+    if (!atomic) {
+        const int n = n0 + (lane & (J - 1));
+        if (n < p.N) add_l = p.negcnt[n] + (p.bias ? p.bias[n] : 0);
+    }
 #pragma unroll
     for (int j = 0; j < J; ++j) {
         const int n = n0 + j;
@@ -458,7 +476,7 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
             for (int r = 0; r < R; ++r)
                 if (live[r]) atomicAdd(at_lane(yc, yoff[r]), acc[r][j]);
         } else {
-            const int32_t add = p.negcnt[n] + (p.bias ? p.bias[n] : 0);
+            const int32_t add = __builtin_amdgcn_readlane(add_l, j);
 #pragma unroll
             for (int r = 0; r < R; ++r)
                 if (live[r]) *at_lane(yc, yoff[r]) = acc[r][j] + add;
@@ -556,7 +574,7 @@ constexpr int kCoopPix = kPlaneRowsWide * kWave;       // pixels of a tile
 constexpr int kCoopTileElems = 64 * kCoopPix;          // int32 sums of a tile
 constexpr int kCoopLdsBytes = kCoopTileElems * 4;
 
-static size_t coop_counter_bytes(int blocks) { return align_up((size_t)blocks * 4, 256); }
+static size_t coop_counter_bytes(int blocks) { return align_up((size_t)blocks * 8, 256); }
 static size_t coop_workspace_bytes(int blocks)
 {
     // a workgroup has at most two partial tiles: the one its share starts in and the one it ends in
@@ -598,7 +616,9 @@ __device__ __forceinline__ int coop_owner(long i, long G, long total) { return (
 struct TileTail {
     const int32_t *negcnt, *bias;
     int32_t *y;
-    int32_t *slots, *counters;
+    int32_t *slots;
+    unsigned long long *counters;
+    unsigned long long token;
     float *out;
     void *q;
     const float *scale, *shift, *residual;
@@ -763,6 +783,25 @@ __device__ __forceinline__ void write_tile(lds_tail *t, lds_i32 *buf, int ntile,
     }
 }
 
+// Counts this workgroup's arrival at a shared tile; true for the last of the `others + 1` contributors.
+// The counter needs no clearing before the launch: its upper 48 bits carry the launch's tag, a word
+// with another tag (whatever the workspace held, or the 0 a finished tile leaves) counts as no arrivals
+// yet, and the last arrival stores 0, so that a replay of the same launch (a captured graph: same tag)
+// starts clean as well.  One compare-and-swap per arrival when the guess holds, never a wait on
+// another workgroup.
+__device__ __forceinline__ bool coop_arrive(unsigned long long *counter, unsigned long long token, int others)
+{
+    unsigned long long seen = 0;  // what a finished launch leaves
+    for (;;) {
+        const unsigned long long count = (seen >> 16) == token ? (seen & 0xffff) : 0;
+        const bool is_last = (int)count == others;
+        const unsigned long long next = is_last ? 0 : (token << 16) | (count + 1);
+        if (__hip_atomic_compare_exchange_strong(counter, &seen, next, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT))
+            return is_last;
+    }
+}
+
 // The tail of one tile segment, after the workgroup's waves have added their sums into `buf` and met
 // at a barrier.  A whole tile (len == comm) is written out.  A partial one is published to this
 // workgroup's slot, its arrival counted, and whichever workgroup arrives last gathers the slots of all
@@ -790,9 +829,7 @@ __device__ __attribute__((noinline)) void coop_finish_tile(lds_tail *t, lds_i32 
         // tile_start: the tile's first iteration in the launch's (tile, K group) space
         const int first = coop_owner(tile_start, G, total);
         const int last = coop_owner(tile_start + comm - 1, G, total);
-        if (threadIdx.x == 0)
-            *flag = __hip_atomic_fetch_add(t->counters + first, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) ==
-                    last - first;
+        if (threadIdx.x == 0) *flag = coop_arrive(t->counters + first, t->token, last - first);
         __syncthreads();
         if (*flag) {
             for (int c = first; c <= last; ++c) {
@@ -814,10 +851,18 @@ __device__ __attribute__((noinline)) void coop_finish_tile(lds_tail *t, lds_i32 
     __syncthreads();
 }
 
+// A whole tile by one wave, from the accumulators straight to the output (a function of its own: a
+// second copy of the main loop inside the kernel body leaves the register allocator no room).
+template <int BITS, int ZT>
+__device__ __attribute__((noinline)) void whole_tile_to_output(const ShiftArgs &p, int ntile, int m0)
+{
+    planes_segment<BITS, ZT, true, false>(p, ntile, m0, 0, p.comm, false);
+}
+
 __device__ __forceinline__ void fill_tail(TileTail &tail, const ShiftArgs &p, long G, long total)
 {
     tail.negcnt = p.negcnt; tail.bias = p.bias; tail.y = p.y;
-    tail.slots = p.coop_slots; tail.counters = p.coop_counters;
+    tail.slots = p.coop_slots; tail.counters = p.coop_counters; tail.token = p.coop_token;
     tail.out = p.ep_out; tail.q = p.ep_q;
     tail.scale = p.ep_scale; tail.shift = p.ep_shift; tail.residual = p.ep_residual;
     tail.y_img_stride = p.y_img_stride; tail.y_pix_stride = p.y_pix_stride; tail.y_ch_stride = p.y_ch_stride;
@@ -853,7 +898,13 @@ void shift_planes_wide_coop_kernel(const ShiftArgs p, const ShiftArgs p2)
     const int span = span1 + (PAIR ? p2.tiles_n * p2.comm : 0);
     const long total = (long)p.tiles_m4 * span;
     long it = w * total / G;
-    const long it_end = (w + 1) * total / G;
+    long it_end = (w + 1) * total / G;
+    if (!FUSED && !PAIR && p.whole_tile_shares) {
+        // shares in whole tiles: no tile is shared between workgroups
+        const long tiles = total / p.comm;
+        it = (w * tiles / G) * p.comm;
+        it_end = ((w + 1) * tiles / G) * p.comm;
+    }
     if (threadIdx.x == 0) {
         fill_tail(tail[0], p, G, total);
         if (PAIR) fill_tail(tail[1], p2, G, total);
@@ -861,6 +912,21 @@ void shift_planes_wide_coop_kernel(const ShiftArgs p, const ShiftArgs p2)
     for (int i = threadIdx.x; i < kCoopTileElems; i += THREADS) tile_sums[i] = 0;
     __syncthreads();
     while (it < it_end) {
+        if (!FUSED && !PAIR && p.whole_tile_shares) {
+            // Many short tiles per workgroup (a 7x7 stem: 12 tiles of 25 K groups): one tile per wave,
+            // straight from the accumulators to the output -- no K split, no LDS, no barrier -- in rounds
+            // of four; the up to three tiles left over are split over the waves like any other.
+            const long run = ((it_end - it) / p.comm) & ~(long)(kCoopWaves - 1);
+            if (run > 0) {
+                const long first_tile = it / p.comm;
+                for (long t = wave; t < run; t += kCoopWaves) {
+                    const long tile = first_tile + t;
+                    whole_tile_to_output<BITS, ZT>(p, (int)(tile % p.tiles_n), (int)(tile / p.tiles_n) * kCoopPix);
+                }
+                it += run * p.comm;
+                continue;
+            }
+        }
         const int mtile = (int)(it / span);
         const int within = (int)(it - (long)mtile * span);
         const bool second = PAIR && within >= span1;
@@ -884,24 +950,30 @@ void shift_planes_wide_coop_kernel(const ShiftArgs p, const ShiftArgs p2)
     }
 }
 
-__global__ void zero_i32_kernel(int32_t *dst, int n)
+// A tag no earlier launch of this process has used: 48 bits, never 0, from a counter that starts at
+// a value drawn from the clock (so that words left by another process are no likelier to match than
+// any other garbage).
+static unsigned long long next_coop_token()
 {
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) dst[i] = 0;
+    static std::atomic<unsigned long long> counter{
+        (unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count() * 0x9E3779B97F4A7C15ull >> 16};
+    unsigned long long t;
+    do t = counter.fetch_add(1, std::memory_order_relaxed) & 0xffffffffffffull;
+    while (t == 0);
+    return t;
 }
 
 template <int BITS, int ZT>
-static int launch_planes_coop(const ShiftArgs &a, long iters, hipStream_t st, const ShiftArgs *second = nullptr)
+static int launch_planes_coop(const ShiftArgs &first, long iters, hipStream_t st, const ShiftArgs *second = nullptr)
 {
     const int blocks = coop_blocks(iters);
-    // the arrival counters start at zero (a fill kernel, not a memset node: callers may capture this)
-    hipLaunchKernelGGL(zero_i32_kernel, dim3(1), dim3(256), 0, st, a.coop_counters, blocks);
     const dim3 grid(blocks), block(kCoopWaves * 64);
+    ShiftArgs a = first;
+    a.coop_token = next_coop_token();
     if (second) {
-        if constexpr (ZT != 1)
-            hipLaunchKernelGGL((shift_planes_wide_coop_kernel<BITS, ZT, true, true>), grid, block, kCoopLdsBytes, st, a,
-                               *second);
-        else
-            return DS_EINVAL;
+        ShiftArgs b = *second;
+        b.coop_token = a.coop_token;
+        hipLaunchKernelGGL((shift_planes_wide_coop_kernel<BITS, ZT, true, true>), grid, block, kCoopLdsBytes, st, a, b);
     } else if (a.fused)
         hipLaunchKernelGGL((shift_planes_wide_coop_kernel<BITS, ZT, true, false>), grid, block, kCoopLdsBytes, st, a, a);
     else
@@ -1033,7 +1105,12 @@ static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
         // is long enough to carry the extra segment ends: from 64 K groups per tile.  Short reductions
         // over many tiles (stems, 1x1 layers) keep the wave-level shares.  A fused epilogue exists only
         // there.  The test hook's "cu" knob (0 / 4) overrides.
-        bool cooperative = WIDE && (a.comm >= 64 || a.fused);
+        // Layers with a short reduction but at least 8 tiles per workgroup also launch this way, with
+        // shares in whole tiles: rounds of four tiles go one per wave, the up to three left over of a
+        // share are split over its waves (6272 tiles on 2048 wave slots: 3 rounds and a quarter, not 4).
+        const bool many_short = !a.alt_y && (long)a.tiles_m4 * a.tiles_n >= 8L * (plane_slots(true) / kCoopWaves);
+        bool cooperative = WIDE && (a.comm >= 64 || a.fused || many_short);
+        a.whole_tile_shares = many_short && a.comm < 64 && !a.fused;
         if (g_tune.cu != kTuneUnset) cooperative = WIDE && (g_tune.cu > 0 || a.fused);
         if (!a.coop_slots) cooperative = false;  // no workspace for the partial tiles
         if (a.fused && !cooperative) return DS_EWORKSPACE;
@@ -1147,7 +1224,12 @@ static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
             int nsplit = plane_regime(a, wide) > 0 ? 1 : 0;
             if (g_tune.split != kTuneUnset) nsplit = g_tune.split;
             if (a.fused) nsplit = 0;
-            // the highest field value unused: the form without its plane
+            // the highest field value unused: the form without its plane -- or, when K leaves a partial
+            // last group, the form that holds that plane at zero, which runs the group's padding codes
+            // in the main loop instead of a scalar-decoded tail
+            if (a.top_unused && a.K % codes_per_word(BITS) != 0)
+                return wide ? launch_planes<BITS, 1, true>(a, nsplit, st)
+                            : launch_planes<BITS, 1, false>(a, nsplit, st);
             if (a.top_unused)
                 return wide ? launch_planes<BITS, 2, true>(a, nsplit, st)
                             : launch_planes<BITS, 2, false>(a, nsplit, st);
@@ -1242,7 +1324,7 @@ static void take_coop_workspace(ShiftArgs &a, void *workspace, size_t workspace_
     const size_t need = coop_bytes_for((size_t)a.M, a.K, a.N, bits);
     if (!need || !workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return;
     const long tiles = (long)ceil_div(a.M, kCoopPix) * (a.N / 64);
-    a.coop_counters = (int32_t *)workspace;
+    a.coop_counters = (unsigned long long *)workspace;
     a.coop_slots = (int32_t *)((char *)workspace + coop_counter_bytes(coop_blocks(tiles * a.comm)));
 }
 
@@ -1478,7 +1560,11 @@ static int pair_args(ShiftArgs &s, const int32_t *x, const ds_fused_conv *f, int
 template <int BITS>
 static int launch_pair(const ShiftArgs &a, const ShiftArgs &b, long iters, hipStream_t st)
 {
-    return a.top_unused ? launch_planes_coop<BITS, 2>(a, iters, st, &b) : launch_planes_coop<BITS, 0>(a, iters, st, &b);
+    if (!a.top_unused) return launch_planes_coop<BITS, 0>(a, iters, st, &b);
+    // a partial last K group in either layer: the form that runs its padding codes on a zero plane
+    constexpr int NUM = codes_per_word(BITS);
+    if (a.K % NUM != 0 || b.K % NUM != 0) return launch_planes_coop<BITS, 1>(a, iters, st, &b);
+    return launch_planes_coop<BITS, 2>(a, iters, st, &b);
 }
 
 DS_EXPORT int ds_conv2d_tiled_fused_pair_i32(const int32_t *x, int Nb, int C, int Hp, int Wp, int sh, int sw, int F_in,
@@ -1497,7 +1583,7 @@ DS_EXPORT int ds_conv2d_tiled_fused_pair_i32(const int32_t *x, int Nb, int C, in
     if (rc) return rc;
     rc = pair_args(sb, x, b, Nb, C, Hp, Wp, sh, sw, OH, OW, F_in);
     if (rc) return rc;
-    sa.coop_counters = sb.coop_counters = (int32_t *)workspace;
+    sa.coop_counters = sb.coop_counters = (unsigned long long *)workspace;
     sa.coop_slots = sb.coop_slots = (int32_t *)((char *)workspace + coop_counter_bytes(blocks));
     hipStream_t st = (hipStream_t)stream;
     switch (a->bits & 0xff) {

@@ -48,8 +48,8 @@ def test_size_queries():
     assert L.ds_tiled_bytes(10, 6, 5) == 256 + 256 + 256
     assert L.ds_tiled_bytes(64, 576, 7) == 0
     # cooperative launch: 25 tiles x 96 K groups on workgroups of 4 waves with >= 8 groups each -> 72
-    # workgroups: their arrival counters (padded to 256 bytes) + two partial tiles of 32 KiB each
-    coop = 512 + 2 * 72 * 32768
+    # workgroups: their 8-byte arrival counters (padded to 256 bytes) + two partial tiles of 32 KiB each
+    coop = 768 + 2 * 72 * 32768
     assert L.ds_conv2d_tiled_workspace_bytes(1, 64, 58, 58, 64, 3, 3, 1, 1, 4) == coop
     assert L.ds_conv2d_tiled_workspace_bytes(1, 64, 58, 58, 64, 3, 3, 1, 1, 4 | 0x200) == coop
     assert L.ds_conv2d_tiled_workspace_bytes(1, 64, 58, 58, 48, 3, 3, 1, 1, 4) == 0    # not 64 channels wide

@@ -121,6 +121,63 @@ def test_cooperative_launch_matches_oracle(oracle, rng, geom, bits):
         np.testing.assert_array_equal(abi_conv_tiled(xp, blob, bias, O, FH, FW, stride, bits, False), want)
 
 
+def test_many_short_tiles_run_in_whole_tile_shares(oracle, rng):
+    """A short reduction over many pixel tiles (a 7x7 stem's shape class): the cooperative launch hands
+    out whole tiles, one per wave in rounds of four, the rest of a share split over its waves.  4616
+    tiles on 512 workgroups leave shares of 9 and 10 tiles: both paths run, and the last tile is ragged."""
+    Nb, C, Hp, Wp, O, FH, FW, stride = 2, 3, 550, 549, 64, 7, 7, (1, 1)
+    xp = random_activations(rng, (Nb, C, Hp, Wp))
+    s, sign = random_codes(rng, (O, C, FH, FW), max_s=14)
+    bias = rng.integers(-2 ** 20, 2 ** 20, size=O).astype(np.int32)
+    want = oracle.conv2d(xp, -s, sign, bias, stride, nthreads=NTHREADS)
+    blob = kernels.tile_weights(_dev(so.np_pack_words(s.reshape(O, -1), sign.reshape(O, -1), 4)).reshape(-1),
+                                O, C, FH, FW, 4, 0)
+    for b in (4, 4 | U):
+        np.testing.assert_array_equal(abi_conv_tiled(xp, blob, bias, O, FH, FW, stride, b), want)
+
+
+def test_cooperative_launch_replays_in_a_graph(oracle, rng):
+    """A captured launch keeps its arguments, the counters' tag among them: every replay must find the
+    arrival counters as a finished launch leaves them.  Replays alternate with eager launches on the
+    same workspace and are checked against the oracle each time."""
+    Nb, C, Hp, Wp, O, FH, FW, stride = 1, 256, 9, 9, 128, 3, 3, (1, 1)   # every tile cut many times
+    s, sign = random_codes(rng, (O, C, FH, FW), max_s=14)
+    blob = kernels.tile_weights(_dev(so.np_pack_words(s.reshape(O, -1), sign.reshape(O, -1), 4)).reshape(-1),
+                                O, C, FH, FW, 4, 0)
+    L = _lib.lib()
+    ws_bytes = L.ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, 1, 1, 4)
+    ws = torch.full((ws_bytes,), 0x77, dtype=torch.uint8, device=DEV)
+    xd = torch.zeros((Nb, C, Hp, Wp), dtype=torch.int32, device=DEV)
+    y = torch.zeros((Nb, O, Hp - 2, Wp - 2), dtype=torch.int32, device=DEV)
+
+    def launch():
+        _lib.call("ds_conv2d_tiled_i32", _lib.ptr(xd), _lib.ptr(blob), None, _lib.ptr(y), Nb, C, Hp, Wp, O, FH, FW,
+                  1, 1, 4, 0, _lib.ptr(ws), ws_bytes, _stream())
+
+    with Tune(planes=1, split=0, cu=4):
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            launch()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            launch()
+        for step in range(4):
+            xp = random_activations(rng, (Nb, C, Hp, Wp))
+            want = oracle.conv2d(xp, -s, sign, None, stride, nthreads=NTHREADS)
+            xd.copy_(_dev(xp))
+            y.fill_(-1)
+            graph.replay()
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(y.cpu().numpy(), want, err_msg="replay %d" % step)
+            y.fill_(-1)
+            launch()
+            torch.cuda.synchronize()
+            np.testing.assert_array_equal(y.cpu().numpy(), want, err_msg="eager after replay %d" % step)
+
+
 @pytest.mark.parametrize("geom", GEOMS, ids=lambda g: "x".join(str(v) for v in g[:7]))
 def test_fused_epilogue_matches_oracle_chain(oracle, rng, geom):
     """Float and fixed-point outputs of the fused call against oracle.conv2d -> np_dequantize_affine ->
