@@ -103,6 +103,23 @@ __device__ __forceinline__ int32_t xor_add(int32_t t, int32_t mask, int32_t acc)
 }
 
 __device__ __forceinline__ int32_t uniform(int32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ float uniform(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int32_t, v)));
+}
+__device__ __forceinline__ uint64_t uniform(uint64_t v)
+{
+    return (uint64_t)(uint32_t)uniform((int32_t)(uint32_t)v) | ((uint64_t)(uint32_t)uniform((int32_t)(uint32_t)(v >> 32)) << 32);
+}
+__device__ __forceinline__ long uniform(long v) { return (long)uniform((uint64_t)v); }
+// A wave-uniform pointer to global memory, for the compiler to keep in scalar registers: values that
+// reach a wave through LDS arrive in vector registers as generic pointers, which makes every access a
+// flat one with its address computed per lane.
+template <typename T>
+__device__ __forceinline__ __attribute__((address_space(1))) T *uniform_global(T *p)
+{
+    return (__attribute__((address_space(1))) T *)uniform((uint64_t)p);
+}
 
 __device__ __forceinline__ int32_t *at_lane(int32_t *uniform_base, uint32_t lane_bytes)
 {
@@ -597,11 +614,13 @@ static int coop_blocks(long iters)
 // exchange (measured: +45 % on a ResNet 3x3 layer, the other workgroups lose their cached activations);
 // instead the slots are written and read with agent-scope (relaxed atomic) accesses, which go through to
 // the level all XCDs share, like the atomic adds of the per-wave launches do.
-__device__ __forceinline__ void store_agent(int32_t *p, int32_t v)
+typedef __attribute__((address_space(1))) int32_t g_i32;
+typedef __attribute__((address_space(1))) float g_f32;
+__device__ __forceinline__ void store_agent(g_i32 *p, int32_t v)
 {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ int32_t load_agent(const int32_t *p)
+__device__ __forceinline__ int32_t load_agent(const g_i32 *p)
 {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -636,15 +655,13 @@ typedef __attribute__((address_space(3))) const TileTail lds_tail;
 // so only NaN (propagated by the clamp, as torch.clamp does) needs the conversion's "NaN -> 0".
 __device__ __forceinline__ int32_t quantize_fixed(float v, float scale, float lo, float hi, bool one_bit)
 {
-    float r = floorf(v * scale);
-    r = (r < lo) ? lo : r;
-    r = (r > hi) ? hi : r;
+    // max / min drop a NaN operand; the select on v == v puts "NaN -> 0" back
+    float r = __builtin_fminf(__builtin_fmaxf(floorf(v * scale), lo), hi);
     if (one_bit) {  // integer_bits == 1: sign(x) - 1 (utils.py:12-13)
-        float s = ((v > 0.0f) ? 1.0f : ((v < 0.0f) ? -1.0f : 0.0f)) - 1.0f;
-        s = (v != v) ? v : s;
+        const float s = ((v > 0.0f) ? 1.0f : ((v < 0.0f) ? -1.0f : 0.0f)) - 1.0f;
         r = s * scale;
     }
-    return (int32_t)((r == r) ? r : 0.0f);
+    return (int32_t)((v == v) ? r : 0.0f);
 }
 
 // The zero padding of the next layer's input around this tile's pixels: the pixels on an image edge
@@ -683,30 +700,35 @@ __device__ __forceinline__ void write_padding(Q *q, size_t plane_base, int oh, i
 template <bool FUSED, typename Q>
 __device__ __forceinline__ void write_tile(lds_tail *t, lds_i32 *buf, int ntile, int m0, int wave, int lane)
 {
+    typedef __attribute__((address_space(1))) Q g_q;
+    typedef __attribute__((address_space(1))) char g_char;
     constexpr int CH = 64 / kCoopWaves, R = kPlaneRowsWide;
-    const int M = t->M, N = t->N, pix_per_img = t->pix_per_img, OW = t->OW;
+    // Every field of the tail block is wave-uniform, but read from LDS it arrives in a vector register:
+    // v_readfirstlane tells the compiler, which then branches on scalars and addresses memory as scalar
+    // base + 32-bit lane offset (the tensors are below 2 GiB) instead of per-lane 64-bit flat addresses.
+    const int M = uniform(t->M), N = uniform(t->N), pix_per_img = uniform(t->pix_per_img), OW = uniform(t->OW);
     const int n0 = ntile * 64 + wave * CH;
     const int mine = n0 + (lane & (CH - 1));
-    const int32_t *bias = t->bias;
-    const int32_t add_l = t->negcnt[mine] + (bias ? bias[mine] : 0);
+    const g_i32 *negcnt = uniform_global(t->negcnt), *bias = uniform_global(t->bias);
+    const int32_t add_l = negcnt[mine] + (bias ? bias[mine] : 0);
     float sa_l = 1.0f, sb_l = 0.0f;
-    const float *residual = nullptr;
-    float *out = nullptr;
-    Q *q = nullptr;
+    const g_f32 *residual = nullptr;
+    g_char *out = nullptr, *q = nullptr;
     if (FUSED) {
-        const float *scale = t->scale, *shift = t->shift;
+        const g_f32 *scale = uniform_global(t->scale), *shift = uniform_global(t->shift);
         if (scale) sa_l = scale[mine];
         if (shift) sb_l = shift[mine];
-        residual = t->residual;
-        out = t->out;
-        q = (Q *)t->q;
+        residual = uniform_global(t->residual);
+        out = (g_char *)uniform_global(t->out);
+        q = (g_char *)uniform_global((char *)t->q);
     }
-    const int ph = FUSED ? t->ph : 0, pw = FUSED ? t->pw : 0;
+    const int ph = FUSED ? uniform(t->ph) : 0, pw = FUSED ? uniform(t->pw) : 0;
     const int OH = pix_per_img / OW;
     const int Hq = OH + 2 * ph, Wq = OW + 2 * pw;
-    const size_t qplane = (size_t)Hq * Wq;
+    const uint32_t qplane = (uint32_t)Hq * Wq;
     bool live[R];
-    size_t pix[R], qpix[R], qimg[R];
+    uint32_t pix[R], qpix[R], qimg[R];  // element indices
+    size_t ypix[R];
     int oh[R], ow[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -717,19 +739,27 @@ __device__ __forceinline__ void write_tile(lds_tail *t, lds_i32 *buf, int ntile,
         oh[r] = rem / OW;
         ow[r] = rem - oh[r] * OW;
         if (FUSED) {
-            pix[r] = ((size_t)img * N + n0) * pix_per_img + rem;
-            qimg[r] = ((size_t)img * N + n0) * qplane;
-            qpix[r] = qimg[r] + (size_t)(oh[r] + ph) * Wq + ow[r] + pw;
+            pix[r] = (uint32_t)(img * N + n0) * (uint32_t)pix_per_img + rem;
+            qimg[r] = (uint32_t)(img * N + n0) * qplane;
+            qpix[r] = qimg[r] + (uint32_t)(oh[r] + ph) * Wq + ow[r] + pw;
         } else {
-            pix[r] = (size_t)img * t->y_img_stride + (size_t)rem * t->y_pix_stride + (size_t)n0 * t->y_ch_stride;
+            ypix[r] = (size_t)img * uniform(t->y_img_stride) + (size_t)rem * uniform(t->y_pix_stride) +
+                      (size_t)n0 * uniform(t->y_ch_stride);
         }
     }
     float res[CH][R];
     if (FUSED && residual) {
 #pragma unroll
-        for (int c = 0; c < CH; ++c)
+        for (int r = 0; r < R; ++r) {
+            if (live[r]) {
 #pragma unroll
-            for (int r = 0; r < R; ++r) res[c][r] = live[r] ? residual[pix[r] + (size_t)c * pix_per_img] : 0.0f;
+                for (int c = 0; c < CH; ++c)
+                    res[c][r] = *(const g_f32 *)((const g_char *)residual + 4u * (pix[r] + (uint32_t)(c * pix_per_img)));
+            } else {
+#pragma unroll
+                for (int c = 0; c < CH; ++c) res[c][r] = 0.0f;
+            }
+        }
     }
     int32_t sums[CH][R];
 #pragma unroll
@@ -741,19 +771,19 @@ __device__ __forceinline__ void write_tile(lds_tail *t, lds_i32 *buf, int ntile,
             *cell = 0;
         }
     if (!FUSED) {
-        int32_t *y = t->y;
-        const size_t ch = (size_t)t->y_ch_stride;
+        g_i32 *y = uniform_global(t->y);
+        const size_t ch = (size_t)uniform(t->y_ch_stride);
 #pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            const int32_t add = __builtin_amdgcn_readlane(add_l, c);
+        for (int r = 0; r < R; ++r) {
+            if (!live[r]) continue;
 #pragma unroll
-            for (int r = 0; r < R; ++r)
-                if (live[r]) y[pix[r] + c * ch] = sums[c][r] + add;
+            for (int c = 0; c < CH; ++c) y[ypix[r] + c * ch] = sums[c][r] + __builtin_amdgcn_readlane(add_l, c);
         }
         return;
     }
-    const float inv = t->inv, qs = t->spec.scale, qlo = t->spec.lo, qhi = t->spec.hi;
-    const bool relu = t->relu != 0, one_bit = t->spec.I == 1, has_res = residual != nullptr;
+    const float inv = uniform(t->inv), qs = uniform(t->spec.scale), qlo = uniform(t->spec.lo), qhi = uniform(t->spec.hi);
+    const bool relu = uniform(t->relu) != 0, one_bit = uniform(t->spec.I) == 1, has_res = residual != nullptr;
+    float f[CH][R];
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         const int32_t add = __builtin_amdgcn_readlane(add_l, c);
@@ -761,24 +791,35 @@ __device__ __forceinline__ void write_tile(lds_tail *t, lds_i32 *buf, int ntile,
         const float sb = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sb_l), c));
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            float f;
-            {
 #pragma clang fp contract(off)
-                f = ((float)(sums[c][r] + add) * inv) * sa + sb;
-                if (has_res) f += res[c][r];
-                if (relu) f = f > 0.0f ? f : 0.0f;
-            }
-            if (!live[r]) continue;
-            if (out) out[pix[r] + (size_t)c * pix_per_img] = f;
-            if (q) q[qpix[r] + c * qplane] = (Q)quantize_fixed(f, qs, qlo, qhi, one_bit);
+            float v = ((float)(sums[c][r] + add) * inv) * sa + sb;
+            if (has_res) v += res[c][r];
+            if (relu) v = v > 0.0f ? v : 0.0f;
+            f[c][r] = v;
         }
     }
-    if (q && (ph | pw) && !t->border_kept) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (!live[r]) continue;
+        if (out) {
+#pragma unroll
+            for (int c = 0; c < CH; ++c) *(g_f32 *)(out + 4u * (pix[r] + (uint32_t)(c * pix_per_img))) = f[c][r];
+        }
+        if (q) {
+#pragma unroll
+            for (int c = 0; c < CH; ++c)
+                *(g_q *)(q + (uint32_t)sizeof(Q) * (qpix[r] + (uint32_t)c * qplane)) =
+                    (Q)quantize_fixed(f[c][r], qs, qlo, qhi, one_bit);
+        }
+    }
+    if (q && (ph | pw) && !uniform(t->border_kept)) {
+        Q *qg = (Q *)t->q;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             if (!live[r]) continue;
             if (!(ow[r] == 0 || ow[r] == OW - 1 || oh[r] == 0 || oh[r] == OH - 1)) continue;
-            for (int c = 0; c < CH; ++c) write_padding(q, qimg[r] + c * qplane, oh[r], ow[r], OH, OW, ph, pw, Wq);
+            for (int c = 0; c < CH; ++c)
+                write_padding(qg, (size_t)qimg[r] + (size_t)c * qplane, oh[r], ow[r], OH, OW, ph, pw, Wq);
         }
     }
 }
@@ -812,11 +853,12 @@ __device__ __attribute__((noinline)) void coop_finish_tile(lds_tail *t, lds_i32 
 {
     constexpr int THREADS = kCoopWaves * 64, PER = kCoopTileElems / THREADS;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & (kWave - 1);
-    const int comm = t->comm;
+    const int comm = uniform(t->comm);
     bool finish = len == comm;
     if (!finish) {
+        g_i32 *slots = uniform_global(t->slots);
         // slot 0 of a workgroup holds the tile its share starts in (g0 > 0), slot 1 the tile it ends in
-        int32_t *slot = t->slots + ((size_t)2 * w + (g0 > 0 ? 0 : 1)) * kCoopTileElems + threadIdx.x;
+        g_i32 *slot = slots + ((size_t)2 * w + (g0 > 0 ? 0 : 1)) * kCoopTileElems + threadIdx.x;
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
             store_agent(slot + k * THREADS, buf[threadIdx.x + k * THREADS]);
@@ -825,7 +867,7 @@ __device__ __attribute__((noinline)) void coop_finish_tile(lds_tail *t, lds_i32 
         // the slot is complete (every store acknowledged) before the arrival is counted
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        const long G = t->G, total = t->total;
+        const long G = uniform(t->G), total = uniform(t->total);
         // tile_start: the tile's first iteration in the launch's (tile, K group) space
         const int first = coop_owner(tile_start, G, total);
         const int last = coop_owner(tile_start + comm - 1, G, total);
@@ -833,7 +875,7 @@ __device__ __attribute__((noinline)) void coop_finish_tile(lds_tail *t, lds_i32 
         __syncthreads();
         if (*flag) {
             for (int c = first; c <= last; ++c) {
-                const int32_t *src = t->slots + ((size_t)2 * c + (c == first ? 1 : 0)) * kCoopTileElems + threadIdx.x;
+                const g_i32 *src = slots + ((size_t)2 * c + (c == first ? 1 : 0)) * kCoopTileElems + threadIdx.x;
                 int32_t v[PER];
 #pragma unroll
                 for (int k = 0; k < PER; ++k) v[k] = load_agent(src + k * THREADS);
@@ -845,7 +887,7 @@ __device__ __attribute__((noinline)) void coop_finish_tile(lds_tail *t, lds_i32 
         __syncthreads();
     }
     if (finish) {
-        if (FUSED && t->q_bytes == 1) write_tile<FUSED, int8_t>(t, buf, ntile, m0, wave, lane);
+        if (FUSED && uniform(t->q_bytes) == 1) write_tile<FUSED, int8_t>(t, buf, ntile, m0, wave, lane);
         else write_tile<FUSED, int32_t>(t, buf, ntile, m0, wave, lane);
     }
     __syncthreads();
@@ -885,6 +927,8 @@ void shift_planes_wide_coop_kernel(const ShiftArgs p, const ShiftArgs p2)
     __shared__ TileTail tail[PAIR ? 2 : 1];
     __shared__ int32_t last_arrival;
     constexpr int THREADS = kCoopWaves * 64;
+    // outside the main loop (which sets its own, by turns) a wave runs at the highest priority
+    __builtin_amdgcn_s_setprio(3);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int bid = blockIdx.x;
     const long G = gridDim.x;

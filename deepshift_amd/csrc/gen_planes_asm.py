@@ -272,7 +272,7 @@ def body(bits, zero_top=False, wide=False, unused_top=False):
                     L += ["v_xad_u32 v%d, v%d, s%d, v%d" % (a, PL + PS * r, MASK, a)]
     L += ["s_sub_u32 s%d, s%d, 1" % (CNT, CNT), "s_cmp_lg_u32 s%d, 0" % CNT, "s_cbranch_scc1 1b"]
     # ---- leave relative addressing, drain the loads that ran ahead of the last slot
-    L += ["s_set_gpr_idx_off", "s_setprio 0", "s_waitcnt vmcnt(0) lgkmcnt(0)"]
+    L += ["s_set_gpr_idx_off", "s_setprio %d" % (3 if wide else 0), "s_waitcnt vmcnt(0) lgkmcnt(0)"]
     return L
 
 
