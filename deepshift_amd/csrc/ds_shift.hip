@@ -1223,7 +1223,10 @@ static int plane_regime(const ShiftArgs &a, bool wide)
     const bool per_tile =
         many_tiles && (a.comm < 24 || (a.comm <= 128 && (fill >= 0.85 || ceil_div(a.N, J) >= 8)));
     const int regime = (per_tile || whole_rounds) ? 1 : 0;
-    const bool eligible = n_ok && ((many_tiles && a.comm >= 6) || (a.comm >= 24 && iters >= slots * 16));
+    // (the 64-channel form with long reductions, which launches workgroup-cooperatively without a
+    // pre-fill, pays from 6 K groups per wave slot: 3x3x64 layers on 8x8 images at batch 256)
+    const long min_per_slot = wide && a.comm >= 64 ? 6 : 16;
+    const bool eligible = n_ok && ((many_tiles && a.comm >= 6) || (a.comm >= 24 && iters >= slots * min_per_slot));
     return eligible ? regime : -1 - regime;
 }
 
