@@ -361,7 +361,8 @@ def pmc_target(device):
     of the byte counters), then one launch each of the kernels of the headline step, three times over:
       * the dominant kernel on the layer1 shape (3x3, 64 -> 64, batch 64, 56x56), with the fused epilogue
         (shift_planes_wide_coop_kernel<4, 2, true, false>) and with the plain int32 output (<.., false, false>);
-      * the stem (7x7 stride 2, 3 -> 64, 224x224): shift_planes_wide_balanced_kernel + its pre-fill;
+      * the stem (7x7 stride 2, 3 -> 64, 224x224): shift_planes_wide_coop_kernel<4, 1, false, false>, whole
+        tiles one per wave (K = 147 leaves a partial last group: the zero-top form runs its padding codes);
       * a down-sampling block's first 3x3 stride-2 convolution with its 1x1 shortcut as one launch
         (<4, 2, true, true>), 64 -> 128 channels at 56x56;
       * the int8 kernel (shift_pairs_cu_kernel) on a ResNet-50 3x3 layer, 128 -> 128 at 28x28, batch 128,
