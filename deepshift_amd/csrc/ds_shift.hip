@@ -376,8 +376,10 @@ DS_PLANES_SPECIALISE(4)
 // One segment of work of the shift-plane kernel: K groups [g_begin, g_end) of the tile made of the J
 // channels of `ntile` and the R*64 pixels starting at m0.  `atomic` selects accumulation into a
 // pre-filled output (several segments share the tile) or a plain store of acc + bias.  WIDE: the
-// 64-channel form (layers with N % 64 == 0).
-template <int BITS, int ZT, bool WIDE, bool TO_LDS = false>
+// 64-channel form (layers with N % 64 == 0).  TO_LDS 1: the sums are added to the workgroup's tile
+// buffer instead; 2: the same if the caller passes a buffer, else the plain store (decided at run
+// time, so that one copy of the main loop serves both).
+template <int BITS, int ZT, bool WIDE, int TO_LDS = 0>
 __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, int m0, int g_begin,
                                                int g_end, bool atomic, int32_t *lds = nullptr)
 {
@@ -466,7 +468,7 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
         }
     }
 
-    if (TO_LDS) {
+    if (TO_LDS == 1 || (TO_LDS == 2 && lds != nullptr)) {
         // the workgroup's tile buffer lds[channel][pixel of the tile]: consecutive lanes, consecutive
         // banks
 #pragma unroll
@@ -893,14 +895,6 @@ __device__ __attribute__((noinline)) void coop_finish_tile(lds_tail *t, lds_i32 
     __syncthreads();
 }
 
-// A whole tile by one wave, from the accumulators straight to the output (a function of its own: a
-// second copy of the main loop inside the kernel body leaves the register allocator no room).
-template <int BITS, int ZT>
-__device__ __attribute__((noinline)) void whole_tile_to_output(const ShiftArgs &p, int ntile, int m0)
-{
-    planes_segment<BITS, ZT, true, false>(p, ntile, m0, 0, p.comm, false);
-}
-
 __device__ __forceinline__ void fill_tail(TileTail &tail, const ShiftArgs &p, long G, long total)
 {
     tail.negcnt = p.negcnt; tail.bias = p.bias; tail.y = p.y;
@@ -956,36 +950,35 @@ void shift_planes_wide_coop_kernel(const ShiftArgs p, const ShiftArgs p2)
     for (int i = threadIdx.x; i < kCoopTileElems; i += THREADS) tile_sums[i] = 0;
     __syncthreads();
     while (it < it_end) {
-        if (!FUSED && !PAIR && p.whole_tile_shares) {
-            // Many short tiles per workgroup (a 7x7 stem: 12 tiles of 25 K groups): one tile per wave,
-            // straight from the accumulators to the output -- no K split, no LDS, no barrier -- in rounds
-            // of four; the up to three tiles left over are split over the waves like any other.
-            const long run = ((it_end - it) / p.comm) & ~(long)(kCoopWaves - 1);
-            if (run > 0) {
-                const long first_tile = it / p.comm;
-                for (long t = wave; t < run; t += kCoopWaves) {
-                    const long tile = first_tile + t;
-                    whole_tile_to_output<BITS, ZT>(p, (int)(tile % p.tiles_n), (int)(tile / p.tiles_n) * kCoopPix);
-                }
-                it += run * p.comm;
-                continue;
-            }
-        }
-        const int mtile = (int)(it / span);
-        const int within = (int)(it - (long)mtile * span);
+        // Many short tiles per workgroup (a 7x7 stem: 12 tiles of 25 K groups): rounds of four whole
+        // tiles go one per wave, straight from the accumulators to the output -- no K split, no LDS, no
+        // barrier; the up to three tiles left over of a share are split over the waves like any other.
+        // (One call of the segment code serves both: a second copy of the main loop in this kernel
+        // leaves the register allocator no room.)
+        const bool direct = !FUSED && !PAIR && p.whole_tile_shares && (it_end - it) / p.comm >= kCoopWaves;
+        const long at = direct ? it + (long)wave * p.comm : it;
+        const int mtile = (int)(at / span);
+        const int within = (int)(at - (long)mtile * span);
         const bool second = PAIR && within >= span1;
         const int comm = second ? p2.comm : p.comm;
         const int ntile = (second ? within - span1 : within) / comm;
         const long tile_start = (long)mtile * span + (second ? span1 : 0) + (long)ntile * comm;
-        const int g0 = (int)(it - tile_start);
-        long g1 = g0 + (it_end - it);
+        const int g0 = (int)(at - tile_start);
+        long g1 = g0 + (it_end - at);
         if (g1 > comm) g1 = comm;
         const int m0 = mtile * kCoopPix;
         const int len = (int)g1 - g0;
-        const int wb = g0 + wave * len / kCoopWaves, we = g0 + (wave + 1) * len / kCoopWaves;
+        // direct: g0 == 0 and len == comm (shares of whole tiles), the wave takes all of it
+        const int wb = direct ? 0 : g0 + wave * len / kCoopWaves;
+        const int we = direct ? comm : g0 + (wave + 1) * len / kCoopWaves;
         if (wb < we) {
-            if (second) planes_segment<BITS, ZT, true, true>(p2, ntile, m0, wb, we, true, tile_sums);
-            else planes_segment<BITS, ZT, true, true>(p, ntile, m0, wb, we, true, tile_sums);
+            if (second) planes_segment<BITS, ZT, true, 1>(p2, ntile, m0, wb, we, false, tile_sums);
+            else planes_segment<BITS, ZT, true, (FUSED || PAIR) ? 1 : 2>(p, ntile, m0, wb, we, false,
+                                                                        direct ? nullptr : tile_sums);
+        }
+        if (direct) {
+            it += (long)kCoopWaves * p.comm;
+            continue;
         }
         __syncthreads();
         coop_finish_tile<FUSED>((lds_tail *)&tail[second ? 1 : 0], (lds_i32 *)tile_sums, (lds_i32 *)&last_arrival, w,
