@@ -56,6 +56,7 @@ SIGNATURES = {
     "ds_linear_tiled_i32": (_c_int, [_ptr, _c_int, _ptr, _ptr, _ptr] + [_c_int] * 5 + [_ptr, _size, _ptr]),
     "ds_linear_tiled_noalloc_max_bytes": (_size, []),
     "ds_linear_tiled_noalloc_i32": (_c_int, [_ptr, _c_int, _ptr, _ptr, _ptr] + [_c_int] * 5 + [_ptr]),
+    "ds_linear_small_f32": (_c_int, [_ptr, _ptr, _ptr, _ptr] + [_c_int] * 8 + [_ptr]),
     "ds_conv2d_workspace_bytes": (_size, [_c_int] * 10),
     "ds_conv2d_i32": (_c_int, [_ptr] * 4 + [_c_int] * 11 + [_ptr, _size, _ptr]),
     "ds_conv2d_tiled_workspace_bytes": (_size, [_c_int] * 10),

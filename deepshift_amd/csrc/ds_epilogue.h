@@ -22,10 +22,11 @@ struct QuantSpec {
 // an out-of-range C++ conversion is undefined).
 __device__ __forceinline__ int32_t f2i_sat(float v)
 {
-    if (v != v) return 0;
-    if (v >= 2147483648.0f) return 2147483647;
-    if (v <= -2147483648.0f) return (int32_t)0x80000000;
-    return (int32_t)v;
+    // selects, not branches: callers convert many independent values between a load and its use
+    const float c = __builtin_fminf(__builtin_fmaxf(v, -2147483648.0f), 2147483520.0f);  // in range; NaN -> a bound
+    int32_t r = (int32_t)c;
+    r = v >= 2147483648.0f ? 2147483647 : r;
+    return v != v ? 0 : r;
 }
 
 __device__ __forceinline__ int32_t quantize_one(float v, const QuantSpec &q)

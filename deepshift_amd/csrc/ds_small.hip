@@ -1,0 +1,171 @@
+// Small LinearShift layers as ONE launch: float activations in, float results out.
+//
+// A fully connected layer at inference batch sizes (ResNet's classifier: 64 x 512 x 1000; the MNIST
+// MLP: 64 x 784 x 512 ...) is a few tens of millions of shift-add pairs -- microseconds of vector
+// issue -- but on the general path it costs five launches: conversion + transpose of the input, the
+// pre-fill, the shift GEMM, the transpose of its channel-major scratch, the dequantisation.  This
+// kernel does the reference's whole chain (modules.py:24-31, modules_q.py:115-125)
+//     x_fixed = (x * 2^F).int()  [or round_to_fixed first]   ->   y = bias + sum_k +-(x_fixed >> s)
+//     ->   y.float() / 2^F
+// per lane = batch row: a workgroup of eight waves owns 64 rows x 8 output channels, its waves split
+// the reduction, the partial sums meet in LDS and each wave writes one channel.  The weights are the
+// tiled blob of ds_tile_weights_i32 / ds_tile_weights_zero_top_i32 (its packed-word section), so a
+// layer keeps one weight format whichever kernel serves it.
+#include "ds_common.h"
+#include "ds_epilogue.h"
+
+namespace ds {
+
+constexpr int kSmallJ = 8;      // output channels per workgroup
+constexpr int kSmallWaves = 8;  // waves per workgroup: eighths of the reduction
+
+struct SmallArgs {
+    const float *x;         // [M][K]
+    const uint32_t *wt;     // tiled words [ceil(N/32)][comm][32]
+    const int32_t *negcnt;  // negative codes per channel
+    const int32_t *bias;    // int32 fixed point, or nullptr
+    float *y;               // [M][N]
+    int M, K, N, comm, nbase;
+    float out_scale;        // 2^F
+    QuantSpec spec;
+};
+
+// MODE 0: every field is a right shift (base 0, fields of at most 5 bits); 1: general codes (a left
+// shift by nbase after the right shift; with 6-bit fields a field >= 32 is a zero weight); 2: the
+// highest field value stands for a zero weight (zero-top blobs).
+template <int BITS, int MODE>
+__global__ __launch_bounds__(kSmallWaves * 64) void linear_small_kernel(const SmallArgs p)
+{
+    constexpr int NUM = 32 / (BITS + 1), CB = BITS + 1, J = kSmallJ;
+    constexpr uint32_t TOP = (1u << BITS) - 1u;
+    __shared__ int32_t part[kSmallWaves][J][kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n0 = blockIdx.x * J;
+    const int m = blockIdx.y * kWave + lane;
+    const bool live = m < p.M;
+    const float *xrow = p.x + (size_t)(live ? m : 0) * p.K;
+    const int g_begin = (int)((long)wave * p.comm / kSmallWaves);
+    const int g_end = (int)((long)(wave + 1) * p.comm / kSmallWaves);
+    // words of the workgroup's channels for K group g: wrow[g * 32 + j] (8 channels never straddle a
+    // 32-channel tile)
+    const uint32_t *wrow = p.wt + (size_t)(n0 / kTileWords) * p.comm * kTileWords + n0 % kTileWords;
+
+    int32_t acc[J];
+#pragma unroll
+    for (int j = 0; j < J; ++j) acc[j] = 0;
+
+    // Activations of one K group: the loads are issued together, unconditionally (reduction indices
+    // past K read the row's last element), one group ahead of their use; the conversion to fixed point
+    // follows the accumulation of the group before, and indices past K convert to 0 whatever the blob
+    // holds there.
+    auto load_group = [&](int g, float (&xf)[NUM]) {
+#pragma unroll
+        for (int i = 0; i < NUM; ++i) {
+            const int k = g * NUM + i;
+            xf[i] = xrow[k < p.K ? k : p.K - 1];
+        }
+    };
+    auto convert_group = [&](int g, const float (&xf)[NUM], int32_t (&xv)[NUM]) {
+#pragma unroll
+        for (int i = 0; i < NUM; ++i) {
+            const int32_t q = quantize_one(xf[i], p.spec);
+            xv[i] = g * NUM + i < p.K ? q : 0;
+        }
+    };
+    float xf[NUM];
+    int32_t xcur[NUM];
+    if (g_begin < g_end) {
+        load_group(g_begin, xf);
+        convert_group(g_begin, xf, xcur);
+    }
+#pragma clang loop unroll(disable)
+    for (int g = g_begin; g < g_end; ++g) {
+        uint32_t w[J];
+#pragma unroll
+        for (int j = 0; j < J; ++j) w[j] = wrow[(size_t)g * kTileWords + j];
+        const int gn = g + 1 < g_end ? g + 1 : g;  // the last iteration re-reads its own group: no branch
+        load_group(gn, xf);
+#pragma unroll
+        for (int i = 0; i < NUM; ++i) {
+#pragma unroll
+            for (int j = 0; j < J; ++j) {
+                const uint32_t code = w[j] >> (i * CB);
+                const int32_t mask = -(int32_t)((code >> BITS) & 1u);  // tiled format: 1 = negative
+                const uint32_t field = code & TOP;
+                int32_t t = xcur[i] >> (field & 31u);
+                if (MODE == 1) {
+                    t = (int32_t)((uint32_t)t << p.nbase);
+                    if (BITS == 6) t &= -(int32_t)(((field >> 5) & 1u) ^ 1u);
+                }
+                if (MODE == 2) t &= field == TOP ? 0 : -1;
+                acc[j] += t ^ mask;  // -t = (t ^ -1) + 1: the + 1 per negative code comes with negcnt
+            }
+        }
+        convert_group(gn, xf, xcur);
+    }
+#pragma unroll
+    for (int j = 0; j < J; ++j) part[wave][j][lane] = acc[j];
+    __syncthreads();
+    // wave j sums the eight partial results of channel n0 + j and writes it
+    static_assert(kSmallJ == kSmallWaves, "one channel per wave in the write-out");
+    const int n = n0 + wave;
+    if (n < p.N && live) {
+        int32_t sum = p.negcnt[n] + (p.bias ? p.bias[n] : 0);
+#pragma unroll
+        for (int w = 0; w < kSmallWaves; ++w) sum += part[w][wave][lane];
+        // out.float() / 2**F: int32 -> fp32 rounds to nearest even, the division is exact
+        p.y[(size_t)m * p.N + n] = (float)sum / p.out_scale;
+    }
+}
+
+template <int BITS>
+static void launch_small(const SmallArgs &a, int mode, hipStream_t st)
+{
+    const dim3 grid(ceil_div(a.N, kSmallJ), ceil_div(a.M, kWave)), block(kSmallWaves * 64);
+    if (mode == 2) hipLaunchKernelGGL((linear_small_kernel<BITS, 2>), grid, block, 0, st, a);
+    else if (mode == 1) hipLaunchKernelGGL((linear_small_kernel<BITS, 1>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((linear_small_kernel<BITS, 0>), grid, block, 0, st, a);
+}
+
+}  // namespace ds
+
+using namespace ds;
+
+DS_EXPORT int ds_linear_small_f32(const float *x, const void *tiled, const int32_t *bias, float *y, int M,
+                                  int K, int N, int bits, int base, int mode, int I, int F,
+                                  ds_stream_t stream)
+{
+    const int zero_top = (bits & DS_BITS_ZERO_TOP) != 0;
+    bits &= ~(DS_BITS_ZERO_TOP | DS_BITS_TOP_UNUSED);  // an unused top value needs no form of its own here
+    if (bits < 1 || bits > 6) return DS_EBITS;
+    if (base > 0 || base < -31) return DS_EBASE;
+    if (zero_top && (bits > 4 || base != 0)) return DS_EBITS;
+    if (M < 0 || K < 0 || N < 0 || F < 0 || F > 31 || I < 1 || I + F > 32) return DS_EINVAL;
+    if (mode != DS_Q_ROUND_TO_FIXED && mode != DS_Q_CAST) return DS_EINVAL;
+    if (M == 0 || N == 0) return DS_OK;
+    if (!tiled || !y || (!x && K > 0)) return DS_EINVAL;
+    if ((size_t)M * K * 4 >= ((size_t)1 << 31) || (size_t)M * N * 4 >= ((size_t)1 << 31)) return DS_ETOOLARGE;
+    if (ceil_div(M, kWave) > 65535) return DS_ETOOLARGE;
+    const TiledGeom g = tiled_geom(N, K, bits);
+    SmallArgs a;
+    a.x = x;
+    a.wt = (const uint32_t *)tiled;
+    a.negcnt = tiled_negcount(tiled, g);
+    a.bias = bias;
+    a.y = y;
+    a.M = M; a.K = K; a.N = N; a.comm = g.comm; a.nbase = -base;
+    a.out_scale = ldexpf(1.0f, F);
+    a.spec = make_spec(I, F, mode);
+    const int kernel_mode = zero_top ? 2 : (base != 0 || bits == 6) ? 1 : 0;
+    hipStream_t st = (hipStream_t)stream;
+    switch (bits) {
+    case 1: launch_small<1>(a, kernel_mode, st); break;
+    case 2: launch_small<2>(a, kernel_mode, st); break;
+    case 3: launch_small<3>(a, kernel_mode, st); break;
+    case 4: launch_small<4>(a, kernel_mode, st); break;
+    case 5: launch_small<5>(a, kernel_mode, st); break;
+    default: launch_small<6>(a, kernel_mode, st); break;
+    }
+    return launch_status();
+}

@@ -461,6 +461,41 @@ def linear_tiled(xT, M, tiled, bias, N, bits, base=0):
     return out
 
 
+# Below this many shift-add pairs a LinearShift layer is launch-bound on the tiled entry point (five
+# launches: conversion, pre-fill, GEMM, transpose, dequantisation) and runs as one launch instead.
+SMALL_LINEAR_PAIRS = 1 << 27
+
+
+def linear_small(x2d, tiled, bias, N, bits, base, integer_bits, fraction_bits, round_to_fixed):
+    """A whole LinearShift layer in one launch (``ds_linear_small_f32``): float32 ``[M, K]`` in, the
+    fixed-point conversion (modules.py:25 or utils.py:7-21), the shift GEMM on the tiled blob and
+    ``y.float() / 2**F`` (modules.py:30-31); returns float32 ``[M, N]``.  Bit-identical to
+    :func:`quantize_transpose` + :func:`linear_tiled` + :func:`dequantize`."""
+    x2d = x2d.contiguous()
+    if x2d.dtype != torch.float32 or not x2d.is_cuda or x2d.dim() != 2:
+        raise TypeError("linear_small expects a 2-D float32 GPU tensor")
+    if bias is not None:
+        bias = _require_device_i32("bias", bias)
+    M, K = x2d.shape
+    out = torch.empty([M, N], dtype=torch.float32, device=x2d.device)
+    with _Timed("linear", M, K, N, x2d.device):
+        _lib.call("ds_linear_small_f32", _lib.ptr(x2d), _lib.ptr(tiled), _lib.ptr(bias), _lib.ptr(out), M, K, N,
+                  int(bits), int(base), _lib.DS_Q_ROUND_TO_FIXED if round_to_fixed else _lib.DS_Q_CAST,
+                  int(integer_bits), int(fraction_bits), _lib.current_stream(x2d.device))
+    return out
+
+
+def linear_layer(x2d, tiled, bias, N, bits, base, integer_bits, fraction_bits, round_to_fixed):
+    """float32 ``[M, K]`` -> float32 ``[M, N]`` through the kernel path of a LinearShift layer: one
+    launch for small problems, conversion + tiled GEMM + dequantisation otherwise (same results)."""
+    M, K = x2d.shape
+    if M * K * N <= SMALL_LINEAR_PAIRS:
+        return linear_small(x2d, tiled, bias, N, bits, base, integer_bits, fraction_bits, round_to_fixed)
+    xT = quantize_transpose(x2d, integer_bits, fraction_bits, round_to_fixed=round_to_fixed)
+    out = linear_tiled(xT, M, tiled, bias, N, bits, base)
+    return dequantize(out, fraction_bits)
+
+
 def linear(input, shift, sign, bias=None, conc_weight=None, use_cuda=True):
     """``out[m, n] = bias[n] + sum_k sign[n,k] * (input[m,k] >> -shift[n,k])`` on packed weights.
 

@@ -155,18 +155,16 @@ class LinearShift(_PackedWeightsMixin, nn.Module):
         I, Fb = self.act_integer_bits, self.act_fraction_bits
         lead = input.shape[:-1]
         x2d = input.reshape(-1, self.in_features).float()
-        M = x2d.shape[0]
         if not self.use_cuda:
             shift, sign = module_codes(self)
             out = linear_cpu_forward(x2d, shift, sign, self.bias, I, Fb, round_to_fixed=False)
             return out.reshape(*lead, self.out_features)
         conc_weight = self.packed_weights()
-        xT = kernels.quantize_transpose(x2d, I, Fb, round_to_fixed=False)
         bias = self._fixed_bias.get(self.bias, I, Fb, round_to_fixed=False)
         tiled = kernels._tiled_of(conc_weight, self.out_features, self.in_features)
-        out = kernels.linear_tiled(xT, M, tiled, bias, self.out_features, kernels.kernel_bits(conc_weight),
-                                   conc_weight.base)
-        return kernels.dequantize(out, Fb).reshape(*lead, self.out_features)
+        out = kernels.linear_layer(x2d, tiled, bias, self.out_features, kernels.kernel_bits(conc_weight),
+                                   conc_weight.base, I, Fb, round_to_fixed=False)
+        return out.reshape(*lead, self.out_features)
 
     def forward(self, input):
         if self.use_kernel:

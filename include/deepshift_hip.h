@@ -210,6 +210,20 @@ int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled, const int
                         int32_t *y, int M, int K, int N, int bits, int base, void *workspace,
                         size_t workspace_bytes, ds_stream_t stream);
 
+/* A whole LinearShift layer as one launch, for small problems (a classifier at inference batch
+ * sizes, the MNIST MLP: launch-bound on the entry points above).  Replaces the kernel branch of
+ * LinearShift.forward (modules.py:24-31) and of LinearShiftQ.forward (modules_q.py:115-125):
+ *   x_fixed = (x * 2**F).int()                      [mode DS_Q_CAST; DS_Q_ROUND_TO_FIXED rounds and
+ *                                                    clamps to I.F first, utils.py:7-21]
+ *   y_fixed = bias + sum_k sgn * ((x_fixed >> field) << -base)      (kernels.py:10-26)
+ *   y       = y_fixed.float() / 2**F
+ * x[M][K] and y[M][N] float, contiguous; tiled: the blob of ds_tile_weights_i32 (or
+ * ds_tile_weights_zero_top_i32 with bits | DS_BITS_ZERO_TOP); bias int32 fixed point or NULL.  No
+ * workspace.  Results are those of ds_quantize_f32_i32 + ds_linear_i32 + ds_dequantize_i32_f32, bit for
+ * bit; any size is accepted, but above some 10^8 shift-add pairs the tiled entry point is faster. */
+int ds_linear_small_f32(const float *x, const void *tiled, const int32_t *bias, float *y, int M, int K,
+                        int N, int bits, int base, int mode, int I, int F, ds_stream_t stream);
+
 /* ds_linear_tiled_i32 for callers that cannot allocate (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc): no workspace argument; the partial-sum scratch lives in a
  * device array inside the library (ds_linear_tiled_noalloc_max_bytes() = 16 MiB per GPU, held until

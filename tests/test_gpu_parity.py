@@ -522,3 +522,93 @@ def test_top_unused_flag_is_ignored_where_it_does_not_apply(oracle, rng):
     np.testing.assert_array_equal(got.cpu().numpy(), want)
     one = ctypes.c_void_p(16)
     assert L.ds_linear_i32(one, one, None, one, 4, 4, 4, 4 | _lib.DS_BITS_TOP_UNUSED, 0, one, 1 << 20, None) == -2
+
+
+# ---- the one-launch LinearShift layer (ds_linear_small_f32) ----------------------------------------
+
+def abi_linear_small(x, blob, bias, N, bits, base, mode, I, F):
+    """ds_linear_small_f32 with canaries around the float output."""
+    M, K = x.shape
+    guard = 64
+    ybuf = torch.full((M * N + 2 * guard,), 12345.0, dtype=torch.float32, device=DEV)
+    y = ybuf[guard:guard + M * N]
+    xd = dev(x)
+    bd = None if bias is None else dev(bias)
+    _lib.call("ds_linear_small_f32", _lib.ptr(xd), _lib.ptr(blob), _lib.ptr(bd), ctypes.c_void_p(y.data_ptr()),
+              M, K, N, bits, base, mode, I, F, stream())
+    torch.cuda.synchronize()
+    host = ybuf.cpu().numpy()
+    assert (host[:guard] == 12345.0).all() and (host[guard + M * N:] == 12345.0).all(), "write outside the output"
+    return host[guard:guard + M * N].reshape(M, N)
+
+
+def _small_inputs(rng, M, K, F):
+    """float activations whose fixed-point images span the range, incl. values the clamp / the
+    saturating cast act on, negative values, exact grid points and +-0."""
+    x = (rng.standard_normal((M, K)) * 2.0 ** rng.integers(-F, 14, size=(M, K))).astype(np.float32)
+    flat = x.reshape(-1)
+    special = np.array([0.0, -0.0, 1.0, -1.0, 32767.99, -32768.0, 1e9, -1e9, 2.0 ** -F, -2.0 ** -F], np.float32)
+    n = min(len(special), flat.size)
+    flat[:n] = special[:n]
+    return x
+
+
+SMALL_SHAPES = [(64, 512, 1000), (1, 7, 3), (63, 100, 10), (65, 784, 512), (200, 96, 24), (256, 64, 10)]
+
+
+@pytest.mark.parametrize("bits", [1, 2, 3, 4, 5])
+@pytest.mark.parametrize("shape", SMALL_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_linear_small_matches_oracle_chain(oracle, rng, bits, shape):
+    """Conversion (cast, modules.py:25, and round_to_fixed, utils.py:7-21) + shift GEMM + y.float() / 2**F in
+    one launch, against the oracle's three steps."""
+    from deepshift_amd import kernels
+    M, K, N = shape
+    s, sign = random_codes(rng, (N, K), max_s=2 ** bits - 1)
+    bias = rng.integers(-2 ** 20, 2 ** 20, size=N).astype(np.int32)
+    blob = kernels.tile_weights(dev(so.np_pack_words(s, sign, bits)).reshape(-1), N, K, 1, 1, bits, 0)
+    for mode, (I, F) in [(_lib.DS_Q_CAST, (16, 16)), (_lib.DS_Q_ROUND_TO_FIXED, (16, 16)),
+                         (_lib.DS_Q_ROUND_TO_FIXED, (3, 5))]:
+        x = _small_inputs(rng, M, K, F)
+        xq = oracle.cast(x, F) if mode == _lib.DS_Q_CAST else oracle.quantize(x, I, F)
+        want = oracle.linear(xq, -s, sign, bias, NTHREADS).astype(np.float32) / np.float32(2.0 ** F)
+        np.testing.assert_array_equal(abi_linear_small(x, blob, bias, N, bits, 0, mode, I, F), want)
+        np.testing.assert_array_equal(abi_linear_small(x, blob, bias, N, bits | _lib.DS_BITS_TOP_UNUSED, 0, mode, I, F),
+                                      want)
+    want = oracle.linear(xq, -s, sign, None, NTHREADS).astype(np.float32) / np.float32(2.0 ** F)
+    np.testing.assert_array_equal(abi_linear_small(x, blob, None, N, bits, 0, mode, I, F), want)
+
+
+def test_linear_small_general_codes_and_zero_top(oracle, rng):
+    from deepshift_amd import kernels
+    M, K, N = 70, 45, 20
+    x = _small_inputs(rng, M, K, 16)
+    xq = oracle.cast(x, 16)
+    # 6-bit words with the reference's zero code (s = 32)
+    s, sign, s_z, sign_z = _ternary_case(rng, (N, K), 31)
+    blob = kernels.tile_weights(dev(so.np_pack_words(s_z, sign_z, 6)).reshape(-1), N, K, 1, 1, 6, 0)
+    want = oracle.linear(xq, -s, sign, None, NTHREADS).astype(np.float32) / np.float32(65536.0)
+    np.testing.assert_array_equal(abi_linear_small(x, blob, None, N, 6, 0, _lib.DS_Q_CAST, 16, 16), want)
+    # left shifts: base != 0
+    for bits, base in [(4, -3), (5, -7), (6, -2)]:
+        s2 = rng.integers(base, base + 2 ** min(bits, 5), size=(N, K)).astype(np.int32)
+        sg = rng.choice(np.array([-1, 1], np.int32), size=(N, K))
+        w2, ovf = oracle.pack_words(s2, sg, bits, base)
+        assert ovf == 0
+        blob = kernels.tile_weights(dev(w2).reshape(-1), N, K, 1, 1, bits, base)
+        want = so.np_linear_planes(xq, s2, sg, None, base).astype(np.float32) / np.float32(65536.0)
+        np.testing.assert_array_equal(abi_linear_small(x, blob, None, N, bits, base, _lib.DS_Q_CAST, 16, 16), want)
+    # ternary words re-packed so that the top field value means zero
+    for width in (1, 2, 4):
+        s, sign, s_z, sign_z = _ternary_case(rng, (N, K), 2 ** width - 2)
+        w6 = dev(so.np_pack_words(s_z, sign_z, 6))
+        blob = kernels.tile_weights_zero_top(w6.reshape(-1), N, K, 1, 1, width)
+        want = oracle.linear(xq, -s, sign, None, NTHREADS).astype(np.float32) / np.float32(65536.0)
+        got = abi_linear_small(x, blob, None, N, width | _lib.DS_BITS_ZERO_TOP, 0, _lib.DS_Q_CAST, 16, 16)
+        np.testing.assert_array_equal(got, want)
+    L = _lib.lib()
+    one = ctypes.c_void_p(16)
+    assert L.ds_linear_small_f32(one, one, None, one, 4, 4, 4, 7, 0, 0, 16, 16, None) == -2
+    assert L.ds_linear_small_f32(one, one, None, one, 4, 4, 4, 4, 1, 0, 16, 16, None) == -3
+    assert L.ds_linear_small_f32(one, one, None, one, -1, 4, 4, 4, 0, 0, 16, 16, None) == -1
+    assert L.ds_linear_small_f32(one, one, None, one, 4, 4, 4, 4, 0, 2, 16, 16, None) == -1
+    assert L.ds_linear_small_f32(None, None, None, None, 0, 4, 4, 4, 0, 0, 16, 16, None) == 0
