@@ -360,6 +360,81 @@ __global__ void requantize_affine_maxpool_kernel(const int32_t *__restrict__ y, 
     }
 }
 
+// The ResNet stem's case -- 3x3 window, stride 2, padding 1, even H and W -- with a third of the
+// loads: a thread fetches columns 2ow and 2ow + 1 of each of its three rows as one 8-byte load (a
+// wave's loads of a row are then contiguous) and takes column 2ow - 1 from the lane to its left,
+// which holds it as the second half of its own pair.  Only the first lane of a wave fetches that
+// column itself.  Rows and columns of index -1 (the pooling's implicit padding) are left out.
+template <typename Q>
+__global__ void requantize_affine_maxpool3s2_kernel(const int32_t *__restrict__ y, float *__restrict__ out,
+                                                    Q *__restrict__ q, const float *__restrict__ scale,
+                                                    const float *__restrict__ shift, uint32_t planes, int C,
+                                                    int H, int W, int OH, int OW, int ph, int pw, float inv,
+                                                    int relu, QuantSpec spec, FastDiv by_plane, FastDiv by_row,
+                                                    FastDiv by_channels)
+{
+    const uint32_t Hp = OH + 2 * ph, Wp = OW + 2 * pw;
+    const uint32_t total = planes * Hp * Wp;
+    const int lane = threadIdx.x & (kWave - 1);
+    // whole waves enter the loop together (the bound is rounded up to the wave), so that the lane to the
+    // left is always there to hand its value over; idx < total guards the stores
+    const uint32_t total_up = (total + kWave - 1) / kWave * kWave;
+    for (uint32_t idx0 = blockIdx.x * blockDim.x + threadIdx.x; idx0 < total_up; idx0 += gridDim.x * blockDim.x) {
+        const bool inside = idx0 < total;
+        const uint32_t idx = inside ? idx0 : total - 1;
+        const uint32_t plane = div_by(idx, by_plane);
+        const uint32_t rem = idx - plane * Hp * Wp;
+        const uint32_t hp = div_by(rem, by_row);
+        const int oh = (int)hp - ph, ow = (int)(rem - hp * Wp) - pw;
+        const bool interior = (unsigned)oh < (unsigned)OH && (unsigned)ow < (unsigned)OW;
+        // clamped coordinates keep every lane's loads inside the plane; what a border lane loads is
+        // never used (its right neighbour, if interior, has ow == 0 and no column to its left)
+        const int ohc = oh < 0 ? 0 : (oh >= OH ? OH - 1 : oh), owc = ow < 0 ? 0 : (ow >= OW ? OW - 1 : ow);
+        const int32_t *yp = y + (size_t)plane * H * W;
+        int2 pair[3];
+        int32_t left[3];
+#pragma unroll
+        for (int i = 0; i < 3; ++i) {
+            const int ih = 2 * ohc - 1 + i;
+            const int ihc = ih < 0 ? 0 : ih;
+            pair[i] = *(const int2 *)(yp + ihc * W + 2 * owc);
+        }
+#pragma unroll
+        for (int i = 0; i < 3; ++i) left[i] = __shfl_up(pair[i].y, 1);
+        if (lane == 0 && owc > 0) {
+#pragma unroll
+            for (int i = 0; i < 3; ++i) {
+                const int ih = 2 * ohc - 1 + i;
+                left[i] = yp[(ih < 0 ? 0 : ih) * W + 2 * owc - 1];
+            }
+        }
+        int32_t v = 0;
+        if (interior) {
+            const uint32_t c = plane - div_by(plane, by_channels) * (uint32_t)C;
+            const float a = scale ? scale[c] : 1.0f, b = shift ? shift[c] : 0.0f;
+            // affine_one is monotonic in y, so the window's maximum is affine_one of its largest int32
+            // (smallest, for a negative scale)
+            const bool flip = a < 0.0f;
+            int32_t ext = flip ? INT32_MAX : INT32_MIN;
+#pragma unroll
+            for (int i = 0; i < 3; ++i) {
+                if (i == 0 && oh == 0) continue;  // row -1
+                int32_t lo = pair[i].x < pair[i].y ? pair[i].x : pair[i].y;
+                int32_t hi = pair[i].x < pair[i].y ? pair[i].y : pair[i].x;
+                if (ow > 0) {
+                    lo = left[i] < lo ? left[i] : lo;
+                    hi = left[i] > hi ? left[i] : hi;
+                }
+                ext = flip ? (lo < ext ? lo : ext) : (hi > ext ? hi : ext);
+            }
+            const float best = affine_one(ext, inv, a, b, nullptr, relu);
+            if (out && inside) out[((size_t)plane * OH + oh) * OW + ow] = best;
+            v = quantize_one(best, spec);
+        }
+        if (q && inside) q[idx] = (Q)v;
+    }
+}
+
 __global__ void copy_kernel(const int4 *__restrict__ src, int4 *__restrict__ dst, long n4)
 {
     const long stride = (long)gridDim.x * blockDim.x;
@@ -582,6 +657,14 @@ static int requantize_affine_maxpool_any(const int32_t *y, float *out, Q *q, con
     if (total == 0) return DS_OK;
     if (total * 4 >= (1L << 31) || (long)Nb * C * H * W * 4 >= (1L << 31)) return DS_ETOOLARGE;
     if (!y || (!q && !out)) return DS_EINVAL;
+    if (pk == 3 && ps == 2 && pp == 1 && H == 2 * OH && W == 2 * OW && ((uintptr_t)y & 7) == 0) {
+        hipLaunchKernelGGL((requantize_affine_maxpool3s2_kernel<Q>), dim3(grid_for(total)), dim3(256), 0,
+                           (hipStream_t)stream, y, out, q, scale, shift, (uint32_t)(Nb * C), C, H, W, OH, OW, ph, pw,
+                           ldexpf(1.0f, -F_in), relu, make_spec(I, F, mode),
+                           fast_div((uint32_t)((OH + 2 * ph) * (OW + 2 * pw))), fast_div((uint32_t)(OW + 2 * pw)),
+                           fast_div((uint32_t)C));
+        return launch_status();
+    }
     hipLaunchKernelGGL((requantize_affine_maxpool_kernel<Q>), dim3(grid_for(total)), dim3(256), 0,
                        (hipStream_t)stream, y, out, q, scale, shift, (uint32_t)(Nb * C), C, H, W, OH, OW, pk,
                        ps, pp, ph, pw, ldexpf(1.0f, -F_in), relu, make_spec(I, F, mode),

@@ -339,8 +339,12 @@ def test_requantize_affine_pad_stays_inside_its_output(rng, dtype):
 
 def test_requantize_affine_maxpool_matches_the_three_passes(rng):
     import torch.nn.functional as F
+    # (even sizes with a 3x3 stride-2 padding-1 window take the pass that shares loads between lanes:
+    # rows of 18, 56 and 19 outputs put the wave boundaries at every column)
     for (Nb, C, H, W), pool, pad in [((2, 5, 12, 12), (3, 2, 1), (1, 1)), ((1, 3, 9, 7), (2, 2, 0), (0, 0)),
-                                     ((3, 4, 11, 13), (3, 1, 1), (2, 1)), ((1, 2, 5, 5), (5, 5, 2), (1, 1))]:
+                                     ((3, 4, 11, 13), (3, 1, 1), (2, 1)), ((1, 2, 5, 5), (5, 5, 2), (1, 1)),
+                                     ((2, 4, 40, 36), (3, 2, 1), (1, 1)), ((1, 2, 112, 112), (3, 2, 1), (0, 0)),
+                                     ((3, 3, 6, 38), (3, 2, 1), (0, 2))]:
         y = torch.from_numpy(rng.integers(-2 ** 27, 2 ** 27, size=(Nb, C, H, W)).astype(np.int32)).to(DEV)
         scale = torch.rand(C, device=DEV) - 0.3          # some channels flip the order of the values
         shift = torch.randn(C, device=DEV)
