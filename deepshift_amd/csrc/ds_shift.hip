@@ -186,50 +186,61 @@ __device__ __forceinline__ void accumulate_code_zero_top(int32_t (&acc)[R][J], c
     }
 }
 
+template <typename Q>
+__device__ __forceinline__ void write_padding(Q *q, size_t plane_base, int oh, int ow, int OH, int OW, int ph,
+                                              int pw, int Wq);
+__device__ __forceinline__ int32_t quantize_fixed(float v, float scale, float lo, float hi, bool one_bit);
+
+// The fused epilogue of the two-instruction kernel (launches without a K split: a lane holds the
+// finished sums of its R pixels x J channels): act(sum / 2^F * scale[c] + shift[c] + residual) stored as
+// float and / or as the next shift convolution's round-to-fixed, zero padded input -- the same
+// arithmetic, in the same order, as the cooperative kernel's write_tile.
+template <typename Q, int R, int J>
+__device__ __forceinline__ void fused_store(const ShiftArgs &p, const int32_t (&acc)[R][J], int n0,
+                                            const bool (&live)[R], const int (&img)[R], const int (&rem)[R])
+{
+    const int OW = p.OW, OH = p.pix_per_img / OW, ph = p.ep_ph, pw = p.ep_pw;
+    const int Wq = OW + 2 * pw;
+    const size_t qplane = (size_t)(OH + 2 * ph) * Wq;
+    float *out = p.ep_out;
+    Q *q = (Q *)p.ep_q;
+    const bool one_bit = p.ep_spec.I == 1;
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        const int n = n0 + j;
+        if (n >= p.N) break;
+        const int32_t add = p.negcnt[n] + (p.bias ? p.bias[n] : 0);
+        const float sa = p.ep_scale ? p.ep_scale[n] : 1.0f, sb = p.ep_shift ? p.ep_shift[n] : 0.0f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (!live[r]) continue;
+            const size_t o = ((size_t)img[r] * p.N + n) * p.pix_per_img + rem[r];
+            float f;
+            {
+#pragma clang fp contract(off)
+                f = ((float)(acc[r][j] + add) * p.ep_inv) * sa + sb;
+                if (p.ep_residual) f += p.ep_residual[o];
+                if (p.ep_relu) f = f > 0.0f ? f : 0.0f;
+            }
+            if (out) out[o] = f;
+            if (q) {
+                const int oh = rem[r] / OW, ow = rem[r] - oh * OW;
+                const size_t plane = ((size_t)img[r] * p.N + n) * qplane;
+                q[plane + (size_t)(oh + ph) * Wq + ow + pw] =
+                    (Q)quantize_fixed(f, p.ep_spec.scale, p.ep_spec.lo, p.ep_spec.hi, one_bit);
+                if ((ph | pw) && !p.ep_border_kept) write_padding(q, plane, oh, ow, OH, OW, ph, pw, Wq);
+            }
+        }
+    }
+}
+
+// K groups [g_begin, g_end) of the tile of channels ntile * J .. and the lane's R pixels (byte offsets
+// xoff), accumulated into acc: two vector instructions per term, codes decoded on the scalar ALU.
 template <int BITS, bool GENERAL, int R, int J>
-__global__ __launch_bounds__(256) void shift_kernel(const ShiftArgs p)
+__device__ __forceinline__ void shift_accumulate(const ShiftArgs &p, int32_t (&acc)[R][J], const uint32_t (&xoff)[R],
+                                                 int ntile, int g_begin, int g_end)
 {
     constexpr int NUM = 32 / (BITS + 1);
-    static_assert(kTileWords % J == 0, "the layout tile must hold whole channel tiles");
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-
-    // XCD-aware tile order: consecutive workgroup ids land on different XCDs, so give each XCD a
-    // contiguous range of tiles (neighbouring pixel tiles and all channel tiles of a pixel range
-    // then share one L2).
-    const int bid = blockIdx.x;
-    const int tile = (bid & 7) * p.blocks_per_xcd + (bid >> 3);
-    if (tile >= p.tiles_m4 * p.tiles_n) return;
-    const int ntile = tile % p.tiles_n;
-    const int mtile = (tile / p.tiles_n) * 4 + wave;
-    const int m0 = mtile * (R * kWave);
-    if (m0 >= p.M) return;
-
-    // per-lane pixel coordinates, as byte offsets (every tensor is < 2^31 bytes)
-    uint32_t xoff[R], yoff[R];
-    bool live[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        int m = m0 + r * kWave + lane;
-        live[r] = m < p.M;
-        if (!live[r]) m = p.M - 1;
-        const int img = m / p.pix_per_img;
-        const int rem = m - img * p.pix_per_img;
-        const int oh = rem / p.OW;
-        const int ow = rem - oh * p.OW;
-        xoff[r] = 4u * (uint32_t)(img * p.x_img_stride + oh * p.x_row_stride + ow * p.x_col_stride);
-        yoff[r] = 4u * (uint32_t)(img * p.y_img_stride + rem * p.y_pix_stride);
-    }
-
-    int32_t acc[R][J];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int j = 0; j < J; ++j) acc[r][j] = 0;
-
-    const int g_begin = blockIdx.y * p.groups_per_split;
-    int g_end = g_begin + p.groups_per_split;
-    if (g_end > p.comm) g_end = p.comm;
     const int full_groups = p.K / NUM;  // groups whose NUM codes are all real
     const int g_full_end = g_end < full_groups ? g_end : full_groups;
 
@@ -274,6 +285,53 @@ __global__ __launch_bounds__(256) void shift_kernel(const ShiftArgs p)
             accumulate_code<BITS, GENERAL, R, J>(acc, xt[i], w, i, p.nbase);
         }
     }
+}
+
+template <int BITS, bool GENERAL, int R, int J>
+__global__ __launch_bounds__(256) void shift_kernel(const ShiftArgs p)
+{
+    constexpr int NUM = 32 / (BITS + 1);
+    static_assert(kTileWords % J == 0, "the layout tile must hold whole channel tiles");
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+
+    // XCD-aware tile order: consecutive workgroup ids land on different XCDs, so give each XCD a
+    // contiguous range of tiles (neighbouring pixel tiles and all channel tiles of a pixel range
+    // then share one L2).
+    const int bid = blockIdx.x;
+    const int tile = (bid & 7) * p.blocks_per_xcd + (bid >> 3);
+    if (tile >= p.tiles_m4 * p.tiles_n) return;
+    const int ntile = tile % p.tiles_n;
+    const int mtile = (tile / p.tiles_n) * 4 + wave;
+    const int m0 = mtile * (R * kWave);
+    if (m0 >= p.M) return;
+
+    // per-lane pixel coordinates, as byte offsets (every tensor is < 2^31 bytes)
+    uint32_t xoff[R], yoff[R];
+    bool live[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        int m = m0 + r * kWave + lane;
+        live[r] = m < p.M;
+        if (!live[r]) m = p.M - 1;
+        const int img = m / p.pix_per_img;
+        const int rem = m - img * p.pix_per_img;
+        const int oh = rem / p.OW;
+        const int ow = rem - oh * p.OW;
+        xoff[r] = 4u * (uint32_t)(img * p.x_img_stride + oh * p.x_row_stride + ow * p.x_col_stride);
+        yoff[r] = 4u * (uint32_t)(img * p.y_img_stride + rem * p.y_pix_stride);
+    }
+
+    int32_t acc[R][J];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int j = 0; j < J; ++j) acc[r][j] = 0;
+
+    const int g_begin = blockIdx.y * p.groups_per_split;
+    int g_end = g_begin + p.groups_per_split;
+    if (g_end > p.comm) g_end = p.comm;
+    shift_accumulate<BITS, GENERAL, R, J>(p, acc, xoff, ntile, g_begin, g_end);
 
     // epilogue
     const int n0 = ntile * J;
@@ -310,6 +368,82 @@ __global__ __launch_bounds__(256) void shift_kernel(const ShiftArgs p)
 #include "ds_planes_asm.inc"
 
 typedef int32_t v16i __attribute__((ext_vector_type(16)));
+// The two-instruction kernel for layers that are narrower than the 64-channel form needs, launched
+// workgroup-cooperatively: a workgroup owns one tile of R x 64 pixels x J channels, its WAVES waves
+// split the tile's reduction (each keeps R pixels per lane, so a code's two scalar instructions serve
+// 2 R vector ones) and add their sums into an LDS tile; after a barrier each wave finishes J / WAVES
+// channels -- with the fused epilogue, or bias + sum as int32.  No K split across workgroups: no
+// pre-fill, no global atomics, and the conversion pass that followed such layers is gone.
+template <int BITS, int R, int J, int WAVES, bool FUSED>
+__global__ __launch_bounds__(WAVES * 64) void shift_coop_kernel(const ShiftArgs p)
+{
+    constexpr int CH = J / WAVES;
+    static_assert(J % WAVES == 0, "whole channels per wave in the write-out");
+    __shared__ int32_t sums[J][R * kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int bid = blockIdx.x;
+    const int tile = (bid & 7) * p.blocks_per_xcd + (bid >> 3);  // an XCD takes a contiguous range of tiles
+    if (tile >= p.tiles_m4 * p.tiles_n) return;                  // (tiles_m4: pixel tiles of this launch)
+    const int ntile = tile % p.tiles_n;
+    const int m0 = (tile / p.tiles_n) * (R * kWave);
+
+    uint32_t xoff[R];
+    bool live[R];
+    int img_of[R], rem_of[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        int m = m0 + r * kWave + lane;
+        live[r] = m < p.M;
+        if (!live[r]) m = p.M - 1;
+        const int img = m / p.pix_per_img;
+        const int rem = m - img * p.pix_per_img;
+        const int oh = rem / p.OW;
+        const int ow = rem - oh * p.OW;
+        img_of[r] = img;
+        rem_of[r] = rem;
+        xoff[r] = 4u * (uint32_t)(img * p.x_img_stride + oh * p.x_row_stride + ow * p.x_col_stride);
+    }
+    for (int i = threadIdx.x; i < J * R * kWave; i += WAVES * kWave) (&sums[0][0])[i] = 0;
+    __syncthreads();
+
+    int32_t acc[R][J];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int j = 0; j < J; ++j) acc[r][j] = 0;
+    const int g_begin = (int)((long)wave * p.comm / WAVES), g_end = (int)((long)(wave + 1) * p.comm / WAVES);
+    shift_accumulate<BITS, false, R, J>(p, acc, xoff, ntile, g_begin, g_end);
+#pragma unroll
+    for (int j = 0; j < J; ++j)
+#pragma unroll
+        for (int r = 0; r < R; ++r) atomicAdd(&sums[j][r * kWave + lane], acc[r][j]);
+    __syncthreads();
+
+    int32_t fin[R][CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+        for (int r = 0; r < R; ++r) fin[r][c] = sums[wave * CH + c][r * kWave + lane];
+    const int n0 = ntile * J + wave * CH;
+    if (FUSED) {
+        if (p.ep_q_bytes == 1) fused_store<int8_t, R, CH>(p, fin, n0, live, img_of, rem_of);
+        else fused_store<int32_t, R, CH>(p, fin, n0, live, img_of, rem_of);
+        return;
+    }
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int n = n0 + c;
+        if (n >= p.N) break;
+        const int32_t add = p.negcnt[n] + (p.bias ? p.bias[n] : 0);
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            if (live[r])
+                p.y[(size_t)img_of[r] * p.y_img_stride + (size_t)rem_of[r] * p.y_pix_stride + (size_t)n * p.y_ch_stride] =
+                    fin[r][c] + add;
+    }
+}
+
 typedef int32_t v32i __attribute__((ext_vector_type(32)));
 typedef int32_t v4i __attribute__((ext_vector_type(4)));
 
@@ -1065,6 +1199,34 @@ static void launch_fill(const ShiftArgs &a, hipStream_t st)
         hipLaunchKernelGGL(fill_bias_kernel, dim3((unsigned)blocks), dim3(256), 0, st, a);
 }
 
+// Tile shapes of the cooperative two-instruction kernel: up to 16 channels 4 pixel rows x 16 channels
+// on four waves, wider layers 2 x 32 on eight (64 accumulators per lane either way).
+static bool narrow_coop_small(const ShiftArgs &a) { return a.N <= 16; }
+static long narrow_coop_waves(const ShiftArgs &a)
+{
+    return narrow_coop_small(a) ? (long)ceil_div(a.M, 4 * kWave) * 4 : (long)ceil_div(a.M, 2 * kWave) * ceil_div(a.N, 32) * 8;
+}
+// Worth it where the waves fill the machine twice over and each gets at least two K groups.
+static bool narrow_coop_fits(const ShiftArgs &a)
+{
+    return narrow_coop_waves(a) >= 2L * 4 * device_cus() && a.comm >= 2 * (narrow_coop_small(a) ? 4 : 8);
+}
+
+template <int BITS, bool FUSED>
+static int launch_shift_coop(ShiftArgs a, hipStream_t st)
+{
+    const bool small = narrow_coop_small(a);
+    a.tiles_m4 = ceil_div(a.M, (small ? 4 : 2) * kWave);  // pixel tiles
+    a.tiles_n = ceil_div(a.N, small ? 16 : 32);
+    a.blocks_per_xcd = ceil_div(a.tiles_m4 * a.tiles_n, 8);
+    a.atomic_out = 0;
+    if (small)
+        hipLaunchKernelGGL((shift_coop_kernel<BITS, 4, 16, 4, FUSED>), dim3(a.blocks_per_xcd * 8), dim3(256), 0, st, a);
+    else
+        hipLaunchKernelGGL((shift_coop_kernel<BITS, 2, 32, 8, FUSED>), dim3(a.blocks_per_xcd * 8), dim3(512), 0, st, a);
+    return launch_status();
+}
+
 template <int BITS, bool GENERAL, int R, int J>
 static int launch_shift(ShiftArgs a, int nsplit, hipStream_t st)
 {
@@ -1256,10 +1418,8 @@ static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
         const bool wide = tiled_wide(a.N, a.K, BITS);  // decided by the shape alone, as at tiling time
         bool planes = plane_regime(a, wide) >= 0;
         if (g_tune.planes != kTuneUnset) planes = g_tune.planes > 0;
-        if (a.fused) {
-            if (!wide) return DS_EINVAL;
-            planes = true;
-        }
+        if (a.fused) planes = wide;  // the fused epilogue exists in the cooperative launch of the 64-channel
+                                     // form and in the two-instruction kernel below
         if (planes) {
             int nsplit = plane_regime(a, wide) > 0 ? 1 : 0;
             if (g_tune.split != kTuneUnset) nsplit = g_tune.split;
@@ -1277,7 +1437,10 @@ static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
                         : launch_planes<BITS, 0, false>(a, nsplit, st);
         }
     }
-    if (a.fused) return DS_EINVAL;  // general codes and 5-bit fields have no fused form
+    if (a.fused) {
+        if constexpr (!GENERAL && BITS <= 5) return launch_shift_coop<BITS, true>(a, st);
+        return DS_EINVAL;  // general codes have no fused form
+    }
     TileChoice c = choose_tile(a);
     if (g_tune.tile != kTuneUnset) { c.R = g_tune.tile / 100; c.J = g_tune.tile % 100; }
     if (g_tune.split != kTuneUnset) c.nsplit = g_tune.split;
@@ -1437,7 +1600,10 @@ static int conv2d_tiled_any(const int32_t *x, const void *tiled, const int32_t *
     a.top_unused = top_unused;
     take_coop_workspace(a, workspace, workspace_bytes, bits_in);
     if (fs) {
-        if (!a.coop_slots) return coop_bytes_for(M, (int)K, O, bits_in) ? DS_EWORKSPACE : DS_EINVAL;
+        // the 64-channel form finishes shared tiles through the workspace; other layers run the fused
+        // form of the two-instruction kernel, which needs none (ordinary codes of at most 5 bits only)
+        if (!a.coop_slots && coop_bytes_for(M, (int)K, O, bits_in)) return DS_EWORKSPACE;
+        if (!a.coop_slots && (zero_top || bits > 5)) return DS_EINVAL;
         if ((size_t)Nb * O * (OH + 2 * fs->ph) * (OW + 2 * fs->pw) * (size_t)fs->q_bytes >= kMaxBytes)
             return DS_ETOOLARGE;
         a.fused = 1;
@@ -1470,14 +1636,22 @@ DS_EXPORT int ds_conv2d_tiled_fusable(int Nb, int C, int Hp, int Wp, int O, int 
                                       int bits, int base)
 {
     const int width = bits & ~(DS_BITS_ZERO_TOP | DS_BITS_TOP_UNUSED);
-    if (base != 0 || width < 1 || width > 4) return 0;
-    if (ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits) == 0) return 0;
-    // where the dispatch would launch cooperatively anyway: long reductions on few tiles
+    if (base != 0 || width < 1 || width > 5) return 0;
+    if (Nb <= 0 || C <= 0 || O <= 0 || FH < 1 || FW < 1 || sh < 1 || sw < 1 || Hp < FH || Wp < FW) return 0;
     ShiftArgs a{};
     a.M = Nb * ((Hp - FH) / sh + 1) * ((Wp - FW) / sw + 1);
     a.N = O;
     a.K = C * FH * FW;
     a.comm = ceil_div(a.K, codes_per_word(width));
+    if (ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits) == 0) {
+        // not the 64-channel form: where the dispatch picks the two-instruction kernel anyway and its
+        // cooperative launch fills the machine, that launch with the fused epilogue saves the pre-fill,
+        // the atomics and the conversion pass (ResNet-20's 16- and 32-channel layers)
+        if (bits & DS_BITS_ZERO_TOP) return 0;
+        const bool two_instruction = width == 5 || plane_regime(a, false) < 0;
+        return two_instruction && narrow_coop_fits(a);
+    }
+    // where the dispatch would launch cooperatively anyway: long reductions on few tiles
     return a.comm >= 64 && plane_regime(a, true) == 0;
 }
 
@@ -1498,7 +1672,7 @@ DS_EXPORT int ds_conv2d_tiled_fused_i32(const int32_t *x, const void *tiled, con
     } else {
         I = 16; F = 16; q_bytes = 4; ph = pw = 0;
     }
-    if (!ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits) || base != 0) return DS_EINVAL;
+    if (base != 0) return DS_EINVAL;
     FusedSpec fs{out, q, scale, shift, residual, F_in, relu, I, F, ph, pw, q_bytes, border_kept};
     return conv2d_tiled_any(x, tiled, bias, nullptr, &fs, Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits, base, workspace,
                             workspace_bytes, stream);

@@ -292,11 +292,16 @@ int ds_cpu_conv2d_i32(const int32_t *x_padded, const int8_t *shift, const int32_
  * layers, and the next layer's round_to_fixed + cast + padding (modules.py:317,:153, kernels.py:32-36):
  * bit-identical to ds_conv2d_tiled_i32 followed by ds_requantize_affine_pad_i32 / _i8.  q_bytes 4:
  * q is int32; 1: int8 (2 <= I, I + F <= 8); | DS_Q_BORDER_KEPT: the caller vouches that the padding of
- * q already holds zeros (a buffer it zeroed once and reuses), and the kernel writes the interior only.  scale, shift, residual may be NULL.  base must be 0.
- * Needs the workspace of ds_conv2d_tiled_workspace_bytes() (DS_EWORKSPACE without it) and a layer
- * the cooperative launch serves: O a multiple of 64, fields of at most 4 bits (DS_EINVAL otherwise);
- * ds_conv2d_tiled_fusable() says whether the fused call is also the faster choice for a shape (long
- * reductions; short ones lose more in the launch form than the separate pass costs).
+ * q already holds zeros (a buffer it zeroed once and reuses), and the kernel writes the interior only.
+ * scale, shift, residual may be NULL.  base must be 0.
+ * Layers of the 64-channel form (O a multiple of 64, fields of at most 4 bits) run the cooperative
+ * launch of the shift-plane kernel and need the workspace of ds_conv2d_tiled_workspace_bytes()
+ * (DS_EWORKSPACE without it).  Other layers (ordinary codes of at most 5 bits; DS_EINVAL for 6-bit
+ * fields and zero-top blobs) run the cooperative launch of the two-instruction kernel, which needs no
+ * workspace.  ds_conv2d_tiled_fusable() says whether the fused call is also the faster choice for a
+ * shape (64-channel form: long reductions -- short ones lose more in the launch form than the
+ * separate pass costs; other layers: where the dispatch would pick the two-instruction kernel anyway
+ * and the launch fills the machine).
  * No counterpart in the reference. */
 #define DS_Q_BORDER_KEPT 0x100
 int ds_conv2d_tiled_fusable(int Nb, int C, int Hp, int Wp, int O, int FH, int FW, int sh, int sw,

@@ -52,8 +52,8 @@ def abi_conv_fused(xp, blob, bias, O, FH, FW, stride, bits, F_in, scale, shift, 
     OH, OW = (Hp - FH) // sh + 1, (Wp - FW) // sw + 1
     L = _lib.lib()
     ws_bytes = L.ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits)
-    assert ws_bytes > 0
-    ws = torch.full((ws_bytes,), 0x77, dtype=torch.uint8, device=DEV)
+    assert ws_bytes > 0 or O % 64 != 0      # the 64-channel form needs the workspace, other layers none
+    ws = torch.full((max(ws_bytes, 1),), 0x77, dtype=torch.uint8, device=DEV)
     guard = 64
     n_out = Nb * O * OH * OW
     obuf = torch.full((n_out + 2 * guard,), 12345.0, dtype=torch.float32, device=DEV)
@@ -72,8 +72,8 @@ def abi_conv_fused(xp, blob, bias, O, FH, FW, stride, bits, F_in, scale, shift, 
     _lib.call("ds_conv2d_tiled_fused_i32", _lib.ptr(xd), _lib.ptr(blob), _lib.ptr(t[0]),
               None if out is None else ctypes.c_void_p(out.data_ptr()),
               None if q is None else ctypes.c_void_p(q.data_ptr()), _lib.ptr(t[1]), _lib.ptr(t[2]), _lib.ptr(t[3]),
-              Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits, 0, F_in, int(relu), I, Fq, ph, pw, qb, _lib.ptr(ws), ws_bytes,
-              _stream())
+              Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits, 0, F_in, int(relu), I, Fq, ph, pw, qb,
+              _lib.ptr(ws) if ws_bytes else None, ws_bytes, _stream())
     torch.cuda.synchronize()
     oh = obuf.cpu().numpy()
     assert (oh[:guard] == 12345.0).all() and (oh[guard + n_out:] == 12345.0).all(), "write outside out"
@@ -97,6 +97,13 @@ GEOMS = [
     (3, 128, 16, 15, 192, 3, 3, (2, 2)),     # strided, three channel tiles
     (5, 384, 12, 12, 64, 1, 1, (1, 1)),      # 1x1 with a long reduction (64 K groups)
     (2, 40, 21, 19, 64, 5, 3, (1, 2)),       # 5x3 filter, K = 600
+]
+# layers that are not a multiple of 64 channels wide: the fused form of the two-instruction kernel
+NARROW_GEOMS = [
+    (3, 16, 34, 34, 16, 3, 3, (1, 1)),       # ResNet-20's first stage
+    (2, 16, 34, 33, 32, 3, 3, (2, 2)),       # strided, 32 channels, ragged pixel count
+    (2, 7, 11, 13, 40, 3, 2, (1, 1)),        # 40 channels: a partial channel tile, K = 42
+    (5, 32, 10, 10, 10, 1, 1, (1, 1)),       # 1x1, fewer channels than a tile holds
 ]
 
 
@@ -178,7 +185,7 @@ def test_cooperative_launch_replays_in_a_graph(oracle, rng):
             np.testing.assert_array_equal(y.cpu().numpy(), want, err_msg="eager after replay %d" % step)
 
 
-@pytest.mark.parametrize("geom", GEOMS, ids=lambda g: "x".join(str(v) for v in g[:7]))
+@pytest.mark.parametrize("geom", GEOMS + NARROW_GEOMS, ids=lambda g: "x".join(str(v) for v in g[:7]))
 def test_fused_epilogue_matches_oracle_chain(oracle, rng, geom):
     """Float and fixed-point outputs of the fused call against oracle.conv2d -> np_dequantize_affine ->
     np_requantize, for every combination of what may follow the layer."""
@@ -243,14 +250,20 @@ def test_fused_entry_point_refuses_what_it_cannot_do(rng):
     args = lambda O, bits, base, ws: (one, one, None, one, None, None, None, None, 2, 64, 30, 30, O, 3, 3, 1, 1,
                                       bits, base, 16, 0, 16, 16, 0, 0, 4, one if ws else None, 1 << 30 if ws else 0,
                                       None)
-    assert L.ds_conv2d_tiled_fused_i32(*args(48, 4, 0, True)) == -1     # not a multiple of 64 channels
-    assert L.ds_conv2d_tiled_fused_i32(*args(64, 5, 0, True)) == -1     # 5-bit fields
+    Z = _lib.DS_BITS_ZERO_TOP
+    assert L.ds_conv2d_tiled_fused_i32(*args(48, 6, 0, True)) == -1     # 6-bit (general) codes
+    assert L.ds_conv2d_tiled_fused_i32(*args(48, 4 | Z, 0, True)) == -1  # zero-top blob on a narrow layer
     assert L.ds_conv2d_tiled_fused_i32(*args(64, 4, -1, True)) == -1    # left shifts
-    assert L.ds_conv2d_tiled_fused_i32(*args(64, 4, 0, False)) == -4    # no workspace
+    assert L.ds_conv2d_tiled_fused_i32(*args(64, 4, 0, False)) == -4    # 64-channel form without its workspace
     assert L.ds_conv2d_tiled_fusable(64, 64, 58, 58, 64, 3, 3, 1, 1, 4 | U, 0) == 1
-    assert L.ds_conv2d_tiled_fusable(64, 64, 58, 58, 64, 3, 3, 1, 1, 5, 0) == 0
-    assert L.ds_conv2d_tiled_fusable(64, 64, 58, 58, 48, 3, 3, 1, 1, 4, 0) == 0
-    assert L.ds_conv2d_tiled_fusable(64, 64, 56, 56, 128, 1, 1, 2, 2, 4, 0) == 0   # short reduction
+    assert L.ds_conv2d_tiled_fusable(64, 64, 56, 56, 128, 1, 1, 2, 2, 4, 0) == 0   # short reduction, 64-channel form
+    # layers the two-instruction kernel serves: fused there when single pixel rows fill the machine
+    assert L.ds_conv2d_tiled_fusable(64, 64, 58, 58, 64, 3, 3, 1, 1, 5, 0) == 1
+    assert L.ds_conv2d_tiled_fusable(64, 64, 58, 58, 48, 3, 3, 1, 1, 4, 0) == 1
+    assert L.ds_conv2d_tiled_fusable(256, 16, 34, 34, 16, 3, 3, 1, 1, 4 | U, 0) == 1
+    assert L.ds_conv2d_tiled_fusable(1, 16, 34, 34, 16, 3, 3, 1, 1, 4, 0) == 0     # 16 waves of pixels
+    assert L.ds_conv2d_tiled_fusable(64, 64, 58, 58, 48, 3, 3, 1, 1, 6, 0) == 0
+    assert L.ds_conv2d_tiled_fusable(64, 64, 58, 58, 48, 3, 3, 1, 1, 4, -2) == 0
 
 
 def test_fused_module_path_equals_the_separate_passes():
