@@ -593,8 +593,9 @@ def main():
         "data": "synthetic",
         "config": {"workload": "ResNet-18, batch 64 x 3x224x224, all 20 conv + FC as shift layers "
                                "(benchmark configuration 4); weight_bits 5 (4-bit shift + sign, 6 codes per "
-                               "word), activations 16.16; BatchNorm/residual/ReLU folded into each "
-                               "conv's dequantisation pass, pooling fp32 PyTorch",
+                               "word), activations 16.16; BatchNorm, residual, ReLU and the next layer's "
+                               "fixed-point conversion in each convolution's epilogue, the stem's max "
+                               "pooling in one conversion pass, global average pooling fp32 PyTorch",
                    "batch": BATCH, "shift_layers": 21, "shift_launches": len(layers), "pairs_per_step": pairs},
         "unfused_images_per_s": BATCH / sec_unfused,
         "shift_kernel_ms_per_step": kernel_s * 1e3,
