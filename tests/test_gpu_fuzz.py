@@ -76,3 +76,38 @@ def test_random_ternary_layers_through_compress_bits(oracle, seed):
     want = oracle.linear(x, -s, sign, None, nthreads=NTHREADS)
     got = kernels.linear(dev(x), torch.from_numpy(-s).float(), torch.from_numpy(sign).float(), None, cw)
     np.testing.assert_array_equal(got.cpu().numpy(), want, err_msg=str((width, M, K, N)))
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_random_fused_convolutions(oracle, seed):
+    """ds_conv2d_tiled_fused_i32 on random geometries -- multiples of 64 channels (cooperative shift-plane
+    launch, shared tiles through the workspace) and narrower layers (cooperative two-instruction launch) --
+    against the oracle's chain: sums, dequantisation, affine, residual, ReLU, round-to-fixed, padding."""
+    from tests.test_gpu_fused import abi_conv_fused
+    rng = np.random.default_rng(4000 + seed)
+    bits = int(rng.integers(2, 5))
+    FH, FW = int(rng.integers(1, 5)), int(rng.integers(1, 5))
+    sh, sw = int(rng.integers(1, 3)), int(rng.integers(1, 3))
+    Nb = int(rng.integers(1, 6))
+    C = int(rng.choice([3, 16, 40, 64, 130]))
+    O = int(rng.choice([8, 16, 32, 48, 64, 128]))
+    Hp, Wp = FH + int(rng.integers(0, 36)), FW + int(rng.integers(0, 36))
+    OH, OW = (Hp - FH) // sh + 1, (Wp - FW) // sw + 1
+    xp = rng.integers(-2 ** 17, 2 ** 19, size=(Nb, C, Hp, Wp)).astype(np.int32)
+    s, sign = random_codes(rng, (O, C, FH, FW), max_s=2 ** bits - 2)
+    bias = rng.integers(-2 ** 16, 2 ** 16, size=O).astype(np.int32) if seed % 2 else None
+    y = oracle.conv2d(xp, -s, sign, bias, (sh, sw), nthreads=NTHREADS)
+    blob = kernels.tile_weights(dev(so.np_pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)).reshape(-1),
+                                O, C, FH, FW, bits, 0)
+    scale = ((rng.random(O) + 0.5) * 2.0 ** -6).astype(np.float32)
+    shift = rng.standard_normal(O).astype(np.float32)
+    res = (rng.standard_normal((Nb, O, OH, OW)) * 2).astype(np.float32) if seed % 3 else None
+    relu = bool(seed % 4)
+    emit = [(1, 1, 16, 16, torch.int32), (0, 0, 16, 16, torch.int32), (2, 1, 3, 5, torch.int8), None][seed % 4]
+    v = so.np_dequantize_affine(y, 16, scale, shift, res, relu)
+    flag = bits | _lib.DS_BITS_TOP_UNUSED
+    out, q = abi_conv_fused(xp, blob, bias, O, FH, FW, (sh, sw), flag, 16, scale, shift, res, relu, True, emit)
+    msg = str((bits, Nb, C, Hp, Wp, O, FH, FW, sh, sw))
+    np.testing.assert_array_equal(out, v, err_msg=msg)
+    if emit is not None:
+        np.testing.assert_array_equal(q, so.np_requantize(v, emit[2], emit[3], emit[:2]), err_msg=msg)
