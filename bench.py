@@ -489,6 +489,8 @@ def main():
                     help="skip config 2 and the VALU calibration (clean kernel-trace profiles)")
     ap.add_argument("--config5-only", action="store_true",
                     help="only benchmark configuration 5 (ResNet-50, 8-bit activations); prints its JSON object")
+    ap.add_argument("--config3-only", action="store_true",
+                    help="only benchmark configuration 3 (ResNet-20, batch 256); prints its JSON object")
     ap.add_argument("--pmc-target", action="store_true",
                     help="only launch the counter targets: a 64 MiB copy kernel and the dominant shift "
                          "kernel (ResNet-18 layer1 3x3 conv, batch 64), 3 times each")
@@ -505,6 +507,9 @@ def main():
         return
     if args.config5_only:
         print(json.dumps(config5(device, args.steps)), flush=True)
+        return
+    if args.config3_only:
+        print(json.dumps(config3(device, args.steps)), flush=True)
         return
 
     from deepshift_amd import workloads
