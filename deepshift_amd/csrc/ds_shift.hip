@@ -789,15 +789,43 @@ typedef __attribute__((address_space(3))) const TileTail lds_tail;
 
 // round_to_fixed + cast of the fused epilogue without branches: the clamp keeps the value inside int32,
 // so only NaN (propagated by the clamp, as torch.clamp does) needs the conversion's "NaN -> 0".
-__device__ __forceinline__ int32_t quantize_fixed(float v, float scale, float lo, float hi, bool one_bit)
+template <bool ONE_BIT>
+__device__ __forceinline__ int32_t quantize_fixed_as(float v, float scale, float lo, float hi)
 {
     // max / min drop a NaN operand; the select on v == v puts "NaN -> 0" back
     float r = __builtin_fminf(__builtin_fmaxf(floorf(v * scale), lo), hi);
-    if (one_bit) {  // integer_bits == 1: sign(x) - 1 (utils.py:12-13)
+    if (ONE_BIT) {  // integer_bits == 1: sign(x) - 1 (utils.py:12-13)
         const float s = ((v > 0.0f) ? 1.0f : ((v < 0.0f) ? -1.0f : 0.0f)) - 1.0f;
         r = s * scale;
     }
     return (int32_t)((v == v) ? r : 0.0f);
+}
+__device__ __forceinline__ int32_t quantize_fixed(float v, float scale, float lo, float hi, bool one_bit)
+{
+    return one_bit ? quantize_fixed_as<true>(v, scale, lo, hi) : quantize_fixed_as<false>(v, scale, lo, hi);
+}
+
+// The float value of a finished tile's sums held by one lane (CH channels x R pixel rows), with what may
+// follow the layer chosen at compile time: the callers branch once, on wave-uniform flags, instead of
+// selecting per element.
+template <int CH, int R, bool HAS_RES, bool RELU>
+__device__ __forceinline__ void tile_affine(float (&f)[CH][R], const int32_t (&sums)[CH][R], const float (&res)[CH][R],
+                                            int32_t add_l, float sa_l, float sb_l, float inv)
+{
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int32_t add = __builtin_amdgcn_readlane(add_l, c);
+        const float sa = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sa_l), c));
+        const float sb = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sb_l), c));
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+#pragma clang fp contract(off)
+            float v = ((float)(sums[c][r] + add) * inv) * sa + sb;
+            if (HAS_RES) v += res[c][r];
+            if (RELU) v = v > 0.0f ? v : 0.0f;
+            f[c][r] = v;
+        }
+    }
 }
 
 // The zero padding of the next layer's input around this tile's pixels: the pixels on an image edge
@@ -920,32 +948,33 @@ __device__ __forceinline__ void write_tile(lds_tail *t, lds_i32 *buf, int ntile,
     const float inv = uniform(t->inv), qs = uniform(t->spec.scale), qlo = uniform(t->spec.lo), qhi = uniform(t->spec.hi);
     const bool relu = uniform(t->relu) != 0, one_bit = uniform(t->spec.I) == 1, has_res = residual != nullptr;
     float f[CH][R];
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        const int32_t add = __builtin_amdgcn_readlane(add_l, c);
-        const float sa = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sa_l), c));
-        const float sb = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sb_l), c));
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-#pragma clang fp contract(off)
-            float v = ((float)(sums[c][r] + add) * inv) * sa + sb;
-            if (has_res) v += res[c][r];
-            if (relu) v = v > 0.0f ? v : 0.0f;
-            f[c][r] = v;
-        }
+    if (has_res) {
+        if (relu) tile_affine<CH, R, true, true>(f, sums, res, add_l, sa_l, sb_l, inv);
+        else tile_affine<CH, R, true, false>(f, sums, res, add_l, sa_l, sb_l, inv);
+    } else {
+        if (relu) tile_affine<CH, R, false, true>(f, sums, res, add_l, sa_l, sb_l, inv);
+        else tile_affine<CH, R, false, false>(f, sums, res, add_l, sa_l, sb_l, inv);
     }
+    const uint32_t ostep = 4u * (uint32_t)pix_per_img, qstep = (uint32_t)sizeof(Q) * qplane;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         if (!live[r]) continue;
         if (out) {
+            uint32_t o = 4u * pix[r];
 #pragma unroll
-            for (int c = 0; c < CH; ++c) *(g_f32 *)(out + 4u * (pix[r] + (uint32_t)(c * pix_per_img))) = f[c][r];
+            for (int c = 0; c < CH; ++c, o += ostep) *(g_f32 *)(out + o) = f[c][r];
         }
         if (q) {
+            uint32_t o = (uint32_t)sizeof(Q) * qpix[r];
+            if (one_bit) {
 #pragma unroll
-            for (int c = 0; c < CH; ++c)
-                *(g_q *)(q + (uint32_t)sizeof(Q) * (qpix[r] + (uint32_t)c * qplane)) =
-                    (Q)quantize_fixed(f[c][r], qs, qlo, qhi, one_bit);
+                for (int c = 0; c < CH; ++c, o += qstep)
+                    *(g_q *)(q + o) = (Q)quantize_fixed_as<true>(f[c][r], qs, qlo, qhi);
+            } else {
+#pragma unroll
+                for (int c = 0; c < CH; ++c, o += qstep)
+                    *(g_q *)(q + o) = (Q)quantize_fixed_as<false>(f[c][r], qs, qlo, qhi);
+            }
         }
     }
     if (q && (ph | pw) && !uniform(t->border_kept)) {
