@@ -45,7 +45,7 @@ struct Tune {
     int planes = kTuneUnset;  // 0 / 1: two-instruction kernel / shift-plane kernel
     int split = kTuneUnset;   // K split (plane kernels: 0 = equal shares, 1 = one tile per wave, -r = r x shares)
     int tile = kTuneUnset;    // R * 100 + J of the two-instruction kernel
-    int cu = kTuneUnset;      // 0 / 4 / 8: cooperative launch off / four / eight waves per workgroup
+    int cu = kTuneUnset;      // 0 / 4: workgroup-cooperative launch off / on (four waves per workgroup)
     int notail = kTuneUnset;  // int8 kernel: keep the last round of tiles on the tile-per-wave launch
 };
 extern Tune g_tune;
