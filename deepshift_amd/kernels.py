@@ -60,6 +60,18 @@ def set_timing_sink(sink):
     _TIMING_SINK = sink
 
 
+_REPLAY_SINK = None
+
+
+def set_replay_sink(sink):
+    """Measurement hook: when ``sink`` is a list, every fused shift-convolution call appends
+    ``(kind, M, K, N, replay)`` to it, where ``replay()`` issues the same launch again (same tensors, same
+    workspace, current stream): a benchmark can then time a run of back-to-back launches between two
+    events instead of bracketing each one.  ``None`` switches the hook off (the default)."""
+    global _REPLAY_SINK
+    _REPLAY_SINK = sink
+
+
 class _Timed:
     def __init__(self, kind, M, K, N, device):
         self.meta = (kind, M, K, N)
@@ -596,11 +608,19 @@ def conv2d_tiled_fused(x_padded, tiled, bias, O, kernel_size, stride, bits, frac
     L = _lib.lib()
     ws_bytes = L.ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, int(bits))
     ws = _workspace(ws_bytes, dev)
-    with _Timed("conv", Nb * OH * OW, C * FH * FW, O, dev):
-        _lib.call("ds_conv2d_tiled_fused_i32", _lib.ptr(x_padded), _lib.ptr(tiled), _lib.ptr(bias), _lib.ptr(out),
-                  _lib.ptr(q), _lib.ptr(scale), _lib.ptr(shift), _lib.ptr(residual), Nb, C, Hp, Wp, O, FH, FW,
+    keep = (x_padded, tiled, bias, out, q, scale, shift, residual, ws)
+
+    def launch():
+        t = keep
+        _lib.call("ds_conv2d_tiled_fused_i32", _lib.ptr(t[0]), _lib.ptr(t[1]), _lib.ptr(t[2]), _lib.ptr(t[3]),
+                  _lib.ptr(t[4]), _lib.ptr(t[5]), _lib.ptr(t[6]), _lib.ptr(t[7]), Nb, C, Hp, Wp, O, FH, FW,
                   sh, sw, int(bits), 0, int(fraction_bits_in), int(bool(relu)), int(I), int(Fq), ph, pw, qb,
-                  _lib.ptr(ws), ws_bytes, _lib.current_stream(dev))
+                  _lib.ptr(t[8]) if ws_bytes else None, ws_bytes, _lib.current_stream(dev))
+
+    with _Timed("conv", Nb * OH * OW, C * FH * FW, O, dev):
+        launch()
+    if _REPLAY_SINK is not None:
+        _REPLAY_SINK.append(("conv", Nb * OH * OW, C * FH * FW, O, launch))
     return out, q
 
 
