@@ -76,7 +76,7 @@ struct ShiftArgs {
     float ep_inv;                         // 2^-F of the sums
     int ep_relu, ep_ph, ep_pw, ep_q_bytes;
     int ep_border_kept;                   // the padding of q already holds zeros: write the interior only
-    int whole_tile_shares;                // cooperative launch: shares end on tile boundaries, tiles go one per wave
+    int whole_tile_shares;                // cooperative launch: rounds of whole tiles, one per wave, before the shared space
     QuantSpec ep_spec;
 };
 
@@ -1100,26 +1100,33 @@ void shift_planes_wide_coop_kernel(const ShiftArgs p, const ShiftArgs p2)
     const long total = (long)p.tiles_m4 * span;
     long it = w * total / G;
     long it_end = (w + 1) * total / G;
+    // Many short tiles per workgroup (a 7x7 stem: 12 tiles of 25 K groups): every workgroup first takes
+    // the same whole number of rounds of four tiles, one tile per wave, straight from the accumulators to
+    // the output -- no K split, no LDS, no barrier.  The tiles left over (fewer than four per workgroup)
+    // form the shared space that follows: equal shares of their (tile, K group) iterations, like any other
+    // launch, so that no workgroup carries a whole tile more than its neighbours.
+    long shared_base = 0, shared_total = total, direct_at = 0;
+    int direct_rounds = 0;
     if (!FUSED && !PAIR && p.whole_tile_shares) {
-        // shares in whole tiles: no tile is shared between workgroups
-        const long tiles = total / p.comm;
-        it = (w * tiles / G) * p.comm;
-        it_end = ((w + 1) * tiles / G) * p.comm;
+        const long per_group = ((total / p.comm) / G) & ~(long)(kCoopWaves - 1);  // direct tiles per workgroup
+        direct_rounds = (int)(per_group / kCoopWaves);
+        direct_at = w * per_group * p.comm;
+        shared_base = G * per_group * p.comm;
+        shared_total = total - shared_base;
+        it = w * shared_total / G;              // from here on relative to shared_base
+        it_end = (w + 1) * shared_total / G;
     }
     if (threadIdx.x == 0) {
-        fill_tail(tail[0], p, G, total);
-        if (PAIR) fill_tail(tail[1], p2, G, total);
+        fill_tail(tail[0], p, G, shared_total);
+        if (PAIR) fill_tail(tail[1], p2, G, shared_total);
     }
     for (int i = threadIdx.x; i < kCoopTileElems; i += THREADS) tile_sums[i] = 0;
     __syncthreads();
-    while (it < it_end) {
-        // Many short tiles per workgroup (a 7x7 stem: 12 tiles of 25 K groups): rounds of four whole
-        // tiles go one per wave, straight from the accumulators to the output -- no K split, no LDS, no
-        // barrier; the up to three tiles left over of a share are split over the waves like any other.
-        // (One call of the segment code serves both: a second copy of the main loop in this kernel
-        // leaves the register allocator no room.)
-        const bool direct = !FUSED && !PAIR && p.whole_tile_shares && (it_end - it) / p.comm >= kCoopWaves;
-        const long at = direct ? it + (long)wave * p.comm : it;
+    while (direct_rounds > 0 || it < it_end) {
+        // (One call of the segment code serves the direct tiles and the shared ones: a second copy of the
+        // main loop in this kernel leaves the register allocator no room.)
+        const bool direct = direct_rounds > 0;
+        const long at = direct ? direct_at + (long)wave * p.comm : shared_base + it;
         const int mtile = (int)(at / span);
         const int within = (int)(at - (long)mtile * span);
         const bool second = PAIR && within >= span1;
@@ -1127,11 +1134,11 @@ void shift_planes_wide_coop_kernel(const ShiftArgs p, const ShiftArgs p2)
         const int ntile = (second ? within - span1 : within) / comm;
         const long tile_start = (long)mtile * span + (second ? span1 : 0) + (long)ntile * comm;
         const int g0 = (int)(at - tile_start);
-        long g1 = g0 + (it_end - at);
+        long g1 = direct ? comm : g0 + (it_end - it);
         if (g1 > comm) g1 = comm;
         const int m0 = mtile * kCoopPix;
         const int len = (int)g1 - g0;
-        // direct: g0 == 0 and len == comm (shares of whole tiles), the wave takes all of it
+        // direct: g0 == 0 and len == comm, the wave takes all of it
         const int wb = direct ? 0 : g0 + wave * len / kCoopWaves;
         const int we = direct ? comm : g0 + (wave + 1) * len / kCoopWaves;
         if (wb < we) {
@@ -1140,12 +1147,14 @@ void shift_planes_wide_coop_kernel(const ShiftArgs p, const ShiftArgs p2)
                                                                         direct ? nullptr : tile_sums);
         }
         if (direct) {
-            it += (long)kCoopWaves * p.comm;
+            direct_at += (long)kCoopWaves * p.comm;
+            --direct_rounds;
             continue;
         }
         __syncthreads();
+        // (the exchange works in the coordinates of the shared space)
         coop_finish_tile<FUSED>((lds_tail *)&tail[second ? 1 : 0], (lds_i32 *)tile_sums, (lds_i32 *)&last_arrival, w,
-                                tile_start, g0, len, ntile, m0);
+                                tile_start - shared_base, g0, len, ntile, m0);
         it += len;
     }
 }
@@ -1333,9 +1342,10 @@ static int launch_planes(ShiftArgs a, int nsplit, hipStream_t st)
         // is long enough to carry the extra segment ends: from 64 K groups per tile.  Short reductions
         // over many tiles (stems, 1x1 layers) keep the wave-level shares.  A fused epilogue exists only
         // there.  The test hook's "cu" knob (0 / 4) overrides.
-        // Layers with a short reduction but at least 8 tiles per workgroup also launch this way, with
-        // shares in whole tiles: rounds of four tiles go one per wave, the up to three left over of a
-        // share are split over its waves (6272 tiles on 2048 wave slots: 3 rounds and a quarter, not 4).
+        // Layers with a short reduction but at least 8 tiles per workgroup also launch this way: every
+        // workgroup first runs the same number of rounds of four whole tiles, one per wave, and the tiles
+        // left over are shared out like any other launch's (6272 tiles on 2048 wave slots: 3 rounds and a
+        // sixteenth of a round for everybody, not 4 for some).
         const bool many_short = !a.alt_y && (long)a.tiles_m4 * a.tiles_n >= 8L * (plane_slots(true) / kCoopWaves);
         bool cooperative = WIDE && (a.comm >= 64 || a.fused || many_short);
         a.whole_tile_shares = many_short && a.comm < 64 && !a.fused;
