@@ -111,3 +111,53 @@ def test_random_fused_convolutions(oracle, seed):
     np.testing.assert_array_equal(out, v, err_msg=msg)
     if emit is not None:
         np.testing.assert_array_equal(q, so.np_requantize(v, emit[2], emit[3], emit[:2]), err_msg=msg)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_pair_launches(oracle, seed):
+    """ds_conv2d_tiled_fused_pair_i32 on random geometries: the two convolutions' tiles have different
+    lengths and the shares are cut in a space that pads each tile, so the ends of the shares fall into
+    tiles, between them and into the padding, at positions that vary with the shape; each output against
+    the oracle's chain for its layer alone."""
+    rng = np.random.default_rng(5000 + seed)
+    bits = int(rng.integers(2, 5))
+    k = int(rng.choice([3, 3, 5]))
+    pad = (k - 1) // 2
+    st = int(rng.integers(1, 3))
+    Nb = int(rng.integers(1, 7))
+    C = int(rng.choice([3, 24, 64, 100]))
+    Oa = int(rng.choice([64, 128]))
+    Ob = int(rng.choice([64, 128, 192]))
+    H, W = int(rng.integers(3, 40)), int(rng.integers(3, 40))
+    x = rng.integers(-2 ** 17, 2 ** 19, size=(Nb, C, H, W)).astype(np.int32)
+    xp = np.pad(x, ((0, 0), (0, 0), (pad, pad), (pad, pad)))
+    sa, ga = random_codes(rng, (Oa, C, k, k), max_s=2 ** bits - 2)
+    sb, gb = random_codes(rng, (Ob, C, 1, 1), max_s=2 ** bits - 2)
+    ba = rng.integers(-2 ** 16, 2 ** 16, size=Oa).astype(np.int32)
+    ya = oracle.conv2d(xp, -sa, ga, ba, (st, st), nthreads=NTHREADS)
+    yb = oracle.conv2d(x, -sb, gb, None, (st, st), nthreads=NTHREADS)
+    assert ya.shape[2:] == yb.shape[2:]
+    scale_a = ((rng.random(Oa) + 0.5) * 2.0 ** -6).astype(np.float32)
+    shift_a = rng.standard_normal(Oa).astype(np.float32)
+    scale_b = ((rng.random(Ob) + 0.5) * 2.0 ** -4).astype(np.float32)
+    shift_b = rng.standard_normal(Ob).astype(np.float32)
+    res_b = rng.standard_normal(yb.shape).astype(np.float32)
+    flag = bits | _lib.DS_BITS_TOP_UNUSED
+
+    def blob(s, g, O, kk):
+        return kernels.tile_weights(dev(so.np_pack_words(s.reshape(O, -1), g.reshape(O, -1), bits)).reshape(-1),
+                                    O, C, kk, kk, bits, 0)
+
+    first = dict(tiled=blob(sa, ga, Oa, k), bias=dev(ba), O=Oa, kernel_size=(k, k), crop=(0, 0), bits=flag,
+                 scale=dev(scale_a), shift=dev(shift_a), relu=True, emit=((1, 1), 16, 16, torch.int32),
+                 want_float=bool(seed % 2))
+    second = dict(tiled=blob(sb, gb, Ob, 1), bias=None, O=Ob, kernel_size=(1, 1), crop=(pad, pad), bits=flag,
+                  scale=dev(scale_b), shift=dev(shift_b), residual=dev(res_b), relu=False, want_float=True)
+    (oa, qa), (ob, _) = kernels.conv2d_tiled_fused_pair(dev(xp), (st, st), 16, first, second)
+    msg = str((bits, Nb, C, H, W, Oa, k, Ob, st))
+    va = so.np_dequantize_affine(ya, 16, scale_a, shift_a, None, True)
+    vb = so.np_dequantize_affine(yb, 16, scale_b, shift_b, res_b, False)
+    np.testing.assert_array_equal(qa.cpu().numpy(), so.np_requantize(va, 16, 16, (1, 1)), err_msg=msg)
+    if oa is not None:
+        np.testing.assert_array_equal(oa.cpu().numpy(), va, err_msg=msg)
+    np.testing.assert_array_equal(ob.cpu().numpy(), vb, err_msg=msg)
