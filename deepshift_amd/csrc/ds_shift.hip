@@ -78,6 +78,7 @@ struct ShiftArgs {
     int ep_border_kept;                   // the padding of q already holds zeros: write the interior only
     int whole_tile_shares;                // cooperative launch: rounds of whole tiles, one per wave, before the shared space
     int coop_pad;                         // cooperative launch: iterations a tile counts for beyond its K groups
+    FastDiv div_pix, div_ow;              // cooperative two-instruction launch: division by pix_per_img, by OW
     QuantSpec ep_spec;
 };
 
@@ -131,18 +132,26 @@ __device__ __forceinline__ int32_t *at_lane(int32_t *uniform_base, uint32_t lane
 // offset of k, ic*x_plane + fh*x_row + fw, is wave-uniform: (ic, fh, fw) come packed from the k
 // table of the weight blob through a scalar load and the offset is formed on the scalar ALU, so a
 // load is one buffer_load_dword (per-lane VGPR offset + SGPR offset) with no vector arithmetic.
-template <int NUM, int R>
-__device__ __forceinline__ void load_group(int32_t (&xv)[NUM][R], __amdgpu_buffer_rsrc_t rsrc,
-                                           const uint32_t (&xoff)[R], const ShiftArgs &p, int g)
+// load_part: the COUNT reduction indices FIRST .. of the group only.
+template <int NUM, int FIRST, int COUNT, int R>
+__device__ __forceinline__ void load_part(int32_t (&xv)[COUNT][R], __amdgpu_buffer_rsrc_t rsrc,
+                                          const uint32_t (&xoff)[R], const ShiftArgs &p, int g)
 {
 #pragma unroll
-    for (int i = 0; i < NUM; ++i) {
-        const uint32_t v = p.ktab[g * NUM + i];
+    for (int i = 0; i < COUNT; ++i) {
+        const uint32_t v = p.ktab[g * NUM + FIRST + i];
         const int koff = (int)(v >> 10) * p.x_plane + (int)((v >> 5) & 31u) * p.x_row + (int)(v & 31u);
 #pragma unroll
         for (int r = 0; r < R; ++r)
             xv[i][r] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, xoff[r], koff * 4, 0);
     }
+}
+
+template <int NUM, int R>
+__device__ __forceinline__ void load_group(int32_t (&xv)[NUM][R], __amdgpu_buffer_rsrc_t rsrc,
+                                           const uint32_t (&xoff)[R], const ShiftArgs &p, int g)
+{
+    load_part<NUM, 0, NUM, R>(xv, rsrc, xoff, p, g);
 }
 
 template <int BITS, bool GENERAL, int R, int J>
@@ -202,35 +211,58 @@ __device__ __forceinline__ void fused_store(const ShiftArgs &p, const int32_t (&
 {
     const int OW = p.OW, OH = p.pix_per_img / OW, ph = p.ep_ph, pw = p.ep_pw;
     const int Wq = OW + 2 * pw;
-    const size_t qplane = (size_t)(OH + 2 * ph) * Wq;
+    const uint32_t qplane = (uint32_t)(OH + 2 * ph) * Wq, plane = (uint32_t)p.pix_per_img;
     float *out = p.ep_out;
     Q *q = (Q *)p.ep_q;
     const bool one_bit = p.ep_spec.I == 1;
+    const int channels = p.N - n0 < J ? p.N - n0 : J;  // wave-uniform
+    // element indices of channel n0 (every tensor is below 2^31 bytes)
+    uint32_t o[R], qo[R];
+    int oh[R], ow[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        oh[r] = (int)div_by((uint32_t)rem[r], p.div_ow);
+        ow[r] = rem[r] - oh[r] * OW;
+        o[r] = (uint32_t)(img[r] * p.N + n0) * plane + rem[r];
+        qo[r] = (uint32_t)(img[r] * p.N + n0) * qplane + (uint32_t)(oh[r] + ph) * Wq + ow[r] + pw;
+    }
+    // all residual loads first: a load that followed the stores of the element before could not be issued
+    // ahead of them (the tensors may overlap as far as the compiler knows), and every element would cost a
+    // round trip to memory
+    float res[J][R];
+    if (p.ep_residual) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int j = 0; j < J; ++j) res[j][r] = live[r] && j < channels ? p.ep_residual[o[r] + j * plane] : 0.0f;
+    }
 #pragma unroll
     for (int j = 0; j < J; ++j) {
+        if (j >= channels) break;
         const int n = n0 + j;
-        if (n >= p.N) break;
         const int32_t add = p.negcnt[n] + (p.bias ? p.bias[n] : 0);
         const float sa = p.ep_scale ? p.ep_scale[n] : 1.0f, sb = p.ep_shift ? p.ep_shift[n] : 0.0f;
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             if (!live[r]) continue;
-            const size_t o = ((size_t)img[r] * p.N + n) * p.pix_per_img + rem[r];
             float f;
             {
 #pragma clang fp contract(off)
                 f = ((float)(acc[r][j] + add) * p.ep_inv) * sa + sb;
-                if (p.ep_residual) f += p.ep_residual[o];
+                if (p.ep_residual) f += res[j][r];
                 if (p.ep_relu) f = f > 0.0f ? f : 0.0f;
             }
-            if (out) out[o] = f;
-            if (q) {
-                const int oh = rem[r] / OW, ow = rem[r] - oh * OW;
-                const size_t plane = ((size_t)img[r] * p.N + n) * qplane;
-                q[plane + (size_t)(oh + ph) * Wq + ow + pw] =
-                    (Q)quantize_fixed(f, p.ep_spec.scale, p.ep_spec.lo, p.ep_spec.hi, one_bit);
-                if ((ph | pw) && !p.ep_border_kept) write_padding(q, plane, oh, ow, OH, OW, ph, pw, Wq);
-            }
+            if (out) out[o[r] + j * plane] = f;
+            if (q) q[qo[r] + j * qplane] = (Q)quantize_fixed(f, p.ep_spec.scale, p.ep_spec.lo, p.ep_spec.hi, one_bit);
+        }
+    }
+    if (q && (ph | pw) && !p.ep_border_kept) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if (!live[r]) continue;
+            if (!(ow[r] == 0 || ow[r] == OW - 1 || oh[r] == 0 || oh[r] == OH - 1)) continue;
+            for (int j = 0; j < channels; ++j)
+                write_padding(q, (size_t)(uint32_t)(img[r] * p.N + n0 + j) * qplane, oh[r], ow[r], OH, OW, ph, pw, Wq);
         }
     }
 }
@@ -251,25 +283,44 @@ __device__ __forceinline__ void shift_accumulate(const ShiftArgs &p, int32_t (&a
     const __amdgpu_buffer_rsrc_t xrsrc =
         __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, (int)p.x_bytes, 0x00020000);
 
-    int32_t xcur[NUM][R];
-    if (g_begin < g_full_end) load_group<NUM, R>(xcur, xrsrc, xoff, p, g_begin);
-
+    // The activations run ahead of their use; the prefetch is unconditional (the k table has a spare zero
+    // group, so group g + 1 always names valid addresses) so that the number of loads in flight is the same
+    // on every path and the wait counts stay exact.
+    if constexpr (R == 1) {
+        // one pixel row: a whole group ahead (NUM loads in flight)
+        int32_t xcur[NUM][R];
+        if (g_begin < g_full_end) load_group<NUM, R>(xcur, xrsrc, xoff, p, g_begin);
 #pragma clang loop unroll(disable)
-    for (int g = g_begin; g < g_full_end; ++g) {
-        uint32_t w[J];
+        for (int g = g_begin; g < g_full_end; ++g) {
+            uint32_t w[J];
 #pragma unroll
-        for (int j = 0; j < J; ++j) w[j] = wrow[(size_t)g * kTileWords + j];
-        // Issue the next group's loads before accumulating this one.  The prefetch is unconditional
-        // (the k table has a spare zero group, so group g + 1 always names valid addresses) so that
-        // the number of loads in flight is the same on every path and the wait counts stay exact.
-        int32_t xnext[NUM][R];
-        load_group<NUM, R>(xnext, xrsrc, xoff, p, g + 1);
+            for (int j = 0; j < J; ++j) w[j] = wrow[(size_t)g * kTileWords + j];
+            int32_t xnext[NUM][R];
+            load_group<NUM, R>(xnext, xrsrc, xoff, p, g + 1);
 #pragma unroll
-        for (int i = 0; i < NUM; ++i) accumulate_code<BITS, GENERAL, R, J>(acc, xcur[i], w, i, p.nbase);
+            for (int i = 0; i < NUM; ++i) accumulate_code<BITS, GENERAL, R, J>(acc, xcur[i], w, i, p.nbase);
 #pragma unroll
-        for (int i = 0; i < NUM; ++i)
+            for (int i = 0; i < NUM; ++i) xcur[i][0] = xnext[i][0];
+        }
+    } else {
+        // several rows: half a group ahead -- while one half of a group's reduction indices is accumulated
+        // the loads of the next half are in flight, in the registers of the half before (NUM x R registers
+        // for activations, not twice that: what lets four waves of the 4 x 16 and 2 x 32 tiles share a SIMD)
+        constexpr int H0 = NUM / 2, H1 = NUM - H0;
+        int32_t xa[H0][R], xb[H1][R];
+        if (g_begin < g_full_end) load_part<NUM, 0, H0, R>(xa, xrsrc, xoff, p, g_begin);
+#pragma clang loop unroll(disable)
+        for (int g = g_begin; g < g_full_end; ++g) {
+            uint32_t w[J];
 #pragma unroll
-            for (int r = 0; r < R; ++r) xcur[i][r] = xnext[i][r];
+            for (int j = 0; j < J; ++j) w[j] = wrow[(size_t)g * kTileWords + j];
+            load_part<NUM, H0, H1, R>(xb, xrsrc, xoff, p, g);
+#pragma unroll
+            for (int i = 0; i < H0; ++i) accumulate_code<BITS, GENERAL, R, J>(acc, xa[i], w, i, p.nbase);
+            load_part<NUM, 0, H0, R>(xa, xrsrc, xoff, p, g + 1);
+#pragma unroll
+            for (int i = 0; i < H1; ++i) accumulate_code<BITS, GENERAL, R, J>(acc, xb[i], w, H0 + i, p.nbase);
+        }
     }
     // tail group: codes with k >= K read as x = 0 (the tiled blob holds neutral codes there)
     for (int g = g_full_end; g < g_end; ++g) {
@@ -376,7 +427,7 @@ typedef int32_t v16i __attribute__((ext_vector_type(16)));
 // channels -- with the fused epilogue, or bias + sum as int32.  No K split across workgroups: no
 // pre-fill, no global atomics, and the conversion pass that followed such layers is gone.
 template <int BITS, int R, int J, int WAVES, bool FUSED>
-__global__ __launch_bounds__(WAVES * 64) void shift_coop_kernel(const ShiftArgs p)
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4))) void shift_coop_kernel(const ShiftArgs p)
 {
     constexpr int CH = J / WAVES;
     static_assert(J % WAVES == 0, "whole channels per wave in the write-out");
@@ -390,19 +441,14 @@ __global__ __launch_bounds__(WAVES * 64) void shift_coop_kernel(const ShiftArgs 
     const int m0 = (tile / p.tiles_n) * (R * kWave);
 
     uint32_t xoff[R];
-    bool live[R];
-    int img_of[R], rem_of[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         int m = m0 + r * kWave + lane;
-        live[r] = m < p.M;
-        if (!live[r]) m = p.M - 1;
-        const int img = m / p.pix_per_img;
+        if (m >= p.M) m = p.M - 1;
+        const int img = (int)div_by((uint32_t)m, p.div_pix);
         const int rem = m - img * p.pix_per_img;
-        const int oh = rem / p.OW;
+        const int oh = (int)div_by((uint32_t)rem, p.div_ow);
         const int ow = rem - oh * p.OW;
-        img_of[r] = img;
-        rem_of[r] = rem;
         xoff[r] = 4u * (uint32_t)(img * p.x_img_stride + oh * p.x_row_stride + ow * p.x_col_stride);
     }
     for (int i = threadIdx.x; i < J * R * kWave; i += WAVES * kWave) (&sums[0][0])[i] = 0;
@@ -421,6 +467,18 @@ __global__ __launch_bounds__(WAVES * 64) void shift_coop_kernel(const ShiftArgs 
         for (int r = 0; r < R; ++r) atomicAdd(&sums[j][r * kWave + lane], acc[r][j]);
     __syncthreads();
 
+    // (the pixel coordinates again: cheaper than twelve registers held across the main loop, which decide
+    // whether four waves fit a SIMD)
+    bool live[R];
+    int img_of[R], rem_of[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        int m = m0 + r * kWave + lane;
+        live[r] = m < p.M;
+        if (!live[r]) m = p.M - 1;
+        img_of[r] = (int)div_by((uint32_t)m, p.div_pix);
+        rem_of[r] = m - img_of[r] * p.pix_per_img;
+    }
     int32_t fin[R][CH];
 #pragma unroll
     for (int c = 0; c < CH; ++c)
@@ -1282,6 +1340,8 @@ static int launch_shift_coop(ShiftArgs a, hipStream_t st)
     a.tiles_n = ceil_div(a.N, small ? 16 : 32);
     a.blocks_per_xcd = ceil_div(a.tiles_m4 * a.tiles_n, 8);
     a.atomic_out = 0;
+    a.div_pix = fast_div((uint32_t)a.pix_per_img);
+    a.div_ow = fast_div((uint32_t)a.OW);
     if (small)
         hipLaunchKernelGGL((shift_coop_kernel<BITS, 4, 16, 4, FUSED>), dim3(a.blocks_per_xcd * 8), dim3(256), 0, st, a);
     else
