@@ -792,12 +792,16 @@ static size_t coop_workspace_bytes(int blocks)
     // a workgroup has at most two partial tiles: the one its share starts in and the one it ends in
     return coop_counter_bytes(blocks) + (size_t)2 * blocks * kCoopTileElems * 4;
 }
-// one workgroup per 8 wave slots (2 waves per SIMD); small layers: >= 8 K groups per wave
+// One workgroup per 8 wave slots (2 waves per SIMD, two workgroups per compute unit).  Small layers: at
+// least 8 K groups per wave, on at most one workgroup per compute unit -- but never a number between one
+// and two per compute unit: the units that hold two would finish last (a wave that shares its SIMD runs
+// at 0.56 of the speed of one that has it alone, so two full rounds beat one and a half: 3x3x64 on 8x8
+// images at batch 256, 6 K groups per wave on 512 workgroups 42 us, 8 on 384 48 us).
 static int coop_blocks(long iters)
 {
     int blocks = plane_slots(true) / kCoopWaves;
     const long fit = (iters / (8 * kCoopWaves)) / 8 * 8;
-    if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
+    if (fit < blocks / 2) blocks = fit < 8 ? 8 : (int)fit;
     // every workgroup must own at least one iteration: a tile is finished by the LAST of the
     // workgroups that its range of iterations names, and an empty share would never arrive
     if (blocks > iters) blocks = iters < 1 ? 1 : (int)iters;
