@@ -1330,10 +1330,12 @@ static long narrow_coop_waves(const ShiftArgs &a)
 {
     return narrow_coop_small(a) ? (long)ceil_div(a.M, 4 * kWave) * 4 : (long)ceil_div(a.M, 2 * kWave) * ceil_div(a.N, 32) * 8;
 }
-// Worth it where the waves fill the machine twice over and each gets at least two K groups.
+// Worth it where the waves fill the machine twice over and each gets at least two K groups -- one on the
+// four-wave shape: a first convolution of 3 x 3 x 3 taps is all tile setup and epilogue either way, and
+// the fused launch replaces three (pre-fill, split-K launch, conversion pass).
 static bool narrow_coop_fits(const ShiftArgs &a)
 {
-    return narrow_coop_waves(a) >= 2L * 4 * device_cus() && a.comm >= 2 * (narrow_coop_small(a) ? 4 : 8);
+    return narrow_coop_waves(a) >= 2L * 4 * device_cus() && a.comm >= (narrow_coop_small(a) ? 4 : 16);
 }
 
 template <int BITS, bool FUSED>
@@ -1545,8 +1547,9 @@ static int dispatch_shape(const ShiftArgs &a, hipStream_t st)
         const bool wide = tiled_wide(a.N, a.K, BITS);  // decided by the shape alone, as at tiling time
         bool planes = plane_regime(a, wide) >= 0;
         if (g_tune.planes != kTuneUnset) planes = g_tune.planes > 0;
-        if (a.fused) planes = wide;  // the fused epilogue exists in the cooperative launch of the 64-channel
-                                     // form and in the two-instruction kernel below
+        // the fused epilogue exists in the cooperative launch of the 64-channel form and in the
+        // two-instruction kernel below, which takes the layers that form has too few K groups for
+        if (a.fused) planes = wide && !(plane_regime(a, true) < 0 && narrow_coop_fits(a));
         if (planes) {
             int nsplit = plane_regime(a, wide) > 0 ? 1 : 0;
             if (g_tune.split != kTuneUnset) nsplit = g_tune.split;
@@ -1778,8 +1781,10 @@ DS_EXPORT int ds_conv2d_tiled_fusable(int Nb, int C, int Hp, int Wp, int O, int 
         const bool two_instruction = width == 5 || plane_regime(a, false) < 0;
         return two_instruction && narrow_coop_fits(a);
     }
-    // where the dispatch would launch cooperatively anyway: long reductions on few tiles
-    return a.comm >= 64 && plane_regime(a, true) == 0;
+    // where the dispatch would launch cooperatively anyway: long reductions on few tiles; shorter ones
+    // through the two-instruction kernel's cooperative launch where that fills the machine
+    const int regime = plane_regime(a, true);
+    return (a.comm >= 64 && regime == 0) || (regime < 0 && narrow_coop_fits(a));
 }
 
 DS_EXPORT int ds_conv2d_tiled_fused_i32(const int32_t *x, const void *tiled, const int32_t *bias, float *out,

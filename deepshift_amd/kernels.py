@@ -555,8 +555,10 @@ def conv2d_tiled(x_padded, tiled, bias, O, kernel_size, stride, bits, base=0):
 
 
 def conv2d_fusable(x_padded_shape, O, kernel_size, stride, bits, base=0):
-    """Whether :func:`conv2d_tiled_fused` serves this layer and is the faster choice for it (long
-    reductions on a multiple of 64 channels, fields of at most 4 bits, base 0)."""
+    """Whether :func:`conv2d_tiled_fused` serves this layer and is the faster choice for it: long
+    reductions on a multiple of 64 channels (cooperative launch of the shift-plane kernel), and other
+    layers whose tiles fill the machine (cooperative launch of the two-instruction kernel); ordinary
+    codes of at most 5 bits, base 0."""
     Nb, C, Hp, Wp = x_padded_shape
     FH, FW = _pair(kernel_size)
     sh, sw = _pair(stride)

@@ -104,6 +104,8 @@ NARROW_GEOMS = [
     (2, 16, 34, 33, 32, 3, 3, (2, 2)),       # strided, 32 channels, ragged pixel count
     (2, 7, 11, 13, 40, 3, 2, (1, 1)),        # 40 channels: a partial channel tile, K = 42
     (5, 32, 10, 10, 10, 1, 1, (1, 1)),       # 1x1, fewer channels than a tile holds
+    (16, 32, 65, 65, 64, 3, 3, (2, 2)),      # 64 channels but only 48 K groups: this kernel, not the 64-channel form
+    (128, 3, 34, 34, 16, 3, 3, (1, 1)),      # a first convolution, K = 27: one or two K groups per wave
 ]
 
 
@@ -388,3 +390,13 @@ def test_fused_resnet18_pairs_its_shortcuts():
         finally:
             modules._FUSE_EPILOGUE = True
     assert torch.equal(got, want)
+
+
+def test_fusable_covers_the_layers_of_a_small_image_network():
+    """ds_conv2d_tiled_fusable at ResNet-20's shapes (batch 256): every convolution, the first one and the
+    stride-2 ones included, has a fused launch; single images do not fill the machine and have none."""
+    shapes = [(3, 34, 16, 1), (16, 34, 16, 1), (16, 34, 32, 2), (32, 18, 32, 1), (32, 18, 64, 2), (64, 10, 64, 1)]
+    for C, Hp, O, st in shapes:
+        assert kernels.conv2d_fusable((256, C, Hp, Hp), O, (3, 3), (st, st), 4 | U), (C, Hp, O, st)
+    assert not kernels.conv2d_fusable((1, 16, 34, 34), 16, (3, 3), (1, 1), 4 | U)
+
