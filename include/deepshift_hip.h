@@ -294,14 +294,15 @@ int ds_cpu_conv2d_i32(const int32_t *x_padded, const int8_t *shift, const int32_
  * q is int32; 1: int8 (2 <= I, I + F <= 8); | DS_Q_BORDER_KEPT: the caller vouches that the padding of
  * q already holds zeros (a buffer it zeroed once and reuses), and the kernel writes the interior only.
  * scale, shift, residual may be NULL.  base must be 0.
- * Layers of the 64-channel form (O a multiple of 64, fields of at most 4 bits) run the cooperative
- * launch of the shift-plane kernel and need the workspace of ds_conv2d_tiled_workspace_bytes()
- * (DS_EWORKSPACE without it).  Other layers (ordinary codes of at most 5 bits; DS_EINVAL for 6-bit
- * fields and zero-top blobs) run the cooperative launch of the two-instruction kernel, which needs no
- * workspace.  ds_conv2d_tiled_fusable() says whether the fused call is also the faster choice for a
- * shape (64-channel form: long reductions -- short ones lose more in the launch form than the
- * separate pass costs; other layers: where the dispatch would pick the two-instruction kernel anyway
- * and the launch fills the machine).
+ * Layers of the 64-channel form (O a multiple of 64, fields of at most 4 bits) must pass the
+ * workspace of ds_conv2d_tiled_workspace_bytes() (DS_EWORKSPACE without it): they run the cooperative
+ * launch of the shift-plane kernel, or, where their reduction is too short for it and the tiles fill
+ * the machine, that of the two-instruction kernel.  Other layers (ordinary codes of at most 5 bits;
+ * DS_EINVAL for 6-bit fields and zero-top blobs) run the cooperative launch of the two-instruction
+ * kernel, which needs no workspace.  ds_conv2d_tiled_fusable() says whether the fused call is also
+ * the faster choice for a shape (long reductions on the 64-channel form, and every shape whose tiles
+ * on the two-instruction kernel give each SIMD two waves; elsewhere the launch form loses more than
+ * the separate pass costs).
  * No counterpart in the reference. */
 #define DS_Q_BORDER_KEPT 0x100
 int ds_conv2d_tiled_fusable(int Nb, int C, int Hp, int Wp, int O, int FH, int FW, int sh, int sw,
