@@ -33,11 +33,19 @@ struct SmallArgs {
 // MODE 0: every field is a right shift (base 0, fields of at most 5 bits); 1: general codes (a left
 // shift by nbase after the right shift; with 6-bit fields a field >= 32 is a zero weight); 2: the
 // highest field value stands for a zero weight (zero-top blobs).
-template <int BITS, int MODE>
+// VEC: a lane reads its row sixteen bytes at a time (K a multiple of 4, x 16-byte aligned).  A lane's row
+// is its own cache line either way -- lane = batch row, the rows are K floats apart -- so a wave's load
+// touches 64 lines and the launch is bound by the number of such loads, not by their bytes: four
+// reduction indices per load instead of one.  The loop then steps through U K groups at a time, the
+// smallest number whose reduction indices are a multiple of four.
+template <int BITS, int MODE, bool VEC>
 __global__ __launch_bounds__(kSmallWaves * 64) void linear_small_kernel(const SmallArgs p)
 {
     constexpr int NUM = 32 / (BITS + 1), CB = BITS + 1, J = kSmallJ;
     constexpr uint32_t TOP = (1u << BITS) - 1u;
+    constexpr int U = !VEC ? 1 : NUM % 4 == 0 ? 1 : NUM % 2 == 0 ? 2 : 4;  // K groups per step
+    constexpr int KS = U * NUM;                                              // reduction indices per step
+    static_assert(!VEC || KS % 4 == 0, "whole 16-byte loads per step");
     __shared__ int32_t part[kSmallWaves][J][kWave];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -45,8 +53,9 @@ __global__ __launch_bounds__(kSmallWaves * 64) void linear_small_kernel(const Sm
     const int m = blockIdx.y * kWave + lane;
     const bool live = m < p.M;
     const float *xrow = p.x + (size_t)(live ? m : 0) * p.K;
-    const int g_begin = (int)((long)wave * p.comm / kSmallWaves);
-    const int g_end = (int)((long)(wave + 1) * p.comm / kSmallWaves);
+    const int steps = (p.comm + U - 1) / U;
+    const int s_begin = (int)((long)wave * steps / kSmallWaves);
+    const int s_end = (int)((long)(wave + 1) * steps / kSmallWaves);
     // words of the workgroup's channels for K group g: wrow[g * 32 + j] (8 channels never straddle a
     // 32-channel tile)
     const uint32_t *wrow = p.wt + (size_t)(n0 / kTileWords) * p.comm * kTileWords + n0 % kTileWords;
@@ -55,54 +64,67 @@ __global__ __launch_bounds__(kSmallWaves * 64) void linear_small_kernel(const Sm
 #pragma unroll
     for (int j = 0; j < J; ++j) acc[j] = 0;
 
-    // Activations of one K group: the loads are issued together, unconditionally (reduction indices
-    // past K read the row's last element), one group ahead of their use; the conversion to fixed point
-    // follows the accumulation of the group before, and indices past K convert to 0 whatever the blob
-    // holds there.
-    auto load_group = [&](int g, float (&xf)[NUM]) {
+    // Activations of one step: the loads are issued together, unconditionally (reduction indices past K
+    // read the end of the row), one step ahead of their use; the conversion to fixed point follows the
+    // accumulation of the step before, and indices past K convert to 0 whatever the blob holds there.
+    auto load_step = [&](int st, float (&xf)[KS]) {
+        if constexpr (VEC) {
 #pragma unroll
-        for (int i = 0; i < NUM; ++i) {
-            const int k = g * NUM + i;
-            xf[i] = xrow[k < p.K ? k : p.K - 1];
-        }
-    };
-    auto convert_group = [&](int g, const float (&xf)[NUM], int32_t (&xv)[NUM]) {
+            for (int c = 0; c < KS / 4; ++c) {
+                const int k = st * KS + 4 * c;
+                const float4 v = *(const float4 *)(xrow + (k < p.K ? k : p.K - 4));
+                xf[4 * c] = v.x; xf[4 * c + 1] = v.y; xf[4 * c + 2] = v.z; xf[4 * c + 3] = v.w;
+            }
+        } else {
 #pragma unroll
-        for (int i = 0; i < NUM; ++i) {
-            const int32_t q = quantize_one(xf[i], p.spec);
-            xv[i] = g * NUM + i < p.K ? q : 0;
-        }
-    };
-    float xf[NUM];
-    int32_t xcur[NUM];
-    if (g_begin < g_end) {
-        load_group(g_begin, xf);
-        convert_group(g_begin, xf, xcur);
-    }
-#pragma clang loop unroll(disable)
-    for (int g = g_begin; g < g_end; ++g) {
-        uint32_t w[J];
-#pragma unroll
-        for (int j = 0; j < J; ++j) w[j] = wrow[(size_t)g * kTileWords + j];
-        const int gn = g + 1 < g_end ? g + 1 : g;  // the last iteration re-reads its own group: no branch
-        load_group(gn, xf);
-#pragma unroll
-        for (int i = 0; i < NUM; ++i) {
-#pragma unroll
-            for (int j = 0; j < J; ++j) {
-                const uint32_t code = w[j] >> (i * CB);
-                const int32_t mask = -(int32_t)((code >> BITS) & 1u);  // tiled format: 1 = negative
-                const uint32_t field = code & TOP;
-                int32_t t = xcur[i] >> (field & 31u);
-                if (MODE == 1) {
-                    t = (int32_t)((uint32_t)t << p.nbase);
-                    if (BITS == 6) t &= -(int32_t)(((field >> 5) & 1u) ^ 1u);
-                }
-                if (MODE == 2) t &= field == TOP ? 0 : -1;
-                acc[j] += t ^ mask;  // -t = (t ^ -1) + 1: the + 1 per negative code comes with negcnt
+            for (int i = 0; i < KS; ++i) {
+                const int k = st * KS + i;
+                xf[i] = xrow[k < p.K ? k : p.K - 1];
             }
         }
-        convert_group(gn, xf, xcur);
+    };
+    auto convert_step = [&](int st, const float (&xf)[KS], int32_t (&xv)[KS]) {
+#pragma unroll
+        for (int i = 0; i < KS; ++i) {
+            const int32_t q = quantize_one(xf[i], p.spec);
+            xv[i] = st * KS + i < p.K ? q : 0;
+        }
+    };
+    float xf[KS];
+    int32_t xcur[KS];
+    if (s_begin < s_end) {
+        load_step(s_begin, xf);
+        convert_step(s_begin, xf, xcur);
+    }
+#pragma clang loop unroll(disable)
+    for (int st = s_begin; st < s_end; ++st) {
+        const int sn = st + 1 < s_end ? st + 1 : st;  // the last step re-reads its own: no branch
+        load_step(sn, xf);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int g = st * U + u;
+            if (g >= p.comm) break;  // (wave-uniform) the last step may hold fewer groups
+            uint32_t w[J];
+#pragma unroll
+            for (int j = 0; j < J; ++j) w[j] = wrow[(size_t)g * kTileWords + j];
+#pragma unroll
+            for (int i = 0; i < NUM; ++i) {
+#pragma unroll
+                for (int j = 0; j < J; ++j) {
+                    const uint32_t code = w[j] >> (i * CB);
+                    const int32_t mask = -(int32_t)((code >> BITS) & 1u);  // tiled format: 1 = negative
+                    const uint32_t field = code & TOP;
+                    int32_t t = xcur[u * NUM + i] >> (field & 31u);
+                    if (MODE == 1) {
+                        t = (int32_t)((uint32_t)t << p.nbase);
+                        if (BITS == 6) t &= -(int32_t)(((field >> 5) & 1u) ^ 1u);
+                    }
+                    if (MODE == 2) t &= field == TOP ? 0 : -1;
+                    acc[j] += t ^ mask;  // -t = (t ^ -1) + 1: the + 1 per negative code comes with negcnt
+                }
+            }
+        }
+        convert_step(sn, xf, xcur);
     }
 #pragma unroll
     for (int j = 0; j < J; ++j) part[wave][j][lane] = acc[j];
@@ -119,13 +141,21 @@ __global__ __launch_bounds__(kSmallWaves * 64) void linear_small_kernel(const Sm
     }
 }
 
+template <int BITS, bool VEC>
+static void launch_small_mode(const SmallArgs &a, int mode, hipStream_t st)
+{
+    const dim3 grid(ceil_div(a.N, kSmallJ), ceil_div(a.M, kWave)), block(kSmallWaves * 64);
+    if (mode == 2) hipLaunchKernelGGL((linear_small_kernel<BITS, 2, VEC>), grid, block, 0, st, a);
+    else if (mode == 1) hipLaunchKernelGGL((linear_small_kernel<BITS, 1, VEC>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((linear_small_kernel<BITS, 0, VEC>), grid, block, 0, st, a);
+}
+
 template <int BITS>
 static void launch_small(const SmallArgs &a, int mode, hipStream_t st)
 {
-    const dim3 grid(ceil_div(a.N, kSmallJ), ceil_div(a.M, kWave)), block(kSmallWaves * 64);
-    if (mode == 2) hipLaunchKernelGGL((linear_small_kernel<BITS, 2>), grid, block, 0, st, a);
-    else if (mode == 1) hipLaunchKernelGGL((linear_small_kernel<BITS, 1>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((linear_small_kernel<BITS, 0>), grid, block, 0, st, a);
+    const bool vec = a.K >= 4 && a.K % 4 == 0 && ((uintptr_t)a.x & 15u) == 0;
+    if (vec) launch_small_mode<BITS, true>(a, mode, st);
+    else launch_small_mode<BITS, false>(a, mode, st);
 }
 
 }  // namespace ds
