@@ -52,7 +52,8 @@ def abi_conv_fused(xp, blob, bias, O, FH, FW, stride, bits, F_in, scale, shift, 
     OH, OW = (Hp - FH) // sh + 1, (Wp - FW) // sw + 1
     L = _lib.lib()
     ws_bytes = L.ds_conv2d_tiled_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, bits)
-    assert ws_bytes > 0 or O % 64 != 0      # the 64-channel form needs the workspace, other layers none
+    # the 64-channel form (fields of at most 4 bits) needs the workspace, other layers none
+    assert ws_bytes > 0 or O % 64 != 0 or (bits & 0xff) > 4
     ws = torch.full((max(ws_bytes, 1),), 0x77, dtype=torch.uint8, device=DEV)
     guard = 64
     n_out = Nb * O * OH * OW
@@ -399,4 +400,27 @@ def test_fusable_covers_the_layers_of_a_small_image_network():
     for C, Hp, O, st in shapes:
         assert kernels.conv2d_fusable((256, C, Hp, Hp), O, (3, 3), (st, st), 4 | U), (C, Hp, O, st)
     assert not kernels.conv2d_fusable((1, 16, 34, 34), 16, (3, 3), (1, 1), 4 | U)
+
+
+@pytest.mark.parametrize("geom", [(3, 16, 34, 34, 16, 3, 3, (1, 1)), (2, 24, 20, 19, 64, 3, 3, (2, 1)),
+                                  (2, 7, 11, 13, 40, 3, 2, (1, 1))], ids=lambda g: "x".join(str(v) for v in g[:7]))
+def test_fused_five_bit_fields(oracle, rng, geom):
+    """Fields of 5 bits (weight_bits 6: shifts down to -31, five codes per word) have no shift-plane form:
+    every layer, 64 channels wide or not, takes the cooperative two-instruction launch."""
+    Nb, C, Hp, Wp, O, FH, FW, stride = geom
+    OH, OW = (Hp - FH) // stride[0] + 1, (Wp - FW) // stride[1] + 1
+    xp = rng.integers(-2 ** 30, 2 ** 30, size=(Nb, C, Hp, Wp)).astype(np.int32)
+    s, sign = random_codes(rng, (O, C, FH, FW), max_s=31)
+    bias = rng.integers(-2 ** 16, 2 ** 16, size=O).astype(np.int32)
+    y = oracle.conv2d(xp, -s, sign, bias, stride, nthreads=NTHREADS)
+    blob = kernels.tile_weights(_dev(so.np_pack_words(s.reshape(O, -1), sign.reshape(O, -1), 5)).reshape(-1),
+                                O, C, FH, FW, 5, 0)
+    scale = ((rng.random(O) + 0.5) * 2.0 ** -10).astype(np.float32)
+    shift = rng.standard_normal(O).astype(np.float32)
+    res = (rng.standard_normal((Nb, O, OH, OW)) * 2).astype(np.float32)
+    for r, emit in ((res, (1, 1, 16, 16, torch.int32)), (None, (0, 2, 3, 5, torch.int8))):
+        v = so.np_dequantize_affine(y, 16, scale, shift, r, True)
+        out, q = abi_conv_fused(xp, blob, bias, O, FH, FW, stride, 5, 16, scale, shift, r, True, True, emit)
+        np.testing.assert_array_equal(out, v)
+        np.testing.assert_array_equal(q, so.np_requantize(v, emit[2], emit[3], emit[:2]))
 
