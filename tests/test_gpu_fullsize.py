@@ -239,3 +239,86 @@ def test_config4_resnet18_batch64_every_layer_shape(oracle):
     assert len(shapes) == 12
     for L in shapes:
         _run_layer_full(oracle, g, L, [0, 63])
+
+
+def _np(t):
+    return None if t is None else t.cpu().numpy()
+
+
+def test_config3_resnet20_batch256_fused_launches(oracle):
+    """The launches benchmark configuration 3 times: every distinct convolution shape of ResNet-20 at batch
+    256 through ds_conv2d_tiled_fused_i32 (the fused cooperative launches of the two-instruction and the
+    64-channel shift-plane kernels), BatchNorm affine + residual + ReLU + the next layer's padded 16.16
+    input, the WHOLE float and fixed-point outputs against the oracle's chain."""
+    from deepshift_amd import workloads
+    from oracle import shift_oracle as so
+    g = torch.Generator().manual_seed(35)
+    shapes = [L for L in _distinct_shapes(workloads.ResNet20(), (3, 32, 32), 256) if L["kind"] == "conv"]
+    assert len(shapes) == 6
+    for L in shapes:
+        ph, pw = L["padding"]
+        x = torch.randint(-2 ** 18, 2 ** 20, (L["Nb"], L["C"], L["H"], L["W"]), generator=g, dtype=torch.int32)
+        xp = torch.nn.functional.pad(x, (pw, pw, ph, ph)).contiguous()
+        shift, sign = _default_init_codes(g, (L["O"], L["C"], L["FH"], L["FW"]))
+        bias = torch.randint(-2 ** 20, 2 ** 20, (L["O"],), generator=g, dtype=torch.int32)
+        cw = utils.compress_bits(shift, sign)
+        kb = kernels.kernel_bits(cw)
+        assert kernels.conv2d_fusable(tuple(xp.shape), L["O"], (L["FH"], L["FW"]), L["stride"], kb), L["name"]
+        tiled = kernels._tiled_of(cw, L["O"], L["C"], L["FH"], L["FW"])
+        scale = (torch.rand(L["O"], generator=g) + 0.5) * 2.0 ** -6
+        shf = torch.randn(L["O"], generator=g)
+        OH = (xp.shape[2] - L["FH"]) // L["stride"][0] + 1
+        OW = (xp.shape[3] - L["FW"]) // L["stride"][1] + 1
+        res = torch.randn(L["Nb"], L["O"], OH, OW, generator=g)
+        out, q = kernels.conv2d_tiled_fused(xp.to(DEV), tiled, bias.to(DEV), L["O"], (L["FH"], L["FW"]), L["stride"],
+                                            kb, 16, scale.to(DEV), shf.to(DEV), res.to(DEV), True,
+                                            emit=((1, 1), 16, 16, torch.int32), want_float=True)
+        y = oracle.conv2d(xp.numpy(), shift.numpy().astype(np.int32), sign.numpy().astype(np.int32), bias.numpy(),
+                          L["stride"], nthreads=NTHREADS)
+        v = so.np_dequantize_affine(y, 16, scale.numpy(), shf.numpy(), res.numpy(), True)
+        np.testing.assert_array_equal(_np(out), v, err_msg=L["name"])
+        np.testing.assert_array_equal(_np(q), so.np_requantize(v, 16, 16, (1, 1)), err_msg=L["name"])
+
+
+def test_config4_resnet18_batch64_pair_launches(oracle):
+    """The three two-convolution launches of a ResNet-18 step at batch 64 (a down-sampling block's 3x3
+    stride-2 convolution and its 1x1 stride-2 shortcut over one padded input, 512 workgroups, shares cut
+    in the padded iteration space): both outputs against the oracle's chain on the first and the last
+    image, and a permutation of the batch permutes both outputs."""
+    from oracle import shift_oracle as so
+    g = torch.Generator().manual_seed(45)
+    for C, H, O in ((64, 56, 128), (128, 28, 256), (256, 14, 512)):
+        Nb = 64
+        x = torch.randint(-2 ** 18, 2 ** 20, (Nb, C, H, H), generator=g, dtype=torch.int32)
+        xp = torch.nn.functional.pad(x, (1, 1, 1, 1)).contiguous()
+        sa, ga = _default_init_codes(g, (O, C, 3, 3))
+        sb, gb = _default_init_codes(g, (O, C, 1, 1))
+        cwa, cwb = utils.compress_bits(sa, ga), utils.compress_bits(sb, gb)
+        ba = torch.randint(-2 ** 20, 2 ** 20, (O,), generator=g, dtype=torch.int32)
+        sc_a, sh_a = (torch.rand(O, generator=g) + 0.5) * 2.0 ** -6, torch.randn(O, generator=g)
+        sc_b, sh_b = (torch.rand(O, generator=g) + 0.5) * 2.0 ** -4, torch.randn(O, generator=g)
+
+        def run(xpad):
+            first = dict(tiled=kernels._tiled_of(cwa, O, C, 3, 3), bias=ba.to(DEV), O=O, kernel_size=(3, 3),
+                         crop=(0, 0), bits=kernels.kernel_bits(cwa), scale=sc_a.to(DEV), shift=sh_a.to(DEV),
+                         relu=True, emit=((1, 1), 16, 16, torch.int32), want_float=False)
+            second = dict(tiled=kernels._tiled_of(cwb, O, C, 1, 1), bias=None, O=O, kernel_size=(1, 1),
+                          crop=(1, 1), bits=kernels.kernel_bits(cwb), scale=sc_b.to(DEV), shift=sh_b.to(DEV),
+                          relu=False, want_float=True)
+            (_, qa), (ob, _) = kernels.conv2d_tiled_fused_pair(xpad.to(DEV), (2, 2), 16, first, second)
+            return qa, ob
+
+        qa, ob = run(xp)
+        for img in (0, Nb - 1):
+            ya = oracle.conv2d(xp[img:img + 1].numpy(), sa.numpy().astype(np.int32), ga.numpy().astype(np.int32),
+                               ba.numpy(), (2, 2), nthreads=NTHREADS)
+            yb = oracle.conv2d(x[img:img + 1].numpy(), sb.numpy().astype(np.int32), gb.numpy().astype(np.int32),
+                               None, (2, 2), nthreads=NTHREADS)
+            va = so.np_dequantize_affine(ya, 16, sc_a.numpy(), sh_a.numpy(), None, True)
+            vb = so.np_dequantize_affine(yb, 16, sc_b.numpy(), sh_b.numpy(), None, False)
+            np.testing.assert_array_equal(_np(qa[img:img + 1]), so.np_requantize(va, 16, 16, (1, 1)),
+                                          err_msg="%d image %d" % (C, img))
+            np.testing.assert_array_equal(_np(ob[img:img + 1]), vb, err_msg="%d image %d" % (C, img))
+        perm = torch.randperm(Nb, generator=g)
+        qa_p, ob_p = run(xp[perm].contiguous())
+        assert torch.equal(qa_p, qa[perm.to(DEV)]) and torch.equal(ob_p, ob[perm.to(DEV)]), C
