@@ -348,6 +348,32 @@ def config1(device, with_cpu=True, reps=50):
     out = {"workload": "MLP 784-512-512-10, batch 64, ternary signs, shifts [-15, 0], activations 16.16",
            "us_per_forward": gpu_s * 1e6, "shift_kernel_us_per_forward": sum(L["seconds"] for L in layers) * 1e6,
            "pairs_per_forward": sum(L["M"] * L["K"] * L["N"] for L in layers)}
+    # The eager forward is bound by the host's five launches; the same forward replayed from a captured HIP
+    # graph shows what the GPU needs for it (replays are checked against the eager result).
+    try:
+        side = torch.cuda.Stream(device)
+        side.wait_stream(torch.cuda.current_stream(device))
+        with torch.no_grad(), torch.cuda.stream(side):
+            for _ in range(3):
+                gpu_model(xd)
+        torch.cuda.current_stream(device).wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.no_grad(), torch.cuda.graph(graph):
+            y_graph = gpu_model(xd)
+        same = True
+        for _ in range(3):
+            graph.replay()
+            torch.cuda.synchronize()
+            same = same and bool(torch.equal(y_graph, y_gpu))
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            graph.replay()
+        torch.cuda.synchronize()
+        out["us_per_forward_graph_replay"] = (time.perf_counter() - t0) / reps * 1e6
+        out["graph_replay_equals_eager"] = same
+    except Exception as exc:  # capture is an extra: the eager figure stands without it
+        out["us_per_forward_graph_replay"] = None
+        out["graph_replay_error"] = str(exc)[:200]
     if with_cpu:
         from oracle import shift_oracle
         oracle = shift_oracle.get()

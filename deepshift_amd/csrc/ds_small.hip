@@ -7,7 +7,7 @@
 // kernel does the reference's whole chain (modules.py:24-31, modules_q.py:115-125)
 //     x_fixed = (x * 2^F).int()  [or round_to_fixed first]   ->   y = bias + sum_k +-(x_fixed >> s)
 //     ->   y.float() / 2^F
-// per lane = batch row: a workgroup of eight waves owns 64 rows x 8 output channels, its waves split
+// per lane = batch row: a workgroup of eight waves owns 64 rows x 8 (4, 2) output channels, its waves split
 // the reduction, the partial sums meet in LDS and each wave writes one channel.  The weights are the
 // tiled blob of ds_tile_weights_i32 / ds_tile_weights_zero_top_i32 (its packed-word section), so a
 // layer keeps one weight format whichever kernel serves it.
@@ -16,7 +16,7 @@
 
 namespace ds {
 
-constexpr int kSmallJ = 8;      // output channels per workgroup
+constexpr int kSmallJ = 8;      // output channels per workgroup, at most: 8, 4 or 2 (launch_small)
 constexpr int kSmallWaves = 8;  // waves per workgroup: eighths of the reduction
 
 struct SmallArgs {
@@ -38,10 +38,10 @@ struct SmallArgs {
 // touches 64 lines and the launch is bound by the number of such loads, not by their bytes: four
 // reduction indices per load instead of one.  The loop then steps through U K groups at a time, the
 // smallest number whose reduction indices are a multiple of four.
-template <int BITS, int MODE, bool VEC>
+template <int BITS, int MODE, bool VEC, int J>
 __global__ __launch_bounds__(kSmallWaves * 64) void linear_small_kernel(const SmallArgs p)
 {
-    constexpr int NUM = 32 / (BITS + 1), CB = BITS + 1, J = kSmallJ;
+    constexpr int NUM = 32 / (BITS + 1), CB = BITS + 1;
     constexpr uint32_t TOP = (1u << BITS) - 1u;
     constexpr int U = !VEC ? 1 : NUM % 4 == 0 ? 1 : NUM % 2 == 0 ? 2 : 4;  // K groups per step
     constexpr int KS = U * NUM;                                              // reduction indices per step
@@ -56,7 +56,7 @@ __global__ __launch_bounds__(kSmallWaves * 64) void linear_small_kernel(const Sm
     const int steps = (p.comm + U - 1) / U;
     const int s_begin = (int)((long)wave * steps / kSmallWaves);
     const int s_end = (int)((long)(wave + 1) * steps / kSmallWaves);
-    // words of the workgroup's channels for K group g: wrow[g * 32 + j] (8 channels never straddle a
+    // words of the workgroup's channels for K group g: wrow[g * 32 + j] (J channels never straddle a
     // 32-channel tile)
     const uint32_t *wrow = p.wt + (size_t)(n0 / kTileWords) * p.comm * kTileWords + n0 % kTileWords;
 
@@ -129,10 +129,10 @@ __global__ __launch_bounds__(kSmallWaves * 64) void linear_small_kernel(const Sm
 #pragma unroll
     for (int j = 0; j < J; ++j) part[wave][j][lane] = acc[j];
     __syncthreads();
-    // wave j sums the eight partial results of channel n0 + j and writes it
-    static_assert(kSmallJ == kSmallWaves, "one channel per wave in the write-out");
+    // wave j < J sums the eight partial results of channel n0 + j and writes it
+    static_assert(J <= kSmallWaves && kTileWords % J == 0, "one channel per wave in the write-out");
     const int n = n0 + wave;
-    if (n < p.N && live) {
+    if (wave < J && n < p.N && live) {
         int32_t sum = p.negcnt[n] + (p.bias ? p.bias[n] : 0);
 #pragma unroll
         for (int w = 0; w < kSmallWaves; ++w) sum += part[w][wave][lane];
@@ -141,21 +141,34 @@ __global__ __launch_bounds__(kSmallWaves * 64) void linear_small_kernel(const Sm
     }
 }
 
-template <int BITS, bool VEC>
+template <int BITS, bool VEC, int J>
 static void launch_small_mode(const SmallArgs &a, int mode, hipStream_t st)
 {
-    const dim3 grid(ceil_div(a.N, kSmallJ), ceil_div(a.M, kWave)), block(kSmallWaves * 64);
-    if (mode == 2) hipLaunchKernelGGL((linear_small_kernel<BITS, 2, VEC>), grid, block, 0, st, a);
-    else if (mode == 1) hipLaunchKernelGGL((linear_small_kernel<BITS, 1, VEC>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((linear_small_kernel<BITS, 0, VEC>), grid, block, 0, st, a);
+    const dim3 grid(ceil_div(a.N, J), ceil_div(a.M, kWave)), block(kSmallWaves * 64);
+    if (mode == 2) hipLaunchKernelGGL((linear_small_kernel<BITS, 2, VEC, J>), grid, block, 0, st, a);
+    else if (mode == 1) hipLaunchKernelGGL((linear_small_kernel<BITS, 1, VEC, J>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((linear_small_kernel<BITS, 0, VEC, J>), grid, block, 0, st, a);
+}
+
+template <int BITS, bool VEC>
+static void launch_small_vec(const SmallArgs &a, int mode, hipStream_t st)
+{
+    // Channels per workgroup: the most that still give every SIMD a wave and a half.  Fewer channels mean
+    // more workgroups, each of which converts its rows' activations again -- worth it while the machine is
+    // not full (64 x 784 x 512: 8 channels 17.4 us, 4 15.0, 2 13.7; 64 x 512 x 1000: 15.9, 13.5, 16.4;
+    // 128 x 2048 x 1000: 44.7, 54.6, 84.3).
+    const long rows = ceil_div(a.M, kWave), enough = 6L * device_cus();
+    if ((long)ceil_div(a.N, 8) * rows * kSmallWaves >= enough) launch_small_mode<BITS, VEC, 8>(a, mode, st);
+    else if ((long)ceil_div(a.N, 4) * rows * kSmallWaves >= enough) launch_small_mode<BITS, VEC, 4>(a, mode, st);
+    else launch_small_mode<BITS, VEC, 2>(a, mode, st);
 }
 
 template <int BITS>
 static void launch_small(const SmallArgs &a, int mode, hipStream_t st)
 {
     const bool vec = a.K >= 4 && a.K % 4 == 0 && ((uintptr_t)a.x & 15u) == 0;
-    if (vec) launch_small_mode<BITS, true>(a, mode, st);
-    else launch_small_mode<BITS, false>(a, mode, st);
+    if (vec) launch_small_vec<BITS, true>(a, mode, st);
+    else launch_small_vec<BITS, false>(a, mode, st);
 }
 
 }  // namespace ds
