@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libdeepshift_hip.so")
 
 DS_Q_ROUND_TO_FIXED = 0
 DS_Q_CAST = 1
+DS_SMALL_RELU = 0x100
 DS_BITS_ZERO_TOP = 0x100
 DS_BITS_TOP_UNUSED = 0x200
 DS_Q_BORDER_KEPT = 0x100

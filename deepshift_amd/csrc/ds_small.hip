@@ -27,6 +27,7 @@ struct SmallArgs {
     float *y;               // [M][N]
     int M, K, N, comm, nbase;
     float out_scale;        // 2^F
+    int relu;               // y = max(y, 0)
     QuantSpec spec;
 };
 
@@ -137,7 +138,9 @@ __global__ __launch_bounds__(kSmallWaves * 64) void linear_small_kernel(const Sm
 #pragma unroll
         for (int w = 0; w < kSmallWaves; ++w) sum += part[w][wave][lane];
         // out.float() / 2**F: int32 -> fp32 rounds to nearest even, the division is exact
-        p.y[(size_t)m * p.N + n] = (float)sum / p.out_scale;
+        float v = (float)sum / p.out_scale;
+        if (p.relu) v = v > 0.0f ? v : 0.0f;  // torch.relu: negative values and -0.0 become +0.0
+        p.y[(size_t)m * p.N + n] = v;
     }
 }
 
@@ -181,6 +184,8 @@ DS_EXPORT int ds_linear_small_f32(const float *x, const void *tiled, const int32
 {
     const int zero_top = (bits & DS_BITS_ZERO_TOP) != 0;
     bits &= ~(DS_BITS_ZERO_TOP | DS_BITS_TOP_UNUSED);  // an unused top value needs no form of its own here
+    const int relu = (mode & DS_SMALL_RELU) != 0;
+    mode &= ~DS_SMALL_RELU;
     if (bits < 1 || bits > 6) return DS_EBITS;
     if (base > 0 || base < -31) return DS_EBASE;
     if (zero_top && (bits > 4 || base != 0)) return DS_EBITS;
@@ -199,6 +204,7 @@ DS_EXPORT int ds_linear_small_f32(const float *x, const void *tiled, const int32
     a.y = y;
     a.M = M; a.K = K; a.N = N; a.comm = g.comm; a.nbase = -base;
     a.out_scale = ldexpf(1.0f, F);
+    a.relu = relu;
     a.spec = make_spec(I, F, mode);
     const int kernel_mode = zero_top ? 2 : (base != 0 || bits == 6) ? 1 : 0;
     hipStream_t st = (hipStream_t)stream;

@@ -24,10 +24,25 @@ import torch.nn.functional as F
 
 from . import kernels, modules, modules_q
 
-__all__ = ["FusedConv2dShift", "fuse_conv_epilogues"]
+__all__ = ["FusedConv2dShift", "FusedLinearShift", "fuse_conv_epilogues"]
 
 _SHIFT_CONVS = (modules.Conv2dShift, modules_q.Conv2dShiftQ)
-_SHIFT_LEAVES = _SHIFT_CONVS + (modules.LinearShift, modules_q.LinearShiftQ)
+_SHIFT_LINEARS = (modules.LinearShift, modules_q.LinearShiftQ)
+_SHIFT_LEAVES = _SHIFT_CONVS + _SHIFT_LINEARS
+
+
+class FusedLinearShift(nn.Module):
+    """A kernel-mode LinearShift / LinearShiftQ layer with the ReLU that follows it (mnist.py:36-38): the
+    one-launch kernel applies it to its output."""
+
+    def __init__(self, linear):
+        super().__init__()
+        self.linear = linear
+
+    def forward(self, input):
+        if not self.linear.use_kernel:
+            return torch.relu(self.linear(input))
+        return self.linear._kernel_forward(input, relu=True)
 
 
 class FusedConv2dShift(nn.Module):
@@ -191,7 +206,8 @@ def _sole_user(node):
 
 def fuse_conv_epilogues(model, handoff=True):
     """Return a ``torch.fx.GraphModule`` equivalent to ``model`` (eval mode) with every kernel-mode
-    shift convolution fused with the BatchNorm / residual add / ReLU that consume its output.
+    shift convolution fused with the BatchNorm / residual add / ReLU that consume its output, and every
+    kernel-mode shift linear layer with its ReLU.
     ``handoff``: fused convolutions that feed each other pass the fixed-point tensor directly."""
     model.eval()
     graph = _Tracer().trace(model)
@@ -202,6 +218,19 @@ def fuse_conv_epilogues(model, handoff=True):
         if node.op != "call_module":
             continue
         conv = mods.get(node.target)
+        if isinstance(conv, _SHIFT_LINEARS) and conv.use_kernel:
+            # a fully connected layer and its ReLU
+            nxt = _sole_user(node)
+            if nxt is not None and _is_relu(nxt, mods):
+                name = "fused_%d" % count
+                count += 1
+                gm.add_module(name, FusedLinearShift(conv))
+                with gm.graph.inserting_after(nxt):
+                    new = gm.graph.call_module(name, (node.args[0],))
+                nxt.replace_all_uses_with(new)
+                gm.graph.erase_node(nxt)
+                gm.graph.erase_node(node)
+            continue
         if not isinstance(conv, _SHIFT_CONVS) or not conv.use_kernel:
             continue
         chain = [node]

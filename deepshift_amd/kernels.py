@@ -478,11 +478,12 @@ def linear_tiled(xT, M, tiled, bias, N, bits, base=0):
 SMALL_LINEAR_PAIRS = 1 << 27
 
 
-def linear_small(x2d, tiled, bias, N, bits, base, integer_bits, fraction_bits, round_to_fixed):
+def linear_small(x2d, tiled, bias, N, bits, base, integer_bits, fraction_bits, round_to_fixed, relu=False):
     """A whole LinearShift layer in one launch (``ds_linear_small_f32``): float32 ``[M, K]`` in, the
     fixed-point conversion (modules.py:25 or utils.py:7-21), the shift GEMM on the tiled blob and
     ``y.float() / 2**F`` (modules.py:30-31); returns float32 ``[M, N]``.  Bit-identical to
-    :func:`quantize_transpose` + :func:`linear_tiled` + :func:`dequantize`."""
+    :func:`quantize_transpose` + :func:`linear_tiled` + :func:`dequantize`.  ``relu``: the ReLU that
+    follows the layer, in the same launch."""
     x2d = x2d.contiguous()
     if x2d.dtype != torch.float32 or not x2d.is_cuda or x2d.dim() != 2:
         raise TypeError("linear_small expects a 2-D float32 GPU tensor")
@@ -492,19 +493,23 @@ def linear_small(x2d, tiled, bias, N, bits, base, integer_bits, fraction_bits, r
     out = torch.empty([M, N], dtype=torch.float32, device=x2d.device)
     with _Timed("linear", M, K, N, x2d.device):
         _lib.call("ds_linear_small_f32", _lib.ptr(x2d), _lib.ptr(tiled), _lib.ptr(bias), _lib.ptr(out), M, K, N,
-                  int(bits), int(base), _lib.DS_Q_ROUND_TO_FIXED if round_to_fixed else _lib.DS_Q_CAST,
+                  int(bits), int(base),
+                  (_lib.DS_Q_ROUND_TO_FIXED if round_to_fixed else _lib.DS_Q_CAST) | (_lib.DS_SMALL_RELU if relu else 0),
                   int(integer_bits), int(fraction_bits), _lib.current_stream(x2d.device))
     return out
 
 
-def linear_layer(x2d, tiled, bias, N, bits, base, integer_bits, fraction_bits, round_to_fixed):
+def linear_layer(x2d, tiled, bias, N, bits, base, integer_bits, fraction_bits, round_to_fixed, relu=False):
     """float32 ``[M, K]`` -> float32 ``[M, N]`` through the kernel path of a LinearShift layer: one
-    launch for small problems, conversion + tiled GEMM + dequantisation otherwise (same results)."""
+    launch for small problems, conversion + tiled GEMM + dequantisation otherwise (same results).
+    ``relu``: a ReLU follows the layer."""
     M, K = x2d.shape
     if M * K * N <= SMALL_LINEAR_PAIRS:
-        return linear_small(x2d, tiled, bias, N, bits, base, integer_bits, fraction_bits, round_to_fixed)
+        return linear_small(x2d, tiled, bias, N, bits, base, integer_bits, fraction_bits, round_to_fixed, relu)
     xT = quantize_transpose(x2d, integer_bits, fraction_bits, round_to_fixed=round_to_fixed)
     out = linear_tiled(xT, M, tiled, bias, N, bits, base)
+    if relu:
+        return dequantize_affine(out, fraction_bits, None, None, None, True)
     return dequantize(out, fraction_bits)
 
 

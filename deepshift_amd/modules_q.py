@@ -86,19 +86,20 @@ class LinearShiftQ(_PackedQMixin, nn.Module):
             bound = 1 / math.sqrt(fan_in)
             init.uniform_(self.bias, -bound, bound)
 
-    def _kernel_forward(self, input):
+    def _kernel_forward(self, input, relu=False):
         I, Fb = self.act_integer_bits, self.act_fraction_bits
         lead = input.shape[:-1]
         x2d = input.reshape(-1, self.in_features).float()
         if not self.use_cuda:
             shift, sign = module_codes_q(self)
             out = linear_cpu_forward(x2d, shift, sign, self.bias, I, Fb, round_to_fixed=True)
+            out = torch.relu(out) if relu else out
             return out.reshape(*lead, self.out_features)
         conc_weight = self.packed_weights()
         bias = self._fixed_bias.get(self.bias, I, Fb, round_to_fixed=True)
         tiled = kernels._tiled_of(conc_weight, self.out_features, self.in_features)
         out = kernels.linear_layer(x2d, tiled, bias, self.out_features, kernels.kernel_bits(conc_weight),
-                                   conc_weight.base, I, Fb, round_to_fixed=True)
+                                   conc_weight.base, I, Fb, round_to_fixed=True, relu=relu)
         return out.reshape(*lead, self.out_features)
 
     def forward(self, input):

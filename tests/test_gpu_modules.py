@@ -495,3 +495,30 @@ def test_forward_pass_replays_as_a_hip_graph():
                 graph.replay()
                 torch.cuda.synchronize()
                 assert torch.equal(static_y, want), (cls.__name__, i)
+
+
+def test_fused_mlp_equals_the_plain_model():
+    """fuse_conv_epilogues on the MNIST MLP (mnist.py:23-39): each LinearShift + ReLU becomes one launch, the
+    output equals the plain converted model's bit for bit -- PS and Q layers, and a ReLU module as well as
+    the function."""
+    from deepshift_amd import convert, fuse, workloads
+    g = torch.Generator().manual_seed(11)
+    x = torch.rand(64, 784, generator=g).to(DEV)
+    for shift_type in ("PS", "Q"):
+        model, _ = convert.convert_to_shift(workloads.MLP(), 0, shift_type, convert_weights=True, use_kernel=True)
+        model = model.to(DEV).eval()
+        with torch.no_grad():
+            want = model(x)
+            fused = fuse.fuse_conv_epilogues(model)
+            assert sum(isinstance(m, fuse.FusedLinearShift) for m in fused.modules()) == 2
+            assert torch.equal(fused(x), want)
+    seq = torch.nn.Sequential(torch.nn.Linear(32, 48), torch.nn.ReLU(), torch.nn.Linear(48, 8))
+    seq, _ = convert.convert_to_shift(seq, 0, "PS", convert_weights=True, use_kernel=True)
+    seq = seq.to(DEV).eval()
+    with torch.no_grad():
+        xs = torch.randn(5, 32, generator=g).to(DEV)
+        want = seq(xs)
+        fused = fuse.fuse_conv_epilogues(seq)
+        assert sum(isinstance(m, fuse.FusedLinearShift) for m in fused.modules()) == 1
+        assert torch.equal(fused(xs), want)
+

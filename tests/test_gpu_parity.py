@@ -576,6 +576,10 @@ def test_linear_small_matches_oracle_chain(oracle, rng, bits, shape):
                                       want)
     want = oracle.linear(xq, -s, sign, None, NTHREADS).astype(np.float32) / np.float32(2.0 ** F)
     np.testing.assert_array_equal(abi_linear_small(x, blob, None, N, bits, 0, mode, I, F), want)
+    # the ReLU that follows the layer, in the same launch (-0.0 and negative values become +0.0)
+    got = abi_linear_small(x, blob, None, N, bits, 0, mode | _lib.DS_SMALL_RELU, I, F)
+    np.testing.assert_array_equal(got, np.maximum(want, np.float32(0)))
+    assert not np.signbit(got).any()
 
 
 def test_linear_small_general_codes_and_zero_top(oracle, rng):
