@@ -436,7 +436,10 @@ def pmc_target(device):
       * a down-sampling block's first 3x3 stride-2 convolution with its 1x1 shortcut as one launch
         (<4, 2, true, true>), 64 -> 128 channels at 56x56;
       * the int8 kernel (shift_pairs_cu_kernel) on a ResNet-50 3x3 layer, 128 -> 128 at 28x28, batch 128,
-        weight_bits 3."""
+        weight_bits 3;
+      * the cooperative two-instruction kernel (shift_coop_kernel) on ResNet-20's 3x3 layers at batch 256:
+        16 -> 16 channels at 32x32 (<4, 4, 16, 4, true>) and 32 -> 32 at 16x16 (<4, 2, 32, 8, true>), both with
+        residual, ReLU, float and fixed-point outputs."""
     from deepshift_amd import _lib, kernels, utils
     g = torch.Generator().manual_seed(0)
     n = 16 * 1024 * 1024
@@ -463,6 +466,13 @@ def pmc_target(device):
     cw8, _, _ = layer(128, 128, 3, lo=-2)
     fields = kernels.paired_fields(cw8, 128, 3, 5)
     blob8 = kernels._paired_of(cw8, fields, 128, 128, 3, 3)
+    narrow = []
+    for ch, size in ((16, 32), (32, 16)):
+        xn = torch.randint(0, 2 ** 20, (256, ch, size + 2, size + 2), generator=g, dtype=torch.int32).to(device)
+        cwn, tiledn, kbn = layer(ch, ch, 3)
+        narrow.append((xn, tiledn, kbn, ch, torch.rand(ch, generator=g).to(device) * 2.0 ** -6,
+                       torch.randn(ch, generator=g).to(device),
+                       torch.randn(256, ch, size, size, generator=g).to(device), {}))
     cache, cache2 = {}, {}
     torch.cuda.synchronize()
     for _ in range(3):
@@ -481,6 +491,9 @@ def pmc_target(device):
             dict(tiled=tiledb, O=128, kernel_size=(1, 1), crop=(1, 1), bits=kbb, scale=scale2, shift=offs2,
                  want_float=True))
         kernels.conv2d_paired(x8, blob8, None, 128, (3, 3), (1, 1), fields[1], 96)
+        for xn, tiledn, kbn, ch, sc, of, res, qc in narrow:
+            kernels.conv2d_tiled_fused(xn, tiledn, None, ch, (3, 3), (1, 1), kbn, 16, sc, of, res, True,
+                                       ((1, 1), 16, 16, torch.int32), True, qc)
     torch.cuda.synchronize()
 
 
