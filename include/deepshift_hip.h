@@ -220,7 +220,7 @@ int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled, const int
  * x[M][K] and y[M][N] float, contiguous; tiled: the blob of ds_tile_weights_i32 (or
  * ds_tile_weights_zero_top_i32 with bits | DS_BITS_ZERO_TOP); bias int32 fixed point or NULL.  No
  * workspace.  Results are those of ds_quantize_f32_i32 + ds_linear_i32 + ds_dequantize_i32_f32, bit for
- * bit; any size is accepted, but above some 10^8 shift-add pairs the tiled entry point is faster.
+ * bit; any size is accepted, but above some 5 * 10^8 shift-add pairs the tiled entry point is faster.
  * mode | DS_SMALL_RELU: a ReLU follows the layer (mnist.py:36-38, F.relu) and is applied to y in the
  * same launch. */
 #define DS_SMALL_RELU 0x100
