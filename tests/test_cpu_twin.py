@@ -173,6 +173,22 @@ def test_modules_use_kernel_on_cpu(oracle):
     assert (got - cq(xi)).abs().max().item() < 27 * 2.0 ** -16 + 1e-4
 
 
+def test_fused_linear_relu_on_the_host_path():
+    """fuse_conv_epilogues folds LinearShift + ReLU into one module; with use_cuda=False it runs the host
+    kernel followed by the ReLU and equals the plain model."""
+    from deepshift_amd import fuse
+    torch.manual_seed(2)
+    model = torch.nn.Sequential(modules.LinearShift(24, 16, use_kernel=True, use_cuda=False), torch.nn.ReLU(),
+                                modules_q.LinearShiftQ(16, 5, use_kernel=True, use_cuda=False)).eval()
+    x = torch.randn(9, 24)
+    with torch.no_grad():
+        want = model(x)
+        fused = fuse.fuse_conv_epilogues(model)
+        assert sum(isinstance(m, fuse.FusedLinearShift) for m in fused.modules()) == 1
+        assert torch.equal(fused(x), want)
+        assert (want >= 0).any() and (model[0](x) < 0).any()   # the ReLU had something to do
+
+
 def test_host_codes_saturate_like_int8():
     shift = torch.tensor([[-1000.0, float("-inf"), 3.7, -3.7, 200.0]])
     sign = torch.tensor([[1.0, 0.0, -1.0, 1.0, 1.0]])
