@@ -80,42 +80,102 @@ def host_threads():
     return max(1, n)
 
 
-def parity_gate(model, x):
-    """Before any timing: the launches that are about to be timed -- the stem, the first 3x3 convolution
-    (the dominant kernel) and the first strided 3x3 / 1x1 pair, each on its real batch-64 input and
-    through kernels.kernel_bits() -- against the oracle on the first and the last image, bit for bit."""
-    from deepshift_amd import kernels, modules
-    from oracle import shift_oracle
-    oracle = shift_oracle.get()
-    convs = [m for m in model.modules() if isinstance(m, modules.Conv2dShift)]
-    strided = [i for i, m in enumerate(convs) if m.stride == (2, 2) and i > 0][:2]
-    picked = {i: convs[i] for i in [0, 1] + strided}
-    captured = {}
+def _oracle_chain(oracle, so, fused_mod, xq_img, residual_img):
+    """What one fused shift convolution must produce for one image, by the oracle: the reference's chain
+    conv kernel -> y.float()/2^F (modules.py:161-162) -> eval BatchNorm -> + residual -> ReLU
+    [-> max pooling] -> the consumer's round_to_fixed + cast + padding (modules.py:317,153,
+    kernels.py:32-36).  Returns (float result, consumer's fixed-point input or None)."""
+    from deepshift_amd import modules
+    conv = fused_mod.conv
+    shift, sign = modules.module_codes(conv)
+    bias = None
+    if conv.bias is not None:
+        bias = oracle.quantize(conv.bias.detach().float().cpu().numpy(), conv.act_integer_bits,
+                               conv.act_fraction_bits)
+    y = oracle.conv2d(xq_img, shift.cpu().numpy().astype(np.int32), sign.cpu().numpy().astype(np.int32), bias,
+                      conv.stride, nthreads=host_threads())
+    scale = None if fused_mod.scale is None else fused_mod.scale.cpu().numpy()
+    offs = None if fused_mod.shift is None else fused_mod.shift.cpu().numpy()
+    v = so.np_dequantize_affine(y, conv.act_fraction_bits, scale, offs, residual_img, fused_mod.relu)
+    if fused_mod.pool is not None:
+        v = so.np_max_pool2d(v, *fused_mod.pool)
+    q = None
+    if fused_mod.emit is not None:
+        padding, I, Fq = fused_mod.emit[:3]
+        q = so.np_requantize(v, I, Fq, tuple(padding))
+    return v, q
 
-    def keep(k):
-        def hook(mod, inp, out):
-            captured[k] = inp[0]   # (a hook's return value would replace the layer's output)
-        return hook
 
-    hooks = [m.register_forward_hook(keep(i)) for i, m in picked.items()]
+def _split_result(fused_mod, result):
+    """(float result or None, fixed-point result or None) of a fused convolution's return value."""
+    if fused_mod.emit is None:
+        return result, None
+    if fused_mod.emit[3]:
+        return result[0], result[1]
+    return None, result
+
+
+def parity_gate(fused, x, images=None):
+    """Before any timing: one forward pass of the FUSED model that is about to be timed, with a hook on every
+    fused shift-convolution launch it issues (ds_conv2d_tiled_fused_i32, ds_conv2d_tiled_fused_pair_i32, the
+    stem's ds_conv2d_tiled_i32 + pooling pass); each launch's own inputs and outputs -- the tensors the
+    timed launches read and write -- are then compared, for the first and the last image, bit for bit with
+    the oracle's restatement of the reference chain on the same inputs.  Returns the number of launches
+    checked."""
+    from deepshift_amd import fuse
+    from oracle import shift_oracle as so
+    oracle = so.get()
+    images = list(images) if images is not None else [0, x.shape[0] - 1]
+    records = []
+
+    def hook(mod, inp, out):
+        records.append((mod, inp, out))   # (a hook's return value would replace the module's output)
+
+    watched = [m for m in fused.modules() if isinstance(m, (fuse.FusedConv2dShift, fuse.FusedShortcutPair))]
+    hooks = [m.register_forward_hook(hook) for m in watched]
     with torch.no_grad():
-        model(x)
+        fused(x)
+    torch.cuda.synchronize()
     for h in hooks:
         h.remove()
-    for i, layer in picked.items():
-        xq = kernels.quantize_pad(captured[i].contiguous(), layer.padding, 16, 16)
-        cw = layer.packed_weights()
-        tiled = kernels._tiled_of(cw, layer.out_channels, layer.in_channels, *layer.kernel_size)
-        y = kernels.conv2d_tiled(xq, tiled, None, layer.out_channels, layer.kernel_size, layer.stride,
-                                 kernels.kernel_bits(cw), cw.base)
-        shift = layer.shift.detach().clamp(*layer.shift_range).round().cpu().numpy().astype(np.int32)
-        sign = layer.sign.detach().round().sign().cpu().numpy().astype(np.int32)
-        for img in (0, x.shape[0] - 1):
-            want = oracle.conv2d(xq[img:img + 1].cpu().numpy(), shift, sign, None, layer.stride,
-                                 nthreads=host_threads())
-            if not np.array_equal(y[img:img + 1].cpu().numpy(), want):
-                raise SystemExit("parity gate failed: shift conv %d, image %d differs from the oracle" % (i, img))
-    return len(picked)
+
+    def img_of(t, i):
+        return None if t is None else t[i:i + 1].cpu().numpy()
+
+    def fixed_input(mod, t, i):
+        conv = mod.conv
+        if mod.prequantized:
+            return t[i:i + 1].cpu().numpy().astype(np.int32)
+        return so.np_requantize(t[i:i + 1].float().cpu().numpy(), conv.act_integer_bits, conv.act_fraction_bits,
+                                tuple(conv.padding))
+
+    def compare(mod, result, xq_img, res_img, i, what):
+        got_f, got_q = _split_result(mod, result)
+        want_f, want_q = _oracle_chain(oracle, so, mod, xq_img, res_img)
+        if got_f is not None and not np.array_equal(got_f[i:i + 1].cpu().numpy(), want_f):
+            raise SystemExit("parity gate failed: %s, image %d: float result differs from the oracle chain" % (what, i))
+        if got_q is not None and not np.array_equal(got_q[i:i + 1].cpu().numpy().astype(np.int32), want_q):
+            raise SystemExit("parity gate failed: %s, image %d: fixed-point result differs from the oracle chain"
+                             % (what, i))
+
+    checked = 0
+    for n, (mod, inp, out) in enumerate(records):
+        for i in images:
+            if isinstance(mod, fuse.FusedShortcutPair):
+                xq = inp[0]
+                res = [inp[k] if len(inp) > k else None for k in (1, 2)]
+                pad = tuple(mod.first.conv.padding)
+                xa = xq[i:i + 1].cpu().numpy()
+                # the shortcut reads the centre taps: the padded tensor without the first convolution's padding
+                xb = xa[:, :, pad[0]:xa.shape[2] - pad[0], pad[1]:xa.shape[3] - pad[1]]
+                compare(mod.first, out[0], xa, img_of(res[0], i), i, "launch %d (pair, k x k)" % n)
+                compare(mod.shortcut, out[1], np.ascontiguousarray(xb), img_of(res[1], i), i,
+                        "launch %d (pair, shortcut)" % n)
+            else:
+                res = inp[1] if len(inp) > 1 else None
+                compare(mod, out, fixed_input(mod, inp[0], i), img_of(res, i), i, "launch %d" % n)
+        checked += 1
+    return checked
 
 
 def time_steps(model, x, steps, warmup):
@@ -594,9 +654,6 @@ def main():
 
     from deepshift_amd import workloads
     model, x, n_conv = build_model(device)
-    checked = parity_gate(model, x)
-    log("parity gate passed on %d timed launches; %d conv + 1 fc shift layers" % (checked, n_conv))
-
     # The measured pipeline: the converted model with the fp32 glue after every shift conv
     # (BatchNorm, residual add, ReLU) folded into that conv's dequantisation pass.  The shift
     # kernels and their int32 results are the same as in the plain converted model, which is timed
@@ -607,6 +664,9 @@ def main():
         want, got = model(x[:4]), fused(x[:4])
     if not torch.allclose(got, want, rtol=0, atol=2e-3 * float(want.abs().max()) + 1e-4):
         raise SystemExit("fused pipeline diverges from the plain converted model")
+    checked = parity_gate(fused, x)
+    log("parity gate passed on the %d convolution launches of the timed model; %d conv + 1 fc shift layers"
+        % (checked, n_conv))
     sec_unfused = time_steps(model, x, max(2, args.steps // 2), args.warmup)
     sec_per_step = time_steps(fused, x, args.steps, args.warmup)
     layers = kernel_timings(fused, x, max(3, min(args.steps, 10)))

@@ -322,3 +322,66 @@ def test_config4_resnet18_batch64_pair_launches(oracle):
         perm = torch.randperm(Nb, generator=g)
         qa_p, ob_p = run(xp[perm].contiguous())
         assert torch.equal(qa_p, qa[perm.to(DEV)]) and torch.equal(ob_p, ob[perm.to(DEV)]), C
+
+
+@pytest.mark.parametrize("C,H", [(64, 56), (128, 28), (256, 14), (512, 7)], ids=lambda v: str(v))
+def test_config4_resnet18_batch64_fused_3x3_launches(oracle, C, H):
+    """The dominant launches of the headline step: the stride-1 3x3 convolutions of ResNet-18 at batch 64
+    through ds_conv2d_tiled_fused_i32 as fuse.py issues them (modules.py:152-162,312-337 followed by the
+    block's BatchNorm, residual add and ReLU and the next layer's round_to_fixed + cast + padding): 512
+    workgroups sharing about three tiles each, partial tiles exchanged through the workspace, the padded
+    fixed-point output kept in a zeroed buffer (`q_cache`).  First and last image against the oracle chain,
+    a second call into the same cached buffer, and a batch permutation on the whole batch."""
+    from oracle import shift_oracle as so
+    g = torch.Generator().manual_seed(46 + C)
+    Nb, O = 64, C
+    x = torch.randint(-2 ** 18, 2 ** 20, (Nb, C, H, H), generator=g, dtype=torch.int32)
+    xp = torch.nn.functional.pad(x, (1, 1, 1, 1)).contiguous()
+    shift, sign = _default_init_codes(g, (O, C, 3, 3))
+    cw = utils.compress_bits(shift, sign)
+    kb = kernels.kernel_bits(cw)
+    assert kb == 4 | 0x200
+    assert kernels.conv2d_fusable(tuple(xp.shape), O, (3, 3), (1, 1), kb)
+    tiled = kernels._tiled_of(cw, O, C, 3, 3)
+    scale = ((torch.rand(O, generator=g) + 0.5) * 2.0 ** -6).to(DEV)
+    shf = torch.randn(O, generator=g).to(DEV)
+    res = torch.randn(Nb, O, H, H, generator=g)
+    cache = {}
+
+    def run(xpad, residual):
+        return kernels.conv2d_tiled_fused(xpad.to(DEV), tiled, None, O, (3, 3), (1, 1), kb, 16, scale, shf,
+                                          residual.to(DEV), True, emit=((1, 1), 16, 16, torch.int32),
+                                          want_float=True, q_cache=cache)
+
+    out, q = run(xp, res)
+    s_np, sg_np = shift.numpy().astype(np.int32), sign.numpy().astype(np.int32)
+    for img in (0, Nb - 1):
+        y = oracle.conv2d(xp[img:img + 1].numpy(), s_np, sg_np, None, (1, 1), nthreads=NTHREADS)
+        v = so.np_dequantize_affine(y, 16, _np(scale), _np(shf), res[img:img + 1].numpy(), True)
+        np.testing.assert_array_equal(_np(out[img:img + 1]), v, err_msg="image %d" % img)
+        np.testing.assert_array_equal(_np(q[img:img + 1]), so.np_requantize(v, 16, 16, (1, 1)),
+                                      err_msg="image %d" % img)
+    out, q = out.clone(), q.clone()
+    perm = torch.randperm(Nb, generator=g)
+    out_p, q_p = run(xp[perm].contiguous(), res[perm].contiguous())
+    assert q_p.data_ptr() == cache[next(iter(cache))].data_ptr(), "the second call reuses the kept buffer"
+    assert torch.equal(out_p, out[perm.to(DEV)]) and torch.equal(q_p, q[perm.to(DEV)])
+    # the form without residual and float output, as the first convolution of a block runs
+    _, q2 = kernels.conv2d_tiled_fused(xp.to(DEV), tiled, None, O, (3, 3), (1, 1), kb, 16, scale, shf, None, True,
+                                       emit=((1, 1), 16, 16, torch.int32), want_float=False, q_cache={})
+    for img in (0, Nb - 1):
+        y = oracle.conv2d(xp[img:img + 1].numpy(), s_np, sg_np, None, (1, 1), nthreads=NTHREADS)
+        v = so.np_dequantize_affine(y, 16, _np(scale), _np(shf), None, True)
+        np.testing.assert_array_equal(_np(q2[img:img + 1]), so.np_requantize(v, 16, 16, (1, 1)))
+
+
+def test_bench_parity_gate_covers_the_timed_model(oracle):
+    """bench.py's gate on a small batch: every fused convolution launch of the fused ResNet-18 (17 of them:
+    stem + pooling pass, 13 single 3x3 launches, three pair launches) against the oracle chain on each
+    launch's own inputs."""
+    import bench
+    from deepshift_amd import fuse
+    model, x, _ = bench.build_model(torch.device(DEV))
+    with torch.no_grad():
+        fused = fuse.fuse_conv_epilogues(model)
+    assert bench.parity_gate(fused, x[:2].contiguous(), images=[0, 1]) == 17
