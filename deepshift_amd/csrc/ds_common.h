@@ -3,7 +3,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stddef.h>
+#include <atomic>
 #include "../../include/deepshift_hip.h"
+#include "../../include/deepshift_hip_test.h"
 
 #define DS_EXPORT extern "C" __attribute__((visibility("default")))
 
@@ -38,15 +40,17 @@ __device__ __forceinline__ uint32_t div_by(uint32_t n, const FastDiv &f)
     return (t + ((n - t) >> f.s1)) >> f.s2;
 }
 
-// Launch-variant overrides for the test-suite (ds_test_tune): kTuneUnset leaves the dispatch's own
-// choice in place.  Process-wide, set only between launches.
+// Launch-variant overrides for the test-suite (ds_test_tune, declared in deepshift_hip_test.h):
+// kTuneUnset leaves the dispatch's own choice in place.  Process-wide; every knob is an atomic that a
+// dispatch reads with a plain (sequentially consistent) load.
 constexpr int kTuneUnset = -2147483647 - 1;
 struct Tune {
-    int planes = kTuneUnset;  // 0 / 1: two-instruction kernel / shift-plane kernel
-    int split = kTuneUnset;   // K split (plane kernels: 0 = equal shares, 1 = one tile per wave, -r = r x shares)
-    int tile = kTuneUnset;    // R * 100 + J of the two-instruction kernel
-    int cu = kTuneUnset;      // 0 / 4: workgroup-cooperative launch off / on (four waves per workgroup)
-    int notail = kTuneUnset;  // int8 kernel: keep the last round of tiles on the tile-per-wave launch
+    std::atomic<int> planes{kTuneUnset};  // 0 / 1: two-instruction kernel / shift-plane kernel
+    std::atomic<int> split{kTuneUnset};   // K split (plane kernels: 0 = equal shares, 1 = one tile per wave, -r = r x shares)
+    std::atomic<int> tile{kTuneUnset};    // R * 100 + J of the two-instruction kernel
+    std::atomic<int> cu{kTuneUnset};      // 0 / 4: workgroup-cooperative launch off / on (four waves per workgroup)
+    std::atomic<int> notail{kTuneUnset};  // int8 kernel: keep the last round of tiles on the tile-per-wave launch
+    void reset() { planes = kTuneUnset; split = kTuneUnset; tile = kTuneUnset; cu = kTuneUnset; notail = kTuneUnset; }
 };
 extern Tune g_tune;
 

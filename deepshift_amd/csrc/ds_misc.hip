@@ -59,7 +59,7 @@ using namespace ds;
 DS_EXPORT int ds_test_tune(const char *knob, int value)
 {
     if (!knob) {
-        g_tune = Tune();
+        g_tune.reset();
         return DS_OK;
     }
     const std::string k(knob);

@@ -431,14 +431,6 @@ int ds_valu_calibrate(int32_t *sink, int blocks, int iters, ds_stream_t stream);
 /* Plain copy kernel of n int32 (used to scale HBM byte counters). */
 int ds_copy_i32(const int32_t *src, int32_t *dst, int64_t n, ds_stream_t stream);
 
-/* Test hook: forces a launch variant of the compute entry points, process-wide, so that the
- * test-suite can run every kernel form on small shapes.  knob: "planes" (0 / 1: two-instruction /
- * shift-plane kernel), "split" (K split; shift-plane kernels: 0 = equal shares, 1 = one tile per
- * wave), "tile" (R * 100 + J of the two-instruction kernel), "cu" (0 / 4 / 8 waves per cooperative
- * workgroup), "notail".  knob == NULL clears every override.  Not for production callers: the
- * dispatch's own choice is the measured best. */
-int ds_test_tune(const char *knob, int value);
-
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,25 @@
+/* libdeepshift_hip.so -- entry points for the library's own test-suite.
+ *
+ * Kept out of deepshift_hip.h on purpose: nothing here is part of the drop-in boundary, and a
+ * production caller has no use for it.  No counterpart in the reference. */
+#ifndef DEEPSHIFT_HIP_TEST_H
+#define DEEPSHIFT_HIP_TEST_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Test hook: forces a launch variant of the compute entry points, process-wide, so that the
+ * test-suite can run every kernel form on small shapes.  knob: "planes" (0 / 1: two-instruction /
+ * shift-plane kernel), "split" (K split; shift-plane kernels: 0 = equal shares, 1 = one tile per
+ * wave), "tile" (R * 100 + J of the two-instruction kernel), "cu" (0 / 4 / 8 waves per cooperative
+ * workgroup), "notail".  knob == NULL clears every override.  Each knob is an atomic integer that an
+ * entry point reads once per call, so a call sees either the old or the new value of a knob, never a
+ * torn one; a thread that changes a knob changes the dispatch of every thread of the process, which
+ * is why this header is not the production one.  The dispatch's own choice is the measured best. */
+int ds_test_tune(const char *knob, int value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DEEPSHIFT_HIP_TEST_H */

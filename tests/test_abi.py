@@ -10,12 +10,21 @@ from deepshift_amd import _lib
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "deepshift_hip.h")
+TEST_HEADER = os.path.join(ROOT, "include", "deepshift_hip_test.h")
 
 
-def declared_symbols():
-    text = open(HEADER).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(ds_[a-z0-9_]+)\s*\(", text)))
+def declared_symbols(headers=(HEADER, TEST_HEADER)):
+    names = set()
+    for header in headers:
+        text = open(header).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names.update(re.findall(r"\b(ds_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
+
+
+def test_the_test_hook_is_not_in_the_production_header():
+    assert declared_symbols((TEST_HEADER,)) == ["ds_test_tune"]
+    assert "ds_test_tune" not in declared_symbols((HEADER,))
 
 
 def test_header_and_binding_agree():
