@@ -19,6 +19,7 @@ Differences from the reference, all deliberate:
 """
 
 import ctypes
+import sys
 
 import torch
 
@@ -47,6 +48,22 @@ def _require_device_i32(name, t):
 
 def _workspace(nbytes, device):
     return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)
+
+
+def _kept_padded_buffer(cache, shape, dtype, device):
+    """The zero padded hand-off buffer of a fused convolution, kept in ``cache`` between calls so that its
+    border is zeroed once and the kernel writes the interior only.  The buffer is reused only while nobody
+    else holds the tensor returned last time (or a view of it): a layer that is called again while an
+    earlier result is still alive -- a weight-shared branch whose consumer has not run yet -- gets a fresh
+    zeroed buffer instead of overwriting what that consumer is about to read."""
+    key = (tuple(shape), dtype, device)
+    q = cache.get(key)
+    if q is not None and sys.getrefcount(q) > 3:   # the cache, the local name, getrefcount's argument
+        q = None
+    if q is None:
+        cache.clear()            # one geometry at a time: a new batch size replaces the buffer
+        q = cache[key] = torch.zeros(shape, dtype=dtype, device=device)
+    return q
 
 
 _TIMING_SINK = None
@@ -479,6 +496,14 @@ def linear_tiled(xT, M, tiled, bias, N, bits, base=0):
 SMALL_LINEAR_PAIRS = 1 << 29
 
 
+def small_linear_serves(M, K, N):
+    """Whether :func:`linear_layer` sends a layer to the one-launch kernel: few enough pairs for it to be
+    the faster path, and within what ``ds_linear_small_f32`` accepts -- one workgroup row per 64 batch rows
+    in ``gridDim.y`` (at most 65535) and 32-bit byte offsets into the activations."""
+    return M * K * N <= SMALL_LINEAR_PAIRS and (M + 63) // 64 <= 65535 and M * K * 4 < 2 ** 31 \
+        and M * N * 4 < 2 ** 31
+
+
 def linear_small(x2d, tiled, bias, N, bits, base, integer_bits, fraction_bits, round_to_fixed, relu=False):
     """A whole LinearShift layer in one launch (``ds_linear_small_f32``): float32 ``[M, K]`` in, the
     fixed-point conversion (modules.py:25 or utils.py:7-21), the shift GEMM on the tiled blob and
@@ -505,7 +530,7 @@ def linear_layer(x2d, tiled, bias, N, bits, base, integer_bits, fraction_bits, r
     launch for small problems, conversion + tiled GEMM + dequantisation otherwise (same results).
     ``relu``: a ReLU follows the layer."""
     M, K = x2d.shape
-    if M * K * N <= SMALL_LINEAR_PAIRS:
+    if small_linear_serves(M, K, N):
         return linear_small(x2d, tiled, bias, N, bits, base, integer_bits, fraction_bits, round_to_fixed, relu)
     xT = quantize_transpose(x2d, integer_bits, fraction_bits, round_to_fixed=round_to_fixed)
     out = linear_tiled(xT, M, tiled, bias, N, bits, base)
@@ -581,7 +606,9 @@ def conv2d_tiled_fused(x_padded, tiled, bias, O, kernel_size, stride, bits, frac
     convolution's round-to-fixed, zero padded input.  Bit-identical to :func:`conv2d_tiled` followed by
     :func:`requantize_affine_pad` / :func:`dequantize_affine`; the int32 sums are never stored.
     ``q_cache``: a dict in which the padded buffer is kept between calls (zeroed once, so the kernel
-    writes the interior only); the returned ``q`` is then that buffer, overwritten by the next call."""
+    writes the interior only).  The returned ``q`` then aliases that buffer: the next call with the same
+    ``q_cache`` overwrites it once the caller has dropped every reference to ``q`` (and its views); while a
+    reference is alive the next call takes a fresh zeroed buffer instead."""
     x_padded = _require_device_i32("x_padded", x_padded)
     Nb, C, Hp, Wp = x_padded.shape
     FH, FW = _pair(kernel_size)
@@ -605,11 +632,7 @@ def conv2d_tiled_fused(x_padded, tiled, bias, O, kernel_size, stride, bits, frac
         qb = 1 if dtype == torch.int8 else 4
         shape = (Nb, O, OH + 2 * ph, OW + 2 * pw)
         if q_cache is not None and (ph or pw):
-            key = (shape, dtype, dev)
-            q = q_cache.get(key)
-            if q is None:
-                q_cache.clear()            # one geometry at a time: a new batch size replaces the buffer
-                q = q_cache[key] = torch.zeros(shape, dtype=dtype, device=dev)
+            q = _kept_padded_buffer(q_cache, shape, dtype, dev)
             qb |= _lib.DS_Q_BORDER_KEPT
         else:
             q = torch.empty(shape, dtype=dtype, device=dev)
@@ -655,11 +678,7 @@ def _fused_conv_struct(x_shape, stride, spec, keep):
         shape = (Nb, O, OH + 2 * ph, OW + 2 * pw)
         cache = spec.get("q_cache")
         if cache is not None and (ph or pw):
-            key = (shape, dtype, dev)
-            q = cache.get(key)
-            if q is None:
-                cache.clear()
-                q = cache[key] = torch.zeros(shape, dtype=dtype, device=dev)
+            q = _kept_padded_buffer(cache, shape, dtype, dev)
             qb |= _lib.DS_Q_BORDER_KEPT
         else:
             q = torch.empty(shape, dtype=dtype, device=dev)

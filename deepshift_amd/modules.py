@@ -73,6 +73,13 @@ class _PackedWeightsMixin:
     def _pack(self):
         return pack_module_weights(self)
 
+    def __getstate__(self):
+        # the hand-off buffers of the fused pipeline (GPU scratch that the next forward pass rebuilds)
+        # do not travel with copy.deepcopy / pickling of the module
+        state = self.__dict__.copy()
+        state.pop("_handoff_buffers", None)
+        return state
+
     def packed_weights(self):
         """The layer's ConcWeight, (re)built if it is missing or older than the parameters."""
         if self._conc_weight is None or (self._packed_from is not None and

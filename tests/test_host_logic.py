@@ -242,3 +242,53 @@ def test_small_layers_stay_on_the_int32_kernels():
     assert modules._small_for_int8(body, (1, 512, 7, 7), 4)                # batch 1
     wide = modules.Conv2dShift(64, 256, 1, use_kernel=True)
     assert not modules._small_for_int8(wide, (128, 64, 56, 56), 2)         # ResNet-50 stage 1
+
+
+def test_small_linear_routing_respects_the_one_launch_kernels_limits():
+    """linear_layer sends a layer to ds_linear_small_f32 only below the break-even in pairs AND within that
+    entry point's limits (65535 workgroup rows of 64 batch rows, 32-bit byte offsets); a tiny layer applied
+    to millions of rows stays on the tiled path, which served it before."""
+    assert kernels.small_linear_serves(64, 784, 512)
+    assert kernels.small_linear_serves(128, 2048, 1000)
+    assert not kernels.small_linear_serves(1024, 1024, 1024)            # above the break-even
+    assert kernels.small_linear_serves(65535 * 64, 8, 8)
+    assert not kernels.small_linear_serves(65535 * 64 + 1, 8, 8)        # gridDim.y
+    assert not kernels.small_linear_serves(5_000_000, 8, 8)
+    assert not kernels.small_linear_serves(2 ** 20, 512, 1)             # M * K * 4 = 2^31
+    assert not kernels.small_linear_serves(2 ** 20, 1, 512)             # M * N * 4 = 2^31
+
+
+def test_kept_hand_off_buffer_is_not_reused_while_its_last_result_is_alive():
+    cache = {}
+    a = kernels._kept_padded_buffer(cache, (1, 2, 4, 4), torch.int32, torch.device("cpu"))
+    assert a.shape == (1, 2, 4, 4) and not a.any()
+    ptr_a = a.data_ptr()
+    del a
+    b = kernels._kept_padded_buffer(cache, (1, 2, 4, 4), torch.int32, torch.device("cpu"))
+    assert b.data_ptr() == ptr_a, "nobody held the buffer: reused"
+    b.fill_(7)
+    c = kernels._kept_padded_buffer(cache, (1, 2, 4, 4), torch.int32, torch.device("cpu"))
+    assert c.data_ptr() != b.data_ptr() and not c.any(), "the earlier result is alive: a fresh zeroed buffer"
+    assert bool((b == 7).all())
+    view = c[:, :1]
+    del c
+    d = kernels._kept_padded_buffer(cache, (1, 2, 4, 4), torch.int32, torch.device("cpu"))
+    assert d.data_ptr() != view.data_ptr(), "a view keeps the buffer taken"
+    del d, view
+    e = kernels._kept_padded_buffer(cache, (2, 2, 4, 4), torch.int32, torch.device("cpu"))
+    assert e.shape[0] == 2 and len(cache) == 1, "a new geometry replaces the buffer"
+
+
+def test_hand_off_buffers_do_not_travel_with_copies_of_a_module():
+    import copy
+    import pickle
+    conv = modules.Conv2dShift(4, 8, 3, padding=1)
+    conv.__dict__["_handoff_buffers"] = {"k": torch.zeros(3)}
+    clone = copy.deepcopy(conv)
+    assert "_handoff_buffers" not in clone.__dict__ and "_handoff_buffers" in conv.__dict__
+    assert torch.equal(clone.shift, conv.shift) and clone.shift_range == conv.shift_range
+    again = pickle.loads(pickle.dumps(conv))
+    assert "_handoff_buffers" not in again.__dict__ and torch.equal(again.sign, conv.sign)
+    convq = modules_q.Conv2dShiftQ(4, 8, 3, padding=1)
+    convq.__dict__["_handoff_buffers"] = {"k": torch.zeros(3)}
+    assert "_handoff_buffers" not in copy.deepcopy(convq).__dict__

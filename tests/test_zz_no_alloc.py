@@ -1,7 +1,8 @@
 """GPU: the allocation-free entry point ds_linear_tiled_noalloc_i32 against ds_linear_tiled_i32, through the
 C ABI, bit for bit: two calls in a row on launches that combine partial sums through the scratch (the second
-with a smaller input, so stale contents of the shared array would show), a launch that needs no scratch, and
-the size limit."""
+with a smaller input, so stale contents of the shared array would show), empty problems, and the size limit.
+"Allocates nothing" is checked at the driver: the device's free memory (hipMemGetInfo, which also sees a
+hipMalloc made inside the library, unlike torch's own allocator statistics) is the same before and after."""
 import ctypes
 
 import numpy as np
@@ -37,11 +38,19 @@ def _both(xT, blob, bias, M, K, N, bits):
     guard = 64
     ybuf = torch.full((M * N + 2 * guard,), 0x5A5A5A5A, dtype=torch.int32, device=DEV)
     y = ybuf[guard:guard + M * N]
-    before = torch.cuda.memory_allocated()
-    _lib.call("ds_linear_tiled_noalloc_i32", _lib.ptr(xT), xT.shape[1], _lib.ptr(blob), _lib.ptr(bd),
-              ctypes.c_void_p(y.data_ptr()), M, K, N, bits, 0, st)
-    assert torch.cuda.memory_allocated() == before
+    def call():
+        _lib.call("ds_linear_tiled_noalloc_i32", _lib.ptr(xT), xT.shape[1], _lib.ptr(blob), _lib.ptr(bd),
+                  ctypes.c_void_p(y.data_ptr()), M, K, N, bits, 0, st)
+
+    call()                       # the first call on a device looks the scratch array's address up
     torch.cuda.synchronize()
+    ybuf.fill_(0x5A5A5A5A)
+    torch.cuda.synchronize()
+    before_torch, before_free = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
+    call()
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before_torch
+    assert torch.cuda.mem_get_info()[0] == before_free, "the device's free memory changed across the call"
     host = ybuf.cpu().numpy()
     assert (host[:guard] == 0x5A5A5A5A).all() and (host[guard + M * N:] == 0x5A5A5A5A).all()
     return want.cpu().numpy(), host[guard:guard + M * N].reshape(M, N)
@@ -75,3 +84,17 @@ def test_noalloc_two_instruction_kernel_and_limit(oracle, rng):
     assert b"scratch" in L.ds_status_string(-6)
     assert 4 * 2048 * 2048 == limit      # the channel-major scratch of a 2048 x 2048 output just fits
     assert L.ds_linear_tiled_noalloc_i32(one, 2048, one, None, one, 2048, 0, 2048, 9, 0, None) == -2   # bits
+
+
+def test_noalloc_empty_problems_touch_nothing():
+    """M == 0 or N == 0: no scratch is needed, nothing is launched, nothing is written."""
+    L = _lib.lib()
+    st = _lib.current_stream(torch.device(DEV))
+    y = torch.full((256,), 0x5A5A5A5A, dtype=torch.int32, device=DEV)
+    xT = torch.zeros((8, 64), dtype=torch.int32, device=DEV)
+    blob = torch.zeros(4096, dtype=torch.uint8, device=DEV)
+    for (M, N) in [(0, 64), (64, 0)]:
+        assert L.ds_linear_tiled_noalloc_i32(_lib.ptr(xT), 64, _lib.ptr(blob), None, _lib.ptr(y), M, 8, N, 4, 0,
+                                             st) == 0
+    torch.cuda.synchronize()
+    assert bool((y == 0x5A5A5A5A).all())
