@@ -557,6 +557,58 @@ def pmc_target(device):
     torch.cuda.synchronize()
 
 
+def pmc_target_other(device):
+    """Counter targets for `rocprofv3 --pmc`, the launches below the 3x3 layers of the headline step: the
+    64 MiB copy (scale of the byte counters), then, three times over,
+      * benchmark configuration 2's convolution (3x3, 64 -> 64, 56x56, batch 32: 784 tiles on 512
+        workgroups) through ds_conv2d_tiled_i32;
+      * its 4096^3 shift GEMM through ds_linear_tiled_i32 (cooperative launch + transpose of the
+        channel-major scratch);
+      * the int8 kernel on ResNet-50's 1x1 convolutions with K = 256 (256 -> 64 at 56x56 and 256 -> 128 at
+        28x28, both at batch 128, weight_bits 3, activations in [0, 96]);
+      * the one-launch LinearShift kernel (ds_linear_small_f32) on the three layers of the MNIST MLP at
+        batch 64 and on ResNet-18's classifier (64 x 512 x 1000)."""
+    from deepshift_amd import _lib, kernels, utils
+    g = torch.Generator().manual_seed(0)
+    n = 16 * 1024 * 1024
+    src = torch.randint(0, 2 ** 20, (n,), generator=g, dtype=torch.int32).to(device)
+    dst = torch.empty_like(src)
+
+    def codes(shape, lo=-14):
+        shift = torch.randint(lo, 1, shape, generator=g).float()
+        sign = (torch.randint(0, 2, shape, generator=g) * 2 - 1).float()
+        return utils.compress_bits(shift, sign)
+
+    x2 = torch.randint(0, 2 ** 20, (32, 64, 58, 58), generator=g, dtype=torch.int32).to(device)
+    cw2 = codes((64, 64, 3, 3), lo=-15)
+    tiled2 = kernels._tiled_of(cw2, 64, 64, 3, 3)
+    xg = torch.randn(4096, 4096, generator=g).clamp_min(0).to(device)
+    cwg = codes((4096, 4096), lo=-15)
+    xT = kernels.quantize_transpose(xg)
+    tiledg = kernels._tiled_of(cwg, 4096, 4096)
+    int8 = []
+    for (C, H, O) in ((256, 56, 64), (256, 28, 128)):
+        x8 = torch.randint(0, 97, (128, C, H, H), generator=g, dtype=torch.int32).to(torch.int8).to(device)
+        cw8 = codes((O, C, 1, 1), lo=-2)
+        fields = kernels.paired_fields(cw8, O, 3, 5)
+        int8.append((x8, kernels._paired_of(cw8, fields, O, C, 1, 1), O, fields[1]))
+    small = []
+    for (M, K, N) in ((64, 784, 512), (64, 512, 512), (64, 512, 10), (64, 512, 1000)):
+        cws = codes((N, K))
+        small.append((torch.rand(M, K, generator=g).to(device), kernels._tiled_of(cws, N, K), N,
+                      kernels.kernel_bits(cws)))
+    torch.cuda.synchronize()
+    for _ in range(3):
+        _lib.call("ds_copy_i32", _lib.ptr(src), _lib.ptr(dst), n, _lib.current_stream(device))
+        kernels.conv2d_tiled(x2, tiled2, None, 64, (3, 3), (1, 1), cw2.bits, cw2.base)
+        kernels.linear_tiled(xT, 4096, tiledg, None, 4096, cwg.bits, cwg.base)
+        for x8, blob8, O, fb in int8:
+            kernels.conv2d_paired(x8, blob8, None, O, (1, 1), (1, 1), fb, 96)
+        for xs, tileds, N, kb in small:
+            kernels.linear_small(xs, tileds, None, N, kb, 0, 16, 16, False, True)
+    torch.cuda.synchronize()
+
+
 def cpu_baseline(shapes):
     """The oracle's restatement of the reference CPU kernel (shift_cpu.cpp loop nests, batch rows /
     images split over threads) on every shift layer of ResNet-18 at a reduced batch."""
@@ -634,6 +686,9 @@ def main():
     ap.add_argument("--pmc-target", action="store_true",
                     help="only launch the counter targets: a 64 MiB copy kernel and the dominant shift "
                          "kernel (ResNet-18 layer1 3x3 conv, batch 64), 3 times each")
+    ap.add_argument("--pmc-target-other", action="store_true",
+                    help="only launch the second set of counter targets: configuration 2's convolution and "
+                         "GEMM, int8 1x1 launches with K = 256, the one-launch linear kernel")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path "
@@ -644,6 +699,9 @@ def main():
 
     if args.pmc_target:
         pmc_target(device)
+        return
+    if args.pmc_target_other:
+        pmc_target_other(device)
         return
     if args.config5_only:
         print(json.dumps(config5(device, args.steps)), flush=True)

@@ -48,6 +48,8 @@ SIGNATURES = {
     "ds_paired_bytes": (_size, [_c_int, _c_int, _c_int]),
     "ds_tile_weights_paired_i32": (_c_int, [_ptr, _ptr] + [_c_int] * 6 + [_ptr]),
     "ds_conv2d_paired_i8": (_c_int, [_ptr] * 4 + [_c_int] * 11 + [_ptr]),
+    "ds_conv2d_paired_fused_workspace_bytes": (_size, [_c_int] * 11),
+    "ds_conv2d_paired_fused_i8": (_c_int, [_ptr] * 8 + [_c_int] * 18 + [_ptr, _size, _ptr]),
     "ds_quantize_pad_f32_i8": (_c_int, [_ptr, _ptr] + [_c_int] * 8 + [_ptr]),
     "ds_requantize_affine_pad_i8": (_c_int, [_ptr] * 6 + [_c_int] * 10 + [_ptr]),
     "ds_requantize_affine_maxpool_i8": (_c_int, [_ptr] * 5 + [_c_int] * 13 + [_ptr]),

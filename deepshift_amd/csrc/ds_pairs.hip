@@ -29,6 +29,7 @@
 // 64-pixel blocks of a tile -- wherever the bias is added.  The highest field value means "no
 // contribution" (zero weights, indices past K); the caller vouches that no real code uses it.
 #include "ds_common.h"
+#include "ds_coop.h"
 #include <atomic>
 #include <cstdlib>
 
@@ -59,6 +60,19 @@ struct PairArgs {
     int blocks_per_xcd;
     int atomic_out;
     uint32_t y_elems;
+    // Fused cooperative launch (shift_pairs_fused_kernel): arrival counters and partial-tile slots in the
+    // caller's workspace, and what follows the layer -- act(sum / 2^F * scale[c] + shift[c] + residual)
+    // stored as float (out) and / or as the next shift convolution's round-to-fixed, zero padded input (q).
+    unsigned long long *coop_counters;
+    unsigned long long coop_token;        // this launch's tag in the counters (never 0)
+    int32_t *coop_slots;
+    float *ep_out;
+    void *ep_q;
+    const float *ep_scale, *ep_shift, *ep_residual;
+    float ep_inv;                         // 2^-F of the sums
+    int ep_relu, ep_ph, ep_pw, ep_q_bytes;
+    int ep_border_kept;                   // the padding of q already holds zeros: write the interior only
+    QuantSpec ep_spec;
 };
 
 struct PairWalk {
@@ -113,6 +127,16 @@ DS_PAIRS_ONE(4, false, DS_PAIRX_ASM_B4, DS_PAIRX_CLOBBERS_B4)
 // that all the waves of the workgroup add up for one tile fit one chunk).
 enum { kStore, kAtomic, kLds, kLdsPacked };
 
+// The lane number, computed where it is called (volatile: not merged with an earlier computation): after
+// the main loop, whose fixed register map leaves eight vector registers free, so that no lane number has
+// to stay live across it.
+__device__ __forceinline__ int lane_now()
+{
+    int lane;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane));
+    return lane;
+}
+
 template <int BITS, int OUT, bool TU>
 __device__ __forceinline__ void pairs_segment(const PairArgs &p, int ntile, int m0, int g_begin, int g_end,
                                               int32_t *lds)
@@ -160,6 +184,7 @@ __device__ __forceinline__ void pairs_segment(const PairArgs &p, int ntile, int 
     }
 
     if (OUT == kLdsPacked) {
+        const int lane = lane_now();
 #pragma unroll
         for (int j = 0; j < 64; ++j)
 #pragma unroll
@@ -169,6 +194,7 @@ __device__ __forceinline__ void pairs_segment(const PairArgs &p, int ntile, int 
     }
     // split the sums into their halves (v = hi * 65536 + lo) and add them to the output
     if (OUT == kLds) {
+        const int lane = lane_now();
 #pragma unroll
         for (int j = 0; j < 64; ++j) {
 #pragma unroll
@@ -371,6 +397,367 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         __syncthreads();
         it += len;
     }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Fused cooperative launch: the scheme of the int32 shift-plane kernel's cooperative launch on the int8
+// tiles.  Equal shares of the (tile, K group) space per workgroup; the workgroup's waves split a tile
+// segment's K range and add their sums into the tile buffer in LDS; a tile whose whole reduction ran here
+// leaves through the fused epilogue; a tile that straddles a share boundary is stored to the workgroup's
+// slot in the workspace, its arrival counted, and the workgroup that arrives LAST at the tile adds the
+// other contributors' slots and writes it.  No pre-fill of an output, no global atomics on it, no int32
+// sums in memory, no separate conversion pass, and nobody waits for anybody.
+// PACKED: reductions of a single chunk on workgroups of four waves, the buffer holds two pixels per word
+// as the registers do (48 KiB, two workgroups per compute unit); otherwise eight waves on widened sums
+// (96 KiB, one workgroup per compute unit).
+struct PairTail {
+    const int32_t *negcnt, *bias;
+    int32_t *slots;
+    unsigned long long *counters;
+    unsigned long long token;
+    float *out;
+    void *q;
+    const float *scale, *shift, *residual;
+    long G, total;
+    int M, N, comm, pix_per_img, OW;
+    float inv;
+    int relu, ph, pw, q_bytes, border_kept;
+    QuantSpec spec;
+};
+typedef __attribute__((address_space(3))) const PairTail lds_ptail;
+
+constexpr int kPairUnit = 8;  // channels that one call of pairs_write_unit finishes
+
+// Eight channels x the tile's six 64-pixel blocks (48 outputs per lane) leave the tile buffer: bias (and,
+// for the xor-mask forms, the count of negative codes for the pixels that lived in low halves), then the
+// arithmetic of the int32 kernel's write_tile in the same order.  Everything that comes from memory is
+// requested up front: the per-channel constants by the lanes (lane c holds those of channel ch0 + c and
+// hands them out with v_readlane), the residuals of all 48 outputs before the first is used.
+template <typename Q, bool PACKED>
+__device__ __forceinline__ void pairs_write_unit(lds_ptail *t, lds_i32 *buf, int ntile, int m0, int ch0, int lane)
+{
+    typedef __attribute__((address_space(1))) Q g_q;
+    typedef __attribute__((address_space(1))) char g_char;
+    constexpr int CH = kPairUnit, PB = 6;
+    const int M = uniform(t->M), N = uniform(t->N), pix_per_img = uniform(t->pix_per_img), OW = uniform(t->OW);
+    const int n0 = ntile * 64 + ch0;
+    const int mine = n0 + (lane & (CH - 1));
+    const g_i32 *negcnt = uniform_global(t->negcnt), *bias = uniform_global(t->bias);
+    const int32_t add_l = bias ? bias[mine] : 0;
+    const int32_t neg_l = negcnt ? negcnt[mine] : 0;
+    float sa_l = 1.0f, sb_l = 0.0f;
+    const g_f32 *scale = uniform_global(t->scale), *shift = uniform_global(t->shift);
+    if (scale) sa_l = scale[mine];
+    if (shift) sb_l = shift[mine];
+    const g_f32 *residual = uniform_global(t->residual);
+    g_char *out = (g_char *)uniform_global(t->out);
+    g_char *q = (g_char *)uniform_global((char *)t->q);
+    const int ph = uniform(t->ph), pw = uniform(t->pw);
+    const int OH = pix_per_img / OW;
+    const int Wq = OW + 2 * pw;
+    const uint32_t qplane = (uint32_t)(OH + 2 * ph) * Wq;
+    bool live[PB];
+    uint32_t pix[PB], qpix[PB], qimg[PB];  // element indices (every tensor is below 2^31 bytes)
+    int oh[PB], ow[PB];
+#pragma unroll
+    for (int b = 0; b < PB; ++b) {
+        const int m = m0 + b * kWave + lane;
+        live[b] = m < M;
+        const int mm = live[b] ? m : 0;
+        const int img = mm / pix_per_img, rem = mm - img * pix_per_img;
+        oh[b] = rem / OW;
+        ow[b] = rem - oh[b] * OW;
+        pix[b] = (uint32_t)(img * N + n0) * (uint32_t)pix_per_img + rem;
+        qimg[b] = (uint32_t)(img * N + n0) * qplane;
+        qpix[b] = qimg[b] + (uint32_t)(oh[b] + ph) * Wq + ow[b] + pw;
+    }
+    float res[CH][PB];
+    if (residual) {
+#pragma unroll
+        for (int b = 0; b < PB; ++b) {
+            if (live[b]) {
+#pragma unroll
+                for (int c = 0; c < CH; ++c)
+                    res[c][b] = *(const g_f32 *)((const g_char *)residual + 4u * (pix[b] + (uint32_t)(c * pix_per_img)));
+            } else {
+#pragma unroll
+                for (int c = 0; c < CH; ++c) res[c][b] = 0.0f;
+            }
+        }
+    }
+    int32_t sums[CH][PB];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int32_t neg = __builtin_amdgcn_readlane(neg_l, c);
+        if (PACKED) {
+#pragma unroll
+            for (int r = 0; r < kPairRows; ++r) {
+                lds_i32 *cell = buf + (ch0 + c) * (kPairRows * kWave) + r * kWave + lane;
+                const int32_t v = *cell;
+                *cell = 0;
+                const int32_t lo = (int32_t)(int16_t)(v & 0xffff), hi = (v - lo) >> 16;
+                sums[c][2 * r] = lo + neg;
+                sums[c][2 * r + 1] = hi;
+            }
+        } else {
+#pragma unroll
+            for (int b = 0; b < PB; ++b) {
+                lds_i32 *cell = buf + (ch0 + c) * kPairPixels + b * kWave + lane;
+                sums[c][b] = *cell + ((b & 1) ? 0 : neg);
+                *cell = 0;
+            }
+        }
+    }
+    const float inv = uniform(t->inv), qs = uniform(t->spec.scale), qlo = uniform(t->spec.lo), qhi = uniform(t->spec.hi);
+    const bool relu = uniform(t->relu) != 0, one_bit = uniform(t->spec.I) == 1, has_res = residual != nullptr;
+    float f[CH][PB];
+    if (has_res) {
+        if (relu) tile_affine<CH, PB, true, true>(f, sums, res, add_l, sa_l, sb_l, inv);
+        else tile_affine<CH, PB, true, false>(f, sums, res, add_l, sa_l, sb_l, inv);
+    } else {
+        if (relu) tile_affine<CH, PB, false, true>(f, sums, res, add_l, sa_l, sb_l, inv);
+        else tile_affine<CH, PB, false, false>(f, sums, res, add_l, sa_l, sb_l, inv);
+    }
+    const uint32_t ostep = 4u * (uint32_t)pix_per_img, qstep = (uint32_t)sizeof(Q) * qplane;
+#pragma unroll
+    for (int b = 0; b < PB; ++b) {
+        if (!live[b]) continue;
+        if (out) {
+            uint32_t o = 4u * pix[b];
+#pragma unroll
+            for (int c = 0; c < CH; ++c, o += ostep) *(g_f32 *)(out + o) = f[c][b];
+        }
+        if (q) {
+            uint32_t o = (uint32_t)sizeof(Q) * qpix[b];
+            if (one_bit) {
+#pragma unroll
+                for (int c = 0; c < CH; ++c, o += qstep)
+                    *(g_q *)(q + o) = (Q)quantize_fixed_as<true>(f[c][b], qs, qlo, qhi);
+            } else {
+#pragma unroll
+                for (int c = 0; c < CH; ++c, o += qstep)
+                    *(g_q *)(q + o) = (Q)quantize_fixed_as<false>(f[c][b], qs, qlo, qhi);
+            }
+        }
+    }
+    if (q && (ph | pw) && !uniform(t->border_kept)) {
+        Q *qg = (Q *)t->q;
+#pragma unroll
+        for (int b = 0; b < PB; ++b) {
+            if (!live[b]) continue;
+            if (!(ow[b] == 0 || ow[b] == OW - 1 || oh[b] == 0 || oh[b] == OH - 1)) continue;
+            for (int c = 0; c < CH; ++c)
+                write_padding(qg, (size_t)qimg[b] + (size_t)c * qplane, oh[b], ow[b], OH, OW, ph, pw, Wq);
+        }
+    }
+}
+
+// The tail of one tile segment, after the workgroup's waves have added their sums into `buf` and met at
+// a barrier (a function of its own, so that its registers are allocated apart from the main loop's fixed
+// map).  A whole tile (len == comm) is written out.  A partial one is published to this workgroup's slot,
+// its arrival counted, and whichever workgroup arrives last gathers the slots of all contributors and
+// writes the tile.  Ends with the buffer cleared and a barrier.
+template <bool PACKED>
+__device__ __attribute__((noinline)) void pairs_finish_tile(lds_ptail *t, lds_i32 *buf, lds_i32 *flag, int w,
+                                                            long tile_start, int g0, int len, int ntile, int m0,
+                                                            int wave)
+{
+    constexpr int WAVES = PACKED ? kPairCu4Waves : kPairCuWaves, THREADS = WAVES * kWave;
+    constexpr int ELEMS = PACKED ? 64 * kPairRows * kWave : 64 * kPairPixels, PER = ELEMS / THREADS;
+    constexpr int UNITS = 64 / kPairUnit / WAVES;  // units of eight channels per wave
+    // (the thread's number from the wave's, which the caller holds in a scalar register, and the lane's:
+    // no work-item id has to stay in a vector register across the caller's main loop)
+    const int lane = lane_now();
+    const int tid = wave * kWave + lane;
+    const int comm = uniform(t->comm);
+    bool finish = len == comm;
+    if (!finish) {
+        g_i32 *slots = uniform_global(t->slots);
+        // slot 0 of a workgroup holds the tile its share starts in (g0 > 0), slot 1 the tile it ends in
+        g_i32 *slot = slots + ((size_t)2 * w + (g0 > 0 ? 0 : 1)) * ELEMS + tid;
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+            store_agent(slot + k * THREADS, buf[tid + k * THREADS]);
+            buf[tid + k * THREADS] = 0;
+        }
+        // the slot is complete (every store acknowledged) before the arrival is counted
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        const long G = uniform(t->G), total = uniform(t->total);
+        const int first = coop_owner(tile_start, G, total);
+        const int last = coop_owner(tile_start + comm - 1, G, total);
+        if (tid == 0) *flag = coop_arrive(t->counters + first, t->token, last - first);
+        __syncthreads();
+        if (*flag) {
+            for (int c = first; c <= last; ++c) {
+                const g_i32 *src = slots + ((size_t)2 * c + (c == first ? 1 : 0)) * ELEMS + tid;
+                int32_t v[PER];
+#pragma unroll
+                for (int k = 0; k < PER; ++k) v[k] = load_agent(src + k * THREADS);
+#pragma unroll
+                for (int k = 0; k < PER; ++k) buf[tid + k * THREADS] += v[k];
+            }
+            finish = true;
+        }
+        __syncthreads();
+    }
+    if (finish) {
+        const bool q8 = uniform(t->q_bytes) == 1;
+#pragma unroll
+        for (int u = 0; u < UNITS; ++u) {
+            const int ch0 = (wave * UNITS + u) * kPairUnit;
+            if (q8) pairs_write_unit<int8_t, PACKED>(t, buf, ntile, m0, ch0, lane);
+            else pairs_write_unit<int32_t, PACKED>(t, buf, ntile, m0, ch0, lane);
+        }
+    }
+    __syncthreads();
+}
+
+// Where a share stands: iteration `it` of [.., it_end) -> the tile it lies in, the K groups [g0, g0 + len)
+// of that tile that belong to the share, the tile's channel tile and first pixel.
+struct PairSegment {
+    int tile, g0, len, ntile, m0;
+};
+__device__ __forceinline__ PairSegment pairs_segment_at(const PairArgs &p, int it, int it_end)
+{
+    PairSegment s;
+    s.tile = uniform(it / p.comm);  // (the division runs on the vector ALU; its result is wave-uniform)
+    s.g0 = it - s.tile * p.comm;
+    int g1 = s.g0 + (it_end - it);
+    if (g1 > p.comm) g1 = p.comm;
+    s.len = g1 - s.g0;
+    const int mt = uniform(s.tile / p.tiles_n);
+    s.ntile = s.tile - mt * p.tiles_n;
+    s.m0 = mt * kPairPixels;
+    return s;
+}
+
+template <int BITS, bool TU, bool PACKED>
+__global__ __launch_bounds__(PACKED ? 256 : 512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void shift_pairs_fused_kernel(const PairArgs p)
+{
+    extern __shared__ int32_t tile_buf[];  // [64][384] sums, or [64][3][64] words of two sums (PACKED)
+    __shared__ PairTail tail;
+    __shared__ int32_t last_arrival;
+    // The share's position lives in LDS, not in registers: the main loop's fixed register map leaves the
+    // compiler a handful of scalar registers, and what is live across it must not need spilling.
+    __shared__ int32_t cursor[2];
+    constexpr int WAVES = PACKED ? kPairCu4Waves : kPairCuWaves, THREADS = WAVES * kWave;
+    constexpr int ELEMS = PACKED ? 64 * kPairRows * kWave : 64 * kPairPixels;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (threadIdx.x == 0) {
+        const long G = gridDim.x;
+        const int bid = blockIdx.x;
+        // an XCD (workgroup ids congruent modulo 8) takes a contiguous range of shares
+        const int w = (gridDim.x & 7) ? bid : (bid & 7) * (int)(gridDim.x >> 3) + (bid >> 3);
+        // (tile, K group) iterations: below 2^31 because every tensor is below 2^31 bytes
+        const int ntiles = p.tile_end - p.tile_begin;
+        const long total = (long)ntiles * p.comm;
+        if (p.whole_tiles) {
+            cursor[0] = (int)((long)w * ntiles / G) * p.comm;
+            cursor[1] = (int)((long)(w + 1) * ntiles / G) * p.comm;
+        } else {
+            cursor[0] = (int)(w * total / G);
+            cursor[1] = (int)((w + 1) * total / G);
+        }
+        tail.negcnt = p.negcnt; tail.bias = p.bias;
+        tail.slots = p.coop_slots; tail.counters = p.coop_counters; tail.token = p.coop_token;
+        tail.out = p.ep_out; tail.q = p.ep_q;
+        tail.scale = p.ep_scale; tail.shift = p.ep_shift; tail.residual = p.ep_residual;
+        tail.G = G; tail.total = total;
+        tail.M = p.M; tail.N = p.N; tail.comm = p.comm; tail.pix_per_img = p.pix_per_img; tail.OW = p.OW;
+        tail.inv = p.ep_inv; tail.relu = p.ep_relu; tail.ph = p.ep_ph; tail.pw = p.ep_pw;
+        tail.q_bytes = p.ep_q_bytes; tail.border_kept = p.ep_border_kept; tail.spec = p.ep_spec;
+    }
+    for (int i = threadIdx.x; i < ELEMS; i += THREADS) tile_buf[i] = 0;
+    __syncthreads();
+    for (;;) {
+        {
+            const int it = uniform(cursor[0]), it_end = uniform(cursor[1]);
+            if (it >= it_end) break;
+            const PairSegment s = pairs_segment_at(p, it, it_end);
+            const int wb = s.g0 + wave * s.len / WAVES, we = s.g0 + (wave + 1) * s.len / WAVES;
+            if (PACKED) {
+                // the whole reduction of a tile fits one chunk: so do the parts of it that meet in the buffer
+                if (wb < we) pairs_segment<BITS, kLdsPacked, TU>(p, s.ntile, s.m0, wb, we, tile_buf);
+            } else {
+                for (int g = wb; g < we; g += p.chunk) {
+                    const int ge = g + p.chunk < we ? g + p.chunk : we;
+                    pairs_segment<BITS, kLds, TU>(p, s.ntile, s.m0, g, ge, tile_buf);
+                }
+            }
+        }
+        __syncthreads();
+        const int it = uniform(cursor[0]), it_end = uniform(cursor[1]);
+        const PairSegment s = pairs_segment_at(p, it, it_end);
+        const int bid = blockIdx.x;
+        const int w = (gridDim.x & 7) ? bid : (bid & 7) * (int)(gridDim.x >> 3) + (bid >> 3);
+        pairs_finish_tile<PACKED>((lds_ptail *)&tail, (lds_i32 *)tile_buf, (lds_i32 *)&last_arrival, w,
+                                  (long)s.tile * p.comm, s.g0, s.len, s.ntile, s.m0, wave);
+        // (pairs_finish_tile ends with a barrier: everybody has read the cursor)
+        if (wave == 0 && lane_now() == 0) cursor[0] = it + s.len;
+        __syncthreads();
+    }
+}
+
+// Workgroups of the fused launch: one per compute unit (eight waves) or two (four waves, PACKED); small
+// layers at least 8 K groups per wave; every workgroup owns at least one iteration (a tile is finished by
+// the last of the workgroups that its range of iterations names: an empty share would never arrive).
+static int pairs_fused_blocks(long iters, bool packed)
+{
+    const int waves = packed ? kPairCu4Waves : kPairCuWaves;
+    int blocks = pair_slots() / waves;
+    const long fit = (iters / (8 * waves)) / 8 * 8;
+    if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
+    if (blocks > iters) blocks = iters < 1 ? 1 : (int)iters;
+    return blocks;
+}
+static size_t pairs_slot_bytes(bool packed) { return (size_t)(packed ? 64 * kPairRows * kWave : 64 * kPairPixels) * 4; }
+static size_t pairs_fused_workspace(long iters, bool packed)
+{
+    const int blocks = pairs_fused_blocks(iters, packed);
+    return coop_counter_bytes(blocks) + (size_t)2 * blocks * pairs_slot_bytes(packed);
+}
+
+template <int BITS, bool TU, bool PACKED>
+static int launch_pairs_fused_as(const PairArgs &a, int blocks, hipStream_t st)
+{
+    constexpr int kBytes = (PACKED ? 64 * kPairRows * kWave : 64 * kPairPixels) * 4;
+    if (!PACKED) {
+        // above the default 64 KiB limit of a workgroup: opt in, once per device
+        static std::atomic<bool> opted_in[64];
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+        if (!opted_in[dev].load(std::memory_order_acquire)) {
+            hipError_t e = hipFuncSetAttribute((const void *)shift_pairs_fused_kernel<BITS, TU, PACKED>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kBytes);
+            if (e != hipSuccess) return hip_status(e);
+            opted_in[dev].store(true, std::memory_order_release);
+        }
+    }
+    hipLaunchKernelGGL((shift_pairs_fused_kernel<BITS, TU, PACKED>), dim3(blocks), dim3(PACKED ? 256 : 512), kBytes, st, a);
+    return launch_status();
+}
+
+template <int BITS, bool TU>
+static int launch_pairs_fused(PairArgs a, void *workspace, size_t workspace_bytes, hipStream_t st)
+{
+    a.tiles_m = ceil_div(a.M, kPairPixels);
+    a.tiles_n = a.N / 64;
+    const long tiles = (long)a.tiles_m * a.tiles_n;
+    const long iters = tiles * a.comm;
+    a.tile_begin = 0;
+    a.tile_end = (int)tiles;
+    a.whole_tiles = 0;
+    const bool packed = a.comm <= a.chunk;
+    const int blocks = pairs_fused_blocks(iters, packed);
+    if (!workspace || workspace_bytes < pairs_fused_workspace(iters, packed) || ((uintptr_t)workspace & 255))
+        return DS_EWORKSPACE;
+    a.coop_counters = (unsigned long long *)workspace;
+    a.coop_slots = (int32_t *)((char *)workspace + coop_counter_bytes(blocks));
+    a.coop_token = next_coop_token();
+    if (packed) return launch_pairs_fused_as<BITS, TU, true>(a, blocks, st);
+    return launch_pairs_fused_as<BITS, TU, false>(a, blocks, st);
 }
 
 // y = bias[n] before an accumulating launch; y is [img][n][pix], dense.  With the xor-mask forms the
@@ -668,5 +1055,92 @@ DS_EXPORT int ds_conv2d_paired_i8(const int8_t *x, const void *paired, const int
     case 2: return top_unused ? launch_pairs<2, true>(a, (hipStream_t)stream) : launch_pairs<2, false>(a, (hipStream_t)stream);
     case 3: return launch_pairs<3, false>(a, (hipStream_t)stream);
     default: return launch_pairs<4, false>(a, (hipStream_t)stream);
+    }
+}
+
+// Fills the geometry part of PairArgs; returns a status (DS_OK with M == 0 for an empty problem).
+static int paired_args(PairArgs &a, const int8_t *x, const void *paired, const int32_t *bias, int Nb, int C, int Hp,
+                       int Wp, int O, int FH, int FW, int sh, int sw, int field_bits, int x_bound)
+{
+    if (Nb < 0 || sh < 1 || sw < 1 || Hp < FH || Wp < FW || x_bound < 1 || x_bound > 128) return DS_EINVAL;
+    const int OH = (Hp - FH) / sh + 1, OW = (Wp - FW) / sw + 1;
+    const size_t M = (size_t)Nb * OH * OW;
+    a = PairArgs{};
+    if (M == 0 || O == 0) return DS_OK;
+    const size_t K = (size_t)C * FH * FW;
+    const size_t x_bytes = (size_t)Nb * C * Hp * Wp;
+    if (x_bytes >= ((size_t)1 << 31) || M * O * 4 >= ((size_t)1 << 31)) return DS_ETOOLARGE;
+    const PairedGeom g = paired_geom(O, (int)K, field_bits);
+    a.x = x;
+    a.x_bytes = (uint32_t)x_bytes;
+    a.codes = (const uint32_t *)paired;
+    a.bias = bias;
+    a.negcnt = field_bits >= 3 ? (const int32_t *)((const char *)paired + g.negcnt_offset) : nullptr;
+    a.M = (int)M; a.N = O; a.K = (int)K; a.comm = g.comm;
+    a.pix_per_img = OH * OW; a.OW = OW;
+    a.x_img_stride = C * Hp * Wp; a.x_row_stride = sh * Wp; a.x_col_stride = sw;
+    a.y_img_stride = O * OH * OW; a.y_ch_stride = OH * OW;
+    a.y_elems = (uint32_t)(M * O);
+    a.x_plane = Hp * Wp; a.x_row = Wp;
+    a.FH = FH; a.FW = FW;
+    a.chunk = pair_chunk(field_bits, x_bound);
+    return DS_OK;
+}
+
+DS_EXPORT size_t ds_conv2d_paired_fused_workspace_bytes(int Nb, int C, int Hp, int Wp, int O, int FH, int FW, int sh,
+                                                        int sw, int field_bits, int x_bound)
+{
+    take_paired_top_unused(field_bits);
+    if (check_paired(O, C, FH, FW, field_bits)) return 0;
+    PairArgs a;
+    if (paired_args(a, nullptr, nullptr, nullptr, Nb, C, Hp, Wp, O, FH, FW, sh, sw, field_bits, x_bound)) return 0;
+    if (a.M == 0 || a.K == 0) return 0;
+    const long iters = (long)ceil_div(a.M, kPairPixels) * (a.N / 64) * a.comm;
+    return pairs_fused_workspace(iters, a.comm <= a.chunk);
+}
+
+DS_EXPORT int ds_conv2d_paired_fused_i8(const int8_t *x, const void *paired, const int32_t *bias, float *out, void *q,
+                                        const float *scale, const float *shift, const float *residual, int Nb,
+                                        int C, int Hp, int Wp, int O, int FH, int FW, int sh, int sw, int field_bits,
+                                        int x_bound, int F_in, int relu, int I, int F, int ph, int pw, int q_bytes,
+                                        void *workspace, size_t workspace_bytes, ds_stream_t stream)
+{
+    const bool top_unused = take_paired_top_unused(field_bits);
+    int rc = check_paired(O, C, FH, FW, field_bits);
+    if (rc) return rc;
+    if (!out && !q) return DS_EINVAL;
+    if (F_in < 0 || F_in > 31 || ph < 0 || pw < 0) return DS_EINVAL;
+    const int border_kept = (q_bytes & DS_Q_BORDER_KEPT) != 0;
+    q_bytes &= ~DS_Q_BORDER_KEPT;
+    if (q) {
+        if (q_bytes != 4 && q_bytes != 1) return DS_EINVAL;
+        if (I < 1 || F < 0 || I + F > 32) return DS_EINVAL;
+        if (q_bytes == 1 && (I < 2 || I + F > 8)) return DS_EINVAL;
+    } else {
+        I = 16; F = 16; q_bytes = 4; ph = pw = 0;
+    }
+    PairArgs a;
+    rc = paired_args(a, x, paired, bias, Nb, C, Hp, Wp, O, FH, FW, sh, sw, field_bits, x_bound);
+    if (rc) return rc;
+    if (a.M == 0) return DS_OK;
+    if (!paired || !x || a.K == 0) return DS_EINVAL;
+    const int OH = a.pix_per_img / a.OW;
+    if ((size_t)Nb * O * (OH + 2 * ph) * (a.OW + 2 * pw) * (size_t)q_bytes >= ((size_t)1 << 31)) return DS_ETOOLARGE;
+    a.ep_out = out;
+    a.ep_q = q;
+    a.ep_scale = scale; a.ep_shift = shift; a.ep_residual = residual;
+    a.ep_inv = ldexpf(1.0f, -F_in);
+    a.ep_relu = relu;
+    a.ep_ph = ph; a.ep_pw = pw; a.ep_q_bytes = q_bytes;
+    a.ep_border_kept = border_kept;
+    a.ep_spec = make_spec(I, F, DS_Q_ROUND_TO_FIXED);
+    hipStream_t st = (hipStream_t)stream;
+    switch (field_bits) {
+    case 1: return top_unused ? launch_pairs_fused<1, true>(a, workspace, workspace_bytes, st)
+                              : launch_pairs_fused<1, false>(a, workspace, workspace_bytes, st);
+    case 2: return top_unused ? launch_pairs_fused<2, true>(a, workspace, workspace_bytes, st)
+                              : launch_pairs_fused<2, false>(a, workspace, workspace_bytes, st);
+    case 3: return launch_pairs_fused<3, false>(a, workspace, workspace_bytes, st);
+    default: return launch_pairs_fused<4, false>(a, workspace, workspace_bytes, st);
     }
 }

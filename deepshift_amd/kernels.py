@@ -27,7 +27,7 @@ from . import _lib
 
 __all__ = ["linear", "conv2d", "compress_sign_and_shift", "quantize", "quantize_pad",
            "quantize_transpose", "dequantize", "tile_weights", "linear_tiled", "conv2d_tiled",
-           "conv2d_tiled_fused", "conv2d_fusable"]
+           "conv2d_tiled_fused", "conv2d_fusable", "conv2d_paired", "conv2d_paired_fused"]
 
 
 def _pair(v):
@@ -749,6 +749,66 @@ def conv2d_paired(x_padded, paired, bias, O, kernel_size, stride, field_bits, x_
                   Nb, C, Hp, Wp, O, FH, FW, sh, sw, int(field_bits), int(x_bound),
                   _lib.current_stream(x_padded.device))
     return out
+
+
+def conv2d_paired_fused(x_padded, paired, bias, O, kernel_size, stride, field_bits, x_bound, fraction_bits_in,
+                        scale=None, shift=None, residual=None, relu=False, emit=None, want_float=True,
+                        q_cache=None):
+    """:func:`conv2d_paired` with what follows the layer done in the kernel's epilogue, the int8 kernel's
+    counterpart of :func:`conv2d_tiled_fused` (same arguments and return value): ``(out, q)`` = the float
+    result ``act(y / 2**F * scale[c] + shift[c] + residual)`` (``None`` unless ``want_float``) and, with
+    ``emit = (padding, integer_bits, fraction_bits, dtype)``, the next shift convolution's round-to-fixed,
+    zero padded input.  Bit-identical to :func:`conv2d_paired` followed by :func:`requantize_affine_pad`
+    / :func:`dequantize_affine`; no pre-fill, no atomics, the int32 sums are never stored."""
+    if x_padded.dtype != torch.int8 or not x_padded.is_cuda or x_padded.dim() != 4:
+        raise TypeError("x_padded must be a 4-D int8 GPU tensor")
+    x_padded = x_padded.contiguous()
+    Nb, C, Hp, Wp = x_padded.shape
+    FH, FW = _pair(kernel_size)
+    sh, sw = _pair(stride)
+    if Hp < FH or Wp < FW:
+        raise ValueError("padded input %dx%d is smaller than the %dx%d filter" % (Hp, Wp, FH, FW))
+    OH, OW = (Hp - FH) // sh + 1, (Wp - FW) // sw + 1
+    dev = x_padded.device
+    for name, t in (("scale", scale), ("shift", shift)):
+        if t is not None and (t.dtype != torch.float32 or t.numel() != O or not t.is_contiguous()):
+            raise ValueError("%s must be a contiguous float32 tensor of %d elements" % (name, O))
+    if residual is not None:
+        if tuple(residual.shape) != (Nb, O, OH, OW) or residual.dtype != torch.float32:
+            raise ValueError("residual must be float32 with the shape of the output")
+        residual = residual.contiguous()
+    if emit is None and not want_float:
+        raise ValueError("nothing to produce")
+    out = torch.empty([Nb, O, OH, OW], dtype=torch.float32, device=dev) if want_float else None
+    q, ph, pw, I, Fq, qb = None, 0, 0, 16, 16, 4
+    if emit is not None:
+        padding, I, Fq, dtype = emit
+        ph, pw = _pair(padding)
+        qb = 1 if dtype == torch.int8 else 4
+        shape = (Nb, O, OH + 2 * ph, OW + 2 * pw)
+        if q_cache is not None and (ph or pw):
+            q = _kept_padded_buffer(q_cache, shape, dtype, dev)
+            qb |= _lib.DS_Q_BORDER_KEPT
+        else:
+            q = torch.empty(shape, dtype=dtype, device=dev)
+    L = _lib.lib()
+    ws_bytes = L.ds_conv2d_paired_fused_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, int(field_bits),
+                                                        int(x_bound))
+    ws = _workspace(ws_bytes, dev)
+    keep = (x_padded, paired, bias, out, q, scale, shift, residual, ws)
+
+    def launch():
+        t = keep
+        _lib.call("ds_conv2d_paired_fused_i8", _lib.ptr(t[0]), _lib.ptr(t[1]), _lib.ptr(t[2]), _lib.ptr(t[3]),
+                  _lib.ptr(t[4]), _lib.ptr(t[5]), _lib.ptr(t[6]), _lib.ptr(t[7]), Nb, C, Hp, Wp, O, FH, FW,
+                  sh, sw, int(field_bits), int(x_bound), int(fraction_bits_in), int(bool(relu)), int(I), int(Fq),
+                  ph, pw, qb, _lib.ptr(t[8]), ws_bytes, _lib.current_stream(dev))
+
+    with _Timed("conv", Nb * OH * OW, C * FH * FW, O, dev):
+        launch()
+    if _REPLAY_SINK is not None:
+        _REPLAY_SINK.append(("conv", Nb * OH * OW, C * FH * FW, O, launch))
+    return out, q
 
 
 def conv2d(input, shift, sign, bias=None, conc_weight=None, stride=1, padding=0, dilation=1,

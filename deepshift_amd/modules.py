@@ -302,6 +302,7 @@ def conv_cpu_forward(module, input, shift, sign):
 # Switch for the fused convolution epilogue (kernels.conv2d_tiled_fused); off = always the separate
 # conversion pass, which the tests compare it with.
 _FUSE_EPILOGUE = True
+_FUSE_INT8 = True   # ... and the int8 kernel's (kernels.conv2d_paired_fused)
 
 
 def _small_for_int8(module, input_shape, field_bits):
@@ -365,6 +366,20 @@ def conv_kernel_forward(module, input, conc_weight, scale=None, shift=None, resi
         # round_to_fixed clamps to [-2^(I-1), 2^(I-1) - 1] (utils.py:7-21): |x| <= 2^(I+F-1), and after
         # a ReLU x <= (2^(I-1) - 1) * 2^F
         bound = (2 ** (I - 1) - 1) * 2 ** Fb if (prequantized and input_nonneg) else 2 ** (I + Fb - 1)
+        if pool is None and _FUSE_EPILOGUE and _FUSE_INT8:
+            # the int8 kernel's fused launch: dequantisation, affine / residual / ReLU and the next layer's
+            # conversion in the epilogue; no pre-fill, no atomics, no int32 sums, no separate pass
+            want_float, spec = True, None
+            if emit is not None:
+                next_padding, next_I, next_F, want_float = emit[:4]
+                spec = (next_padding, next_I, next_F, emit[4] if len(emit) == 5 else torch.int32)
+            cache = module.__dict__.setdefault("_handoff_buffers", {})
+            f, q = kernels.conv2d_paired_fused(xq, blob, bias, module.out_channels, module.kernel_size,
+                                               module.stride, fields[1], max(1, bound), Fb, scale, shift,
+                                               residual, relu, spec, want_float, cache)
+            if emit is None:
+                return f
+            return (f, q) if want_float else q
         out = kernels.conv2d_paired(xq, blob, bias, module.out_channels, module.kernel_size, module.stride,
                                     fields[1], max(1, bound))
     else:

@@ -171,6 +171,28 @@ int ds_conv2d_paired_i8(const int8_t *x, const void *paired, const int32_t *bias
                         int C, int Hp, int Wp, int O, int FH, int FW, int sh, int sw, int field_bits,
                         int x_bound, ds_stream_t stream);
 
+/* ds_conv2d_paired_i8 with what follows the layer at inference time done in the kernel's epilogue, as
+ * ds_conv2d_tiled_fused_i32 does for int32 activations (Conv2dShiftFunction's out.float() / 2**F,
+ * modules.py:161-162, the ops between two shift layers, and the next layer's round_to_fixed + cast +
+ * padding, modules.py:317,:153, kernels.py:32-36):
+ *   v = act(float(sum) / 2^F_in * scale[c] + shift[c] + residual)
+ *   out [Nb][O][OH][OW] float = v                                                  (or NULL)
+ *   q   [Nb][O][OH+2ph][OW+2pw] = round_to_fixed(v, I, F) * 2^F, zero padded      (or NULL)
+ * bit-identical to ds_conv2d_paired_i8 followed by ds_requantize_affine_pad_i8 / _i32; the int32 sums
+ * are never stored.  q_bytes 1: q is int8 (2 <= I, I + F <= 8); 4: int32; | DS_Q_BORDER_KEPT: the
+ * padding of q already holds zeros and only the interior is written.  The launch cuts the (tile, K
+ * group) space into equal shares per workgroup; tiles that two workgroups share are finished by the
+ * last arrival through partial tiles in the workspace: ds_conv2d_paired_fused_workspace_bytes() bytes,
+ * 256-byte aligned, contents arbitrary on entry (DS_EWORKSPACE otherwise).  Every geometry that
+ * ds_conv2d_paired_i8 takes is served, C > 0. */
+size_t ds_conv2d_paired_fused_workspace_bytes(int Nb, int C, int Hp, int Wp, int O, int FH, int FW, int sh,
+                                              int sw, int field_bits, int x_bound);
+int ds_conv2d_paired_fused_i8(const int8_t *x, const void *paired, const int32_t *bias, float *out, void *q,
+                              const float *scale, const float *shift, const float *residual, int Nb, int C,
+                              int Hp, int Wp, int O, int FH, int FW, int sh, int sw, int field_bits,
+                              int x_bound, int F_in, int relu, int I, int F, int ph, int pw, int q_bytes,
+                              void *workspace, size_t workspace_bytes, ds_stream_t stream);
+
 /* The conversion passes with an int8 result, for that kernel's input: ds_quantize_pad_f32_i32,
  * ds_requantize_affine_pad_i32 and ds_requantize_affine_maxpool_i32 with q int8, always in mode
  * DS_Q_ROUND_TO_FIXED (utils.py:7-21, whose clamp is what bounds the values).  DS_EINVAL unless

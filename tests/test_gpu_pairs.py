@@ -237,8 +237,9 @@ def test_models_with_8_bit_activations_take_the_int8_kernel_and_keep_their_outpu
     model = model.to(DEV)
     x = torch.randn(2, 3, 64, 64, generator=g).to(DEV)
     calls = []
-    real = kernels.conv2d_paired
+    real, real_fused = kernels.conv2d_paired, kernels.conv2d_paired_fused
     monkeypatch.setattr(kernels, "conv2d_paired", lambda *a, **k: calls.append(1) or real(*a, **k))
+    monkeypatch.setattr(kernels, "conv2d_paired_fused", lambda *a, **k: calls.append(1) or real_fused(*a, **k))
     with torch.no_grad():
         fused = fuse.fuse_conv_epilogues(model)
         got = fused(x)
@@ -255,6 +256,13 @@ def test_models_with_8_bit_activations_take_the_int8_kernel_and_keep_their_outpu
     assert len(calls) == taken
     assert torch.equal(got, want)
     assert torch.equal(unfused, want_unfused)
+    # ... and neither does switching the int8 kernel's fused launch off (int8 kernel + conversion pass)
+    monkeypatch.undo()
+    from deepshift_amd import modules
+    monkeypatch.setattr(modules, "_FUSE_INT8", False)
+    with torch.no_grad():
+        assert torch.equal(fuse.fuse_conv_epilogues(model)(x), got)
+        assert torch.equal(model(x), unfused)
 
 
 @pytest.mark.parametrize("seed", range(24))
@@ -338,3 +346,144 @@ def test_paired_launch_regimes(oracle, rng, form, regime):
         with _Tune(**env):
             got = abi_conv_paired(x8, blob, bias, O, FH, FW, stride, form)
         np.testing.assert_array_equal(got, want, err_msg=str((Nb, C, Hp, Wp, O, FH, FW)))
+
+
+# ---- the fused cooperative launch (ds_conv2d_paired_fused_i8) --------------------------------------------
+
+def abi_conv_paired_fused(x8, blob, bias, O, FH, FW, stride, field_bits, x_bound, F_in, scale, shift, res, relu,
+                          want_float, emit, border_kept=False):
+    """emit = (ph, pw, I, F, torch dtype) or None; returns (out or None, q or None); guard bands around both
+    outputs are checked, the workspace starts with stale contents."""
+    from oracle import shift_oracle as so  # noqa: F401  (the callers use it)
+    Nb, C, Hp, Wp = x8.shape
+    sh, sw = stride
+    OH, OW = (Hp - FH) // sh + 1, (Wp - FW) // sw + 1
+    L = _lib.lib()
+    ws_bytes = L.ds_conv2d_paired_fused_workspace_bytes(Nb, C, Hp, Wp, O, FH, FW, sh, sw, field_bits, x_bound)
+    assert ws_bytes > 0
+    ws = torch.full((ws_bytes,), 0x77, dtype=torch.uint8, device=DEV)
+    guard = 64
+    n_out = Nb * O * OH * OW
+    obuf = torch.full((n_out + 2 * guard,), 12345.0, dtype=torch.float32, device=DEV)
+    out = obuf[guard:guard + n_out] if want_float else None
+    q = qbuf = None
+    ph = pw = 0
+    I, Fq, qb = 16, 16, 4
+    n_q = 0
+    if emit is not None:
+        ph, pw, I, Fq, dtype = emit
+        n_q = Nb * O * (OH + 2 * ph) * (OW + 2 * pw)
+        qbuf = torch.full((n_q + 2 * guard,), 0x5A, dtype=dtype, device=DEV)
+        q = qbuf[guard:guard + n_q]
+        if border_kept:
+            q.zero_()
+        qb = (1 if dtype == torch.int8 else 4) | (_lib.DS_Q_BORDER_KEPT if border_kept else 0)
+    xd = torch.from_numpy(x8).to(DEV)
+    t = [None if a is None else dev(a) for a in (bias, scale, shift, res)]
+    _lib.call("ds_conv2d_paired_fused_i8", _lib.ptr(xd), _lib.ptr(blob), _lib.ptr(t[0]),
+              None if out is None else ctypes.c_void_p(out.data_ptr()),
+              None if q is None else ctypes.c_void_p(q.data_ptr()), _lib.ptr(t[1]), _lib.ptr(t[2]), _lib.ptr(t[3]),
+              Nb, C, Hp, Wp, O, FH, FW, sh, sw, field_bits, x_bound, F_in, int(relu), I, Fq, ph, pw, qb,
+              _lib.ptr(ws), ws_bytes, stream())
+    torch.cuda.synchronize()
+    oh = obuf.cpu().numpy()
+    assert (oh[:guard] == 12345.0).all() and (oh[guard + n_out:] == 12345.0).all(), "write outside out"
+    got_out = oh[guard:guard + n_out].reshape(Nb, O, OH, OW) if want_float else None
+    if not want_float:
+        assert (oh == 12345.0).all()
+    got_q = None
+    if q is not None:
+        qh = qbuf.cpu().numpy()
+        assert (qh[:guard] == 0x5A).all() and (qh[guard + n_q:] == 0x5A).all(), "write outside q"
+        got_q = qh[guard:guard + n_q].reshape(Nb, O, OH + 2 * ph, OW + 2 * pw).astype(np.int32)
+    return got_out, got_q
+
+
+def _chain(oracle, x8, s, sign, bias, stride, F_in, scale, shift, res, relu, emit):
+    from oracle import shift_oracle as so
+    y = oracle.conv2d(x8.astype(np.int32), -s, sign, bias, stride, nthreads=NTHREADS)
+    v = so.np_dequantize_affine(y, F_in, scale, shift, res, relu)
+    q = None if emit is None else so.np_requantize(v, emit[2], emit[3], (emit[0], emit[1]))
+    return v, q
+
+
+FUSED_SHAPES = [
+    # Nb, C, Hp, Wp, O, FH, FW, stride
+    (2, 64, 18, 18, 128, 3, 3, (1, 1)),        # K = 576: several chunks per wave, few tiles: every tile shared
+    (1, 300, 9, 9, 64, 3, 3, (1, 1)),          # one ragged pixel tile, K = 2700: cut many times
+    (2, 64, 16, 16, 64, 1, 1, (1, 1)),         # K = 64: a single chunk (packed tile buffer), partial last group
+    (16, 32, 30, 30, 64, 1, 1, (1, 1)),        # many tiles, one chunk: several whole tiles per workgroup
+    (4, 128, 14, 14, 256, 1, 1, (2, 2)),       # strided 1x1, four channel tiles
+    (3, 3, 37, 37, 64, 7, 7, (2, 2)),          # stem-like, strided, K = 147
+    (5, 256, 9, 11, 64, 1, 1, (1, 1)),         # K = 256: one chunk only with the post-ReLU bound
+]
+
+
+@pytest.mark.parametrize("form", FORMS, ids=form_id)
+@pytest.mark.parametrize("shape", FUSED_SHAPES, ids=lambda s: "x".join(map(str, s[:7])))
+def test_paired_fused_matches_oracle_chain(oracle, rng, form, shape):
+    """BatchNorm affine + residual + ReLU + the next layer's padded 3.5 input (int8), float result too."""
+    Nb, C, Hp, Wp, O, FH, FW, stride = shape
+    bits = form & 0xff
+    x8 = random_int8(rng, (Nb, C, Hp, Wp))
+    s, sign = random_codes(rng, (O, C, FH, FW), max_s=top_field(form))
+    bias = rng.integers(-2 ** 8, 2 ** 8, size=O).astype(np.int32)
+    w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)
+    blob = abi_tile_paired(w, O, C, FH, FW, bits, form)
+    OH, OW = (Hp - FH) // stride[0] + 1, (Wp - FW) // stride[1] + 1
+    scale = (rng.random(O).astype(np.float32) + 0.5) * np.float32(2.0 ** -4)
+    shift = rng.standard_normal(O).astype(np.float32)
+    res = rng.standard_normal((Nb, O, OH, OW)).astype(np.float32)
+    emit = (1, 1, 3, 5, torch.int8)
+    want_v, want_q = _chain(oracle, x8, s, sign, bias, stride, 5, scale, shift, res, True, emit)
+    out, q = abi_conv_paired_fused(x8, blob, bias, O, FH, FW, stride, form, 128, 5, scale, shift, res, True, True, emit)
+    np.testing.assert_array_equal(out, want_v)
+    np.testing.assert_array_equal(q, want_q)
+
+
+@pytest.mark.parametrize("shape", FUSED_SHAPES[:4], ids=lambda s: "x".join(map(str, s[:7])))
+def test_paired_fused_output_forms(oracle, rng, shape):
+    """Every combination the fused pipeline asks for: float only; fixed point only (int8 and int32, other
+    formats and paddings, kept border); no affine, no bias, no ReLU; non-negative input under the tighter
+    bound."""
+    Nb, C, Hp, Wp, O, FH, FW, stride = shape
+    form = 2 | U
+    x8 = rng.integers(0, 97, size=(Nb, C, Hp, Wp)).astype(np.int8)
+    s, sign = random_codes(rng, (O, C, FH, FW), max_s=2)
+    w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), 2)
+    blob = abi_tile_paired(w, O, C, FH, FW, 2, form)
+    OH, OW = (Hp - FH) // stride[0] + 1, (Wp - FW) // stride[1] + 1
+    scale = (rng.random(O).astype(np.float32) + 0.5) * np.float32(2.0 ** -5)
+    shift = rng.standard_normal(O).astype(np.float32)
+    res = rng.standard_normal((Nb, O, OH, OW)).astype(np.float32)
+    cases = [
+        # bound, scale, shift, res, relu, want_float, emit, border_kept
+        (96, scale, shift, None, True, True, None, False),
+        (96, scale, shift, None, True, False, (1, 1, 3, 5, torch.int8), False),
+        (96, scale, shift, None, True, False, (1, 1, 3, 5, torch.int8), True),
+        (128, scale, shift, res, False, True, (0, 0, 3, 5, torch.int8), False),
+        (128, None, None, None, False, True, (2, 1, 16, 16, torch.int32), False),
+        (96, scale, None, res, True, False, (1, 2, 4, 4, torch.int8), True),
+    ]
+    for bound, sc, sf, rs, relu, want_float, emit, kept in cases:
+        want_v, want_q = _chain(oracle, x8, s, sign, None, stride, 5, sc, sf, rs, relu, emit)
+        out, q = abi_conv_paired_fused(x8, blob, None, O, FH, FW, stride, form, bound, 5, sc, sf, rs, relu,
+                                       want_float, emit, kept)
+        if want_float:
+            np.testing.assert_array_equal(out, want_v)
+        if emit is not None:
+            np.testing.assert_array_equal(q, want_q)
+
+
+def test_paired_fused_rejects_bad_arguments():
+    L = _lib.lib()
+    one = ctypes.c_void_p(256)
+    args = (2, 64, 16, 16, 64, 1, 1, 1, 1, 2, 128, 5, 1, 3, 5, 1, 1, 1)
+    assert L.ds_conv2d_paired_fused_i8(one, one, None, None, None, None, None, None, *args, one, 1 << 30, None) == -1
+    assert L.ds_conv2d_paired_fused_i8(one, one, None, one, None, None, None, None, *args, None, 0, None) == -4
+    assert L.ds_conv2d_paired_fused_i8(one, one, None, one, None, None, None, None, *args, one, 16, None) == -4
+    bad_bits = args[:9] + (5,) + args[10:]
+    assert L.ds_conv2d_paired_fused_i8(one, one, None, one, None, None, None, None, *bad_bits, one, 1 << 30, None) == -2
+    bad_q = args[:13] + (16, 16) + args[15:]   # an int8 q cannot hold 16.16
+    assert L.ds_conv2d_paired_fused_i8(one, one, None, None, one, None, None, None, *bad_q, one, 1 << 30, None) == -1
+    assert L.ds_conv2d_paired_fused_workspace_bytes(2, 64, 16, 16, 48, 1, 1, 1, 1, 2, 128) == 0   # not 64 channels wide
