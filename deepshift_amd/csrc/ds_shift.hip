@@ -1643,10 +1643,13 @@ DS_EXPORT int ds_conv2d_tiled_fusable(int Nb, int C, int Hp, int Wp, int O, int 
         const bool two_instruction = width == 5 || plane_regime(a, false) < 0;
         return two_instruction && narrow_coop_fits(a);
     }
-    // where the dispatch would launch cooperatively anyway: long reductions on few tiles; shorter ones
-    // through the two-instruction kernel's cooperative launch where that fills the machine
-    const int regime = plane_regime(a, true);
-    return (a.comm >= 64 && regime == 0) || (regime < 0 && narrow_coop_fits(a));
+    // The 64-channel form: every layer.  Long reductions launch cooperatively anyway; for short ones (1x1
+    // convolutions, K below 64 groups) the unfused launches are faster by themselves, but the fused one
+    // also replaces the pass that follows them, which costs more than the difference on every layer shape
+    // of a ResNet-50 at batch 128 (64 -> 256 at 56x56: 742 us for launch + pass, 539 fused; 256 -> 64:
+    // 381 / 341; 256 -> 1024 at 14x14: 447 / 347).  Where the plane kernels have too few K groups the
+    // dispatch hands the layer to the two-instruction kernel's cooperative launch if that fills the machine.
+    return 1;
 }
 
 DS_EXPORT int ds_conv2d_tiled_fused_i32(const int32_t *x, const void *tiled, const int32_t *bias, float *out,

@@ -325,9 +325,9 @@ int ds_cpu_conv2d_i32(const int32_t *x_padded, const int8_t *shift, const int32_
  * the machine, that of the two-instruction kernel.  Other layers (ordinary codes of at most 5 bits;
  * DS_EINVAL for 6-bit fields and zero-top blobs) run the cooperative launch of the two-instruction
  * kernel, which needs no workspace.  ds_conv2d_tiled_fusable() says whether the fused call is also
- * the faster choice for a shape (long reductions on the 64-channel form, and every shape whose tiles
- * on the two-instruction kernel give each SIMD two waves; elsewhere the launch form loses more than
- * the separate pass costs).
+ * the faster choice for a shape than the plain launch followed by a conversion pass (every shape of the
+ * 64-channel form, and every other shape whose tiles on the two-instruction kernel give each SIMD two
+ * waves; elsewhere the launch form loses more than the separate pass costs).
  * No counterpart in the reference. */
 #define DS_Q_BORDER_KEPT 0x100
 int ds_conv2d_tiled_fusable(int Nb, int C, int Hp, int Wp, int O, int FH, int FW, int sh, int sw,

@@ -13,6 +13,10 @@ DEV = "cuda:0"
 NTHREADS = min(16, os.cpu_count() or 1)
 
 
+def _np(t):
+    return None if t is None else t.cpu().numpy()
+
+
 def _codes(g, shape, lo=-15):
     shift = torch.randint(lo, 1, shape, generator=g).float()
     sign = (torch.randint(0, 2, shape, generator=g) * 2 - 1).float()
@@ -149,6 +153,22 @@ def test_config5_int8_layers_full_size(oracle, layer):
     perm = torch.randperm(Nb, generator=g).to(DEV)
     assert torch.equal(kernels.conv2d_paired(x8[perm].contiguous(), blob, bias, O, (F, F), (stride, stride), 2, 96),
                        want[perm])
+    # the fused launch the 8-bit pipeline issues (ds_conv2d_paired_fused_i8: BatchNorm affine, residual, ReLU,
+    # float result and the next layer's padded int8 input from the epilogue): the first image against the
+    # oracle chain, the whole batch against the conversion pass on the int32 kernel's sums
+    from oracle import shift_oracle as so
+    OH = want.shape[2]
+    scale = ((torch.rand(O, generator=g) + 0.5) * 2.0 ** -5).to(DEV)
+    shf = torch.randn(O, generator=g).to(DEV)
+    res = torch.randn(Nb, O, OH, OH, generator=g).to(DEV)
+    for bound in (128, 96):
+        out, q = kernels.conv2d_paired_fused(x8, blob, bias, O, (F, F), (stride, stride), 2, bound, 5, scale, shf,
+                                             res, True, ((1, 1), 3, 5, torch.int8), True, {})
+        v = so.np_dequantize_affine(first, 5, _np(scale), _np(shf), _np(res[:1]), True)
+        np.testing.assert_array_equal(_np(out[:1]), v)
+        np.testing.assert_array_equal(_np(q[:1]).astype(np.int32), so.np_requantize(v, 3, 5, (1, 1)))
+        want_f, want_q = kernels.requantize_affine_pad(want, 5, scale, shf, res, True, (1, 1), 3, 5, True, torch.int8)
+        assert torch.equal(out, want_f) and torch.equal(q, want_q), bound
 
 
 def _default_init_codes(g, shape, weight_bits=5):
@@ -239,10 +259,6 @@ def test_config4_resnet18_batch64_every_layer_shape(oracle):
     assert len(shapes) == 12
     for L in shapes:
         _run_layer_full(oracle, g, L, [0, 63])
-
-
-def _np(t):
-    return None if t is None else t.cpu().numpy()
 
 
 def test_config3_resnet20_batch256_fused_launches(oracle):

@@ -98,6 +98,12 @@ GEOMS = [
     (3, 128, 16, 15, 192, 3, 3, (2, 2)),     # strided, three channel tiles
     (5, 384, 12, 12, 64, 1, 1, (1, 1)),      # 1x1 with a long reduction (64 K groups)
     (2, 40, 21, 19, 64, 5, 3, (1, 2)),       # 5x3 filter, K = 600
+    # short reductions on the 64-channel form: the 1x1 convolutions of a bottleneck block (modules.py:312-340
+    # followed by the same glue as every other layer)
+    (4, 64, 20, 20, 256, 1, 1, (1, 1)),      # 64 -> 256, 11 K groups: less than a group per wave of some tiles
+    (3, 256, 14, 14, 64, 1, 1, (1, 1)),      # 256 -> 64, 43 K groups
+    (2, 256, 17, 16, 512, 1, 1, (2, 2)),     # strided shortcut, eight channel tiles
+    (6, 3, 37, 37, 64, 7, 7, (2, 2)),        # a stem without its pooling: K = 147, a partial last group
 ]
 # layers that are not a multiple of 64 channels wide: the fused form of the two-instruction kernel
 NARROW_GEOMS = [
@@ -259,7 +265,7 @@ def test_fused_entry_point_refuses_what_it_cannot_do(rng):
     assert L.ds_conv2d_tiled_fused_i32(*args(64, 4, -1, True)) == -1    # left shifts
     assert L.ds_conv2d_tiled_fused_i32(*args(64, 4, 0, False)) == -4    # 64-channel form without its workspace
     assert L.ds_conv2d_tiled_fusable(64, 64, 58, 58, 64, 3, 3, 1, 1, 4 | U, 0) == 1
-    assert L.ds_conv2d_tiled_fusable(64, 64, 56, 56, 128, 1, 1, 2, 2, 4, 0) == 0   # short reduction, 64-channel form
+    assert L.ds_conv2d_tiled_fusable(64, 64, 56, 56, 128, 1, 1, 2, 2, 4, 0) == 1   # short reduction, 64-channel form
     # layers the two-instruction kernel serves: fused there when single pixel rows fill the machine
     assert L.ds_conv2d_tiled_fusable(64, 64, 58, 58, 64, 3, 3, 1, 1, 5, 0) == 1
     assert L.ds_conv2d_tiled_fusable(64, 64, 58, 58, 48, 3, 3, 1, 1, 4, 0) == 1
