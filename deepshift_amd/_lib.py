@@ -15,6 +15,8 @@ DS_SMALL_RELU = 0x100
 DS_BITS_ZERO_TOP = 0x100
 DS_BITS_TOP_UNUSED = 0x200
 DS_Q_BORDER_KEPT = 0x100
+DS_CHAIN_CONTROL_BYTES = 12288
+DS_CHAIN_STATUS_AT = 1536
 
 _c_int = ctypes.c_int
 _c_i64 = ctypes.c_int64
@@ -30,6 +32,14 @@ class FusedConv(ctypes.Structure):
 
 
 _fcp = ctypes.POINTER(FusedConv)
+
+
+class ChainLayer(ctypes.Structure):
+    """``ds_chain_layer`` of the header: one layer of a one-launch chain of small linear layers."""
+    _fields_ = [("tiled", _ptr), ("bias", _ptr)] + [(name, _c_int) for name in ("K", "N", "bits", "base", "relu")]
+
+
+_clp = ctypes.POINTER(ChainLayer)
 
 # name -> (restype, argtypes); mirrors include/deepshift_hip.h one to one
 SIGNATURES = {
@@ -60,6 +70,8 @@ SIGNATURES = {
     "ds_linear_tiled_noalloc_max_bytes": (_size, []),
     "ds_linear_tiled_noalloc_i32": (_c_int, [_ptr, _c_int, _ptr, _ptr, _ptr] + [_c_int] * 5 + [_ptr]),
     "ds_linear_small_f32": (_c_int, [_ptr, _ptr, _ptr, _ptr] + [_c_int] * 8 + [_ptr]),
+    "ds_linear_chain_workspace_bytes": (_size, [_c_int, _clp, _c_int]),
+    "ds_linear_chain_f32": (_c_int, [_ptr, _clp, _c_int, _ptr, _c_int, _c_int, _c_int, _c_int, _ptr, _size, _ptr]),
     "ds_conv2d_workspace_bytes": (_size, [_c_int] * 10),
     "ds_conv2d_i32": (_c_int, [_ptr] * 4 + [_c_int] * 11 + [_ptr, _size, _ptr]),
     "ds_conv2d_tiled_workspace_bytes": (_size, [_c_int] * 10),

@@ -50,9 +50,17 @@ struct Tune {
     std::atomic<int> tile{kTuneUnset};    // R * 100 + J of the two-instruction kernel
     std::atomic<int> cu{kTuneUnset};      // 0 / 4: workgroup-cooperative launch off / on (four waves per workgroup)
     std::atomic<int> notail{kTuneUnset};  // int8 kernel: keep the last round of tiles on the tile-per-wave launch
-    void reset() { planes = kTuneUnset; split = kTuneUnset; tile = kTuneUnset; cu = kTuneUnset; notail = kTuneUnset; }
+    std::atomic<int> chain_spin_us{-1};   // layer-chain launch: bound of a barrier wait in microseconds (-1: default)
+    std::atomic<int> chain_extra{-1};     // ... arrivals a barrier waits for beyond the grid (they never come)
+    void reset()
+    {
+        planes = kTuneUnset; split = kTuneUnset; tile = kTuneUnset; cu = kTuneUnset; notail = kTuneUnset;
+        chain_spin_us = -1; chain_extra = -1;
+    }
 };
 extern Tune g_tune;
+// Test hook of the layer-chain launch (ds_small.hip): spin_us < 0 / extra_arrivals < 0 restore the defaults.
+void chain_test_knobs(int spin_us, int extra_arrivals);
 
 // Compute units of the current device (cached per device; 256 on an MI355X).
 int device_cus();

@@ -13,6 +13,7 @@
 // layer keeps one weight format whichever kernel serves it.
 #include "ds_common.h"
 #include "ds_epilogue.h"
+#include "ds_coop.h"
 
 namespace ds {
 
@@ -28,6 +29,7 @@ struct SmallArgs {
     int M, K, N, comm, nbase;
     float out_scale;        // 2^F
     int relu;               // y = max(y, 0)
+    int agent_out;          // y is read by other workgroups of this launch: store it through to memory
     QuantSpec spec;
 };
 
@@ -40,18 +42,17 @@ struct SmallArgs {
 // reduction indices per load instead of one.  The loop then steps through U K groups at a time, the
 // smallest number whose reduction indices are a multiple of four.
 template <int BITS, int MODE, bool VEC, int J>
-__global__ __launch_bounds__(kSmallWaves * 64) void linear_small_kernel(const SmallArgs p)
+__device__ __forceinline__ void small_tile(const SmallArgs &p, const int n0, const int mblock,
+                                           int32_t (&part)[kSmallWaves][J][kWave])
 {
     constexpr int NUM = 32 / (BITS + 1), CB = BITS + 1;
     constexpr uint32_t TOP = (1u << BITS) - 1u;
     constexpr int U = !VEC ? 1 : NUM % 4 == 0 ? 1 : NUM % 2 == 0 ? 2 : 4;  // K groups per step
     constexpr int KS = U * NUM;                                              // reduction indices per step
     static_assert(!VEC || KS % 4 == 0, "whole 16-byte loads per step");
-    __shared__ int32_t part[kSmallWaves][J][kWave];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int n0 = blockIdx.x * J;
-    const int m = blockIdx.y * kWave + lane;
+    const int m = mblock * kWave + lane;
     const bool live = m < p.M;
     const float *xrow = p.x + (size_t)(live ? m : 0) * p.K;
     const int steps = (p.comm + U - 1) / U;
@@ -140,8 +141,18 @@ __global__ __launch_bounds__(kSmallWaves * 64) void linear_small_kernel(const Sm
         // out.float() / 2**F: int32 -> fp32 rounds to nearest even, the division is exact
         float v = (float)sum / p.out_scale;
         if (p.relu) v = v > 0.0f ? v : 0.0f;  // torch.relu: negative values and -0.0 become +0.0
-        p.y[(size_t)m * p.N + n] = v;
+        float *dst = p.y + (size_t)m * p.N + n;
+        if (p.agent_out) __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else *dst = v;
     }
+}
+
+
+template <int BITS, int MODE, bool VEC, int J>
+__global__ __launch_bounds__(kSmallWaves * 64) void linear_small_kernel(const SmallArgs p)
+{
+    __shared__ int32_t part[kSmallWaves][J][kWave];
+    small_tile<BITS, MODE, VEC, J>(p, blockIdx.x * J, blockIdx.y, part);
 }
 
 template <int BITS, bool VEC, int J>
@@ -172,6 +183,142 @@ static void launch_small(const SmallArgs &a, int mode, hipStream_t st)
     const bool vec = a.K >= 4 && a.K % 4 == 0 && ((uintptr_t)a.x & 15u) == 0;
     if (vec) launch_small_vec<BITS, true>(a, mode, st);
     else launch_small_vec<BITS, false>(a, mode, st);
+}
+
+
+// ---------------------------------------------------------------------------------------------
+// A chain of small LinearShift layers (the MNIST MLP, mnist.py:23-39: 784-512-512-10 at batch 64) as ONE
+// launch.  Each layer is a few microseconds of work, and a launch per layer costs more than the layer.
+// One persistent workgroup per compute unit runs the tiles of layer 1 (the code of linear_small_kernel),
+// then every workgroup meets at a barrier in device memory, runs the tiles of layer 2 on the hidden
+// activations (float, in the caller's workspace, as the separate launches would hand them on), and so on.
+//
+// The barrier is a two-level counter in the workspace's control block (which the caller zeroes once).  The
+// workgroups form kChainGroups groups (workgroup w belongs to group w mod kChainGroups); an arrival is one
+// fetch-and-add on the group's counter, the last of a group clears that counter and adds to the top
+// counter, and the last group clears the top counter and bumps every group's release word.  A workgroup
+// then polls its group's release word until it differs from the value read at kernel start.  No word is
+// hit by more than a few dozen read-modify-writes per barrier (a single counter for 256 workgroups,
+// arrivals and polls on one address, cost 650 us per barrier: atomics on one address are served one after
+// the other where all XCDs see them), counters are back at zero when the barrier has passed, and the
+// release words only ever count up: a launch needs no tag and no clearing, and a replay of a captured
+// launch finds what it needs.  Polls are read-modify-writes too (fetch-and-add of 0), which are performed
+// where every XCD sees them.
+// The hidden activations cross XCDs, whose L2 caches are not coherent with each other: they are written
+// with agent-scope stores, which go through to memory, every wave waits for its stores to be acknowledged
+// (s_waitcnt vmcnt(0)) before the workgroup's arrival is counted, and after the barrier one wave of the
+// workgroup invalidates the caches (an agent-scope acquire fence) before anybody loads them; each layer's
+// result has a buffer of its own, so no line of it was read earlier in the launch.
+// All workgroups of the launch must be resident for the barrier to complete: the grid never exceeds the
+// number of compute units, and a workgroup (512 threads, 8 KiB of LDS) fits every one of them, so the
+// hardware places the whole grid as soon as other work leaves room.  The wait is BOUNDED all the same
+// (spin_ticks of the 100 MHz clock): a workgroup that gives up stores the barrier's number in the status
+// word of the workspace and returns, the others follow, every wave exits; the output is then undefined,
+// the status says so, and the control block has to be zeroed again before the workspace is reused.
+constexpr int kChainMax = 4;  // layers per chain
+constexpr int kChainJ = 2;    // output channels per tile: 256 tiles for 512 channels, one per compute unit
+
+struct ChainLayer {
+    const uint32_t *wt;
+    const int32_t *negcnt, *bias;
+    int K, N, comm, relu;
+};
+struct ChainArgs {
+    const float *x;
+    float *y;
+    float *hidden[kChainMax - 1];
+    ChainLayer layer[kChainMax];
+    int nlayers, M, nbase;
+    float out_scale;
+    QuantSpec spec;
+    char *control;               // the control block: kChainBarrierBytes per barrier (see chain_word)
+    int *status;                 // 0, or the number (1 ..) of the barrier that gave up
+    int extra_arrivals;          // test hook: arrivals group 0 waits for beyond its members (they never come)
+    unsigned spin_ticks;         // bound of one wait, in ticks of the 100 MHz clock
+};
+
+// Control block: per barrier the groups' arrival counters (64 bytes apart), the top counter, the groups'
+// release words; the status word sits in an unused part of the first barrier's block.
+constexpr int kChainGroups = 16;
+constexpr int kChainBarrierBytes = 4096;
+constexpr int kChainStatusAt = 1536;
+enum { kChainGroupCounter = 0, kChainTopCounter = 1024, kChainRelease = 2048 };
+__device__ __forceinline__ unsigned *chain_word(char *control, int barrier, int what, int group)
+{
+    return (unsigned *)(control + barrier * kChainBarrierBytes + what + group * 64);
+}
+__device__ __forceinline__ unsigned chain_rmw(unsigned *word, unsigned add)
+{
+    return __hip_atomic_fetch_add(word, add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int BITS, int MODE>
+__global__ __launch_bounds__(kSmallWaves * 64) void linear_chain_kernel(const ChainArgs c)
+{
+    __shared__ int32_t part[kSmallWaves][kChainJ][kWave];
+    __shared__ int32_t proceed;
+    const int G = (int)gridDim.x, w = (int)blockIdx.x;
+    const int mblocks = ceil_div(c.M, kWave);
+    // the release words of this workgroup's group as the launch finds them (they cannot move before every
+    // workgroup, this one included, has arrived at their barrier); only thread 0 uses them
+    unsigned release_before[kChainMax - 1] = {};
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int l = 0; l < kChainMax - 1; ++l)
+            if (l + 1 < c.nlayers) release_before[l] = chain_rmw(chain_word(c.control, l, kChainRelease, w % kChainGroups), 0u);
+    }
+    for (int l = 0; l < c.nlayers; ++l) {
+        const bool last = l == c.nlayers - 1;
+        SmallArgs p;
+        p.x = l == 0 ? c.x : c.hidden[l - 1];
+        p.y = last ? c.y : c.hidden[l];
+        p.agent_out = !last;
+        p.wt = c.layer[l].wt; p.negcnt = c.layer[l].negcnt; p.bias = c.layer[l].bias;
+        p.M = c.M; p.K = c.layer[l].K; p.N = c.layer[l].N; p.comm = c.layer[l].comm; p.nbase = c.nbase;
+        p.out_scale = c.out_scale;
+        p.relu = c.layer[l].relu;
+        p.spec = c.spec;
+        const int ntiles = ceil_div(p.N, kChainJ);
+        for (int item = (int)blockIdx.x; item < ntiles * mblocks; item += G) {
+            const int mb = item / ntiles;
+            small_tile<BITS, MODE, true, kChainJ>(p, (item - mb * ntiles) * kChainJ, mb, part);
+            __syncthreads();  // `part` is reused by the next tile
+        }
+        // every wave's write-through stores are acknowledged before the workgroup's arrival is counted
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (last) return;
+        if (threadIdx.x == 0) {
+            int ok = 1;
+            const int group = w % kChainGroups;
+            const int ngroups = G < kChainGroups ? G : kChainGroups;
+            const int members = (G - group + kChainGroups - 1) / kChainGroups + (group == 0 ? c.extra_arrivals : 0);
+            if ((int)chain_rmw(chain_word(c.control, l, kChainGroupCounter, group), 1u) == members - 1) {
+                // the last of the group: nobody polls the counters, so they can go back to zero at once
+                __hip_atomic_store(chain_word(c.control, l, kChainGroupCounter, group), 0u, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+                if ((int)chain_rmw(chain_word(c.control, l, kChainTopCounter, 0), 1u) == ngroups - 1) {
+                    __hip_atomic_store(chain_word(c.control, l, kChainTopCounter, 0), 0u, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                    for (int g = 0; g < ngroups; ++g) chain_rmw(chain_word(c.control, l, kChainRelease, g), 1u);
+                }
+            }
+            const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();
+            while (chain_rmw(chain_word(c.control, l, kChainRelease, group), 0u) == release_before[l]) {
+                if (__builtin_amdgcn_s_memrealtime() - t0 > (unsigned long long)c.spin_ticks) {
+                    ok = 0;
+                    __hip_atomic_store(c.status, l + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(16);
+            }
+            proceed = ok;
+        }
+        __syncthreads();
+        if (!proceed) return;
+        if (threadIdx.x < kWave) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // one wave: the caches are the workgroup's
+        __syncthreads();
+    }
 }
 
 }  // namespace ds
@@ -205,6 +352,7 @@ DS_EXPORT int ds_linear_small_f32(const float *x, const void *tiled, const int32
     a.M = M; a.K = K; a.N = N; a.comm = g.comm; a.nbase = -base;
     a.out_scale = ldexpf(1.0f, F);
     a.relu = relu;
+    a.agent_out = 0;
     a.spec = make_spec(I, F, mode);
     const int kernel_mode = zero_top ? 2 : (base != 0 || bits == 6) ? 1 : 0;
     hipStream_t st = (hipStream_t)stream;
@@ -215,6 +363,117 @@ DS_EXPORT int ds_linear_small_f32(const float *x, const void *tiled, const int32
     case 4: launch_small<4>(a, kernel_mode, st); break;
     case 5: launch_small<5>(a, kernel_mode, st); break;
     default: launch_small<6>(a, kernel_mode, st); break;
+    }
+    return launch_status();
+}
+
+// ---- a chain of small layers in one launch --------------------------------------------------------
+
+static constexpr size_t kChainControlBytes = (size_t)(kChainMax - 1) * kChainBarrierBytes;
+static_assert(kChainControlBytes == DS_CHAIN_CONTROL_BYTES && kChainStatusAt == DS_CHAIN_STATUS_AT, "the header's layout");
+static std::atomic<unsigned> g_chain_spin_ticks{200000000u};  // 2 s of the 100 MHz clock
+static std::atomic<int> g_chain_extra_arrivals{0};            // test hook: arrivals that never come
+
+namespace ds {
+void chain_test_knobs(int spin_us, int extra_arrivals)
+{
+    g_chain_spin_ticks = spin_us < 0 ? 200000000u : (unsigned)spin_us * 100u;
+    g_chain_extra_arrivals = extra_arrivals < 0 ? 0 : extra_arrivals;
+}
+}  // namespace ds
+
+static int chain_check(const ds_chain_layer *layers, int nlayers, int M, int *width, int *kernel_mode)
+{
+    if (!layers || nlayers < 2 || nlayers > kChainMax || M < 0) return DS_EINVAL;
+    int bits0 = 0, base0 = 0, zt0 = 0;
+    for (int l = 0; l < nlayers; ++l) {
+        const ds_chain_layer &L = layers[l];
+        const int zero_top = (L.bits & DS_BITS_ZERO_TOP) != 0;
+        const int bits = L.bits & ~(DS_BITS_ZERO_TOP | DS_BITS_TOP_UNUSED);
+        if (bits < 1 || bits > 6) return DS_EBITS;
+        if (L.base > 0 || L.base < -31) return DS_EBASE;
+        if (zero_top && (bits > 4 || L.base != 0)) return DS_EBITS;
+        if (L.K < 4 || L.N < 1 || L.K % 4 != 0) return DS_EINVAL;     // rows are read sixteen bytes at a time
+        if (l > 0 && L.K != layers[l - 1].N) return DS_EINVAL;
+        if (l == 0) { bits0 = bits; base0 = L.base; zt0 = zero_top; }
+        else if (bits != bits0 || L.base != base0 || zero_top != zt0) return DS_EINVAL;  // one kernel form
+        if ((size_t)M * L.K * 4 >= ((size_t)1 << 31) || (size_t)M * L.N * 4 >= ((size_t)1 << 31)) return DS_ETOOLARGE;
+    }
+    if (ceil_div(M, kWave) > 65535) return DS_ETOOLARGE;
+    *width = bits0;
+    *kernel_mode = zt0 ? 2 : (base0 != 0 || bits0 == 6) ? 1 : 0;
+    return DS_OK;
+}
+
+static size_t chain_hidden_bytes(const ds_chain_layer *layers, int nlayers, int M)
+{
+    int widest = 0;
+    for (int l = 0; l + 1 < nlayers; ++l) widest = layers[l].N > widest ? layers[l].N : widest;
+    return align_up((size_t)M * widest * 4, 256);
+}
+
+DS_EXPORT size_t ds_linear_chain_workspace_bytes(int M, const ds_chain_layer *layers, int nlayers)
+{
+    int width, mode;
+    if (chain_check(layers, nlayers, M, &width, &mode)) return 0;
+    return kChainControlBytes + (size_t)(nlayers - 1) * chain_hidden_bytes(layers, nlayers, M);
+}
+
+template <int BITS>
+static void launch_chain(const ChainArgs &a, int mode, int blocks, hipStream_t st)
+{
+    const dim3 grid(blocks), block(kSmallWaves * 64);
+    if (mode == 2) hipLaunchKernelGGL((linear_chain_kernel<BITS, 2>), grid, block, 0, st, a);
+    else if (mode == 1) hipLaunchKernelGGL((linear_chain_kernel<BITS, 1>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((linear_chain_kernel<BITS, 0>), grid, block, 0, st, a);
+}
+
+DS_EXPORT int ds_linear_chain_f32(const float *x, const ds_chain_layer *layers, int nlayers, float *y, int M, int mode,
+                                  int I, int F, void *workspace, size_t workspace_bytes, ds_stream_t stream)
+{
+    int width = 0, kernel_mode = 0;
+    int rc = chain_check(layers, nlayers, M, &width, &kernel_mode);
+    if (rc) return rc;
+    if (F < 0 || F > 31 || I < 1 || I + F > 32) return DS_EINVAL;
+    if (mode != DS_Q_ROUND_TO_FIXED && mode != DS_Q_CAST) return DS_EINVAL;
+    if (M == 0) return DS_OK;
+    if (!x || !y || ((uintptr_t)x & 15u)) return DS_EINVAL;
+    const size_t hidden = chain_hidden_bytes(layers, nlayers, M);
+    if (!workspace || workspace_bytes < kChainControlBytes + (size_t)(nlayers - 1) * hidden || ((uintptr_t)workspace & 255))
+        return DS_EWORKSPACE;
+    ChainArgs a{};
+    a.x = x;
+    a.y = y;
+    for (int l = 0; l + 1 < nlayers; ++l) a.hidden[l] = (float *)((char *)workspace + kChainControlBytes + l * hidden);
+    int most_tiles = 1;
+    for (int l = 0; l < nlayers; ++l) {
+        if (!layers[l].tiled) return DS_EINVAL;
+        const TiledGeom g = tiled_geom(layers[l].N, layers[l].K, width);
+        a.layer[l].wt = (const uint32_t *)layers[l].tiled;
+        a.layer[l].negcnt = tiled_negcount(layers[l].tiled, g);
+        a.layer[l].bias = layers[l].bias;
+        a.layer[l].K = layers[l].K; a.layer[l].N = layers[l].N; a.layer[l].comm = g.comm;
+        a.layer[l].relu = layers[l].relu != 0;
+        const int tiles = ceil_div(layers[l].N, kChainJ) * ceil_div(M, kWave);
+        most_tiles = tiles > most_tiles ? tiles : most_tiles;
+    }
+    a.nlayers = nlayers; a.M = M; a.nbase = -layers[0].base;
+    a.out_scale = ldexpf(1.0f, F);
+    a.spec = make_spec(I, F, mode);
+    a.control = (char *)workspace;
+    a.status = (int *)((char *)workspace + kChainStatusAt);
+    // never more workgroups than compute units: all of them must be resident for the barriers
+    const int blocks = most_tiles < device_cus() ? most_tiles : device_cus();
+    a.extra_arrivals = g_chain_extra_arrivals;
+    a.spin_ticks = g_chain_spin_ticks;
+    hipStream_t st = (hipStream_t)stream;
+    switch (width) {
+    case 1: launch_chain<1>(a, kernel_mode, blocks, st); break;
+    case 2: launch_chain<2>(a, kernel_mode, blocks, st); break;
+    case 3: launch_chain<3>(a, kernel_mode, blocks, st); break;
+    case 4: launch_chain<4>(a, kernel_mode, blocks, st); break;
+    case 5: launch_chain<5>(a, kernel_mode, blocks, st); break;
+    default: launch_chain<6>(a, kernel_mode, blocks, st); break;
     }
     return launch_status();
 }

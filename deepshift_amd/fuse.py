@@ -24,7 +24,7 @@ import torch.nn.functional as F
 
 from . import kernels, modules, modules_q
 
-__all__ = ["FusedConv2dShift", "FusedLinearShift", "fuse_conv_epilogues"]
+__all__ = ["FusedConv2dShift", "FusedLinearShift", "FusedLinearChain", "fuse_conv_epilogues"]
 
 _SHIFT_CONVS = (modules.Conv2dShift, modules_q.Conv2dShiftQ)
 _SHIFT_LINEARS = (modules.LinearShift, modules_q.LinearShiftQ)
@@ -43,6 +43,69 @@ class FusedLinearShift(nn.Module):
         if not self.linear.use_kernel:
             return torch.relu(self.linear(input))
         return self.linear._kernel_forward(input, relu=True)
+
+
+class FusedLinearChain(nn.Module):
+    """Kernel-mode LinearShift / LinearShiftQ layers that feed each other directly, each optionally followed by
+    a ReLU -- the shape of the MNIST MLP, mnist.py:23-39 -- as ONE launch (``kernels.linear_chain``) where
+    that is the faster way: narrow layers, whose persistent grid is small enough for its barriers to cost
+    less than the launches they save (``kernels.linear_chain_pays``).  Bit-identical to the layers run one
+    by one, which is what happens everywhere else: wide layers (the 512-wide MNIST MLP at batch 64 takes
+    50 us as one launch, 39 us as three), layers of different field widths or activation formats, a layer
+    too large for the one-launch kernel, host execution."""
+
+    def __init__(self, linears, relus):
+        super().__init__()
+        self.linears = nn.ModuleList(linears)
+        self.relus = [bool(r) for r in relus]
+        self.force = False   # True: one launch whatever the size (tests, measurements)
+
+    def _one_by_one(self, input):
+        x = input
+        for linear, relu in zip(self.linears, self.relus):
+            if linear.use_kernel:
+                x = linear._kernel_forward(x, relu=relu)
+            else:
+                x = torch.relu(linear(x)) if relu else linear(x)
+        return x
+
+    def forward(self, input):
+        first = self.linears[0]
+        kind = type(first)
+        I, Fb = first.act_integer_bits, first.act_fraction_bits
+        if not all(type(m) is kind and m.use_kernel and m.use_cuda and
+                   (m.act_integer_bits, m.act_fraction_bits) == (I, Fb) for m in self.linears):
+            return self._one_by_one(input)
+        lead = input.shape[:-1]
+        x2d = input.reshape(-1, first.in_features).float()
+        M = x2d.shape[0]
+        if not x2d.is_cuda or not all(kernels.small_linear_serves(M, m.in_features, m.out_features)
+                                      for m in self.linears):
+            return self._one_by_one(input)
+        if not self.force and not kernels.linear_chain_pays(M, [(m.in_features, m.out_features) for m in self.linears]):
+            return self._one_by_one(input)   # wide layers: the barriers cost more than the launches they save
+        round_to_fixed = isinstance(first, modules_q.LinearShiftQ)   # modules_q.py:115-125 / modules.py:24-31
+        layers = []
+        for m, relu in zip(self.linears, self.relus):
+            cw = m.packed_weights()
+            bias = m._fixed_bias.get(m.bias, I, Fb, round_to_fixed=round_to_fixed)
+            layers.append((kernels._tiled_of(cw, m.out_features, m.in_features), bias, m.in_features,
+                           m.out_features, kernels.kernel_bits(cw), cw.base, relu))
+        cache = self.__dict__.setdefault("_chain_workspace", {})
+        out = kernels.linear_chain(x2d, layers, I, Fb, round_to_fixed, cache)
+        if out is None:
+            return self._one_by_one(input)
+        return out.reshape(*lead, self.linears[-1].out_features)
+
+    def status(self):
+        """0, or the number of the barrier at which a launch gave up waiting for the grid to be resident (its
+        result was undefined); synchronises with the device."""
+        return kernels.linear_chain_status(self.__dict__.get("_chain_workspace", {}))
+
+    def __getstate__(self):
+        state = self.__dict__.copy()
+        state.pop("_chain_workspace", None)
+        return state
 
 
 class FusedConv2dShift(nn.Module):
@@ -274,9 +337,52 @@ def fuse_conv_epilogues(model, handoff=True):
     if handoff:
         _hand_off_fixed_point(gm)
         _pair_shortcuts(gm)
+    _chain_linears(gm)
     gm.graph.lint()
     gm.recompile()
     return gm
+
+
+def _chain_linears(gm):
+    """Kernel-mode linear layers (with or without their fused ReLU) that feed each other directly become one
+    :class:`FusedLinearChain` (two to four layers per chain)."""
+    mods = dict(gm.named_modules())
+
+    def linear_of(n):
+        """(LinearShift module, relu) if node ``n`` is a kernel-mode linear layer call, else None."""
+        m = mods.get(n.target) if n.op == "call_module" else None
+        if isinstance(m, FusedLinearShift) and m.linear.use_kernel:
+            return m.linear, True
+        if isinstance(m, _SHIFT_LINEARS) and m.use_kernel:
+            return m, False
+        return None
+
+    count = 0
+    taken = set()
+    for node in list(gm.graph.nodes):
+        if node in taken or linear_of(node) is None or len(node.args) != 1 or node.kwargs:
+            continue
+        chain = [node]
+        while len(chain) < 4:
+            nxt = _sole_user(chain[-1])
+            if nxt is None or linear_of(nxt) is None or tuple(nxt.args) != (chain[-1],) or nxt.kwargs:
+                break
+            if linear_of(nxt)[0].in_features != linear_of(chain[-1])[0].out_features:
+                break
+            chain.append(nxt)
+        if len(chain) < 2:
+            continue
+        taken.update(chain)
+        pairs = [linear_of(n) for n in chain]
+        name = "chain_%d" % count
+        count += 1
+        gm.add_module(name, FusedLinearChain([m for m, _ in pairs], [r for _, r in pairs]))
+        with gm.graph.inserting_after(chain[-1]):
+            new = gm.graph.call_module(name, (chain[0].args[0],))
+        chain[-1].replace_all_uses_with(new)
+        for old in reversed(chain):
+            gm.graph.erase_node(old)
+    return count
 
 
 def _input_key(conv):
