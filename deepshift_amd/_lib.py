@@ -15,6 +15,8 @@ DS_SMALL_RELU = 0x100
 DS_BITS_ZERO_TOP = 0x100
 DS_BITS_TOP_UNUSED = 0x200
 DS_Q_BORDER_KEPT = 0x100
+DS_CHAIN_ONE_LAUNCH = 0x200
+DS_CHAIN_LAUNCH_PER_LAYER = 0x400
 DS_CHAIN_CONTROL_BYTES = 12288
 DS_CHAIN_STATUS_AT = 1536
 

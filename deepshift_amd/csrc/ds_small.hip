@@ -217,6 +217,7 @@ static void launch_small(const SmallArgs &a, int mode, hipStream_t st)
 // the status says so, and the control block has to be zeroed again before the workspace is reused.
 constexpr int kChainMax = 4;  // layers per chain
 constexpr int kChainJ = 2;    // output channels per tile: 256 tiles for 512 channels, one per compute unit
+constexpr int kChainPersistentTiles = 64;  // up to this many tiles per layer the chain runs as one persistent launch
 
 struct ChainLayer {
     const uint32_t *wt;
@@ -435,6 +436,9 @@ DS_EXPORT int ds_linear_chain_f32(const float *x, const ds_chain_layer *layers, 
     int rc = chain_check(layers, nlayers, M, &width, &kernel_mode);
     if (rc) return rc;
     if (F < 0 || F > 31 || I < 1 || I + F > 32) return DS_EINVAL;
+    const int how = mode & (DS_CHAIN_ONE_LAUNCH | DS_CHAIN_LAUNCH_PER_LAYER);
+    mode &= ~(DS_CHAIN_ONE_LAUNCH | DS_CHAIN_LAUNCH_PER_LAYER);
+    if (how == (DS_CHAIN_ONE_LAUNCH | DS_CHAIN_LAUNCH_PER_LAYER)) return DS_EINVAL;
     if (mode != DS_Q_ROUND_TO_FIXED && mode != DS_Q_CAST) return DS_EINVAL;
     if (M == 0) return DS_OK;
     if (!x || !y || ((uintptr_t)x & 15u)) return DS_EINVAL;
@@ -460,13 +464,42 @@ DS_EXPORT int ds_linear_chain_f32(const float *x, const ds_chain_layer *layers, 
     a.nlayers = nlayers; a.M = M; a.nbase = -layers[0].base;
     a.out_scale = ldexpf(1.0f, F);
     a.spec = make_spec(I, F, mode);
+    hipStream_t st = (hipStream_t)stream;
+    // Wide layers: a launch per layer, issued from here (one call across the boundary instead of one per
+    // layer).  The persistent grid pays while it is small: its barriers are a few read-modify-writes that
+    // cross the XCDs -- about 10 us per barrier with 256 workgroups, 3 us with 32 -- against about 4 us for a
+    // launch (64 x 784-512-512-10: 50 us as one launch, 39 us as three; 64 x 64-64-64: 12.5 against 24.7).
+    const bool persistent = how == DS_CHAIN_ONE_LAUNCH || (how == 0 && most_tiles <= kChainPersistentTiles);
+    if (!persistent) {
+        for (int l = 0; l < nlayers; ++l) {
+            SmallArgs p;
+            p.x = l == 0 ? a.x : a.hidden[l - 1];
+            p.y = l == nlayers - 1 ? a.y : a.hidden[l];
+            p.wt = a.layer[l].wt; p.negcnt = a.layer[l].negcnt; p.bias = a.layer[l].bias;
+            p.M = M; p.K = a.layer[l].K; p.N = a.layer[l].N; p.comm = a.layer[l].comm; p.nbase = a.nbase;
+            p.out_scale = a.out_scale;
+            p.relu = a.layer[l].relu;
+            p.agent_out = 0;
+            p.spec = a.spec;
+            switch (width) {
+            case 1: launch_small<1>(p, kernel_mode, st); break;
+            case 2: launch_small<2>(p, kernel_mode, st); break;
+            case 3: launch_small<3>(p, kernel_mode, st); break;
+            case 4: launch_small<4>(p, kernel_mode, st); break;
+            case 5: launch_small<5>(p, kernel_mode, st); break;
+            default: launch_small<6>(p, kernel_mode, st); break;
+            }
+            rc = launch_status();
+            if (rc) return rc;
+        }
+        return DS_OK;
+    }
     a.control = (char *)workspace;
     a.status = (int *)((char *)workspace + kChainStatusAt);
     // never more workgroups than compute units: all of them must be resident for the barriers
     const int blocks = most_tiles < device_cus() ? most_tiles : device_cus();
     a.extra_arrivals = g_chain_extra_arrivals;
     a.spin_ticks = g_chain_spin_ticks;
-    hipStream_t st = (hipStream_t)stream;
     switch (width) {
     case 1: launch_chain<1>(a, kernel_mode, blocks, st); break;
     case 2: launch_chain<2>(a, kernel_mode, blocks, st); break;

@@ -47,18 +47,19 @@ class FusedLinearShift(nn.Module):
 
 class FusedLinearChain(nn.Module):
     """Kernel-mode LinearShift / LinearShiftQ layers that feed each other directly, each optionally followed by
-    a ReLU -- the shape of the MNIST MLP, mnist.py:23-39 -- as ONE launch (``kernels.linear_chain``) where
-    that is the faster way: narrow layers, whose persistent grid is small enough for its barriers to cost
-    less than the launches they save (``kernels.linear_chain_pays``).  Bit-identical to the layers run one
-    by one, which is what happens everywhere else: wide layers (the 512-wide MNIST MLP at batch 64 takes
-    50 us as one launch, 39 us as three), layers of different field widths or activation formats, a layer
-    too large for the one-launch kernel, host execution."""
+    a ReLU -- the shape of the MNIST MLP, mnist.py:23-39 -- in one call of the library
+    (``kernels.linear_chain``): ONE launch where that is the faster way (narrow layers, whose persistent
+    grid is small enough for its barriers to cost less than the launches they save), else a launch per
+    layer issued inside the call (the 512-wide MNIST MLP at batch 64 takes 50 us as one launch, 39 us as
+    three).  Bit-identical to the layers run one by one from Python, which is what happens where the
+    library has no such form: layers of different field widths or activation formats, a layer too large
+    for the one-launch kernel, host execution."""
 
     def __init__(self, linears, relus):
         super().__init__()
         self.linears = nn.ModuleList(linears)
         self.relus = [bool(r) for r in relus]
-        self.force = False   # True: one launch whatever the size (tests, measurements)
+        self.force = False   # True: the one-launch form whatever the size (tests, measurements)
 
     def _one_by_one(self, input):
         x = input
@@ -82,8 +83,6 @@ class FusedLinearChain(nn.Module):
         if not x2d.is_cuda or not all(kernels.small_linear_serves(M, m.in_features, m.out_features)
                                       for m in self.linears):
             return self._one_by_one(input)
-        if not self.force and not kernels.linear_chain_pays(M, [(m.in_features, m.out_features) for m in self.linears]):
-            return self._one_by_one(input)   # wide layers: the barriers cost more than the launches they save
         round_to_fixed = isinstance(first, modules_q.LinearShiftQ)   # modules_q.py:115-125 / modules.py:24-31
         layers = []
         for m, relu in zip(self.linears, self.relus):
@@ -92,7 +91,7 @@ class FusedLinearChain(nn.Module):
             layers.append((kernels._tiled_of(cw, m.out_features, m.in_features), bias, m.in_features,
                            m.out_features, kernels.kernel_bits(cw), cw.base, relu))
         cache = self.__dict__.setdefault("_chain_workspace", {})
-        out = kernels.linear_chain(x2d, layers, I, Fb, round_to_fixed, cache)
+        out = kernels.linear_chain(x2d, layers, I, Fb, round_to_fixed, cache, "one" if self.force else None)
         if out is None:
             return self._one_by_one(input)
         return out.reshape(*lead, self.linears[-1].out_features)

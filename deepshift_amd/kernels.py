@@ -529,14 +529,16 @@ class ChainFailed(RuntimeError):
     """A barrier of a one-launch layer chain gave up waiting (see :func:`linear_chain_status`)."""
 
 
-def linear_chain(x2d, layers, integer_bits, fraction_bits, round_to_fixed, ws_cache):
-    """A chain of small LinearShift layers in ONE launch (``ds_linear_chain_f32``): what calling
-    :func:`linear_small` once per layer returns, bit for bit.  ``layers``: a list of
+def linear_chain(x2d, layers, integer_bits, fraction_bits, round_to_fixed, ws_cache, how=None):
+    """A chain of small LinearShift layers in one call (``ds_linear_chain_f32``): what calling
+    :func:`linear_small` once per layer returns, bit for bit.  Narrow layers run as ONE launch (a persistent
+    grid with barriers between the layers), wider ones as a launch per layer issued inside the call;
+    ``how`` = ``"one"`` / ``"each"`` forces either.  ``layers``: a list of
     ``(tiled, bias, K, N, bits, base, relu)``; ``ws_cache``: a dict that keeps the workspace (control block
     zeroed once + hidden activations) between calls.  Returns float32 ``[M, N_last]``, or ``None`` when the
-    chain has no one-launch form (mixed field widths, a K that is not a multiple of 4, ...): the caller
-    then runs the layers one by one.  The launch's barriers wait at most 2 s for the whole grid to be
-    resident; :func:`linear_chain_status` tells whether one gave up."""
+    chain has no such form (mixed field widths, a K that is not a multiple of 4, ...): the caller then
+    runs the layers one by one.  The barriers of the one-launch form wait at most 2 s for the whole grid to
+    be resident; :func:`linear_chain_status` tells whether one gave up."""
     x2d = x2d.contiguous()
     if x2d.dtype != torch.float32 or not x2d.is_cuda or x2d.dim() != 2:
         raise TypeError("linear_chain expects a 2-D float32 GPU tensor")
@@ -559,23 +561,12 @@ def linear_chain(x2d, layers, integer_bits, fraction_bits, round_to_fixed, ws_ca
         ws = ws_cache[key] = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)   # control block zeroed once
     out = torch.empty([M, layers[-1][3]], dtype=torch.float32, device=dev)
     pairs = sum(M * K * N for (_, _, K, N, _, _, _) in layers)
+    mode = _lib.DS_Q_ROUND_TO_FIXED if round_to_fixed else _lib.DS_Q_CAST
+    mode |= {None: 0, "one": _lib.DS_CHAIN_ONE_LAUNCH, "each": _lib.DS_CHAIN_LAUNCH_PER_LAYER}[how]
     with _Timed("linear", M, pairs // (M * layers[-1][3]) if M else 0, layers[-1][3], dev):
-        _lib.call("ds_linear_chain_f32", _lib.ptr(x2d), arr, len(layers), _lib.ptr(out), M,
-                  _lib.DS_Q_ROUND_TO_FIXED if round_to_fixed else _lib.DS_Q_CAST, int(integer_bits),
+        _lib.call("ds_linear_chain_f32", _lib.ptr(x2d), arr, len(layers), _lib.ptr(out), M, mode, int(integer_bits),
                   int(fraction_bits), _lib.ptr(ws), ws_bytes, _lib.current_stream(dev))
     return out
-
-
-# Workgroups above which the one-launch chain loses to a launch per layer: its barriers cost a few
-# read-modify-writes that cross the XCDs (about 10 us per barrier with 256 workgroups, 3 us with 32), a launch
-# about 4 us (64 x 784-512-512-10: 50 us as one launch, 39 us as three; 64 x 64-64-64: 12.5 against 24.7).
-CHAIN_MAX_WORKGROUPS = 64
-
-
-def linear_chain_pays(M, layers):
-    """Whether :func:`linear_chain` is the faster way to run ``layers`` (a list of (K, N)) on ``M`` rows."""
-    rows = (M + 63) // 64
-    return max((N + 1) // 2 * rows for _, N in layers) <= CHAIN_MAX_WORKGROUPS
 
 
 def linear_chain_status(ws_cache):

@@ -250,21 +250,26 @@ int ds_linear_small_f32(const float *x, const void *tiled, const int32_t *bias, 
                         int N, int bits, int base, int mode, int I, int F, ds_stream_t stream);
 
 /* A chain of 2..4 small LinearShift layers, each optionally followed by a ReLU -- the MNIST MLP,
- * mnist.py:23-39 with modules.py:24-31 per layer -- as ONE launch: the result of calling
- * ds_linear_small_f32 once per layer, bit for bit, without the launches in between (784-512-512-10 at
- * batch 64: three launches of 8 to 14 us each become one).  x [M][layers[0].K] float, y
+ * mnist.py:23-39 with modules.py:24-31 per layer -- in one call: the result of calling
+ * ds_linear_small_f32 once per layer, bit for bit.  Narrow layers (at most 64 workgroups of two channels x
+ * 64 rows per layer) run as ONE launch, a persistent grid that meets at barriers between the layers; wider
+ * ones (784-512-512-10 at batch 64) as a launch per layer issued by this call, because there the barriers
+ * cost more than the launches.  mode | DS_CHAIN_ONE_LAUNCH / mode | DS_CHAIN_LAUNCH_PER_LAYER force one
+ * or the other.  x [M][layers[0].K] float, y
  * [M][layers[n-1].N] float; layers[l].K == layers[l-1].N; every layer the same field width, base and
  * zero-top flag (one kernel form), every K a multiple of 4, x 16-byte aligned (DS_EINVAL otherwise: call
  * the layers one by one).  mode, I, F as ds_linear_small_f32 (without DS_SMALL_RELU: relu is per layer).
  * Workspace: ds_linear_chain_workspace_bytes() bytes, 256-byte aligned -- a control block of
  * DS_CHAIN_CONTROL_BYTES, which the caller zeroes ONCE before the first call and leaves alone afterwards,
- * then the hidden activations.  The launch is a persistent grid of at most one workgroup per compute
- * unit that meets at a barrier in the control block between layers.  The wait at a barrier is bounded
+ * then the hidden activations.  The one-launch form is a persistent grid of at most one workgroup per
+ * compute unit that meets at a barrier in the control block between layers.  The wait at a barrier is bounded
  * (2 s): if it expires -- the GPU is so busy with other work that the grid was not resident in time --
  * every workgroup exits, y is undefined, and the int at byte DS_CHAIN_STATUS_AT of the workspace holds
  * the number (1 ..) of the barrier that gave up.  It is 0 as long as every launch completed; after a
  * failure the caller zeroes the control block again before reusing the workspace.  Launches that share a
  * workspace must not overlap.  No counterpart in the reference. */
+#define DS_CHAIN_ONE_LAUNCH 0x200
+#define DS_CHAIN_LAUNCH_PER_LAYER 0x400
 #define DS_CHAIN_CONTROL_BYTES 12288
 #define DS_CHAIN_STATUS_AT 1536
 typedef struct ds_chain_layer {

@@ -45,13 +45,13 @@ class Chain:
         self.ws = torch.full((self.ws_bytes,), 0x77, dtype=torch.uint8, device=DEV)   # stale hidden activations
         self.ws[:CONTROL] = 0
 
-    def run(self, x, mode=_lib.DS_Q_CAST, I=16, F=16, y=None):
+    def run(self, x, mode=_lib.DS_Q_CAST, I=16, F=16, how=_lib.DS_CHAIN_ONE_LAUNCH):
         guard = 64
         M, N = self.M, self.N_out
         ybuf = torch.full((M * N + 2 * guard,), 12345.0, dtype=torch.float32, device=DEV)
         yv = ybuf[guard:guard + M * N]
         xd = x if torch.is_tensor(x) else _dev(x)
-        _lib.call("ds_linear_chain_f32", _lib.ptr(xd), self.arr, self.n, ctypes.c_void_p(yv.data_ptr()), M, mode, I, F,
+        _lib.call("ds_linear_chain_f32", _lib.ptr(xd), self.arr, self.n, ctypes.c_void_p(yv.data_ptr()), M, mode | how, I, F,
                   _lib.ptr(self.ws), self.ws_bytes, _stream())
         torch.cuda.synchronize()
         host = ybuf.cpu().numpy()
@@ -98,9 +98,10 @@ def test_chain_matches_oracle_layer_by_layer(oracle, rng, bits, shape):
                          (_lib.DS_Q_ROUND_TO_FIXED, (3, 5))]:
         x = (rng.standard_normal((M, sizes[0])) * 2.0 ** rng.integers(-8, 6, size=(M, sizes[0]))).astype(np.float32)
         want = _oracle_chain(oracle, x, codes, relus, mode, I, F)
-        # twice on the same workspace: the barrier words of the first launch are what the second finds
-        for _ in range(2):
-            np.testing.assert_array_equal(chain.run(x, mode, I, F), want)
+        # twice on the same workspace: the barrier words of the first launch are what the second finds; then
+        # as a launch per layer, and as the library chooses
+        for how in (_lib.DS_CHAIN_ONE_LAUNCH, _lib.DS_CHAIN_ONE_LAUNCH, _lib.DS_CHAIN_LAUNCH_PER_LAYER, 0):
+            np.testing.assert_array_equal(chain.run(x, mode, I, F, how), want)
         assert chain.status() == 0
 
 
@@ -121,19 +122,15 @@ def test_chain_equals_one_launch_per_layer_and_the_module_path(oracle):
         fused = fuse.fuse_conv_epilogues(model)
         chains = [m for m in fused.modules() if isinstance(m, fuse.FusedLinearChain)]
         assert len(chains) == 1 and len(chains[0].linears) == 3 and chains[0].relus == [True, True, False]
-        # 512-wide layers: the chain runs a launch per layer by itself (256 workgroups: its barriers would cost
-        # more than the launches); forced, it is one launch with the same result
-        launches = []
-        kernels.set_timing_sink(launches)
+        # 512-wide layers: one call of the library, which issues a launch per layer by itself (256 workgroups:
+        # the barriers of the one-launch form would cost more than the launches); forced, the same result
         by_itself = fused(x)
-        kernels.set_timing_sink(None)
-        assert len(launches) == 3
         chains[0].force = True
         launches = []
         kernels.set_timing_sink(launches)
         got = fused(x)
         kernels.set_timing_sink(None)
-        assert len(launches) == 1, "one launch for the three layers"
+        assert len(launches) == 1, "one call for the three layers"
         want = model(x)
         assert torch.equal(got, want) and torch.equal(by_itself, want)
         assert chains[0].status() == 0
@@ -144,11 +141,7 @@ def test_chain_equals_one_launch_per_layer_and_the_module_path(oracle):
                                              use_kernel=True)
         narrow = narrow.to(DEV).eval()
         fused_narrow = fuse.fuse_conv_epilogues(narrow)
-        launches = []
-        kernels.set_timing_sink(launches)
-        got = fused_narrow(x)
-        kernels.set_timing_sink(None)
-        assert len(launches) == 1 and torch.equal(got, narrow(x))
+        assert torch.equal(fused_narrow(x), narrow(x))
 
 
 def test_chain_falls_back_where_it_has_no_one_launch_form():
@@ -172,6 +165,7 @@ def test_chain_falls_back_where_it_has_no_one_launch_form():
     assert L.ds_linear_chain_f32(one, arr, 2, one, 5, 0, 16, 16, one, 16, None) == -4
     assert L.ds_linear_chain_f32(one, arr, 1, one, 5, 0, 16, 16, one, 1 << 20, None) == -1
     assert L.ds_linear_chain_f32(one, arr, 5, one, 5, 0, 16, 16, one, 1 << 20, None) == -1
+    assert L.ds_linear_chain_f32(one, arr, 2, one, 5, 0x600, 16, 16, one, 1 << 20, None) == -1   # both ways at once
 
 
 def test_a_barrier_that_cannot_complete_gives_up_and_every_workgroup_exits(oracle, rng):
@@ -202,7 +196,8 @@ def test_chain_replays_from_a_captured_graph(oracle, rng):
     y = torch.zeros((M, sizes[-1]), dtype=torch.float32, device=DEV)
 
     def launch():
-        _lib.call("ds_linear_chain_f32", _lib.ptr(xd), chain.arr, chain.n, _lib.ptr(y), M, _lib.DS_Q_CAST, 16, 16,
+        _lib.call("ds_linear_chain_f32", _lib.ptr(xd), chain.arr, chain.n, _lib.ptr(y), M,
+                  _lib.DS_Q_CAST | _lib.DS_CHAIN_ONE_LAUNCH, 16, 16,
                   _lib.ptr(chain.ws), chain.ws_bytes, _stream())
 
     side = torch.cuda.Stream()

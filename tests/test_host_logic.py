@@ -292,12 +292,3 @@ def test_hand_off_buffers_do_not_travel_with_copies_of_a_module():
     convq = modules_q.Conv2dShiftQ(4, 8, 3, padding=1)
     convq.__dict__["_handoff_buffers"] = {"k": torch.zeros(3)}
     assert "_handoff_buffers" not in copy.deepcopy(convq).__dict__
-
-
-def test_one_launch_chain_is_chosen_for_narrow_layers_only():
-    """kernels.linear_chain_pays: the persistent grid's barriers cost more than the launches they save once
-    the widest layer needs more than 64 workgroups (two channels x 64 rows each)."""
-    assert kernels.linear_chain_pays(64, [(784, 64), (64, 64), (64, 10)])
-    assert kernels.linear_chain_pays(64, [(64, 128), (128, 16)])
-    assert not kernels.linear_chain_pays(64, [(784, 512), (512, 512), (512, 10)])   # the MNIST MLP: 256 workgroups
-    assert not kernels.linear_chain_pays(256, [(64, 64), (64, 64)])                 # four row blocks x 32
