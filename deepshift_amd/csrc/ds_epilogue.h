@@ -18,15 +18,15 @@ struct QuantSpec {
     int mode, I;
 };
 
-// float -> int32 toward zero, saturating, NaN -> 0 (what v_cvt_i32_f32 returns; spelled out because
-// an out-of-range C++ conversion is undefined).
+// float -> int32 toward zero, saturating, NaN -> 0: v_cvt_i32_f32 itself (out-of-range values and
+// infinities saturate, NaN converts to 0), asked for by name because an out-of-range C++ conversion is
+// undefined and spelling the clamps out costs five more instructions per value -- which is most of the
+// vector work of a small fully connected layer, whose every workgroup converts its rows' activations.
 __device__ __forceinline__ int32_t f2i_sat(float v)
 {
-    // selects, not branches: callers convert many independent values between a load and its use
-    const float c = __builtin_fminf(__builtin_fmaxf(v, -2147483648.0f), 2147483520.0f);  // in range; NaN -> a bound
-    int32_t r = (int32_t)c;
-    r = v >= 2147483648.0f ? 2147483647 : r;
-    return v != v ? 0 : r;
+    int32_t r;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(r) : "v"(v));
+    return r;
 }
 
 __device__ __forceinline__ int32_t quantize_one(float v, const QuantSpec &q)
