@@ -517,8 +517,9 @@ def pmc_target(device):
         tiles one per wave (K = 147 leaves a partial last group: the zero-top form runs its padding codes);
       * a down-sampling block's first 3x3 stride-2 convolution with its 1x1 shortcut as one launch
         (<4, 2, true, true>), 64 -> 128 channels at 56x56;
-      * the int8 kernel (shift_pairs_cu_kernel) on a ResNet-50 3x3 layer, 128 -> 128 at 28x28, batch 128,
-        weight_bits 3;
+      * the int8 kernel's fused launch (shift_pairs_fused_kernel<2, true, false>: eight-wave workgroups,
+        BatchNorm affine, ReLU and the next 1x1 layer's int8 input from the epilogue) on a ResNet-50 3x3 layer,
+        128 -> 128 at 28x28, batch 128, weight_bits 3;
       * the cooperative two-instruction kernel (shift_coop_kernel) on ResNet-20's 3x3 layers at batch 256:
         16 -> 16 channels at 32x32 (<4, 4, 16, 4, true>) and 32 -> 32 at 16x16 (<4, 2, 32, 8, true>), both with
         residual, ReLU, float and fixed-point outputs."""
@@ -555,7 +556,7 @@ def pmc_target(device):
         narrow.append((xn, tiledn, kbn, ch, torch.rand(ch, generator=g).to(device) * 2.0 ** -6,
                        torch.randn(ch, generator=g).to(device),
                        torch.randn(256, ch, size, size, generator=g).to(device), {}))
-    cache, cache2 = {}, {}
+    cache, cache2, cache8 = {}, {}, {}
     torch.cuda.synchronize()
     for _ in range(3):
         _lib.call("ds_copy_i32", _lib.ptr(src), _lib.ptr(dst), n, _lib.current_stream(device))
@@ -572,7 +573,8 @@ def pmc_target(device):
                  emit=((1, 1), 16, 16, torch.int32), want_float=False, q_cache=cache2),
             dict(tiled=tiledb, O=128, kernel_size=(1, 1), crop=(1, 1), bits=kbb, scale=scale2, shift=offs2,
                  want_float=True))
-        kernels.conv2d_paired(x8, blob8, None, 128, (3, 3), (1, 1), fields[1], 96)
+        kernels.conv2d_paired_fused(x8, blob8, None, 128, (3, 3), (1, 1), fields[1], 96, 5, scale2, offs2, None, True,
+                                    ((0, 0), 3, 5, torch.int8), False, cache8)
         for xn, tiledn, kbn, ch, sc, of, res, qc in narrow:
             kernels.conv2d_tiled_fused(xn, tiledn, None, ch, (3, 3), (1, 1), kbn, 16, sc, of, res, True,
                                        ((1, 1), 16, 16, torch.int32), True, qc)

@@ -426,13 +426,16 @@ struct PairTail {
 };
 typedef __attribute__((address_space(3))) const PairTail lds_ptail;
 
-constexpr int kPairUnit = 8;  // channels that one call of pairs_write_unit finishes
+// channels that one call of pairs_write_unit finishes: 4 x 6 blocks = 24 outputs per lane keep the tail
+// function within the registers it need not save (with 8 it saved and restored 61 registers through scratch
+// memory on every call: 100 MB of extra traffic per launch of a ResNet-50 3x3 layer)
+constexpr int kPairUnit = 4;
 
-// Eight channels x the tile's six 64-pixel blocks (48 outputs per lane) leave the tile buffer: bias (and,
+// kPairUnit channels x the tile's six 64-pixel blocks (24 outputs per lane) leave the tile buffer: bias (and,
 // for the xor-mask forms, the count of negative codes for the pixels that lived in low halves), then the
 // arithmetic of the int32 kernel's write_tile in the same order.  Everything that comes from memory is
 // requested up front: the per-channel constants by the lanes (lane c holds those of channel ch0 + c and
-// hands them out with v_readlane), the residuals of all 48 outputs before the first is used.
+// hands them out with v_readlane), the residuals of all 24 outputs before the first is used.
 template <typename Q, bool PACKED>
 __device__ __forceinline__ void pairs_write_unit(lds_ptail *t, lds_i32 *buf, int ntile, int m0, int ch0, int lane)
 {
@@ -564,7 +567,7 @@ __device__ __attribute__((noinline)) void pairs_finish_tile(lds_ptail *t, lds_i3
 {
     constexpr int WAVES = PACKED ? kPairCu4Waves : kPairCuWaves, THREADS = WAVES * kWave;
     constexpr int ELEMS = PACKED ? 64 * kPairRows * kWave : 64 * kPairPixels, PER = ELEMS / THREADS;
-    constexpr int UNITS = 64 / kPairUnit / WAVES;  // units of eight channels per wave
+    constexpr int UNITS = 64 / kPairUnit / WAVES;  // units of kPairUnit channels per wave
     // (the thread's number from the wave's, which the caller holds in a scalar register, and the lane's:
     // no work-item id has to stay in a vector register across the caller's main loop)
     const int lane = lane_now();

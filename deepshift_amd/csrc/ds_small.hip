@@ -202,8 +202,9 @@ static void launch_small(const SmallArgs &a, int mode, hipStream_t st)
 // arrivals and polls on one address, cost 650 us per barrier: atomics on one address are served one after
 // the other where all XCDs see them), counters are back at zero when the barrier has passed, and the
 // release words only ever count up: a launch needs no tag and no clearing, and a replay of a captured
-// launch finds what it needs.  Polls are read-modify-writes too (fetch-and-add of 0), which are performed
-// where every XCD sees them.
+// launch finds what it needs.  A poll is an agent-scope atomic load (global_load_dword ... sc1; the
+// compiler turns a fetch-and-add of 0 into the same instruction), which is not served from a stale line
+// of the XCD's own L2: the release is seen within a poll interval.
 // The hidden activations cross XCDs, whose L2 caches are not coherent with each other: they are written
 // with agent-scope stores, which go through to memory, every wave waits for its stores to be acknowledged
 // (s_waitcnt vmcnt(0)) before the workgroup's arrival is counted, and after the barrier one wave of the
@@ -252,6 +253,10 @@ __device__ __forceinline__ unsigned chain_rmw(unsigned *word, unsigned add)
 {
     return __hip_atomic_fetch_add(word, add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+__device__ __forceinline__ unsigned chain_peek(unsigned *word)
+{
+    return __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 template <int BITS, int MODE>
 __global__ __launch_bounds__(kSmallWaves * 64) void linear_chain_kernel(const ChainArgs c)
@@ -266,7 +271,7 @@ __global__ __launch_bounds__(kSmallWaves * 64) void linear_chain_kernel(const Ch
     if (threadIdx.x == 0) {
 #pragma unroll
         for (int l = 0; l < kChainMax - 1; ++l)
-            if (l + 1 < c.nlayers) release_before[l] = chain_rmw(chain_word(c.control, l, kChainRelease, w % kChainGroups), 0u);
+            if (l + 1 < c.nlayers) release_before[l] = chain_peek(chain_word(c.control, l, kChainRelease, w % kChainGroups));
     }
     for (int l = 0; l < c.nlayers; ++l) {
         const bool last = l == c.nlayers - 1;
@@ -305,7 +310,7 @@ __global__ __launch_bounds__(kSmallWaves * 64) void linear_chain_kernel(const Ch
                 }
             }
             const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();
-            while (chain_rmw(chain_word(c.control, l, kChainRelease, group), 0u) == release_before[l]) {
+            while (chain_peek(chain_word(c.control, l, kChainRelease, group)) == release_before[l]) {
                 if (__builtin_amdgcn_s_memrealtime() - t0 > (unsigned long long)c.spin_ticks) {
                     ok = 0;
                     __hip_atomic_store(c.status, l + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
