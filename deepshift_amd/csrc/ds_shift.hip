@@ -494,7 +494,8 @@ struct PlaneWalk {
 constexpr int kPlaneRows = 3;      // pixels per lane of the 32-channel form (R of gen_planes_asm.py)
 constexpr int kPlaneRowsWide = 2;  // ... of the 64-channel form (ROWS_WIDE): two scalar and two vector
                                    // instructions per code, which two waves interleave without gaps
-constexpr int plane_rows(bool wide) { return wide ? kPlaneRowsWide : kPlaneRows; }
+constexpr int kPlaneRowsNarrow = 2;  // ... of the 32-channel form that runs four waves per SIMD (128 registers)
+constexpr int plane_rows(bool wide, bool narrow = false) { return wide ? kPlaneRowsWide : narrow ? kPlaneRowsNarrow : kPlaneRows; }
 // Wave slots of the machine: the 32-channel form runs 3 waves per SIMD, the 64-channel form 2 (they
 // interleave best); 4 SIMDs per compute unit -- 3072 and 2048 on the 256 CUs of an MI355X.
 static int plane_slots(bool wide) { return device_cus() * 4 * (wide ? 2 : 3); }
@@ -514,8 +515,15 @@ static int plane_slots(bool wide) { return device_cus() * 4 * (wide ? 2 : 3); }
       "s"(w.fw), "s"(w.fh), "s"(w.FW), "s"(w.FH), "s"(w.row_step), "s"(w.plane_step),             \
       "s"(w.koff_max)
 
-// Main loop of the 32-channel form (six 16-register accumulator vectors) and of the 64-channel form
-// (six of 32 registers).
+// the 32-channel form with two pixel rows: 64 accumulators in v[64:127], four waves per SIMD
+#define DS_PLANES_OPERANDS_NARROW                                                                 \
+    : "+{v[64:79]}"(a[0]), "+{v[80:95]}"(a[1]), "+{v[96:111]}"(a[2]), "+{v[112:127]}"(a[3])       \
+    : "v"(xoff[0]), "v"(xoff[1]), "s"(rsrc), "s"(wptr), "s"(groups), "s"(w.koff),                 \
+      "s"(w.fw), "s"(w.fh), "s"(w.FW), "s"(w.FH), "s"(w.row_step), "s"(w.plane_step),             \
+      "s"(w.koff_max)
+
+// Main loop of the 32-channel form (six 16-register accumulator vectors), of the 64-channel form
+// (six of 32 registers) and of the 32-channel form with two pixel rows (four of 16).
 // ZT 1: the blob's highest field value stands for a zero weight (its plane is held at 0); 2: no code
 // carries the highest field value (its plane does not exist); 0: every field value is a shift.
 template <int BITS, int ZT>
@@ -524,6 +532,10 @@ __device__ __forceinline__ void planes_main_loop(v16i (&a)[6], const uint32_t (&
 template <int BITS, int ZT>
 __device__ __forceinline__ void planes_main_loop(v32i (&a)[2 * kPlaneRowsWide],
                                                  const uint32_t (&xoff)[kPlaneRowsWide], v4i rsrc,
+                                                 const uint32_t *wptr, int groups, const PlaneWalk &w);
+template <int BITS, int ZT>
+__device__ __forceinline__ void planes_main_loop(v16i (&a)[2 * kPlaneRowsNarrow],
+                                                 const uint32_t (&xoff)[kPlaneRowsNarrow], v4i rsrc,
                                                  const uint32_t *wptr, int groups, const PlaneWalk &w);
 #define DS_PLANES_ONE(B, ZT, VEC, ROWS, ASM, OPERANDS, CLOBBERS)                                   \
     template <>                                                                                    \
@@ -539,7 +551,10 @@ __device__ __forceinline__ void planes_main_loop(v32i (&a)[2 * kPlaneRowsWide],
     DS_PLANES_ONE(B, 2, v16i, kPlaneRows, DS_PLANES_ASM_B##B##U, DS_PLANES_OPERANDS, DS_PLANES_CLOBBERS_B##B##U) \
     DS_PLANES_ONE(B, 0, v32i, kPlaneRowsWide, DS_PLANES_ASM_B##B##W, DS_PLANES_OPERANDS_WIDE, DS_PLANES_CLOBBERS_B##B##W) \
     DS_PLANES_ONE(B, 1, v32i, kPlaneRowsWide, DS_PLANES_ASM_B##B##ZW, DS_PLANES_OPERANDS_WIDE, DS_PLANES_CLOBBERS_B##B##W) \
-    DS_PLANES_ONE(B, 2, v32i, kPlaneRowsWide, DS_PLANES_ASM_B##B##UW, DS_PLANES_OPERANDS_WIDE, DS_PLANES_CLOBBERS_B##B##UW)
+    DS_PLANES_ONE(B, 2, v32i, kPlaneRowsWide, DS_PLANES_ASM_B##B##UW, DS_PLANES_OPERANDS_WIDE, DS_PLANES_CLOBBERS_B##B##UW) \
+    DS_PLANES_ONE(B, 0, v16i, kPlaneRowsNarrow, DS_PLANES_ASM_B##B##N, DS_PLANES_OPERANDS_NARROW, DS_PLANES_CLOBBERS_B##B##N) \
+    DS_PLANES_ONE(B, 1, v16i, kPlaneRowsNarrow, DS_PLANES_ASM_B##B##ZN, DS_PLANES_OPERANDS_NARROW, DS_PLANES_CLOBBERS_B##B##N) \
+    DS_PLANES_ONE(B, 2, v16i, kPlaneRowsNarrow, DS_PLANES_ASM_B##B##UN, DS_PLANES_OPERANDS_NARROW, DS_PLANES_CLOBBERS_B##B##UN)
 DS_PLANES_SPECIALISE(1)
 DS_PLANES_SPECIALISE(2)
 DS_PLANES_SPECIALISE(3)
@@ -551,12 +566,14 @@ DS_PLANES_SPECIALISE(4)
 // 64-channel form (layers with N % 64 == 0).  TO_LDS 1: the sums are added to the workgroup's tile
 // buffer instead; 2: the same if the caller passes a buffer, else the plain store (decided at run
 // time, so that one copy of the main loop serves both).
-template <int BITS, int ZT, bool WIDE, int TO_LDS = 0>
+// NARROW: the 32-channel form with two pixel rows.
+template <int BITS, int ZT, bool WIDE, int TO_LDS = 0, bool NARROW = false>
 __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, int m0, int g_begin,
                                                int g_end, bool atomic, int32_t *lds = nullptr)
 {
+    static_assert(!(WIDE && NARROW), "two pixel rows of 32 channels, or 64 channels");
     constexpr int NUM = 32 / (BITS + 1);
-    constexpr int R = plane_rows(WIDE), J = WIDE ? 64 : 32;
+    constexpr int R = plane_rows(WIDE, NARROW), J = WIDE ? 64 : 32;
     constexpr int VEC = WIDE ? 32 : 16;  // registers per accumulator operand of the asm loop
     using acc_vec = typename std::conditional<WIDE, v32i, v16i>::type;
     const int lane = threadIdx.x & (kWave - 1);
@@ -744,6 +761,52 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void shift_planes_wide_balanced_kernel(const ShiftArgs p)
 {
     planes_balanced_body<BITS, ZT, true>(p);
+}
+
+// The 32-channel form inside the one-tile-per-workgroup scheme of shift_coop_kernel, for layers of 32, 96,
+// 160 ... channels that the 64-channel form cannot take: a workgroup owns a tile of 2 x 64 pixels x 32
+// channels, its eight waves split the tile's reduction, each runs the shift-plane loop on its part
+// (1 + 15/32 vector instructions per term instead of two) and adds its sums into the LDS tile; after the
+// barrier each wave finishes four channels through the fused epilogue.  128 registers: four waves per
+// SIMD, like the kernel it replaces.
+template <int BITS, int ZT, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(4, 4)))
+void shift_planes_narrow_coop_kernel(const ShiftArgs p)
+{
+    constexpr int R = kPlaneRowsNarrow, J = 32, CH = J / WAVES;
+    static_assert(J % WAVES == 0, "whole channels per wave in the write-out");
+    __shared__ int32_t sums[J][R * kWave];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int bid = blockIdx.x;
+    const int tile = (bid & 7) * p.blocks_per_xcd + (bid >> 3);  // an XCD takes a contiguous range of tiles
+    if (tile >= p.tiles_m4 * p.tiles_n) return;
+    const int ntile = tile % p.tiles_n;
+    const int m0 = (tile / p.tiles_n) * (R * kWave);
+    for (int i = threadIdx.x; i < J * R * kWave; i += WAVES * kWave) (&sums[0][0])[i] = 0;
+    __syncthreads();
+    const int g_begin = (int)((long)wave * p.comm / WAVES), g_end = (int)((long)(wave + 1) * p.comm / WAVES);
+    planes_segment<BITS, ZT, false, 1, true>(p, ntile, m0, g_begin, g_end, false, &sums[0][0]);
+    __syncthreads();
+
+    bool live[R];
+    int img_of[R], rem_of[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        int m = m0 + r * kWave + lane;
+        live[r] = m < p.M;
+        if (!live[r]) m = p.M - 1;
+        img_of[r] = (int)div_by((uint32_t)m, p.div_pix);
+        rem_of[r] = m - img_of[r] * p.pix_per_img;
+    }
+    int32_t fin[R][CH];
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+        for (int r = 0; r < R; ++r) fin[r][c] = sums[wave * CH + c][r * kWave + lane];
+    const int n0 = ntile * J + wave * CH;
+    if (p.ep_q_bytes == 1) fused_store<int8_t, R, CH>(p, fin, n0, live, img_of, rem_of);
+    else fused_store<int32_t, R, CH>(p, fin, n0, live, img_of, rem_of);
 }
 
 // Workgroup-cooperative launch of the 64-channel form: the (tile, K group) space is cut into one
@@ -1210,10 +1273,27 @@ static int launch_shift_coop(ShiftArgs a, hipStream_t st)
     a.atomic_out = 0;
     a.div_pix = fast_div((uint32_t)a.pix_per_img);
     a.div_ow = fast_div((uint32_t)a.OW);
-    if (small)
+    if (small) {
         hipLaunchKernelGGL((shift_coop_kernel<BITS, 4, 16, 4, FUSED>), dim3(a.blocks_per_xcd * 8), dim3(256), 0, st, a);
-    else
-        hipLaunchKernelGGL((shift_coop_kernel<BITS, 2, 32, 8, FUSED>), dim3(a.blocks_per_xcd * 8), dim3(512), 0, st, a);
+        return launch_status();
+    }
+    if constexpr (BITS <= 4 && FUSED) {
+        // whole tiles of 32 channels whose codes are there in the 32-channel 16-bit layout: the shift-plane
+        // loop (the test hook's "planes" knob, 0, keeps the two-instruction loop)
+        bool planes = a.N % 32 == 0 && a.wt16 != nullptr && !tiled_wide(a.N, a.K, BITS) && a.comm >= 8;
+        if (g_tune.planes != kTuneUnset) planes = planes && g_tune.planes > 0;
+        if (planes) {
+            const dim3 grid(a.blocks_per_xcd * 8), block(512);
+            if (a.top_unused && a.K % codes_per_word(BITS) != 0)
+                hipLaunchKernelGGL((shift_planes_narrow_coop_kernel<BITS, 1, 8>), grid, block, 0, st, a);
+            else if (a.top_unused)
+                hipLaunchKernelGGL((shift_planes_narrow_coop_kernel<BITS, 2, 8>), grid, block, 0, st, a);
+            else
+                hipLaunchKernelGGL((shift_planes_narrow_coop_kernel<BITS, 0, 8>), grid, block, 0, st, a);
+            return launch_status();
+        }
+    }
+    hipLaunchKernelGGL((shift_coop_kernel<BITS, 2, 32, 8, FUSED>), dim3(a.blocks_per_xcd * 8), dim3(512), 0, st, a);
     return launch_status();
 }
 

@@ -67,6 +67,7 @@ R = 3                                    # pixel rows per lane (the int8 forms: 
 ROWS_WIDE = 2                            # ... of the 64-channel int32 form
 DEPTH = {1: 4, 2: 5, 3: 4, 4: 3}        # prefetch ring depth, 32-channel form
 DEPTH_WIDE = {1: 4, 2: 5, 3: 4, 4: 3}   # 64-channel form
+DEPTH_NARROW = {1: 4, 2: 5, 3: 4, 4: 3} # 32-channel form with two pixel rows
 DEPTH_WIDE_U = {1: 4, 2: 5, 3: 4, 4: 3}  # 64-channel form without the top plane: its registers buy a third slot
 DEPTH_PAIRED = {1: 4, 2: 2, 3: 1, 4: 1}  # int8 forms: six activation registers per slot
 DEPTH_PAIRED_U = {1: 4, 2: 5}            # index forms without the planes of the top field value
@@ -75,13 +76,13 @@ DEPTH_PAIRED_U = {1: 4, 2: 5}            # index forms without the planes of the
 class Form:
     """Register and operand layout of the 32-channel (wide=False) or 64-channel loop."""
 
-    def __init__(self, bits, wide, paired=False):
+    def __init__(self, bits, wide, paired=False, narrow=False):
         self.paired = paired
         self.J = 64 if wide else 32
-        self.acc = 64 if wide else 66
-        self.depth = (DEPTH_WIDE if wide else DEPTH)[bits]
-        self.waves = 2 if wide else 3
-        self.R = ROWS_WIDE if wide and not paired else R
+        self.acc = 64 if wide or narrow else 66
+        self.depth = (DEPTH_WIDE if wide else DEPTH_NARROW if narrow else DEPTH)[bits]
+        self.waves = 2 if wide else 4 if narrow else 3
+        self.R = ROWS_WIDE if (wide and not paired) or narrow else R
         nacc = 2 * self.R                       # accumulator operands, 16 or 32 registers each
         nx = 2 * R if paired else self.R        # activation offsets: one per pixel held by a lane
         if paired:
@@ -155,6 +156,8 @@ def take_turn(tag, waves):
     should take over is the one that is running slowly.  Three waves rotate through priorities 2, 1,
     0; two waves swap 2 and 0."""
     hi, mid, end = "%d" % (20 + tag), "%d" % (40 + tag), "%d" % (60 + tag)
+    if waves == 4:
+        return []   # four waves of one workgroup meet at its barrier anyway: no turns
     if waves == 2:
         return ["s_bfe_u32 s%d, s%d, 0x1000c" % (T0, TIME),
                 "s_and_b32 s%d, s%d, 1" % (T1, PRIO),
@@ -179,12 +182,12 @@ def take_turn(tag, waves):
             end + ":"]
 
 
-def body(bits, zero_top=False, wide=False, unused_top=False):
+def body(bits, zero_top=False, wide=False, unused_top=False, narrow=False):
     """zero_top: the plane of the highest field value is held at 0 (it stands for a zero weight).
     unused_top: no code carries the highest field value, so its plane does not exist: PS planes per
     row instead of P, and in the 64-channel form of 4-bit fields room for a third prefetch slot."""
-    assert not (zero_top and unused_top)
-    f = Form(bits, wide)
+    assert not (zero_top and unused_top) and not (wide and narrow)
+    f = Form(bits, wide, narrow=narrow)
     if unused_top and wide:
         f.depth = DEPTH_WIDE_U[bits]
     R = f.R
@@ -195,7 +198,7 @@ def body(bits, zero_top=False, wide=False, unused_top=False):
     D, ACC = f.depth, f.acc
     assert num % D == 0 and num % 2 == 0
     PL = XP + R * D
-    assert PL + PS * R <= ACC and ACC + R * f.J <= 256
+    assert PL + PS * R <= ACC and ACC + R * f.J <= (128 if narrow else 256)
     L = []
     # ---- prologue: mutable copies of the inputs, the first activation loads and code row
     L += ["s_getreg_b32 s%d, hwreg(HW_REG_HW_ID, 0, 4)" % PRIO,  # the wave's slot on its SIMD
@@ -276,8 +279,8 @@ def body(bits, zero_top=False, wide=False, unused_top=False):
     return L
 
 
-def clobbers(bits, wide=False, unused_top=False):
-    f = Form(bits, wide)
+def clobbers(bits, wide=False, unused_top=False, narrow=False):
+    f = Form(bits, wide, narrow=narrow)
     if unused_top and wide:
         f.depth = DEPTH_WIDE_U[bits]
     P = (1 << bits) - (1 if unused_top else 0)
@@ -457,6 +460,15 @@ def main():
             out.append("#define DS_PLANES_CLOBBERS_B%d%s %s" % (bits, wtag, clobbers(bits, wide)))
             out.append("#define DS_PLANES_CLOBBERS_B%dU%s %s" % (bits, wtag, clobbers(bits, wide, True)))
             out.append("")
+    for bits in (1, 2, 3, 4):
+        for zero_top, tag in ((False, ""), (True, "Z"), (False, "U")):
+            lines = body(bits, zero_top, False, unused_top=tag == "U", narrow=True)
+            out.append("#define DS_PLANES_ASM_B%d%sN \\" % (bits, tag))
+            out.append(" \\\n".join('    "%s\\n"' % line for line in lines))
+            out.append("")
+        out.append("#define DS_PLANES_CLOBBERS_B%dN %s" % (bits, clobbers(bits, narrow=True)))
+        out.append("#define DS_PLANES_CLOBBERS_B%dUN %s" % (bits, clobbers(bits, unused_top=True, narrow=True)))
+        out.append("")
     for bits in (1, 2):
         out.append("#define DS_PAIRS_ASM_B%d \\" % bits)
         out.append(" \\\n".join('    "%s\\n"' % line for line in body_paired(bits)))

@@ -226,6 +226,56 @@ def test_fused_epilogue_matches_oracle_chain(oracle, rng, geom):
             np.testing.assert_array_equal(q, so.np_requantize(v, emit[2], emit[3], emit[:2]))
 
 
+# layers of 32, 96 ... channels: the shift-plane loop inside the one-tile-per-workgroup launch (two pixel rows x
+# 32 channels per lane), every form of it
+PLANE32_CASES = [
+    # Nb, C, Hp, Wp, O, FH, FW, stride, bits, top value unused
+    (3, 16, 34, 33, 32, 3, 3, (2, 2), 4, True),     # K = 144: whole groups, the form without the top plane
+    (3, 16, 18, 18, 32, 3, 3, (1, 1), 4, False),    # shifts up to 15: every plane
+    (2, 7, 25, 23, 96, 3, 3, (1, 1), 4, True),      # K = 63: a partial last group, top plane held at zero
+    (2, 7, 25, 23, 32, 3, 3, (1, 1), 4, False),     # ... decoded by the scalar tail
+    (4, 32, 18, 18, 32, 3, 3, (1, 1), 4, True),     # ResNet-20's second stage in small
+    (2, 40, 14, 15, 64 + 32, 3, 3, (1, 1), 3, True),   # 3-bit fields, 8 codes per word
+    (2, 40, 14, 15, 32, 3, 3, (1, 1), 2, False),    # 2-bit fields, 10 codes per word
+    (2, 150, 12, 12, 32, 1, 1, (1, 1), 1, False),   # 1-bit fields, 16 codes per word: K = 150 leaves a partial group
+    (1, 24, 9, 9, 160, 3, 3, (1, 1), 4, True),      # 49 pixels: one ragged tile, five channel tiles
+]
+
+
+@pytest.mark.parametrize("case", PLANE32_CASES, ids=lambda c: "x".join(str(v) for v in c[:7]) + "-b%d%s" % (c[8], "u" if c[9] else ""))
+def test_narrow_plane_form_matches_oracle_chain(oracle, rng, case):
+    """The fused launch of layers whose channel count is a multiple of 32 but not of 64 against the oracle
+    chain, and against the two-instruction loop it replaces (forced through the test hook)."""
+    Nb, C, Hp, Wp, O, FH, FW, stride, bits, unused = case
+    OH, OW = (Hp - FH) // stride[0] + 1, (Wp - FW) // stride[1] + 1
+    xp = random_activations(rng, (Nb, C, Hp, Wp))
+    s, sign = random_codes(rng, (O, C, FH, FW), max_s=2 ** bits - (2 if unused else 1))
+    bias = rng.integers(-2 ** 16, 2 ** 16, size=O).astype(np.int32)
+    y = oracle.conv2d(xp, -s, sign, bias, stride, nthreads=NTHREADS)
+    blob = kernels.tile_weights(_dev(so.np_pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)).reshape(-1),
+                                O, C, FH, FW, bits, 0)
+    scale = ((rng.random(O) + 0.5) * 2.0 ** -6).astype(np.float32)
+    shift = rng.standard_normal(O).astype(np.float32)
+    res = (rng.standard_normal((Nb, O, OH, OW)) * 2).astype(np.float32)
+    flag = bits | (U if unused else 0)
+    for sc, sh, r, relu, want_float, emit in [
+        (scale, shift, res, True, True, (1, 1, 16, 16, torch.int32)),
+        (None, None, None, False, True, None),
+        (scale, shift, None, True, False, (1, 2, 3, 5, torch.int8)),
+    ]:
+        v = so.np_dequantize_affine(y, 16, sc, sh, r, relu)
+        out, q = abi_conv_fused(xp, blob, bias, O, FH, FW, stride, flag, 16, sc, sh, r, relu, want_float, emit)
+        with Tune(planes=0):
+            out2, q2 = abi_conv_fused(xp, blob, bias, O, FH, FW, stride, flag, 16, sc, sh, r, relu, want_float, emit)
+        if want_float:
+            np.testing.assert_array_equal(out, v)
+            np.testing.assert_array_equal(out2, v)
+        if emit is not None:
+            want_q = so.np_requantize(v, emit[2], emit[3], emit[:2])
+            np.testing.assert_array_equal(q, want_q)
+            np.testing.assert_array_equal(q2, want_q)
+
+
 def test_border_kept_writes_the_interior_only(oracle, rng):
     """q_bytes | DS_Q_BORDER_KEPT: the caller's buffer keeps its padding (zeroed once by the caller), the
     kernel overwrites the interior; with the flag off the kernel writes the padding itself."""
