@@ -315,7 +315,7 @@ def config2(device, reps=10):
 
 
 def fused_model_timing(device, cls, batch, weight_bits, integer_bits, fraction_bits, workload, steps=5,
-                       chw=CHW, peak=PEAK_PAIRS):
+                       chw=CHW, peak=PEAK_PAIRS, graph_replay=False):
     """Steps/s and shift-kernel rate of a converted, fused network on synthetic input."""
     from deepshift_amd import convert, fuse
     g = torch.Generator().manual_seed(0)
@@ -338,11 +338,48 @@ def fused_model_timing(device, cls, batch, weight_bits, integer_bits, fraction_b
     layers = kernel_timings(fused, x, 3)
     pairs = sum(L["M"] * L["K"] * L["N"] for L in layers)
     kernel_s = sum(L["seconds"] for L in layers)
-    return dict(workload=workload, ms_per_step=sec * 1e3, images_per_s=batch / sec, shift_layers=len(layers),
-                pairs_per_step=pairs, shift_kernel_ms_per_step=kernel_s * 1e3,
-                shift_tpairs_per_s=pairs / kernel_s / 1e12,
-                valu_bound_tpairs_per_s=peak / 1e12, valu_frac=pairs / kernel_s / peak,
-                frac_of_two_instruction_peak=pairs / kernel_s / PEAK_PAIRS_TWO_INSTR)
+    out = dict(workload=workload, ms_per_step=sec * 1e3, images_per_s=batch / sec, shift_layers=len(layers),
+               pairs_per_step=pairs, shift_kernel_ms_per_step=kernel_s * 1e3,
+               shift_tpairs_per_s=pairs / kernel_s / 1e12,
+               valu_bound_tpairs_per_s=peak / 1e12, valu_frac=pairs / kernel_s / peak,
+               frac_of_two_instruction_peak=pairs / kernel_s / PEAK_PAIRS_TWO_INSTR)
+    if graph_replay:
+        out.update(graph_replay_timing(fused, x, steps))
+    return out
+
+
+def graph_replay_timing(fused, x, steps):
+    """The step replayed from a captured HIP graph (what the GPU needs for it, with no launch left on the host),
+    beside the eager figure.  Every replay is checked against the eager result, with eager steps and
+    synchronisations between the replays."""
+    try:
+        with torch.no_grad():
+            want = fused(x).clone()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(2):
+                    fused(x)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                y_graph = fused(x)
+            same = True
+            for _ in range(3):
+                graph.replay()
+                torch.cuda.synchronize()
+                same = same and bool(torch.equal(y_graph, want))
+                same = same and bool(torch.equal(fused(x), want))
+                torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                graph.replay()
+            torch.cuda.synchronize()
+            sec = (time.perf_counter() - t0) / steps
+        return dict(ms_per_step_graph_replay=sec * 1e3, graph_replay_equals_eager=same)
+    except Exception as exc:  # capture is an extra: the eager figure stands without it
+        return dict(ms_per_step_graph_replay=None, graph_replay_error=str(exc)[:200])
 
 
 def config5(device, steps=5):
@@ -371,7 +408,7 @@ def config3(device, steps=10):
     from deepshift_amd import workloads
     return fused_model_timing(device, workloads.ResNet20, 256, 5, 16, 16,
                               "ResNet-20, batch 256 x 3x32x32, weight_bits 5, activations 16.16", steps,
-                              chw=(3, 32, 32))
+                              chw=(3, 32, 32), graph_replay=True)
 
 
 def config1(device, with_cpu=True, reps=50):
