@@ -159,9 +159,9 @@ def take_turn(tag, waves):
     if waves == 4:
         return []   # four waves of one workgroup meet at its barrier anyway: no turns
     if waves == 2:
+        # (the prologue of the 64-channel form reduced PRIO to its low bit: T1 holds a constant there)
         return ["s_bfe_u32 s%d, s%d, 0x1000c" % (T0, TIME),
-                "s_and_b32 s%d, s%d, 1" % (T1, PRIO),
-                "s_cmp_eq_u32 s%d, s%d" % (T0, T1), "s_cbranch_scc1 %sf" % hi,
+                "s_cmp_eq_u32 s%d, s%d" % (T0, PRIO), "s_cbranch_scc1 %sf" % hi,
                 "s_setprio 0", "s_branch %sf" % end,
                 hi + ":", "s_setprio 2",
                 end + ":"]
@@ -219,6 +219,12 @@ def body(bits, zero_top=False, wide=False, unused_top=False, narrow=False):
         # the highest field value contributes nothing: its plane is 0, once and for all
         L += ["v_mov_b32 v%d, 0" % (PL + PS * r + P - 1) for r in range(R)]
     L += ["s_mov_b32 s%d, 0" % IDX, "s_set_gpr_idx_on s%d, 0x1" % IDX]  # src0 of vector ops is M0-relative
+    if wide:
+        # The bit-field descriptors of the two sign bits (width 1, offset 8 / 24) live in scalar registers:
+        # as literals they would make each s_bfe_i32 eight bytes long, 4 of the 28 bytes of code per weight
+        # code, and the loop draws close to what the instruction cache delivers.
+        L += ["s_and_b32 s%d, s%d, 1" % (PRIO, PRIO),
+              "s_mov_b32 s%d, 0x10008" % IDX, "s_mov_b32 s%d, 0x10018" % T1]
     # ---- one K group per iteration
     L += ["1:"]
     for i in range(num):
@@ -268,7 +274,10 @@ def body(bits, zero_top=False, wide=False, unused_top=False, narrow=False):
                     L += ["s_mov_b32 m0, s%d" % (cur + j)]
                 else:
                     L += ["s_lshr_b32 m0, s%d, 16" % (cur + j)]
-                L += ["s_bfe_i32 s%d, s%d, 0x%x" % (MASK, cur + j, (1 << 16) | (16 * half + 8))]
+                if wide:
+                    L += ["s_bfe_i32 s%d, s%d, s%d" % (MASK, cur + j, T1 if half else IDX)]
+                else:
+                    L += ["s_bfe_i32 s%d, s%d, 0x%x" % (MASK, cur + j, (1 << 16) | (16 * half + 8))]
                 ch = j + 32 * half if wide else j
                 for r in range(R):
                     a = ACC + f.J * r + ch
@@ -309,7 +318,8 @@ def body_paired(bits, unused_top=False):
           "s_mov_b64 s[%d:%d], %%%d" % (WP, WP + 1, f.op_wptr),
           "s_mov_b32 s%d, %%%d" % (KOFF, f.op_walk), "s_mov_b32 s%d, %%%d" % (FWC, f.op_walk + 1),
           "s_mov_b32 s%d, %%%d" % (FHC, f.op_walk + 2),
-          "s_mov_b32 s%d, 0x05040100" % MASK]   # v_perm_b32 selector: low halves of (src0, src1)
+          "s_mov_b32 s%d, 0x05040100" % MASK,   # v_perm_b32 selector: low halves of (src0, src1)
+          "s_and_b32 s%d, s%d, 1" % (PRIO, PRIO)]
     L += load_words(W)
     L += ["s_memrealtime s[%d:%d]" % (TIME, TIME + 1)]
     for i in range(D):
@@ -385,7 +395,8 @@ def body_pairx(bits):
           "s_mov_b64 s[%d:%d], %%%d" % (WP, WP + 1, f.op_wptr),
           "s_mov_b32 s%d, %%%d" % (KOFF, f.op_walk), "s_mov_b32 s%d, %%%d" % (FWC, f.op_walk + 1),
           "s_mov_b32 s%d, %%%d" % (FHC, f.op_walk + 2),
-          "s_mov_b32 s%d, 0x05040100" % SEL]    # v_perm_b32 selector: low halves of (src0, src1)
+          "s_mov_b32 s%d, 0x05040100" % SEL,    # v_perm_b32 selector: low halves of (src0, src1)
+          "s_and_b32 s%d, s%d, 1" % (PRIO, PRIO)]
     L += load_words(W)
     L += ["s_memrealtime s[%d:%d]" % (TIME, TIME + 1)]
     L += walk_and_load(0, f)
