@@ -623,7 +623,7 @@ def pmc_target_other(device):
     64 MiB copy (scale of the byte counters), then, three times over,
       * benchmark configuration 2's convolution (3x3, 64 -> 64, 56x56, batch 32: 784 tiles on 512
         workgroups) through ds_conv2d_tiled_i32;
-      * its 4096^3 shift GEMM through ds_linear_tiled_i32 (cooperative launch + transpose of the
+      * its 4096^3 shift GEMM through ds_linear_tiled_i32 (one tile per wave + transpose of the
         channel-major scratch);
       * the int8 kernel's fused launch (ds_conv2d_paired_fused_i8: BatchNorm affine, ReLU and the next layer's
         padded int8 input from the epilogue) on ResNet-50's 1x1 convolutions with K = 256 (256 -> 64 at 56x56
