@@ -39,6 +39,13 @@ __device__ __forceinline__ uint32_t div_by(uint32_t n, const FastDiv &f)
     const uint32_t t = __umulhi(f.m, n);
     return (t + ((n - t) >> f.s1)) >> f.s2;
 }
+// The same on a wave-uniform dividend: the multiply-high goes to the scalar ALU (the compiler keeps a
+// product of two uniform values there; __umulhi as such it treats as a vector operation).
+__device__ __forceinline__ uint32_t div_by_uniform(uint32_t n, const FastDiv &f)
+{
+    const uint32_t t = (uint32_t)(((uint64_t)f.m * n) >> 32);
+    return (t + ((n - t) >> f.s1)) >> f.s2;
+}
 
 // Launch-variant overrides for the test-suite (ds_test_tune, declared in deepshift_hip_test.h):
 // kTuneUnset leaves the dispatch's own choice in place.  Process-wide; every knob is an atomic that a

@@ -73,7 +73,27 @@ struct PairArgs {
     int ep_relu, ep_ph, ep_pw, ep_q_bytes;
     int ep_border_kept;                   // the padding of q already holds zeros: write the interior only
     QuantSpec ep_spec;
+    // divisions by launch-invariant numbers as multiply-shift (ds_common.h): by pix_per_img, OW, FH * FW, FW,
+    // comm and the number of channel tiles
+    FastDiv div_pix, div_ow, div_ff, div_fw, div_comm, div_tiles_n;
+    int OH;                               // pix_per_img / OW
+    int koff_max;                         // element offset of the last real reduction index
 };
+
+// The derived fields, once M, N, K, comm, pix_per_img, OW, FH, FW, x_plane and x_row stand.
+static void derive_pair_geometry(PairArgs &a)
+{
+    const int ff = a.FH * a.FW;
+    a.div_pix = fast_div((uint32_t)a.pix_per_img);
+    a.div_ow = fast_div((uint32_t)a.OW);
+    a.div_ff = fast_div((uint32_t)ff);
+    a.div_fw = fast_div((uint32_t)a.FW);
+    a.div_comm = fast_div((uint32_t)a.comm);
+    a.div_tiles_n = fast_div((uint32_t)(a.N / 64));
+    a.OH = a.OW > 0 ? a.pix_per_img / a.OW : 0;
+    // reduction indices past K (the codes there select the zero plane) read the last real one
+    a.koff_max = ff > 0 && a.K >= ff ? (a.K / ff - 1) * a.x_plane + (a.FH - 1) * a.x_row + a.FW - 1 : 0;
+}
 
 struct PairWalk {
     int koff, fw, fh, FW, FH, row_step, plane_step, koff_max;
@@ -149,9 +169,9 @@ __device__ __forceinline__ void pairs_segment(const PairArgs &p, int ntile, int 
     for (int q = 0; q < 6; ++q) {
         int m = m0 + q * kWave + lane;
         if (m >= p.M) m = p.M - 1;
-        const int img = m / p.pix_per_img;
+        const int img = (int)div_by((uint32_t)m, p.div_pix);
         const int rem = m - img * p.pix_per_img;
-        const int oh = rem / p.OW;
+        const int oh = (int)div_by((uint32_t)rem, p.div_ow);
         const int ow = rem - oh * p.OW;
         xoff[q] = (uint32_t)(img * p.x_img_stride + oh * p.x_row_stride + ow * p.x_col_stride);
     }
@@ -168,16 +188,15 @@ __device__ __forceinline__ void pairs_segment(const PairArgs &p, int ntile, int 
         rsrc.w = 0x00020000;
         PairWalk w;
         const int k0 = g_begin * NUM, ff = p.FH * p.FW;
-        const int ic = k0 / ff, rem = k0 - ic * ff;
-        w.fh = rem / p.FW;
+        const int ic = (int)div_by_uniform((uint32_t)k0, p.div_ff), rem = k0 - ic * ff;
+        w.fh = (int)div_by_uniform((uint32_t)rem, p.div_fw);
         w.fw = rem - w.fh * p.FW;
         w.koff = ic * p.x_plane + w.fh * p.x_row + w.fw;
         w.FW = p.FW;
         w.FH = p.FH;
         w.row_step = p.x_row - p.FW;
         w.plane_step = p.x_plane - p.FH * p.x_row;
-        // reduction indices past K (the codes there select the zero plane) read the last real one
-        w.koff_max = (p.K / ff - 1) * p.x_plane + (p.FH - 1) * p.x_row + p.FW - 1;
+        w.koff_max = p.koff_max;
         pairs_main_loop<BITS, TU>(a, xoff, rsrc,
                               p.codes + ((size_t)ntile * p.comm + g_begin) * NUM * kTileWords,
                               __builtin_amdgcn_readfirstlane(g_end - g_begin), w);
@@ -214,7 +233,7 @@ __device__ __forceinline__ void pairs_segment(const PairArgs &p, int ntile, int 
         const int m = m0 + q * kWave + lane;
         live[q] = m < p.M;
         const int mc = live[q] ? m : p.M - 1;
-        const int img = mc / p.pix_per_img;
+        const int img = (int)div_by((uint32_t)mc, p.div_pix);
         yoff[q] = 4u * (uint32_t)(img * p.y_img_stride + (mc - img * p.pix_per_img));
     }
     const int n0 = ntile * 64;
@@ -330,7 +349,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             for (int q = 0; q < 6; ++q) {
                 const int m = m0 + q * kWave + lane;
                 if (m >= p.M) break;
-                const int img = m / p.pix_per_img;
+                const int img = (int)div_by((uint32_t)m, p.div_pix);
                 int32_t *dst = p.y + (size_t)img * p.y_img_stride + (size_t)n * p.y_ch_stride +
                                (m - img * p.pix_per_img);
                 const int32_t v = tile_sums[j * kPairPixels + q * kWave + lane];
@@ -385,7 +404,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 for (int h = 0; h < 2; ++h) {
                     const int m = m0 + (2 * r + h) * kWave + lane;
                     if (m >= p.M) break;
-                    const int img = m / p.pix_per_img;
+                    const int img = (int)div_by((uint32_t)m, p.div_pix);
                     int32_t *dst = p.y + (size_t)img * p.y_img_stride + (size_t)n * p.y_ch_stride +
                                    (m - img * p.pix_per_img);
                     const int32_t sum = h ? hi : lo;
@@ -419,7 +438,8 @@ struct PairTail {
     void *q;
     const float *scale, *shift, *residual;
     long G, total;
-    int M, N, comm, pix_per_img, OW;
+    int M, N, comm, pix_per_img, OW, OH;
+    FastDiv div_pix, div_ow;
     float inv;
     int relu, ph, pw, q_bytes, border_kept;
     QuantSpec spec;
@@ -456,7 +476,11 @@ __device__ __forceinline__ void pairs_write_unit(lds_ptail *t, lds_i32 *buf, int
     g_char *out = (g_char *)uniform_global(t->out);
     g_char *q = (g_char *)uniform_global((char *)t->q);
     const int ph = uniform(t->ph), pw = uniform(t->pw);
-    const int OH = pix_per_img / OW;
+    const int OH = uniform(t->OH);
+    const FastDiv div_pix{(uint32_t)uniform((int32_t)t->div_pix.d), (uint32_t)uniform((int32_t)t->div_pix.m),
+                          (uint32_t)uniform((int32_t)t->div_pix.s1), (uint32_t)uniform((int32_t)t->div_pix.s2)};
+    const FastDiv div_ow{(uint32_t)uniform((int32_t)t->div_ow.d), (uint32_t)uniform((int32_t)t->div_ow.m),
+                         (uint32_t)uniform((int32_t)t->div_ow.s1), (uint32_t)uniform((int32_t)t->div_ow.s2)};
     const int Wq = OW + 2 * pw;
     const uint32_t qplane = (uint32_t)(OH + 2 * ph) * Wq;
     bool live[PB];
@@ -467,8 +491,8 @@ __device__ __forceinline__ void pairs_write_unit(lds_ptail *t, lds_i32 *buf, int
         const int m = m0 + b * kWave + lane;
         live[b] = m < M;
         const int mm = live[b] ? m : 0;
-        const int img = mm / pix_per_img, rem = mm - img * pix_per_img;
-        oh[b] = rem / OW;
+        const int img = (int)div_by((uint32_t)mm, div_pix), rem = mm - img * pix_per_img;
+        oh[b] = (int)div_by((uint32_t)rem, div_ow);
         ow[b] = rem - oh[b] * OW;
         pix[b] = (uint32_t)(img * N + n0) * (uint32_t)pix_per_img + rem;
         qimg[b] = (uint32_t)(img * N + n0) * qplane;
@@ -624,12 +648,12 @@ struct PairSegment {
 __device__ __forceinline__ PairSegment pairs_segment_at(const PairArgs &p, int it, int it_end)
 {
     PairSegment s;
-    s.tile = uniform(it / p.comm);  // (the division runs on the vector ALU; its result is wave-uniform)
+    s.tile = uniform((int)div_by_uniform((uint32_t)it, p.div_comm));
     s.g0 = it - s.tile * p.comm;
     int g1 = s.g0 + (it_end - it);
     if (g1 > p.comm) g1 = p.comm;
     s.len = g1 - s.g0;
-    const int mt = uniform(s.tile / p.tiles_n);
+    const int mt = uniform((int)div_by_uniform((uint32_t)s.tile, p.div_tiles_n));
     s.ntile = s.tile - mt * p.tiles_n;
     s.m0 = mt * kPairPixels;
     return s;
@@ -669,6 +693,7 @@ void shift_pairs_fused_kernel(const PairArgs p)
         tail.scale = p.ep_scale; tail.shift = p.ep_shift; tail.residual = p.ep_residual;
         tail.G = G; tail.total = total;
         tail.M = p.M; tail.N = p.N; tail.comm = p.comm; tail.pix_per_img = p.pix_per_img; tail.OW = p.OW;
+        tail.OH = p.OH; tail.div_pix = p.div_pix; tail.div_ow = p.div_ow;
         tail.inv = p.ep_inv; tail.relu = p.ep_relu; tail.ph = p.ep_ph; tail.pw = p.ep_pw;
         tail.q_bytes = p.ep_q_bytes; tail.border_kept = p.ep_border_kept; tail.spec = p.ep_spec;
     }
@@ -1043,6 +1068,7 @@ DS_EXPORT int ds_conv2d_paired_i8(const int8_t *x, const void *paired, const int
     a.y_elems = (uint32_t)(M * O);
     a.x_plane = Hp * Wp; a.x_row = Wp;
     a.FH = FH; a.FW = FW;
+    derive_pair_geometry(a);
     a.chunk = pair_chunk(field_bits, x_bound);
     if (K == 0) {
         // no terms: the output is the bias
@@ -1086,6 +1112,7 @@ static int paired_args(PairArgs &a, const int8_t *x, const void *paired, const i
     a.y_elems = (uint32_t)(M * O);
     a.x_plane = Hp * Wp; a.x_row = Wp;
     a.FH = FH; a.FW = FW;
+    derive_pair_geometry(a);
     a.chunk = pair_chunk(field_bits, x_bound);
     return DS_OK;
 }

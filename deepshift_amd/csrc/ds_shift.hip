@@ -79,9 +79,27 @@ struct ShiftArgs {
     int ep_border_kept;                   // the padding of q already holds zeros: write the interior only
     int whole_tile_shares;                // cooperative launch: rounds of whole tiles, one per wave, before the shared space
     int coop_pad;                         // cooperative launch: iterations a tile counts for beyond its K groups
-    FastDiv div_pix, div_ow;              // cooperative two-instruction launch: division by pix_per_img, by OW
+    // Divisions by launch-invariant numbers as multiply-shift (a general 32-bit division costs the vector
+    // ALU about 40 instructions, and every segment of a tile needs a dozen): by pix_per_img, OW, FH * FW, FW,
+    // and -- cooperative launch -- by the length of a tile and of a pixel tile's span in the share space.
+    FastDiv div_pix, div_ow, div_ff, div_fw, div_len, div_span;
+    int OH;                               // pix_per_img / OW
+    int koff_max;                         // element offset of the last real reduction index
     QuantSpec ep_spec;
 };
+
+// The derived fields above, once M, K, pix_per_img, OW, FH, FW, x_plane and x_row stand.
+static void derive_geometry(ShiftArgs &a)
+{
+    a.div_pix = fast_div((uint32_t)a.pix_per_img);
+    a.div_ow = fast_div((uint32_t)a.OW);
+    a.div_ff = fast_div((uint32_t)(a.FH * a.FW));
+    a.div_fw = fast_div((uint32_t)a.FW);
+    a.div_len = a.div_span = fast_div(1u);  // set by the cooperative launch
+    a.OH = a.OW > 0 ? a.pix_per_img / a.OW : 0;
+    const int ff = a.FH * a.FW;
+    a.koff_max = ff > 0 && a.K >= ff ? (a.K / ff - 1) * a.x_plane + (a.FH - 1) * a.x_row + a.FW - 1 : 0;
+}
 
 // Redirects an atomic LinearShift launch to its channel-major scratch; returns the final y or nullptr.
 static int32_t *redirect_to_scratch(ShiftArgs &a)
@@ -188,7 +206,7 @@ template <typename Q, int R, int J>
 __device__ __forceinline__ void fused_store(const ShiftArgs &p, const int32_t (&acc)[R][J], int n0,
                                             const bool (&live)[R], const int (&img)[R], const int (&rem)[R])
 {
-    const int OW = p.OW, OH = p.pix_per_img / OW, ph = p.ep_ph, pw = p.ep_pw;
+    const int OW = p.OW, OH = p.OH, ph = p.ep_ph, pw = p.ep_pw;
     const int Wq = OW + 2 * pw;
     const uint32_t qplane = (uint32_t)(OH + 2 * ph) * Wq, plane = (uint32_t)p.pix_per_img;
     float *out = p.ep_out;
@@ -345,9 +363,9 @@ __global__ __launch_bounds__(256) void shift_kernel(const ShiftArgs p)
         int m = m0 + r * kWave + lane;
         live[r] = m < p.M;
         if (!live[r]) m = p.M - 1;
-        const int img = m / p.pix_per_img;
+        const int img = (int)div_by((uint32_t)m, p.div_pix);
         const int rem = m - img * p.pix_per_img;
-        const int oh = rem / p.OW;
+        const int oh = (int)div_by((uint32_t)rem, p.div_ow);
         const int ow = rem - oh * p.OW;
         xoff[r] = 4u * (uint32_t)(img * p.x_img_stride + oh * p.x_row_stride + ow * p.x_col_stride);
         yoff[r] = 4u * (uint32_t)(img * p.y_img_stride + rem * p.y_pix_stride);
@@ -585,9 +603,9 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
         int m = m0 + r * kWave + lane;
         live[r] = m < p.M;
         if (!live[r]) m = p.M - 1;
-        const int img = m / p.pix_per_img;
+        const int img = (int)div_by((uint32_t)m, p.div_pix);
         const int rem = m - img * p.pix_per_img;
-        const int oh = rem / p.OW;
+        const int oh = (int)div_by((uint32_t)rem, p.div_ow);
         const int ow = rem - oh * p.OW;
         xoff[r] = 4u * (uint32_t)(img * p.x_img_stride + oh * p.x_row_stride + ow * p.x_col_stride);
         yoff[r] = 4u * (uint32_t)(img * p.y_img_stride + rem * p.y_pix_stride);
@@ -612,8 +630,8 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
         PlaneWalk w;
         const int FH = uniform(p.FH), FW = uniform(p.FW), x_plane = uniform(p.x_plane), x_row = uniform(p.x_row);
         const int k0 = uniform(g_begin) * NUM, ff = FH * FW;
-        const int ic = k0 / ff, rem = k0 - ic * ff;
-        w.fh = uniform(rem / FW);
+        const int ic = (int)div_by_uniform((uint32_t)k0, p.div_ff), rem = k0 - ic * ff;
+        w.fh = uniform((int)div_by_uniform((uint32_t)rem, p.div_fw));
         w.fw = uniform(rem - w.fh * FW);
         // byte offsets; row_step is the whole step of an fw wrap (the element step included)
         w.koff = uniform(4 * (ic * x_plane + w.fh * x_row + w.fw));
@@ -621,7 +639,7 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
         w.FH = FH;
         w.row_step = 4 * (x_row - FW + 1);
         w.plane_step = 4 * (x_plane - FH * x_row);
-        w.koff_max = uniform(4 * ((uniform(p.K) / ff - 1) * x_plane + (FH - 1) * x_row + FW - 1));
+        w.koff_max = uniform(4 * p.koff_max);
         // rows of 16-bit codes per K group: NUM/2 (two slots per row) or NUM (one slot, 64 channels)
         constexpr int ROWS = WIDE ? NUM : NUM / 2;
         const uint64_t waddr = (uint64_t)(p.wt16 + ((size_t)ntile * p.comm + g_begin) * ROWS * kTileWords);
@@ -864,7 +882,8 @@ struct TileTail {
     const float *scale, *shift, *residual;
     long y_img_stride, y_pix_stride, y_ch_stride;
     long G, total;
-    int M, N, comm, pix_per_img, OW;
+    int M, N, comm, pix_per_img, OW, OH;
+    FastDiv div_pix, div_ow;
     float inv;
     int relu, ph, pw, q_bytes, border_kept;
     QuantSpec spec;
@@ -905,7 +924,11 @@ __device__ __forceinline__ void write_tile(lds_tail *t, lds_i32 *buf, int ntile,
         q = (g_char *)uniform_global((char *)t->q);
     }
     const int ph = FUSED ? uniform(t->ph) : 0, pw = FUSED ? uniform(t->pw) : 0;
-    const int OH = pix_per_img / OW;
+    const int OH = uniform(t->OH);
+    const FastDiv div_pix{(uint32_t)uniform((int32_t)t->div_pix.d), (uint32_t)uniform((int32_t)t->div_pix.m),
+                          (uint32_t)uniform((int32_t)t->div_pix.s1), (uint32_t)uniform((int32_t)t->div_pix.s2)};
+    const FastDiv div_ow{(uint32_t)uniform((int32_t)t->div_ow.d), (uint32_t)uniform((int32_t)t->div_ow.m),
+                         (uint32_t)uniform((int32_t)t->div_ow.s1), (uint32_t)uniform((int32_t)t->div_ow.s2)};
     const int Hq = OH + 2 * ph, Wq = OW + 2 * pw;
     const uint32_t qplane = (uint32_t)Hq * Wq;
     bool live[R];
@@ -917,8 +940,8 @@ __device__ __forceinline__ void write_tile(lds_tail *t, lds_i32 *buf, int ntile,
         const int m = m0 + r * kWave + lane;
         live[r] = m < M;
         const int mm = live[r] ? m : 0;
-        const int img = mm / pix_per_img, rem = mm - img * pix_per_img;
-        oh[r] = rem / OW;
+        const int img = (int)div_by((uint32_t)mm, div_pix), rem = mm - img * pix_per_img;
+        oh[r] = (int)div_by((uint32_t)rem, div_ow);
         ow[r] = rem - oh[r] * OW;
         if (FUSED) {
             pix[r] = (uint32_t)(img * N + n0) * (uint32_t)pix_per_img + rem;
@@ -1067,6 +1090,7 @@ __device__ __forceinline__ void fill_tail(TileTail &tail, const ShiftArgs &p, lo
     tail.y_img_stride = p.y_img_stride; tail.y_pix_stride = p.y_pix_stride; tail.y_ch_stride = p.y_ch_stride;
     tail.G = G; tail.total = total;
     tail.M = p.M; tail.N = p.N; tail.comm = p.comm; tail.pix_per_img = p.pix_per_img; tail.OW = p.OW;
+    tail.OH = p.OH; tail.div_pix = p.div_pix; tail.div_ow = p.div_ow;
     tail.inv = p.ep_inv; tail.relu = p.ep_relu; tail.ph = p.ep_ph; tail.pw = p.ep_pw;
     tail.q_bytes = p.ep_q_bytes; tail.border_kept = p.ep_border_kept; tail.spec = p.ep_spec;
 }
@@ -1135,12 +1159,13 @@ void shift_planes_wide_coop_kernel(const ShiftArgs p, const ShiftArgs p2)
         // main loop in this kernel leaves the register allocator no room.)
         const bool direct = direct_rounds > 0;
         const long at = direct ? direct_at + (long)wave * len1 : shared_base + it;
-        const int mtile = (int)(at / span);
+        // (the launch's iterations stay below 2^31: 32-bit multiply-shift divisions)
+        const int mtile = (int)div_by_uniform((uint32_t)at, p.div_span);
         const int within = (int)(at - (long)mtile * span);
         const bool second = PAIR && within >= span1;
         const int comm = second ? p2.comm : p.comm;
         const int padded = comm + pad;
-        const int ntile = (second ? within - span1 : within) / padded;
+        const int ntile = (int)div_by_uniform((uint32_t)(second ? within - span1 : within), second ? p2.div_len : p.div_len);
         const long tile_start = (long)mtile * span + (second ? span1 : 0) + (long)ntile * padded;
         // position in the padded tile -> K groups [g0, g1)
         const int v0 = (int)(at - tile_start);
@@ -1189,10 +1214,17 @@ static int launch_planes_coop(const ShiftArgs &first, long iters, hipStream_t st
     ShiftArgs a = first;
     a.coop_token = next_coop_token();
     a.coop_pad = second ? kCoopPairPad : 0;
+    // the share space of the kernel: a tile counts for comm + pad iterations, a pixel tile for its channel tiles'
+    const long span = (long)a.tiles_n * (a.comm + a.coop_pad) + (second ? (long)second->tiles_n * (second->comm + a.coop_pad) : 0);
+    if (span <= 0 || (long)a.tiles_m4 * span >= (1L << 31)) return DS_ETOOLARGE;
+    a.div_len = fast_div((uint32_t)(a.comm + a.coop_pad));
+    a.div_span = fast_div((uint32_t)span);
     if (second) {
         ShiftArgs b = *second;
         b.coop_token = a.coop_token;
         b.coop_pad = a.coop_pad;
+        b.div_len = fast_div((uint32_t)(b.comm + b.coop_pad));
+        b.div_span = a.div_span;
         hipLaunchKernelGGL((shift_planes_wide_coop_kernel<BITS, ZT, true, true>), grid, block, kCoopLdsBytes, st, a, b);
     } else if (a.fused)
         hipLaunchKernelGGL((shift_planes_wide_coop_kernel<BITS, ZT, true, false>), grid, block, kCoopLdsBytes, st, a, a);
@@ -1271,8 +1303,6 @@ static int launch_shift_coop(ShiftArgs a, hipStream_t st)
     a.tiles_n = ceil_div(a.N, small ? 16 : 32);
     a.blocks_per_xcd = ceil_div(a.tiles_m4 * a.tiles_n, 8);
     a.atomic_out = 0;
-    a.div_pix = fast_div((uint32_t)a.pix_per_img);
-    a.div_ow = fast_div((uint32_t)a.OW);
     if (small) {
         hipLaunchKernelGGL((shift_coop_kernel<BITS, 4, 16, 4, FUSED>), dim3(a.blocks_per_xcd * 8), dim3(256), 0, st, a);
         return launch_status();
@@ -1667,6 +1697,7 @@ static int conv2d_tiled_any(const int32_t *x, const void *tiled, const int32_t *
     a.ktab = tiled_ktab(tiled, g);
     a.x_plane = Hp * Wp; a.x_row = Wp;
     a.FH = FH; a.FW = FW;
+    derive_geometry(a);
     a.nbase = -base;
     a.zero_top = zero_top;
     a.top_unused = top_unused;
@@ -1834,6 +1865,7 @@ static int pair_args(ShiftArgs &s, const int32_t *x, const ds_fused_conv *f, int
     s.ktab = tiled_ktab(f->tiled, g);
     s.x_plane = Hp * Wp; s.x_row = Wp;
     s.FH = f->FH; s.FW = f->FW;
+    derive_geometry(s);
     s.top_unused = (f->bits & DS_BITS_TOP_UNUSED) != 0;
     s.tiles_m4 = ceil_div((int)M, kCoopPix);
     s.tiles_n = f->O / 64;
@@ -1972,6 +2004,7 @@ DS_EXPORT int ds_linear_tiled_i32(const int32_t *xT, int ldx, const void *tiled,
     a.ktab = tiled_ktab(tiled, g);
     a.x_plane = ldx; a.x_row = 1;
     a.FH = 1; a.FW = 1;
+    derive_geometry(a);
     a.nbase = -base;
     a.zero_top = zero_top;
     a.top_unused = top_unused;
