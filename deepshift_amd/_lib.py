@@ -100,6 +100,7 @@ SIGNATURES = {
     "ds_valu_calibrate": (_c_int, [_ptr, _c_int, _c_int, _ptr]),
     "ds_copy_i32": (_c_int, [_ptr, _ptr, _c_i64, _ptr]),
     "ds_test_tune": (_c_int, [ctypes.c_char_p, _c_int]),
+    "ds_test_fast_div": (_c_int, [_ptr, _ptr, ctypes.c_long, ctypes.c_uint, _c_int, _ptr]),
 }
 
 _LIB = None

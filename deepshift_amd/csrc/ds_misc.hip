@@ -75,6 +75,25 @@ DS_EXPORT int ds_test_tune(const char *knob, int value)
     return DS_OK;
 }
 
+__global__ void fast_div_kernel(const uint32_t *n, uint32_t *q, long count, ds::FastDiv f, int uniform_form)
+{
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    q[i] = uniform_form ? ds::div_by_uniform(n[i], f) : ds::div_by(n[i], f);
+}
+
+DS_EXPORT int ds_test_fast_div(const unsigned int *n, unsigned int *q, long count, unsigned int d, int uniform_form,
+                               ds_stream_t stream)
+{
+    if (count < 0 || d < 1 || (count > 0 && (!n || !q))) return DS_EINVAL;
+    if (count == 0) return DS_OK;
+    const long blocks = (count + 255) / 256;
+    if (blocks > 0x7fffffffL) return DS_ETOOLARGE;
+    hipLaunchKernelGGL(fast_div_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, n, q, count,
+                       ds::fast_div(d), uniform_form);
+    return ds::launch_status();
+}
+
 DS_EXPORT int ds_version(void) { return 100; }
 
 DS_EXPORT const char *ds_status_string(int status)

@@ -22,6 +22,15 @@ extern "C" {
  * is why this header is not the production one.  The dispatch's own choice is the measured best. */
 int ds_test_tune(const char *knob, int value);
 
+/* q[i] = n[i] / d (and, uniform != 0, the same through the form the kernels use on wave-uniform
+ * dividends) by the multiply-shift division with which every shift kernel turns flat indices into
+ * (image, row, column) and share positions into tiles: the host derives the constants for the divisor,
+ * the device applies them.  Device pointers, count elements, d >= 1; asynchronous on `stream` (a
+ * hipStream_t, NULL = the default stream).  For the tests, which compare it with plain division over
+ * divisors and dividends up to 2^32 - 1.  Returns 0 or a negative status. */
+int ds_test_fast_div(const unsigned int *n, unsigned int *q, long count, unsigned int d, int uniform,
+                     void *stream);
+
 #ifdef __cplusplus
 }
 #endif
