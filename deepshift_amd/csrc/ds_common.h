@@ -39,6 +39,12 @@ __device__ __forceinline__ uint32_t div_by(uint32_t n, const FastDiv &f)
     const uint32_t t = __umulhi(f.m, n);
     return (t + ((n - t) >> f.s1)) >> f.s2;
 }
+// A copy of the constants, wherever the block that holds them lives (kernel-argument segment, LDS ...).
+template <typename F>
+__device__ __forceinline__ FastDiv fast_div_of(const F &f)
+{
+    return FastDiv{f.d, f.m, f.s1, f.s2};
+}
 // The same on a wave-uniform dividend: the multiply-high goes to the scalar ALU (the compiler keeps a
 // product of two uniform values there; __umulhi as such it treats as a vector operation).
 __device__ __forceinline__ uint32_t div_by_uniform(uint32_t n, const FastDiv &f)

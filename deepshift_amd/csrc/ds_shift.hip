@@ -101,6 +101,9 @@ static void derive_geometry(ShiftArgs &a)
     a.koff_max = ff > 0 && a.K >= ff ? (a.K / ff - 1) * a.x_plane + (a.FH - 1) * a.x_row + a.FW - 1 : 0;
 }
 
+// A ShiftArgs block where a kernel finds it: in the kernel-argument segment (constant address space).
+typedef __attribute__((address_space(4))) const ShiftArgs KernargShiftArgs;
+
 // Redirects an atomic LinearShift launch to its channel-major scratch; returns the final y or nullptr.
 static int32_t *redirect_to_scratch(ShiftArgs &a)
 {
@@ -134,9 +137,9 @@ __device__ __forceinline__ int32_t *at_lane(int32_t *uniform_base, uint32_t lane
 // table of the weight blob through a scalar load and the offset is formed on the scalar ALU, so a
 // load is one buffer_load_dword (per-lane VGPR offset + SGPR offset) with no vector arithmetic.
 // load_part: the COUNT reduction indices FIRST .. of the group only.
-template <int NUM, int FIRST, int COUNT, int R>
+template <int NUM, int FIRST, int COUNT, int R, typename ARGS>
 __device__ __forceinline__ void load_part(int32_t (&xv)[COUNT][R], __amdgpu_buffer_rsrc_t rsrc,
-                                          const uint32_t (&xoff)[R], const ShiftArgs &p, int g)
+                                          const uint32_t (&xoff)[R], const ARGS &p, int g)
 {
 #pragma unroll
     for (int i = 0; i < COUNT; ++i) {
@@ -148,9 +151,9 @@ __device__ __forceinline__ void load_part(int32_t (&xv)[COUNT][R], __amdgpu_buff
     }
 }
 
-template <int NUM, int R>
+template <int NUM, int R, typename ARGS>
 __device__ __forceinline__ void load_group(int32_t (&xv)[NUM][R], __amdgpu_buffer_rsrc_t rsrc,
-                                           const uint32_t (&xoff)[R], const ShiftArgs &p, int g)
+                                           const uint32_t (&xoff)[R], const ARGS &p, int g)
 {
     load_part<NUM, 0, NUM, R>(xv, rsrc, xoff, p, g);
 }
@@ -585,8 +588,9 @@ DS_PLANES_SPECIALISE(4)
 // buffer instead; 2: the same if the caller passes a buffer, else the plain store (decided at run
 // time, so that one copy of the main loop serves both).
 // NARROW: the 32-channel form with two pixel rows.
-template <int BITS, int ZT, bool WIDE, int TO_LDS = 0, bool NARROW = false>
-__device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, int m0, int g_begin,
+// ARGS: ShiftArgs, or the same block read in place in the kernel-argument segment (KernargShiftArgs).
+template <int BITS, int ZT, bool WIDE, int TO_LDS = 0, bool NARROW = false, typename ARGS = ShiftArgs>
+__device__ __forceinline__ void planes_segment(const ARGS &p, int ntile, int m0, int g_begin,
                                                int g_end, bool atomic, int32_t *lds = nullptr)
 {
     static_assert(!(WIDE && NARROW), "two pixel rows of 32 channels, or 64 channels");
@@ -598,14 +602,15 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
 
     uint32_t xoff[R], yoff[R];
     bool live[R];
+    const FastDiv div_pix = fast_div_of(p.div_pix), div_ow = fast_div_of(p.div_ow);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         int m = m0 + r * kWave + lane;
         live[r] = m < p.M;
         if (!live[r]) m = p.M - 1;
-        const int img = (int)div_by((uint32_t)m, p.div_pix);
+        const int img = (int)div_by((uint32_t)m, div_pix);
         const int rem = m - img * p.pix_per_img;
-        const int oh = (int)div_by((uint32_t)rem, p.div_ow);
+        const int oh = (int)div_by((uint32_t)rem, div_ow);
         const int ow = rem - oh * p.OW;
         xoff[r] = 4u * (uint32_t)(img * p.x_img_stride + oh * p.x_row_stride + ow * p.x_col_stride);
         yoff[r] = 4u * (uint32_t)(img * p.y_img_stride + rem * p.y_pix_stride);
@@ -630,8 +635,8 @@ __device__ __forceinline__ void planes_segment(const ShiftArgs &p, int ntile, in
         PlaneWalk w;
         const int FH = uniform(p.FH), FW = uniform(p.FW), x_plane = uniform(p.x_plane), x_row = uniform(p.x_row);
         const int k0 = uniform(g_begin) * NUM, ff = FH * FW;
-        const int ic = (int)div_by_uniform((uint32_t)k0, p.div_ff), rem = k0 - ic * ff;
-        w.fh = uniform((int)div_by_uniform((uint32_t)rem, p.div_fw));
+        const int ic = (int)div_by_uniform((uint32_t)k0, fast_div_of(p.div_ff)), rem = k0 - ic * ff;
+        w.fh = uniform((int)div_by_uniform((uint32_t)rem, fast_div_of(p.div_fw)));
         w.fw = uniform(rem - w.fh * FW);
         // byte offsets; row_step is the whole step of an fw wrap (the element step included)
         w.koff = uniform(4 * (ic * x_plane + w.fh * x_row + w.fw));
@@ -1154,18 +1159,31 @@ void shift_planes_wide_coop_kernel(const ShiftArgs p, const ShiftArgs p2)
     }
     for (int i = threadIdx.x; i < kCoopTileElems; i += THREADS) tile_sums[i] = 0;
     __syncthreads();
+    // Inside the loop the two argument blocks are read where they lie, in the kernel-argument segment, through
+    // a pointer that every iteration makes opaque again: what an iteration needs of them it loads (scalar loads
+    // that hit the scalar cache) instead of keeping several dozen values alive across the main loop, whose fixed
+    // register map leaves the compiler two dozen scalar registers -- it kept them in lanes of vector registers,
+    // 370 lane writes and reads per segment.
+    const KernargShiftArgs *ka = (const KernargShiftArgs *)__builtin_amdgcn_kernarg_segment_ptr();
     while (direct_rounds > 0 || it < it_end) {
+        asm volatile("" : "+s"(ka));
+        const KernargShiftArgs &pa = ka[0], &pb = ka[1];
+        const int pad = PAIR ? pa.coop_pad : 0;
+        const int len1 = pa.comm + pad, len2 = PAIR ? pb.comm + pad : 0;
+        const int span1 = pa.tiles_n * len1;
+        const int span = span1 + (PAIR ? pb.tiles_n * len2 : 0);
         // (One call of the segment code serves the direct tiles and the shared ones: a second copy of the
         // main loop in this kernel leaves the register allocator no room.)
         const bool direct = direct_rounds > 0;
         const long at = direct ? direct_at + (long)wave * len1 : shared_base + it;
         // (the launch's iterations stay below 2^31: 32-bit multiply-shift divisions)
-        const int mtile = (int)div_by_uniform((uint32_t)at, p.div_span);
+        const int mtile = (int)div_by_uniform((uint32_t)at, fast_div_of(pa.div_span));
         const int within = (int)(at - (long)mtile * span);
         const bool second = PAIR && within >= span1;
-        const int comm = second ? p2.comm : p.comm;
+        const int comm = second ? pb.comm : pa.comm;
         const int padded = comm + pad;
-        const int ntile = (int)div_by_uniform((uint32_t)(second ? within - span1 : within), second ? p2.div_len : p.div_len);
+        const int ntile = (int)div_by_uniform((uint32_t)(second ? within - span1 : within),
+                                              second ? fast_div_of(pb.div_len) : fast_div_of(pa.div_len));
         const long tile_start = (long)mtile * span + (second ? span1 : 0) + (long)ntile * padded;
         // position in the padded tile -> K groups [g0, g1)
         const int v0 = (int)(at - tile_start);
@@ -1183,8 +1201,8 @@ void shift_planes_wide_coop_kernel(const ShiftArgs p, const ShiftArgs p2)
         const int wb = direct ? 0 : g0 + wave * len / kCoopWaves;
         const int we = direct ? comm : g0 + (wave + 1) * len / kCoopWaves;
         if (wb < we) {
-            if (second) planes_segment<BITS, ZT, true, 1>(p2, ntile, m0, wb, we, false, tile_sums);
-            else planes_segment<BITS, ZT, true, (FUSED || PAIR) ? 1 : 2>(p, ntile, m0, wb, we, false,
+            if (second) planes_segment<BITS, ZT, true, 1>(pb, ntile, m0, wb, we, false, tile_sums);
+            else planes_segment<BITS, ZT, true, (FUSED || PAIR) ? 1 : 2>(pa, ntile, m0, wb, we, false,
                                                                         direct ? nullptr : tile_sums);
         }
         if (direct) {
