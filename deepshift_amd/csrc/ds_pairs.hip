@@ -95,6 +95,9 @@ static void derive_pair_geometry(PairArgs &a)
     a.koff_max = ff > 0 && a.K >= ff ? (a.K / ff - 1) * a.x_plane + (a.FH - 1) * a.x_row + a.FW - 1 : 0;
 }
 
+// A PairArgs block where a kernel finds it: in the kernel-argument segment (constant address space).
+typedef __attribute__((address_space(4))) const PairArgs KernargPairArgs;
+
 struct PairWalk {
     int koff, fw, fh, FW, FH, row_step, plane_step, koff_max;
 };
@@ -157,21 +160,23 @@ __device__ __forceinline__ int lane_now()
     return lane;
 }
 
-template <int BITS, int OUT, bool TU>
-__device__ __forceinline__ void pairs_segment(const PairArgs &p, int ntile, int m0, int g_begin, int g_end,
+// ARGS: PairArgs, or the same block read in place in the kernel-argument segment (KernargPairArgs).
+template <int BITS, int OUT, bool TU, typename ARGS = PairArgs>
+__device__ __forceinline__ void pairs_segment(const ARGS &p, int ntile, int m0, int g_begin, int g_end,
                                               int32_t *lds)
 {
     constexpr int NUM = 32 / (BITS + 1);
     const int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
 
     uint32_t xoff[6];
+    const FastDiv div_pix = fast_div_of(p.div_pix), div_ow = fast_div_of(p.div_ow);
 #pragma unroll
     for (int q = 0; q < 6; ++q) {
         int m = m0 + q * kWave + lane;
         if (m >= p.M) m = p.M - 1;
-        const int img = (int)div_by((uint32_t)m, p.div_pix);
+        const int img = (int)div_by((uint32_t)m, div_pix);
         const int rem = m - img * p.pix_per_img;
-        const int oh = (int)div_by((uint32_t)rem, p.div_ow);
+        const int oh = (int)div_by((uint32_t)rem, div_ow);
         const int ow = rem - oh * p.OW;
         xoff[q] = (uint32_t)(img * p.x_img_stride + oh * p.x_row_stride + ow * p.x_col_stride);
     }
@@ -188,8 +193,8 @@ __device__ __forceinline__ void pairs_segment(const PairArgs &p, int ntile, int 
         rsrc.w = 0x00020000;
         PairWalk w;
         const int k0 = g_begin * NUM, ff = p.FH * p.FW;
-        const int ic = (int)div_by_uniform((uint32_t)k0, p.div_ff), rem = k0 - ic * ff;
-        w.fh = (int)div_by_uniform((uint32_t)rem, p.div_fw);
+        const int ic = (int)div_by_uniform((uint32_t)k0, fast_div_of(p.div_ff)), rem = k0 - ic * ff;
+        w.fh = (int)div_by_uniform((uint32_t)rem, fast_div_of(p.div_fw));
         w.fw = rem - w.fh * p.FW;
         w.koff = ic * p.x_plane + w.fh * p.x_row + w.fw;
         w.FW = p.FW;
@@ -233,7 +238,7 @@ __device__ __forceinline__ void pairs_segment(const PairArgs &p, int ntile, int 
         const int m = m0 + q * kWave + lane;
         live[q] = m < p.M;
         const int mc = live[q] ? m : p.M - 1;
-        const int img = (int)div_by((uint32_t)mc, p.div_pix);
+        const int img = (int)div_by((uint32_t)mc, div_pix);
         yoff[q] = 4u * (uint32_t)(img * p.y_img_stride + (mc - img * p.pix_per_img));
     }
     const int n0 = ntile * 64;
@@ -645,15 +650,16 @@ __device__ __attribute__((noinline)) void pairs_finish_tile(lds_ptail *t, lds_i3
 struct PairSegment {
     int tile, g0, len, ntile, m0;
 };
-__device__ __forceinline__ PairSegment pairs_segment_at(const PairArgs &p, int it, int it_end)
+template <typename ARGS>
+__device__ __forceinline__ PairSegment pairs_segment_at(const ARGS &p, int it, int it_end)
 {
     PairSegment s;
-    s.tile = uniform((int)div_by_uniform((uint32_t)it, p.div_comm));
+    s.tile = uniform((int)div_by_uniform((uint32_t)it, fast_div_of(p.div_comm)));
     s.g0 = it - s.tile * p.comm;
     int g1 = s.g0 + (it_end - it);
     if (g1 > p.comm) g1 = p.comm;
     s.len = g1 - s.g0;
-    const int mt = uniform((int)div_by_uniform((uint32_t)s.tile, p.div_tiles_n));
+    const int mt = uniform((int)div_by_uniform((uint32_t)s.tile, fast_div_of(p.div_tiles_n)));
     s.ntile = s.tile - mt * p.tiles_n;
     s.m0 = mt * kPairPixels;
     return s;
@@ -699,7 +705,14 @@ void shift_pairs_fused_kernel(const PairArgs p)
     }
     for (int i = threadIdx.x; i < ELEMS; i += THREADS) tile_buf[i] = 0;
     __syncthreads();
+    // Inside the loop the argument block is read where it lies, in the kernel-argument segment, through a
+    // pointer that every iteration makes opaque again: an iteration loads what it needs (scalar loads that hit
+    // the scalar cache) instead of keeping the block's fields alive across the main loop in lanes of vector
+    // registers.
+    const KernargPairArgs *ka = (const KernargPairArgs *)__builtin_amdgcn_kernarg_segment_ptr();
     for (;;) {
+        asm volatile("" : "+s"(ka));
+        const KernargPairArgs &p = *ka;
         {
             const int it = uniform(cursor[0]), it_end = uniform(cursor[1]);
             if (it >= it_end) break;
