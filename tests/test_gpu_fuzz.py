@@ -161,3 +161,60 @@ def test_random_pair_launches(oracle, seed):
     if oa is not None:
         np.testing.assert_array_equal(oa.cpu().numpy(), va, err_msg=msg)
     np.testing.assert_array_equal(ob.cpu().numpy(), vb, err_msg=msg)
+
+
+@pytest.mark.parametrize("seed", range(36))
+def test_random_fused_launches(oracle, seed):
+    """Seeded random geometries through the fused entry points -- the 64-channel form, the narrow forms (16, 32, 40,
+    96, 160 channels: two-instruction and shift-plane loops) and the int8 kernel -- with random choices of what
+    follows the layer (residual, ReLU, float and / or fixed-point output, padding), against the oracle chain."""
+    from tests import test_gpu_fused as tf, test_gpu_pairs as tp
+    U = _lib.DS_BITS_TOP_UNUSED
+    rng = np.random.default_rng(3000 + seed)
+    kind = seed % 3
+    FH = int(rng.choice([1, 1, 3, 3, 5]))
+    FW = 1 if FH == 1 else int(rng.choice([1, 3]))
+    sh = int(rng.choice([1, 1, 2]))
+    stride = (sh, sh)
+    Nb, C = int(rng.integers(1, 7)), int(rng.choice([3, 7, 16, 32, 40, 64, 100]))
+    Hp, Wp = FH + int(rng.integers(4, 40)), FW + int(rng.integers(4, 40))
+    OH, OW = (Hp - FH) // sh + 1, (Wp - FW) // sh + 1
+    relu, use_res, want_float = (bool(rng.integers(0, 2)) for _ in range(3))
+    int8 = kind == 2
+    if int8:
+        O = int(rng.choice([64, 128, 256]))
+        form = int(rng.choice([1, 2, 3, 4, 1 | U, 2 | U]))
+        bits, F_in = form & 0xff, 5
+        x = tp.random_int8(rng, (Nb, C, Hp, Wp))
+        s, sign = random_codes(rng, (O, C, FH, FW), max_s=tp.top_field(form))
+        bias = rng.integers(-2 ** 8, 2 ** 8, size=O).astype(np.int32)
+        scale = (rng.random(O).astype(np.float32) + 0.5) * np.float32(2.0 ** -4)
+        fmt = (3, 5, torch.int8)
+    else:
+        O = int(rng.choice([64, 128, 192] if kind == 0 else [16, 32, 96, 160, 40]))
+        bits, unused, F_in = int(rng.choice([4, 4, 3, 2])), bool(rng.integers(0, 2)), 16
+        form = bits | (U if unused else 0)
+        x = random_activations(rng, (Nb, C, Hp, Wp))
+        s, sign = random_codes(rng, (O, C, FH, FW), max_s=2 ** bits - (2 if unused else 1))
+        bias = rng.integers(-2 ** 16, 2 ** 16, size=O).astype(np.int32)
+        scale = ((rng.random(O) + 0.5) * 2.0 ** -6).astype(np.float32)
+        fmt = (16, 16, torch.int32)
+    shift = rng.standard_normal(O).astype(np.float32)
+    res = (rng.standard_normal((Nb, O, OH, OW)) * 2).astype(np.float32) if use_res else None
+    emit = (int(rng.integers(0, 3)), int(rng.integers(0, 3))) + fmt if (rng.integers(0, 3) or not want_float) else None
+    want_float = want_float or emit is None
+    w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)
+    y = oracle.conv2d(x.astype(np.int32), -s, sign, bias, stride, nthreads=NTHREADS)
+    v = so.np_dequantize_affine(y, F_in, scale, shift, res, relu)
+    if int8:
+        blob = tp.abi_tile_paired(w, O, C, FH, FW, bits, form)
+        out, q = tp.abi_conv_paired_fused(x, blob, bias, O, FH, FW, stride, form, 128, F_in, scale, shift, res, relu,
+                                          want_float, emit)
+    else:
+        blob = kernels.tile_weights(dev(w).reshape(-1), O, C, FH, FW, bits, 0)
+        out, q = tf.abi_conv_fused(x, blob, bias, O, FH, FW, stride, form, F_in, scale, shift, res, relu, want_float, emit)
+    what = str((kind, Nb, C, Hp, Wp, O, FH, FW, sh, form, relu, use_res, want_float, emit))
+    if want_float:
+        np.testing.assert_array_equal(out, v, err_msg=what)
+    if emit is not None:
+        np.testing.assert_array_equal(q, so.np_requantize(v, emit[2], emit[3], emit[:2]), err_msg=what)
