@@ -49,18 +49,22 @@ __device__ __forceinline__ int coop_owner(long i, long G, long total) { return (
 
 typedef __attribute__((address_space(3))) int32_t lds_i32;
 
-// round_to_fixed + cast of the fused epilogue without branches: the clamp keeps the value inside int32,
-// so only NaN (propagated by the clamp, as torch.clamp does) needs the conversion's "NaN -> 0".
+// round_to_fixed + cast of the fused epilogue in four instructions: floor(v * scale), converted to int32 by
+// v_cvt_i32_f32 (saturating, NaN -> 0), then the clamp on integers (v_med3_i32).  lo and hi are integers within
+// int32 (make_spec), so clamping the saturated integer equals clamping the float and converting; a NaN becomes
+// 0, which lies between them, as in the conversion kernels.  (As float operations -- multiply, floor, max, min,
+// the "NaN -> 0" select, convert -- the same took seven.  v_cvt_flr_i32_f32 would fold the floor into the
+// conversion, but it turns a NaN into the largest integer.)
 template <bool ONE_BIT>
 __device__ __forceinline__ int32_t quantize_fixed_as(float v, float scale, float lo, float hi)
 {
-    // max / min drop a NaN operand; the select on v == v puts "NaN -> 0" back
-    float r = __builtin_fminf(__builtin_fmaxf(floorf(v * scale), lo), hi);
     if (ONE_BIT) {  // integer_bits == 1: sign(x) - 1 (utils.py:12-13)
         const float s = ((v > 0.0f) ? 1.0f : ((v < 0.0f) ? -1.0f : 0.0f)) - 1.0f;
-        r = s * scale;
+        return (int32_t)((v == v) ? s * scale : 0.0f);
     }
-    return (int32_t)((v == v) ? r : 0.0f);
+    int32_t q;
+    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(q) : "v"(f2i_sat(floorf(v * scale))), "v"((int32_t)lo), "v"((int32_t)hi));
+    return q;
 }
 
 __device__ __forceinline__ int32_t quantize_fixed(float v, float scale, float lo, float hi, bool one_bit)

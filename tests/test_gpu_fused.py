@@ -276,6 +276,37 @@ def test_narrow_plane_form_matches_oracle_chain(oracle, rng, case):
             np.testing.assert_array_equal(q2, want_q)
 
 
+@pytest.mark.parametrize("geom", [GEOMS[0], NARROW_GEOMS[0], NARROW_GEOMS[1]], ids=["64-channel", "16-channel", "32-channel"])
+def test_fused_round_to_fixed_saturates(oracle, rng, geom):
+    """Values beyond the fixed-point range clamp to its ends (utils.py:7-21), infinities included, and a NaN
+    (a broken BatchNorm constant) becomes 0 as in the conversion kernels: the epilogue converts with the
+    hardware's saturating floor conversion and clamps on integers."""
+    Nb, C, Hp, Wp, O, FH, FW, stride = geom
+    xp = rng.integers(-2 ** 17, 2 ** 19, size=(Nb, C, Hp, Wp)).astype(np.int32)
+    s, sign = random_codes(rng, (O, C, FH, FW), max_s=14)
+    y = oracle.conv2d(xp, -s, sign, None, stride, nthreads=NTHREADS)
+    blob = kernels.tile_weights(_dev(so.np_pack_words(s.reshape(O, -1), sign.reshape(O, -1), 4)).reshape(-1),
+                                O, C, FH, FW, 4, 0)
+    scale = (rng.choice([1e-3, 1.0, 3e4, 1e9], size=O) * rng.choice([-1.0, 1.0], size=O)).astype(np.float32)
+    shift = rng.standard_normal(O).astype(np.float32)
+    shift[1], shift[2], shift[3] = np.inf, -np.inf, np.nan
+    for I, F, dtype in ((16, 16, torch.int32), (12, 4, torch.int32), (3, 5, torch.int8)):
+        out, q = abi_conv_fused(xp, blob, None, O, FH, FW, stride, 4 | U, 16, scale, shift, None, False, True,
+                                (1, 1, I, F, dtype))
+        with np.errstate(invalid="ignore", over="ignore"):
+            v = so.np_dequantize_affine(y, 16, scale, shift, None, False)
+            finite = v.copy()
+            finite[:, 3] = 0.0
+            want = so.np_requantize(finite, I, F, (1, 1))
+        np.testing.assert_array_equal(out[:, :3], v[:, :3])
+        np.testing.assert_array_equal(out[:, 4:], v[:, 4:])
+        assert np.isnan(out[:, 3]).all()
+        np.testing.assert_array_equal(q, want)
+        hi, lo = (2 ** (I - 1) - 1) * 2 ** F, -2 ** (I - 1 + F)
+        assert (q[:, 1, 1:-1, 1:-1] == hi).all() and (q[:, 2, 1:-1, 1:-1] == lo).all() and (q[:, 3] == 0).all()
+        assert (q == hi).sum() > q[:, 1, 1:-1, 1:-1].size and (q == lo).sum() > q[:, 2, 1:-1, 1:-1].size
+
+
 def test_border_kept_writes_the_interior_only(oracle, rng):
     """q_bytes | DS_Q_BORDER_KEPT: the caller's buffer keeps its padding (zeroed once by the caller), the
     kernel overwrites the interior; with the flag off the kernel writes the padding itself."""
