@@ -142,6 +142,17 @@ __device__ __forceinline__ bool coop_arrive(unsigned long long *counter, unsigne
     }
 }
 
+// True when every one of a shared tile's `others` other contributors has arrived already: the caller is then
+// the tile's last contributor whatever it does, needs no slot of its own and no arrival -- it adds the others'
+// slots to the sums it still holds and, having read them, leaves the counter as a finished tile does (0).  A
+// count that is not complete yet says nothing (the caller goes the ordinary way).  The same observation as the
+// last arrival's compare-and-swap makes, by an agent-scope load.
+__device__ __forceinline__ bool coop_others_all_arrived(unsigned long long *counter, unsigned long long token, int others)
+{
+    const unsigned long long seen = __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return (seen >> 16) == token && (int)(seen & 0xffff) == others;
+}
+
 // A tag no earlier launch of this process has used: 48 bits, never 0, from a counter that starts at
 // a value drawn from the clock (so that words left by another process are no likelier to match than
 // any other garbage).

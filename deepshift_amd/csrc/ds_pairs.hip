@@ -605,23 +605,36 @@ __device__ __attribute__((noinline)) void pairs_finish_tile(lds_ptail *t, lds_i3
     bool finish = len == comm;
     if (!finish) {
         g_i32 *slots = uniform_global(t->slots);
-        // slot 0 of a workgroup holds the tile its share starts in (g0 > 0), slot 1 the tile it ends in
-        g_i32 *slot = slots + ((size_t)2 * w + (g0 > 0 ? 0 : 1)) * ELEMS + tid;
-#pragma unroll
-        for (int k = 0; k < PER; ++k) {
-            store_agent(slot + k * THREADS, buf[tid + k * THREADS]);
-            buf[tid + k * THREADS] = 0;
-        }
-        // the slot is complete (every store acknowledged) before the arrival is counted
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
         const long G = uniform(t->G), total = uniform(t->total);
         const int first = coop_owner(tile_start, G, total);
         const int last = coop_owner(tile_start + comm - 1, G, total);
-        if (tid == 0) *flag = coop_arrive(t->counters + first, t->token, last - first);
-        __syncthreads();
-        if (*flag) {
+        // The tile a share ENDS in (g0 == 0): the workgroups that hold the rest of it ran it first thing and have
+        // as a rule published their parts long ago; one look at the counter then saves this workgroup its own
+        // slot, the wait for the stores and the arrival (as in the int32 kernel's coop_finish_tile).
+        bool skip_own = false;
+        if (g0 == 0) {
+            if (tid == 0) *flag = coop_others_all_arrived(t->counters + first, t->token, last - first);
+            __syncthreads();
+            skip_own = *flag != 0;
+            __syncthreads();  // (everybody has read the flag before anybody writes it again)
+        }
+        if (!skip_own) {
+            // slot 0 of a workgroup holds the tile its share starts in (g0 > 0), slot 1 the tile it ends in
+            g_i32 *slot = slots + ((size_t)2 * w + (g0 > 0 ? 0 : 1)) * ELEMS + tid;
+#pragma unroll
+            for (int k = 0; k < PER; ++k) {
+                store_agent(slot + k * THREADS, buf[tid + k * THREADS]);
+                buf[tid + k * THREADS] = 0;
+            }
+            // the slot is complete (every store acknowledged) before the arrival is counted
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (tid == 0) *flag = coop_arrive(t->counters + first, t->token, last - first);
+            __syncthreads();
+        }
+        if (skip_own || *flag) {
             for (int c = first; c <= last; ++c) {
+                if (skip_own && c == w) continue;  // this workgroup's part is still in the buffer
                 const g_i32 *src = slots + ((size_t)2 * c + (c == first ? 1 : 0)) * ELEMS + tid;
                 int32_t v[PER];
 #pragma unroll
@@ -629,6 +642,9 @@ __device__ __attribute__((noinline)) void pairs_finish_tile(lds_ptail *t, lds_i3
 #pragma unroll
                 for (int k = 0; k < PER; ++k) buf[tid + k * THREADS] += v[k];
             }
+            // (the counter is left as a finished tile leaves it: a replay of the launch starts clean)
+            if (skip_own && tid == 0)
+                __hip_atomic_store(t->counters + first, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             finish = true;
         }
         __syncthreads();

@@ -1050,24 +1050,39 @@ __device__ __attribute__((noinline)) void coop_finish_tile(lds_tail *t, lds_i32 
     bool finish = len == comm;
     if (!finish) {
         g_i32 *slots = uniform_global(t->slots);
-        // slot 0 of a workgroup holds the tile its share starts in (g0 > 0), slot 1 the tile it ends in
-        g_i32 *slot = slots + ((size_t)2 * w + (g0 > 0 ? 0 : 1)) * kCoopTileElems + threadIdx.x;
-#pragma unroll
-        for (int k = 0; k < PER; ++k) {
-            store_agent(slot + k * THREADS, buf[threadIdx.x + k * THREADS]);
-            buf[threadIdx.x + k * THREADS] = 0;
-        }
-        // the slot is complete (every store acknowledged) before the arrival is counted
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
         const long G = uniform(t->G), total = uniform(t->total);
         // tile_start: the tile's first iteration in the launch's (tile, K group) space
         const int first = coop_owner(tile_start, G, total);
         const int last = coop_owner(tile_start + comm - 1, G, total);
-        if (threadIdx.x == 0) *flag = coop_arrive(t->counters + first, t->token, last - first);
-        __syncthreads();
-        if (*flag) {
+        // The tile a share ENDS in (g0 == 0: the share holds the tile's first K groups, the following workgroups
+        // the rest, and for them it is the tile their shares START in, which they ran first thing): by the time
+        // this workgroup gets there, at the end of its share, the others have as a rule published their parts
+        // long ago.  One look at the counter then saves this workgroup its own slot, the wait for the stores
+        // and the arrival -- at the very end of the launch, where nothing else hides them.
+        bool skip_own = false;
+        if (g0 == 0) {
+            if (threadIdx.x == 0) *flag = coop_others_all_arrived(t->counters + first, t->token, last - first);
+            __syncthreads();
+            skip_own = *flag != 0;
+            __syncthreads();  // (everybody has read the flag before anybody writes it again)
+        }
+        if (!skip_own) {
+            // slot 0 of a workgroup holds the tile its share starts in (g0 > 0), slot 1 the tile it ends in
+            g_i32 *slot = slots + ((size_t)2 * w + (g0 > 0 ? 0 : 1)) * kCoopTileElems + threadIdx.x;
+#pragma unroll
+            for (int k = 0; k < PER; ++k) {
+                store_agent(slot + k * THREADS, buf[threadIdx.x + k * THREADS]);
+                buf[threadIdx.x + k * THREADS] = 0;
+            }
+            // the slot is complete (every store acknowledged) before the arrival is counted
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (threadIdx.x == 0) *flag = coop_arrive(t->counters + first, t->token, last - first);
+            __syncthreads();
+        }
+        if (skip_own || *flag) {
             for (int c = first; c <= last; ++c) {
+                if (skip_own && c == w) continue;  // this workgroup's part is still in the buffer
                 const g_i32 *src = slots + ((size_t)2 * c + (c == first ? 1 : 0)) * kCoopTileElems + threadIdx.x;
                 int32_t v[PER];
 #pragma unroll
@@ -1075,6 +1090,9 @@ __device__ __attribute__((noinline)) void coop_finish_tile(lds_tail *t, lds_i32 
 #pragma unroll
                 for (int k = 0; k < PER; ++k) buf[threadIdx.x + k * THREADS] += v[k];
             }
+            // (the counter is left as a finished tile leaves it: a replay of the launch starts clean)
+            if (skip_own && threadIdx.x == 0)
+                __hip_atomic_store(t->counters + first, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             finish = true;
         }
         __syncthreads();
