@@ -77,13 +77,14 @@ __device__ __forceinline__ int32_t quantize_fixed(float v, float scale, float lo
 // selecting per element.
 template <int CH, int R, bool HAS_RES, bool RELU>
 __device__ __forceinline__ void tile_affine(float (&f)[CH][R], const int32_t (&sums)[CH][R], const float (&res)[CH][R],
-                                            int32_t add_l, float sa_l, float sb_l, float inv)
+                                            int32_t add_l, float sa_l, float sb_l, float inv, int first = 0)
 {
+    // (lane first + c holds the constants of channel c)
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
-        const int32_t add = __builtin_amdgcn_readlane(add_l, c);
-        const float sa = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sa_l), c));
-        const float sb = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sb_l), c));
+        const int32_t add = __builtin_amdgcn_readlane(add_l, first + c);
+        const float sa = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sa_l), first + c));
+        const float sb = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, sb_l), first + c));
 #pragma unroll
         for (int r = 0; r < R; ++r) {
 #pragma clang fp contract(off)

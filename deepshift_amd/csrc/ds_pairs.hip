@@ -148,7 +148,11 @@ DS_PAIRS_ONE(4, false, DS_PAIRX_ASM_B4, DS_PAIRX_CLOBBERS_B4)
 // they are, two pixels per word, kLdsPacked (add to lds[channel][row][lane]: the sum of such words is
 // the word of the sums as long as every 16-bit half stays in range, i.e. while the reduction indices
 // that all the waves of the workgroup add up for one tile fit one chunk).
-enum { kStore, kAtomic, kLds, kLdsPacked };
+// kLdsThree: three sums per 64-bit word, s0 + s1 * 2^21 + s2 * 2^42 (the lane's six pixels of a channel in two
+// words, lds[channel][2][lane]): again the sum of such words is the word of the sums, here as long as every
+// sum stays within 21 bits, sign included -- reductions of thousands of indices at two thirds of the widened
+// buffer's size.
+enum { kStore, kAtomic, kLds, kLdsPacked, kLdsThree };
 
 // The lane number, computed where it is called (volatile: not merged with an earlier computation): after
 // the main loop, whose fixed register map leaves eight vector registers free, so that no lane number has
@@ -214,6 +218,24 @@ __device__ __forceinline__ void pairs_segment(const ARGS &p, int ntile, int m0, 
 #pragma unroll
             for (int r = 0; r < kPairRows; ++r)
                 atomicAdd(lds + j * (kPairRows * kWave) + r * kWave + lane, a[2 * r + j / 32][j % 32]);
+        return;
+    }
+    if (OUT == kLdsThree) {
+        const int lane = lane_now();
+        unsigned long long *l64 = (unsigned long long *)lds;
+#pragma unroll
+        for (int j = 0; j < 64; ++j) {
+            long long s[6];  // the lane's pixels in the tile's block order: row r holds blocks 2r (low half), 2r + 1
+#pragma unroll
+            for (int r = 0; r < kPairRows; ++r) {
+                const int32_t v = a[2 * r + j / 32][j % 32];
+                const int32_t lo = (int32_t)(int16_t)(v & 0xffff), hi = (v - lo) >> 16;
+                s[2 * r] = lo;
+                s[2 * r + 1] = hi;
+            }
+            atomicAdd(l64 + (j * 2 + 0) * kWave + lane, (unsigned long long)(s[0] + (s[1] << 21) + (s[2] << 42)));
+            atomicAdd(l64 + (j * 2 + 1) * kWave + lane, (unsigned long long)(s[3] + (s[4] << 21) + (s[5] << 42)));
+        }
         return;
     }
     // split the sums into their halves (v = hi * 65536 + lo) and add them to the output
@@ -340,7 +362,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int i = threadIdx.x; i < 64 * kPairPixels; i += 512) tile_sums[i] = 0;
         __syncthreads();
         const int len = g1 - g0;
-        const int wb = g0 + wave * len / kPairCuWaves, we = g0 + (wave + 1) * len / kPairCuWaves;
+        // (equal parts; the groups left over go one each to waves 0, 1, ..: the first four sit on different
+        // vector units)
+        const int part = len / kPairCuWaves, extra = len % kPairCuWaves;
+        const int wb = g0 + wave * part + (wave < extra ? wave : extra), we = wb + part + (wave < extra ? 1 : 0);
         for (int g = wb; g < we; g += p.chunk) {
             const int ge = g + p.chunk < we ? g + p.chunk : we;
             pairs_segment<BITS, kLds, TU>(p, ntile, m0, g, ge, tile_sums);
@@ -431,9 +456,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // slot in the workspace, its arrival counted, and the workgroup that arrives LAST at the tile adds the
 // other contributors' slots and writes it.  No pre-fill of an output, no global atomics on it, no int32
 // sums in memory, no separate conversion pass, and nobody waits for anybody.
-// PACKED: reductions of a single chunk on workgroups of four waves, the buffer holds two pixels per word
-// as the registers do (48 KiB, two workgroups per compute unit); otherwise eight waves on widened sums
-// (96 KiB, one workgroup per compute unit).
+// Three forms of the tile buffer (FORM): kTilePacked, reductions of a single chunk on workgroups of four waves,
+// the buffer holds two pixels per word as the registers do (48 KiB, two workgroups per compute unit);
+// kTileThree, reductions whose sums stay within 21 bits, four waves, three sums per 64-bit word (64 KiB, two
+// workgroups per compute unit: one's tile tail and barrier waits run beside the other's main loop);
+// kTileWide, anything longer, eight waves on widened sums (96 KiB, one workgroup per compute unit).
+enum { kTileWide, kTilePacked, kTileThree };
+constexpr int pair_tile_waves(int form) { return form == kTileWide ? 8 : 4; }
+constexpr int pair_tile_words(int form)  // 32-bit words of the buffer (and of a slot in the workspace)
+{
+    return form == kTilePacked ? 64 * 3 * kWave : form == kTileThree ? 64 * 4 * kWave : 64 * 6 * kWave;
+}
 struct PairTail {
     const int32_t *negcnt, *bias;
     int32_t *slots;
@@ -451,25 +484,27 @@ struct PairTail {
 };
 typedef __attribute__((address_space(3))) const PairTail lds_ptail;
 
-// channels that one call of pairs_write_unit finishes: 4 x 6 blocks = 24 outputs per lane keep the tail
-// function within the registers it need not save (with 8 it saved and restored 61 registers through scratch
-// memory on every call: 100 MB of extra traffic per launch of a ResNet-50 3x3 layer)
+// channels per step of pairs_write_tile: 4 x 6 blocks = 24 outputs per lane
 constexpr int kPairUnit = 4;
 
-// kPairUnit channels x the tile's six 64-pixel blocks (24 outputs per lane) leave the tile buffer: bias (and,
-// for the xor-mask forms, the count of negative codes for the pixels that lived in low halves), then the
-// arithmetic of the int32 kernel's write_tile in the same order.  Everything that comes from memory is
-// requested up front: the per-channel constants by the lanes (lane c holds those of channel ch0 + c and
-// hands them out with v_readlane), the residuals of all 24 outputs before the first is used.
-template <typename Q, bool PACKED>
-__device__ __forceinline__ void pairs_write_unit(lds_ptail *t, lds_i32 *buf, int ntile, int m0, int ch0, int lane)
+// One wave's channels of a finished tile (64 / WAVES of them x the tile's six 64-pixel blocks) leave the tile
+// buffer: bias (and, for the xor-mask forms, the count of negative codes for the pixels that lived in low
+// halves), then the arithmetic of the int32 kernel's write_tile in the same order, kPairUnit channels (24
+// outputs per lane) at a time.  What comes from memory is asked for ahead of its use: the per-channel constants
+// of all the wave's channels once, by the lanes (lane c holds those of the wave's channel c and hands them out
+// with v_readlane), the residuals of a step before the step ahead of it is computed and its stores are issued.
+template <typename Q, int FORM>
+__device__ __forceinline__ void pairs_write_tile(lds_ptail *t, lds_i32 *buf, int ntile, int m0, int wave, int lane)
 {
     typedef __attribute__((address_space(1))) Q g_q;
     typedef __attribute__((address_space(1))) char g_char;
-    constexpr int CH = kPairUnit, PB = 6;
+    typedef __attribute__((address_space(3))) long long lds_i64;
+    constexpr int WAVES = pair_tile_waves(FORM);
+    constexpr int CH = kPairUnit, PB = 6, WCH = 64 / WAVES, UNITS = WCH / CH;
     const int M = uniform(t->M), N = uniform(t->N), pix_per_img = uniform(t->pix_per_img), OW = uniform(t->OW);
-    const int n0 = ntile * 64 + ch0;
-    const int mine = n0 + (lane & (CH - 1));
+    const int ch_base = wave * WCH;
+    const int n0 = ntile * 64 + ch_base;
+    const int mine = n0 + (lane & (WCH - 1));
     const g_i32 *negcnt = uniform_global(t->negcnt), *bias = uniform_global(t->bias);
     const int32_t add_l = bias ? bias[mine] : 0;
     const int32_t neg_l = negcnt ? negcnt[mine] : 0;
@@ -488,87 +523,107 @@ __device__ __forceinline__ void pairs_write_unit(lds_ptail *t, lds_i32 *buf, int
                          (uint32_t)uniform((int32_t)t->div_ow.s1), (uint32_t)uniform((int32_t)t->div_ow.s2)};
     const int Wq = OW + 2 * pw;
     const uint32_t qplane = (uint32_t)(OH + 2 * ph) * Wq;
+    const uint32_t ostep = 4u * (uint32_t)pix_per_img, qstep = (uint32_t)sizeof(Q) * qplane;
     bool live[PB];
-    uint32_t pix[PB], qpix[PB], qimg[PB];  // element indices (every tensor is below 2^31 bytes)
-    int oh[PB], ow[PB];
+    uint32_t pix[PB], qpix[PB];  // element indices of the wave's first channel (every tensor is below 2^31 bytes)
 #pragma unroll
     for (int b = 0; b < PB; ++b) {
         const int m = m0 + b * kWave + lane;
         live[b] = m < M;
         const int mm = live[b] ? m : 0;
         const int img = (int)div_by((uint32_t)mm, div_pix), rem = mm - img * pix_per_img;
-        oh[b] = (int)div_by((uint32_t)rem, div_ow);
-        ow[b] = rem - oh[b] * OW;
+        const int oh = (int)div_by((uint32_t)rem, div_ow), ow = rem - oh * OW;
         pix[b] = (uint32_t)(img * N + n0) * (uint32_t)pix_per_img + rem;
-        qimg[b] = (uint32_t)(img * N + n0) * qplane;
-        qpix[b] = qimg[b] + (uint32_t)(oh[b] + ph) * Wq + ow[b] + pw;
-    }
-    float res[CH][PB];
-    if (residual) {
-#pragma unroll
-        for (int b = 0; b < PB; ++b) {
-            if (live[b]) {
-#pragma unroll
-                for (int c = 0; c < CH; ++c)
-                    res[c][b] = *(const g_f32 *)((const g_char *)residual + 4u * (pix[b] + (uint32_t)(c * pix_per_img)));
-            } else {
-#pragma unroll
-                for (int c = 0; c < CH; ++c) res[c][b] = 0.0f;
-            }
-        }
-    }
-    int32_t sums[CH][PB];
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        const int32_t neg = __builtin_amdgcn_readlane(neg_l, c);
-        if (PACKED) {
-#pragma unroll
-            for (int r = 0; r < kPairRows; ++r) {
-                lds_i32 *cell = buf + (ch0 + c) * (kPairRows * kWave) + r * kWave + lane;
-                const int32_t v = *cell;
-                *cell = 0;
-                const int32_t lo = (int32_t)(int16_t)(v & 0xffff), hi = (v - lo) >> 16;
-                sums[c][2 * r] = lo + neg;
-                sums[c][2 * r + 1] = hi;
-            }
-        } else {
-#pragma unroll
-            for (int b = 0; b < PB; ++b) {
-                lds_i32 *cell = buf + (ch0 + c) * kPairPixels + b * kWave + lane;
-                sums[c][b] = *cell + ((b & 1) ? 0 : neg);
-                *cell = 0;
-            }
-        }
+        qpix[b] = (uint32_t)(img * N + n0) * qplane + (uint32_t)(oh + ph) * Wq + ow + pw;
     }
     const float inv = uniform(t->inv), qs = uniform(t->spec.scale), qlo = uniform(t->spec.lo), qhi = uniform(t->spec.hi);
     const bool relu = uniform(t->relu) != 0, one_bit = uniform(t->spec.I) == 1, has_res = residual != nullptr;
-    float f[CH][PB];
-    if (has_res) {
-        if (relu) tile_affine<CH, PB, true, true>(f, sums, res, add_l, sa_l, sb_l, inv);
-        else tile_affine<CH, PB, true, false>(f, sums, res, add_l, sa_l, sb_l, inv);
-    } else {
-        if (relu) tile_affine<CH, PB, false, true>(f, sums, res, add_l, sa_l, sb_l, inv);
-        else tile_affine<CH, PB, false, false>(f, sums, res, add_l, sa_l, sb_l, inv);
-    }
-    const uint32_t ostep = 4u * (uint32_t)pix_per_img, qstep = (uint32_t)sizeof(Q) * qplane;
+    float res[2][CH][PB];
+    auto load_residuals = [&](int u, float (&r)[CH][PB]) {
 #pragma unroll
-    for (int b = 0; b < PB; ++b) {
-        if (!live[b]) continue;
-        if (out) {
-            uint32_t o = 4u * pix[b];
+        for (int b = 0; b < PB; ++b) {
+            if (live[b]) {
+                const g_char *at = (const g_char *)residual + 4u * pix[b] + (uint32_t)(u * CH) * ostep;
 #pragma unroll
-            for (int c = 0; c < CH; ++c, o += ostep) *(g_f32 *)(out + o) = f[c][b];
-        }
-        if (q) {
-            uint32_t o = (uint32_t)sizeof(Q) * qpix[b];
-            if (one_bit) {
-#pragma unroll
-                for (int c = 0; c < CH; ++c, o += qstep)
-                    *(g_q *)(q + o) = (Q)quantize_fixed_as<true>(f[c][b], qs, qlo, qhi);
+                for (int c = 0; c < CH; ++c) r[c][b] = *(const g_f32 *)(at + (uint32_t)c * ostep);
             } else {
 #pragma unroll
-                for (int c = 0; c < CH; ++c, o += qstep)
-                    *(g_q *)(q + o) = (Q)quantize_fixed_as<false>(f[c][b], qs, qlo, qhi);
+                for (int c = 0; c < CH; ++c) r[c][b] = 0.0f;
+            }
+        }
+    };
+    if (has_res) load_residuals(0, res[0]);
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u) {
+        if (has_res && u + 1 < UNITS) load_residuals(u + 1, res[(u + 1) & 1]);
+        int32_t sums[CH][PB];
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int32_t neg = __builtin_amdgcn_readlane(neg_l, u * CH + c);
+            const int ch = ch_base + u * CH + c;
+            if (FORM == kTileThree) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    lds_i64 *cell = (lds_i64 *)buf + (ch * 2 + h) * kWave + lane;
+                    long long v = *cell;
+                    *cell = 0;
+                    // s0 + s1 * 2^21 + s2 * 2^42, every sum within 21 bits: take the lowest, sign-extended, off
+                    const int32_t s0 = (int32_t)((v << 43) >> 43);
+                    v = (v - s0) >> 21;
+                    const int32_t s1 = (int32_t)((v << 43) >> 43);
+                    const int32_t s2 = (int32_t)((v - s1) >> 21);
+                    // (pixels that lived in low halves: the even blocks)
+                    sums[c][3 * h] = s0 + (h == 0 ? neg : 0);
+                    sums[c][3 * h + 1] = s1 + (h == 1 ? neg : 0);
+                    sums[c][3 * h + 2] = s2 + (h == 0 ? neg : 0);
+                }
+            } else if (FORM == kTilePacked) {
+#pragma unroll
+                for (int r = 0; r < kPairRows; ++r) {
+                    lds_i32 *cell = buf + ch * (kPairRows * kWave) + r * kWave + lane;
+                    const int32_t v = *cell;
+                    *cell = 0;
+                    const int32_t lo = (int32_t)(int16_t)(v & 0xffff), hi = (v - lo) >> 16;
+                    sums[c][2 * r] = lo + neg;
+                    sums[c][2 * r + 1] = hi;
+                }
+            } else {
+#pragma unroll
+                for (int b = 0; b < PB; ++b) {
+                    lds_i32 *cell = buf + ch * kPairPixels + b * kWave + lane;
+                    sums[c][b] = *cell + ((b & 1) ? 0 : neg);
+                    *cell = 0;
+                }
+            }
+        }
+        float f[CH][PB];
+        const float (&r)[CH][PB] = res[u & 1];
+        if (has_res) {
+            if (relu) tile_affine<CH, PB, true, true>(f, sums, r, add_l, sa_l, sb_l, inv, u * CH);
+            else tile_affine<CH, PB, true, false>(f, sums, r, add_l, sa_l, sb_l, inv, u * CH);
+        } else {
+            if (relu) tile_affine<CH, PB, false, true>(f, sums, r, add_l, sa_l, sb_l, inv, u * CH);
+            else tile_affine<CH, PB, false, false>(f, sums, r, add_l, sa_l, sb_l, inv, u * CH);
+        }
+#pragma unroll
+        for (int b = 0; b < PB; ++b) {
+            if (!live[b]) continue;
+            if (out) {
+                uint32_t o = 4u * pix[b] + (uint32_t)(u * CH) * ostep;
+#pragma unroll
+                for (int c = 0; c < CH; ++c, o += ostep) *(g_f32 *)(out + o) = f[c][b];
+            }
+            if (q) {
+                uint32_t o = (uint32_t)sizeof(Q) * qpix[b] + (uint32_t)(u * CH) * qstep;
+                if (one_bit) {
+#pragma unroll
+                    for (int c = 0; c < CH; ++c, o += qstep)
+                        *(g_q *)(q + o) = (Q)quantize_fixed_as<true>(f[c][b], qs, qlo, qhi);
+                } else {
+#pragma unroll
+                    for (int c = 0; c < CH; ++c, o += qstep)
+                        *(g_q *)(q + o) = (Q)quantize_fixed_as<false>(f[c][b], qs, qlo, qhi);
+                }
             }
         }
     }
@@ -577,9 +632,13 @@ __device__ __forceinline__ void pairs_write_unit(lds_ptail *t, lds_i32 *buf, int
 #pragma unroll
         for (int b = 0; b < PB; ++b) {
             if (!live[b]) continue;
-            if (!(ow[b] == 0 || ow[b] == OW - 1 || oh[b] == 0 || oh[b] == OH - 1)) continue;
-            for (int c = 0; c < CH; ++c)
-                write_padding(qg, (size_t)qimg[b] + (size_t)c * qplane, oh[b], ow[b], OH, OW, ph, pw, Wq);
+            const int m = m0 + b * kWave + lane;
+            const int img = (int)div_by((uint32_t)m, div_pix), rem = m - img * pix_per_img;
+            const int oh = (int)div_by((uint32_t)rem, div_ow), ow = rem - oh * OW;
+            if (!(ow == 0 || ow == OW - 1 || oh == 0 || oh == OH - 1)) continue;
+            const size_t qimg = (size_t)((uint32_t)(img * N + n0) * qplane);
+            for (int c = 0; c < WCH; ++c)
+                write_padding(qg, qimg + (size_t)c * qplane, oh, ow, OH, OW, ph, pw, Wq);
         }
     }
 }
@@ -589,14 +648,18 @@ __device__ __forceinline__ void pairs_write_unit(lds_ptail *t, lds_i32 *buf, int
 // map).  A whole tile (len == comm) is written out.  A partial one is published to this workgroup's slot,
 // its arrival counted, and whichever workgroup arrives last gathers the slots of all contributors and
 // writes the tile.  Ends with the buffer cleared and a barrier.
-template <bool PACKED>
+template <int FORM>
 __device__ __attribute__((noinline)) void pairs_finish_tile(lds_ptail *t, lds_i32 *buf, lds_i32 *flag, int w,
                                                             long tile_start, int g0, int len, int ntile, int m0,
                                                             int wave)
 {
-    constexpr int WAVES = PACKED ? kPairCu4Waves : kPairCuWaves, THREADS = WAVES * kWave;
-    constexpr int ELEMS = PACKED ? 64 * kPairRows * kWave : 64 * kPairPixels, PER = ELEMS / THREADS;
-    constexpr int UNITS = 64 / kPairUnit / WAVES;  // units of kPairUnit channels per wave
+    // (the buffer's elements as they are added: 64-bit words where a word holds three sums)
+    typedef typename std::conditional<FORM == kTileThree, long long, int32_t>::type elem_t;
+    typedef __attribute__((address_space(3))) elem_t lds_elem;
+    typedef __attribute__((address_space(1))) elem_t g_elem;
+    constexpr int WAVES = pair_tile_waves(FORM), THREADS = WAVES * kWave;
+    constexpr int ELEMS = pair_tile_words(FORM) * 4 / (int)sizeof(elem_t), PER = ELEMS / THREADS;
+    lds_elem *ebuf = (lds_elem *)buf;
     // (the thread's number from the wave's, which the caller holds in a scalar register, and the lane's:
     // no work-item id has to stay in a vector register across the caller's main loop)
     const int lane = lane_now();
@@ -620,11 +683,11 @@ __device__ __attribute__((noinline)) void pairs_finish_tile(lds_ptail *t, lds_i3
         }
         if (!skip_own) {
             // slot 0 of a workgroup holds the tile its share starts in (g0 > 0), slot 1 the tile it ends in
-            g_i32 *slot = slots + ((size_t)2 * w + (g0 > 0 ? 0 : 1)) * ELEMS + tid;
+            g_elem *slot = (g_elem *)slots + ((size_t)2 * w + (g0 > 0 ? 0 : 1)) * ELEMS + tid;
 #pragma unroll
             for (int k = 0; k < PER; ++k) {
-                store_agent(slot + k * THREADS, buf[tid + k * THREADS]);
-                buf[tid + k * THREADS] = 0;
+                __hip_atomic_store(slot + k * THREADS, ebuf[tid + k * THREADS], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                ebuf[tid + k * THREADS] = 0;
             }
             // the slot is complete (every store acknowledged) before the arrival is counted
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -635,12 +698,13 @@ __device__ __attribute__((noinline)) void pairs_finish_tile(lds_ptail *t, lds_i3
         if (skip_own || *flag) {
             for (int c = first; c <= last; ++c) {
                 if (skip_own && c == w) continue;  // this workgroup's part is still in the buffer
-                const g_i32 *src = slots + ((size_t)2 * c + (c == first ? 1 : 0)) * ELEMS + tid;
-                int32_t v[PER];
+                const g_elem *src = (const g_elem *)slots + ((size_t)2 * c + (c == first ? 1 : 0)) * ELEMS + tid;
+                elem_t v[PER];
 #pragma unroll
-                for (int k = 0; k < PER; ++k) v[k] = load_agent(src + k * THREADS);
+                for (int k = 0; k < PER; ++k)
+                    v[k] = __hip_atomic_load(src + k * THREADS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
-                for (int k = 0; k < PER; ++k) buf[tid + k * THREADS] += v[k];
+                for (int k = 0; k < PER; ++k) ebuf[tid + k * THREADS] += v[k];
             }
             // (the counter is left as a finished tile leaves it: a replay of the launch starts clean)
             if (skip_own && tid == 0)
@@ -650,13 +714,8 @@ __device__ __attribute__((noinline)) void pairs_finish_tile(lds_ptail *t, lds_i3
         __syncthreads();
     }
     if (finish) {
-        const bool q8 = uniform(t->q_bytes) == 1;
-#pragma unroll
-        for (int u = 0; u < UNITS; ++u) {
-            const int ch0 = (wave * UNITS + u) * kPairUnit;
-            if (q8) pairs_write_unit<int8_t, PACKED>(t, buf, ntile, m0, ch0, lane);
-            else pairs_write_unit<int32_t, PACKED>(t, buf, ntile, m0, ch0, lane);
-        }
+        if (uniform(t->q_bytes) == 1) pairs_write_tile<int8_t, FORM>(t, buf, ntile, m0, wave, lane);
+        else pairs_write_tile<int32_t, FORM>(t, buf, ntile, m0, wave, lane);
     }
     __syncthreads();
 }
@@ -681,18 +740,19 @@ __device__ __forceinline__ PairSegment pairs_segment_at(const ARGS &p, int it, i
     return s;
 }
 
-template <int BITS, bool TU, bool PACKED>
-__global__ __launch_bounds__(PACKED ? 256 : 512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+template <int BITS, bool TU, int FORM>
+__global__ __launch_bounds__(pair_tile_waves(FORM) * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void shift_pairs_fused_kernel(const PairArgs p)
 {
-    extern __shared__ int32_t tile_buf[];  // [64][384] sums, or [64][3][64] words of two sums (PACKED)
+    // [64][384] sums, [64][3][64] words of two sums (kTilePacked) or [64][2][64] 64-bit words of three (kTileThree)
+    extern __shared__ __attribute__((aligned(8))) int32_t tile_buf[];
     __shared__ PairTail tail;
     __shared__ int32_t last_arrival;
     // The share's position lives in LDS, not in registers: the main loop's fixed register map leaves the
     // compiler a handful of scalar registers, and what is live across it must not need spilling.
     __shared__ int32_t cursor[2];
-    constexpr int WAVES = PACKED ? kPairCu4Waves : kPairCuWaves, THREADS = WAVES * kWave;
-    constexpr int ELEMS = PACKED ? 64 * kPairRows * kWave : 64 * kPairPixels;
+    constexpr int WAVES = pair_tile_waves(FORM), THREADS = WAVES * kWave;
+    constexpr int ELEMS = pair_tile_words(FORM);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (threadIdx.x == 0) {
         const long G = gridDim.x;
@@ -733,14 +793,23 @@ void shift_pairs_fused_kernel(const PairArgs p)
             const int it = uniform(cursor[0]), it_end = uniform(cursor[1]);
             if (it >= it_end) break;
             const PairSegment s = pairs_segment_at(p, it, it_end);
-            const int wb = s.g0 + wave * s.len / WAVES, we = s.g0 + (wave + 1) * s.len / WAVES;
-            if (PACKED) {
+            // The segment's K groups go to the waves in equal parts; the groups left over, one each, to the waves
+            // of the lowest rank.  Eight waves sit two to a vector unit (wave w and w + 4): ranks in wave order
+            // put the first four extra groups on four different units (the proportional cut wave * len / 8 gave
+            // two left-over groups to waves 3 and 7 -- one unit -- and everybody waited for it at the barrier).
+            // Four waves share their units with the waves of the compute unit's other workgroup: the ranks
+            // rotate with the tile, so that the two workgroups' extra groups meet on one unit only now and then.
+            const int rank = WAVES == 4 ? ((wave + s.tile) & (WAVES - 1)) : wave;
+            const int part = s.len / WAVES, extra = s.len % WAVES;
+            const int wb = s.g0 + rank * part + (rank < extra ? rank : extra);
+            const int we = wb + part + (rank < extra ? 1 : 0);
+            if (FORM == kTilePacked) {
                 // the whole reduction of a tile fits one chunk: so do the parts of it that meet in the buffer
                 if (wb < we) pairs_segment<BITS, kLdsPacked, TU>(p, s.ntile, s.m0, wb, we, tile_buf);
             } else {
                 for (int g = wb; g < we; g += p.chunk) {
                     const int ge = g + p.chunk < we ? g + p.chunk : we;
-                    pairs_segment<BITS, kLds, TU>(p, s.ntile, s.m0, g, ge, tile_buf);
+                    pairs_segment<BITS, FORM == kTileThree ? kLdsThree : kLds, TU>(p, s.ntile, s.m0, g, ge, tile_buf);
                 }
             }
         }
@@ -749,7 +818,7 @@ void shift_pairs_fused_kernel(const PairArgs p)
         const PairSegment s = pairs_segment_at(p, it, it_end);
         const int bid = blockIdx.x;
         const int w = (gridDim.x & 7) ? bid : (bid & 7) * (int)(gridDim.x >> 3) + (bid >> 3);
-        pairs_finish_tile<PACKED>((lds_ptail *)&tail, (lds_i32 *)tile_buf, (lds_i32 *)&last_arrival, w,
+        pairs_finish_tile<FORM>((lds_ptail *)&tail, (lds_i32 *)tile_buf, (lds_i32 *)&last_arrival, w,
                                   (long)s.tile * p.comm, s.g0, s.len, s.ntile, s.m0, wave);
         // (pairs_finish_tile ends with a barrier: everybody has read the cursor)
         if (wave == 0 && lane_now() == 0) cursor[0] = it + s.len;
@@ -757,42 +826,57 @@ void shift_pairs_fused_kernel(const PairArgs p)
     }
 }
 
-// Workgroups of the fused launch: one per compute unit (eight waves) or two (four waves, PACKED); small
+// Workgroups of the fused launch: one per compute unit (eight waves) or two (four waves); small
 // layers at least 8 K groups per wave; every workgroup owns at least one iteration (a tile is finished by
 // the last of the workgroups that its range of iterations names: an empty share would never arrive).
-static int pairs_fused_blocks(long iters, bool packed)
+static int pairs_fused_blocks(long iters, int form)
 {
-    const int waves = packed ? kPairCu4Waves : kPairCuWaves;
+    const int waves = pair_tile_waves(form);
     int blocks = pair_slots() / waves;
     const long fit = (iters / (8 * waves)) / 8 * 8;
     if (fit < blocks) blocks = fit < 8 ? 8 : (int)fit;
     if (blocks > iters) blocks = iters < 1 ? 1 : (int)iters;
     return blocks;
 }
-static size_t pairs_slot_bytes(bool packed) { return (size_t)(packed ? 64 * kPairRows * kWave : 64 * kPairPixels) * 4; }
-static size_t pairs_fused_workspace(long iters, bool packed)
+// The form of the tile buffer that serves a reduction of `comm` K groups, run `chunk` groups at a time, over
+// `tiles` tiles.  A chunk's sums stay within 16 bits by construction, so the whole reduction's stay below
+// comm / chunk * 2^15: within 21 bits, sign included, up to 31 chunks' worth.  Three sums per 64-bit word pay
+// where every four-wave workgroup gets a tile or more (measured on ResNet-50's layers, batch 128: 3-10 % faster
+// there, 2-6 % slower where a tile is shared by two to four workgroups -- twice the partial tiles of the
+// eight-wave form, all of them exchanged).
+static int pairs_tile_form(const PairArgs &a, long tiles)
 {
-    const int blocks = pairs_fused_blocks(iters, packed);
-    return coop_counter_bytes(blocks) + (size_t)2 * blocks * pairs_slot_bytes(packed);
+    if (a.comm <= a.chunk) return kTilePacked;
+    if (g_tune.wide != kTuneUnset) return g_tune.wide > 0 || a.comm > 31L * a.chunk ? kTileWide : kTileThree;
+    if (a.comm <= 31L * a.chunk && tiles >= pairs_fused_blocks(tiles * a.comm, kTileThree)) return kTileThree;
+    return kTileWide;
 }
 
-template <int BITS, bool TU, bool PACKED>
+static size_t pairs_slot_bytes(int form) { return (size_t)pair_tile_words(form) * 4; }
+static size_t pairs_fused_workspace(long iters, int form)
+{
+    const int blocks = pairs_fused_blocks(iters, form);
+    return coop_counter_bytes(blocks) + (size_t)2 * blocks * pairs_slot_bytes(form);
+}
+
+template <int BITS, bool TU, int FORM>
 static int launch_pairs_fused_as(const PairArgs &a, int blocks, hipStream_t st)
 {
-    constexpr int kBytes = (PACKED ? 64 * kPairRows * kWave : 64 * kPairPixels) * 4;
-    if (!PACKED) {
+    constexpr int kBytes = pair_tile_words(FORM) * 4;
+    if (FORM != kTilePacked) {
         // above the default 64 KiB limit of a workgroup: opt in, once per device
         static std::atomic<bool> opted_in[64];
         int dev = 0;
         if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
         if (!opted_in[dev].load(std::memory_order_acquire)) {
-            hipError_t e = hipFuncSetAttribute((const void *)shift_pairs_fused_kernel<BITS, TU, PACKED>,
+            hipError_t e = hipFuncSetAttribute((const void *)shift_pairs_fused_kernel<BITS, TU, FORM>,
                                                hipFuncAttributeMaxDynamicSharedMemorySize, kBytes);
             if (e != hipSuccess) return hip_status(e);
             opted_in[dev].store(true, std::memory_order_release);
         }
     }
-    hipLaunchKernelGGL((shift_pairs_fused_kernel<BITS, TU, PACKED>), dim3(blocks), dim3(PACKED ? 256 : 512), kBytes, st, a);
+    hipLaunchKernelGGL((shift_pairs_fused_kernel<BITS, TU, FORM>), dim3(blocks), dim3(pair_tile_waves(FORM) * 64), kBytes,
+                       st, a);
     return launch_status();
 }
 
@@ -806,15 +890,16 @@ static int launch_pairs_fused(PairArgs a, void *workspace, size_t workspace_byte
     a.tile_begin = 0;
     a.tile_end = (int)tiles;
     a.whole_tiles = 0;
-    const bool packed = a.comm <= a.chunk;
-    const int blocks = pairs_fused_blocks(iters, packed);
-    if (!workspace || workspace_bytes < pairs_fused_workspace(iters, packed) || ((uintptr_t)workspace & 255))
+    const int form = pairs_tile_form(a, tiles);
+    const int blocks = pairs_fused_blocks(iters, form);
+    if (!workspace || workspace_bytes < pairs_fused_workspace(iters, form) || ((uintptr_t)workspace & 255))
         return DS_EWORKSPACE;
     a.coop_counters = (unsigned long long *)workspace;
     a.coop_slots = (int32_t *)((char *)workspace + coop_counter_bytes(blocks));
     a.coop_token = next_coop_token();
-    if (packed) return launch_pairs_fused_as<BITS, TU, true>(a, blocks, st);
-    return launch_pairs_fused_as<BITS, TU, false>(a, blocks, st);
+    if (form == kTilePacked) return launch_pairs_fused_as<BITS, TU, kTilePacked>(a, blocks, st);
+    if (form == kTileThree) return launch_pairs_fused_as<BITS, TU, kTileThree>(a, blocks, st);
+    return launch_pairs_fused_as<BITS, TU, kTileWide>(a, blocks, st);
 }
 
 // y = bias[n] before an accumulating launch; y is [img][n][pix], dense.  With the xor-mask forms the
@@ -1155,7 +1240,10 @@ DS_EXPORT size_t ds_conv2d_paired_fused_workspace_bytes(int Nb, int C, int Hp, i
     if (paired_args(a, nullptr, nullptr, nullptr, Nb, C, Hp, Wp, O, FH, FW, sh, sw, field_bits, x_bound)) return 0;
     if (a.M == 0 || a.K == 0) return 0;
     const long iters = (long)ceil_div(a.M, kPairPixels) * (a.N / 64) * a.comm;
-    return pairs_fused_workspace(iters, a.comm <= a.chunk);
+    // (room for the larger of the forms that the launch may take)
+    const size_t need = pairs_fused_workspace(iters, pairs_tile_form(a, iters / a.comm));
+    const size_t wide = pairs_fused_workspace(iters, kTileWide);
+    return need > wide ? need : wide;
 }
 
 DS_EXPORT int ds_conv2d_paired_fused_i8(const int8_t *x, const void *paired, const int32_t *bias, float *out, void *q,

@@ -441,6 +441,61 @@ def test_paired_fused_matches_oracle_chain(oracle, rng, form, shape):
     np.testing.assert_array_equal(q, want_q)
 
 
+@pytest.mark.parametrize("wide", [0, 1], ids=["three-sums-per-word", "widened"])
+@pytest.mark.parametrize("form", [2, 3, 2 | U], ids=form_id)
+@pytest.mark.parametrize("shape", [FUSED_SHAPES[0], FUSED_SHAPES[1], (24, 64, 18, 18, 128, 3, 3, (1, 1))],
+                         ids=lambda s: "x".join(map(str, s[:7])))
+def test_paired_fused_tile_buffer_forms(oracle, rng, wide, form, shape):
+    """Reductions longer than a chunk on either tile buffer -- three sums per 64-bit word (four-wave workgroups)
+    and widened sums (eight waves) -- whatever the dispatch would pick for the shape: shared tiles only, one
+    ragged tile cut many times, and more tiles than workgroups."""
+    Nb, C, Hp, Wp, O, FH, FW, stride = shape
+    bits = form & 0xff
+    x8 = random_int8(rng, (Nb, C, Hp, Wp))
+    s, sign = random_codes(rng, (O, C, FH, FW), max_s=top_field(form))
+    bias = rng.integers(-2 ** 8, 2 ** 8, size=O).astype(np.int32)
+    w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)
+    blob = abi_tile_paired(w, O, C, FH, FW, bits, form)
+    OH, OW = (Hp - FH) // stride[0] + 1, (Wp - FW) // stride[1] + 1
+    scale = (rng.random(O).astype(np.float32) + 0.5) * np.float32(2.0 ** -4)
+    shift = rng.standard_normal(O).astype(np.float32)
+    res = rng.standard_normal((Nb, O, OH, OW)).astype(np.float32)
+    emit = (1, 1, 3, 5, torch.int8)
+    want_v, want_q = _chain(oracle, x8, s, sign, bias, stride, 5, scale, shift, res, True, emit)
+    with _Tune(wide=wide):
+        out, q = abi_conv_paired_fused(x8, blob, bias, O, FH, FW, stride, form, 128, 5, scale, shift, res, True, True,
+                                       emit)
+    np.testing.assert_array_equal(out, want_v)
+    np.testing.assert_array_equal(q, want_q)
+
+
+@pytest.mark.parametrize("form", [2, 3], ids=form_id)
+def test_paired_fused_three_sums_per_word_at_their_bound(oracle, form):
+    """Every activation -128 (or 127), every code the unshifted value with one sign, and the longest reduction
+    that the three-sums-per-word buffer takes (31 chunks): the 21-bit fields reach their bound without a carry
+    into their neighbours.  int32 fixed-point output of 16.16 so that nothing saturates on the way out."""
+    bits = form & 0xff
+    num = 32 // (bits + 1)
+    chunk = (32767 // (129 if bits >= 3 else 128)) // num
+    C, O, Nb, Hp, Wp = 31 * chunk * num, 64, 1, 5, 5
+    for fill, sgn in ((-128, 1), (-128, -1), (127, 1), (127, -1)):
+        x8 = np.full((Nb, C, Hp, Wp), fill, np.int8)
+        x8[0, :, 1, 2] = -fill - 1  # one pixel of the other extreme next to them
+        s = np.zeros((O, C, 1, 1), np.int32)
+        sign = np.full((O, C, 1, 1), sgn, np.int32)
+        sign[1::2] = -sgn             # every other channel the other way
+        w, _ = oracle.pack_words(s.reshape(O, -1), sign.reshape(O, -1), bits)
+        blob = abi_tile_paired(w, O, C, 1, 1, bits, form)
+        emit = (0, 0, 16, 16, torch.int32)
+        want_v, want_q = _chain(oracle, x8, s, sign, None, (1, 1), 5, None, None, None, False, emit)
+        assert np.abs(want_v).max() * 32 > 2 ** 19, "the case does not reach the upper bits of a field"
+        with _Tune(wide=0):
+            out, q = abi_conv_paired_fused(x8, blob, None, O, 1, 1, (1, 1), form, 128, 5, None, None, None, False,
+                                           True, emit)
+        np.testing.assert_array_equal(out, want_v)
+        np.testing.assert_array_equal(q, want_q)
+
+
 @pytest.mark.parametrize("shape", FUSED_SHAPES[:4], ids=lambda s: "x".join(map(str, s[:7])))
 def test_paired_fused_output_forms(oracle, rng, shape):
     """Every combination the fused pipeline asks for: float only; fixed point only (int8 and int32, other
