@@ -543,9 +543,9 @@ __device__ __forceinline__ void pairs_write_tile(lds_ptail *t, lds_i32 *buf, int
 #pragma unroll
         for (int b = 0; b < PB; ++b) {
             if (live[b]) {
-                const g_char *at = (const g_char *)residual + 4u * pix[b] + (uint32_t)(u * CH) * ostep;
 #pragma unroll
-                for (int c = 0; c < CH; ++c) r[c][b] = *(const g_f32 *)(at + (uint32_t)c * ostep);
+                for (int c = 0; c < CH; ++c)
+                    r[c][b] = *(const g_f32 *)((const g_char *)residual + (uint32_t)(u * CH + c) * ostep + 4u * pix[b]);
             } else {
 #pragma unroll
                 for (int c = 0; c < CH; ++c) r[c][b] = 0.0f;
@@ -605,24 +605,29 @@ __device__ __forceinline__ void pairs_write_tile(lds_ptail *t, lds_i32 *buf, int
             if (relu) tile_affine<CH, PB, false, true>(f, sums, r, add_l, sa_l, sb_l, inv, u * CH);
             else tile_affine<CH, PB, false, false>(f, sums, r, add_l, sa_l, sb_l, inv, u * CH);
         }
+        // (a channel's plane is a scalar base, a pixel's place in it the lane's offset: no address arithmetic on
+        // the vector unit)
+        g_char *out_c[CH], *q_c[CH];
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            out_c[c] = out ? out + (uint32_t)(u * CH + c) * ostep : nullptr;
+            q_c[c] = q ? q + (uint32_t)(u * CH + c) * qstep : nullptr;
+        }
 #pragma unroll
         for (int b = 0; b < PB; ++b) {
             if (!live[b]) continue;
             if (out) {
-                uint32_t o = 4u * pix[b] + (uint32_t)(u * CH) * ostep;
 #pragma unroll
-                for (int c = 0; c < CH; ++c, o += ostep) *(g_f32 *)(out + o) = f[c][b];
+                for (int c = 0; c < CH; ++c) *(g_f32 *)(out_c[c] + 4u * pix[b]) = f[c][b];
             }
             if (q) {
-                uint32_t o = (uint32_t)sizeof(Q) * qpix[b] + (uint32_t)(u * CH) * qstep;
+                const uint32_t o = (uint32_t)sizeof(Q) * qpix[b];
                 if (one_bit) {
 #pragma unroll
-                    for (int c = 0; c < CH; ++c, o += qstep)
-                        *(g_q *)(q + o) = (Q)quantize_fixed_as<true>(f[c][b], qs, qlo, qhi);
+                    for (int c = 0; c < CH; ++c) *(g_q *)(q_c[c] + o) = (Q)quantize_fixed_as<true>(f[c][b], qs, qlo, qhi);
                 } else {
 #pragma unroll
-                    for (int c = 0; c < CH; ++c, o += qstep)
-                        *(g_q *)(q + o) = (Q)quantize_fixed_as<false>(f[c][b], qs, qlo, qhi);
+                    for (int c = 0; c < CH; ++c) *(g_q *)(q_c[c] + o) = (Q)quantize_fixed_as<false>(f[c][b], qs, qlo, qhi);
                 }
             }
         }
