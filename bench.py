@@ -42,10 +42,10 @@ CHW = (3, 224, 224)
 
 # the kernel behind the 3x3 convolutions of the headline network, as rocprofv3 names it
 DOMINANT_KERNEL = "ds::shift_planes_wide_coop_kernel<4, 2, true, false>"
-# HBM bytes of one launch of that kernel on the layer1 shape: 126.3 MB read + 72.5 MB written (FETCH_SIZE /
+# HBM bytes of one launch of that kernel on the layer1 shape: 77.0 MB read + 69.5 MB written (FETCH_SIZE /
 # WRITE_SIZE counters scaled by a 64 MiB copy kernel's readings); 106.6 MB are algorithmic, the rest are
-# the partial tiles that workgroups exchange through the workspace and re-read halo rows of the input
-TRAFFIC_LAYER1_BYTES = 198.8e6
+# the partial tiles that workgroups exchange through the workspace and what is left of the re-read halo rows
+TRAFFIC_LAYER1_BYTES = 146.5e6
 
 
 def log(*a):

@@ -63,13 +63,14 @@ struct Tune {
     std::atomic<int> tile{kTuneUnset};    // R * 100 + J of the two-instruction kernel
     std::atomic<int> cu{kTuneUnset};      // 0 / 4: workgroup-cooperative launch off / on (four waves per workgroup)
     std::atomic<int> notail{kTuneUnset};  // int8 kernel: keep the last round of tiles on the tile-per-wave launch
+    std::atomic<int> perm{kTuneUnset};    // int32 cooperative launch: 0 = the share space walks the pixel tiles as they lie
     std::atomic<int> wide{kTuneUnset};    // int8 fused launch: 1 = widened tile buffer (eight waves) for every reduction longer than a chunk
     std::atomic<int> chain_spin_us{-1};   // layer-chain launch: bound of a barrier wait in microseconds (-1: default)
     std::atomic<int> chain_extra{-1};     // ... arrivals a barrier waits for beyond the grid (they never come)
     void reset()
     {
         planes = kTuneUnset; split = kTuneUnset; tile = kTuneUnset; cu = kTuneUnset; notail = kTuneUnset;
-        wide = kTuneUnset;
+        wide = kTuneUnset; perm = kTuneUnset;
         chain_spin_us = -1; chain_extra = -1;
     }
 };

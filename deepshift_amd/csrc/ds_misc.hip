@@ -70,6 +70,7 @@ DS_EXPORT int ds_test_tune(const char *knob, int value)
     else if (k == "cu") g_tune.cu = value;
     else if (k == "notail") g_tune.notail = value;
     else if (k == "wide") g_tune.wide = value;
+    else if (k == "perm") g_tune.perm = value;
     else if (k == "chain_spin_us") { g_tune.chain_spin_us = value; chain_test_knobs(g_tune.chain_spin_us, g_tune.chain_extra); }
     else if (k == "chain_extra") { g_tune.chain_extra = value; chain_test_knobs(g_tune.chain_spin_us, g_tune.chain_extra); }
     else return DS_EINVAL;

@@ -83,6 +83,9 @@ struct ShiftArgs {
     // ALU about 40 instructions, and every segment of a tile needs a dozen): by pix_per_img, OW, FH * FW, FW,
     // and -- cooperative launch -- by the length of a tile and of a pixel tile's span in the share space.
     FastDiv div_pix, div_ow, div_ff, div_fw, div_len, div_span;
+    // cooperative launch: the order in which the share space walks the pixel tiles (0: as they lie)
+    int perm_t, perm_edge;
+    FastDiv div_perm;
     int OH;                               // pix_per_img / OW
     int koff_max;                         // element offset of the last real reduction index
     QuantSpec ep_spec;
@@ -95,7 +98,8 @@ static void derive_geometry(ShiftArgs &a)
     a.div_ow = fast_div((uint32_t)a.OW);
     a.div_ff = fast_div((uint32_t)(a.FH * a.FW));
     a.div_fw = fast_div((uint32_t)a.FW);
-    a.div_len = a.div_span = fast_div(1u);  // set by the cooperative launch
+    a.div_len = a.div_span = a.div_perm = fast_div(1u);  // set by the cooperative launch
+    a.perm_t = a.perm_edge = 0;
     a.OH = a.OW > 0 ? a.pix_per_img / a.OW : 0;
     const int ff = a.FH * a.FW;
     a.koff_max = ff > 0 && a.K >= ff ? (a.K / ff - 1) * a.x_plane + (a.FH - 1) * a.x_row + a.FW - 1 : 0;
@@ -1209,7 +1213,19 @@ void shift_planes_wide_coop_kernel(const ShiftArgs p, const ShiftArgs p2)
         if (v1 > padded) v1 = padded;
         const int g0 = v0 > pad ? v0 - pad : 0;
         const int g1 = (int)v1 > pad ? (int)v1 - pad : 0;
-        const int m0 = mtile * kCoopPix;
+        // Where the pixel tile lies.  A workgroup's share is a run of T and a bit consecutive tiles of the share
+        // space; were they consecutive in the image too, the tiles that the compute units work on at one time
+        // would lie T tiles apart, and the rows that neighbouring tiles both read (a 3x3 window: two of the
+        // four or so rows of a 128-pixel tile) would come from memory twice -- by the time a workgroup reaches
+        // its next tile the L2 has long been overwritten.  So the first T * G tiles of the space are laid out
+        // transposed, index j at tile (j mod T) * G + j / T: at any moment neighbouring workgroups (the same
+        // XCD, the same L2) work on neighbouring tiles.
+        int mphys = mtile;
+        if (!PAIR && pa.perm_t && mtile < pa.perm_edge) {
+            const int q = (int)div_by_uniform((uint32_t)mtile, fast_div_of(pa.div_perm));
+            mphys = (mtile - q * pa.perm_t) * (int)gridDim.x + q;
+        }
+        const int m0 = mphys * kCoopPix;
         const int len = g1 - g0;
         if (!direct && len == 0) {  // the share ends inside the tile's padding: nothing of it to do here
             it += v1 - v0;
@@ -1255,6 +1271,13 @@ static int launch_planes_coop(const ShiftArgs &first, long iters, hipStream_t st
     if (span <= 0 || (long)a.tiles_m4 * span >= (1L << 31)) return DS_ETOOLARGE;
     a.div_len = fast_div((uint32_t)(a.comm + a.coop_pad));
     a.div_span = fast_div((uint32_t)span);
+    // (tile order of the share space, see the kernel: transposed where a workgroup holds two tiles or more)
+    const int per_group = a.tiles_m4 / blocks;
+    if (!second && !a.whole_tile_shares && per_group >= 2 && !(g_tune.perm != kTuneUnset && g_tune.perm == 0)) {
+        a.perm_t = per_group;
+        a.perm_edge = per_group * blocks;
+        a.div_perm = fast_div((uint32_t)per_group);
+    }
     if (second) {
         ShiftArgs b = *second;
         b.coop_token = a.coop_token;

@@ -14,7 +14,8 @@ extern "C" {
  * shift-plane kernel), "split" (K split; shift-plane kernels: 0 = equal shares, 1 = one tile per
  * wave), "tile" (R * 100 + J of the two-instruction kernel), "cu" (0 / 4 / 8 waves per cooperative
  * workgroup), "notail", "wide" (1: the int8 fused launch keeps reductions longer than a chunk on the
- * widened tile buffer of eight-wave workgroups); "chain_spin_us" (bound of a barrier wait of ds_linear_chain_f32 in
+ * widened tile buffer of eight-wave workgroups), "perm" (0: the int32 cooperative launch walks the pixel
+ * tiles in image order); "chain_spin_us" (bound of a barrier wait of ds_linear_chain_f32 in
  * microseconds) and "chain_extra" (arrivals its barriers wait for beyond the grid, which never come: with
  * a small bound every workgroup gives up and exits, which is how the tests reach that path without
  * hanging anything).  knob == NULL clears every override.  Each knob is an atomic integer that an

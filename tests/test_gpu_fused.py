@@ -104,6 +104,9 @@ GEOMS = [
     (3, 256, 14, 14, 64, 1, 1, (1, 1)),      # 256 -> 64, 43 K groups
     (2, 256, 17, 16, 512, 1, 1, (2, 2)),     # strided shortcut, eight channel tiles
     (6, 3, 37, 37, 64, 7, 7, (2, 2)),        # a stem without its pooling: K = 147, a partial last group
+    # 100 pixel tiles on 32 workgroups: three tiles and a bit per share, so the share space walks the first 96
+    # tiles transposed (index j at tile (j mod 3) * 32 + j / 3) and the last four as they lie
+    (8, 64, 40, 40, 64, 1, 1, (1, 1)),
 ]
 # layers that are not a multiple of 64 channels wide: the fused form of the two-instruction kernel
 NARROW_GEOMS = [
