@@ -876,6 +876,8 @@ def main():
                                "pooling in one conversion pass, global average pooling fp32 PyTorch",
                    "batch": BATCH, "shift_layers": 21, "shift_launches": len(layers), "pairs_per_step": pairs},
         "unfused_images_per_s": BATCH / sec_unfused,
+        # the same step replayed from a captured HIP graph: an extra beside `value`, which is the eager step
+        **graph_replay_timing(fused, x, args.steps),
         "shift_kernel_ms_per_step": kernel_s * 1e3,
         "shift_gops": 2 * pairs / kernel_s / 1e9,
         "shift_layers_images_per_s": BATCH / kernel_s,
