@@ -233,8 +233,9 @@ __device__ __forceinline__ void pairs_segment(const ARGS &p, int ntile, int m0, 
                 s[2 * r] = lo;
                 s[2 * r + 1] = hi;
             }
-            atomicAdd(l64 + (j * 2 + 0) * kWave + lane, (unsigned long long)(s[0] + (s[1] << 21) + (s[2] << 42)));
-            atomicAdd(l64 + (j * 2 + 1) * kWave + lane, (unsigned long long)(s[3] + (s[4] << 21) + (s[5] << 42)));
+            // (multiplications, not shifts: the sums are signed)
+            atomicAdd(l64 + (j * 2 + 0) * kWave + lane, (unsigned long long)(s[0] + s[1] * (1LL << 21) + s[2] * (1LL << 42)));
+            atomicAdd(l64 + (j * 2 + 1) * kWave + lane, (unsigned long long)(s[3] + s[4] * (1LL << 21) + s[5] * (1LL << 42)));
         }
         return;
     }
@@ -568,9 +569,9 @@ __device__ __forceinline__ void pairs_write_tile(lds_ptail *t, lds_i32 *buf, int
                     long long v = *cell;
                     *cell = 0;
                     // s0 + s1 * 2^21 + s2 * 2^42, every sum within 21 bits: take the lowest, sign-extended, off
-                    const int32_t s0 = (int32_t)((v << 43) >> 43);
+                    const int32_t s0 = (int32_t)((long long)((unsigned long long)v << 43) >> 43);
                     v = (v - s0) >> 21;
-                    const int32_t s1 = (int32_t)((v << 43) >> 43);
+                    const int32_t s1 = (int32_t)((long long)((unsigned long long)v << 43) >> 43);
                     const int32_t s2 = (int32_t)((v - s1) >> 21);
                     // (pixels that lived in low halves: the even blocks)
                     sums[c][3 * h] = s0 + (h == 0 ? neg : 0);
