@@ -627,7 +627,8 @@ def pmc_target_other(device):
         channel-major scratch);
       * the int8 kernel's fused launch (ds_conv2d_paired_fused_i8: BatchNorm affine, ReLU and the next layer's
         padded int8 input from the epilogue) on ResNet-50's 1x1 convolutions with K = 256 (256 -> 64 at 56x56
-        and 256 -> 128 at 28x28, both at batch 128, weight_bits 3, activations in [0, 96]);
+        and 256 -> 128 at 28x28, both at batch 128, weight_bits 3, activations in [0, 96]) and on a block end
+        of its first stage (64 -> 256 at 56x56: residual in, float result and unpadded int8 input out);
       * the one-launch LinearShift kernel (ds_linear_small_f32) on the three layers of the MNIST MLP at
         batch 64 and on ResNet-18's classifier (64 x 512 x 1000)."""
     from deepshift_amd import _lib, kernels, utils
@@ -649,12 +650,14 @@ def pmc_target_other(device):
     xT = kernels.quantize_transpose(xg)
     tiledg = kernels._tiled_of(cwg, 4096, 4096)
     int8 = []
-    for (C, H, O) in ((256, 56, 64), (256, 28, 128)):
+    for (C, H, O, block_end) in ((256, 56, 64, False), (256, 28, 128, False), (64, 56, 256, True)):
         x8 = torch.randint(0, 97, (128, C, H, H), generator=g, dtype=torch.int32).to(torch.int8).to(device)
         cw8 = codes((O, C, 1, 1), lo=-2)
         fields = kernels.paired_fields(cw8, O, 3, 5)
+        res8 = torch.randn(128, O, H, H, generator=g).to(device) if block_end else None
         int8.append((x8, kernels._paired_of(cw8, fields, O, C, 1, 1), O, fields[1],
-                     (torch.rand(O, generator=g) * 2.0 ** -5).to(device), torch.randn(O, generator=g).to(device), {}))
+                     (torch.rand(O, generator=g) * 2.0 ** -5).to(device), torch.randn(O, generator=g).to(device), {},
+                     res8))
     small = []
     for (M, K, N) in ((64, 784, 512), (64, 512, 512), (64, 512, 10), (64, 512, 1000)):
         cws = codes((N, K))
@@ -665,9 +668,10 @@ def pmc_target_other(device):
         _lib.call("ds_copy_i32", _lib.ptr(src), _lib.ptr(dst), n, _lib.current_stream(device))
         kernels.conv2d_tiled(x2, tiled2, None, 64, (3, 3), (1, 1), cw2.bits, cw2.base)
         kernels.linear_tiled(xT, 4096, tiledg, None, 4096, cwg.bits, cwg.base)
-        for x8, blob8, O, fb, sc8, of8, cache8 in int8:
-            kernels.conv2d_paired_fused(x8, blob8, None, O, (1, 1), (1, 1), fb, 96, 5, sc8, of8, None, True,
-                                        ((1, 1), 3, 5, torch.int8), False, cache8)
+        for x8, blob8, O, fb, sc8, of8, cache8, res8 in int8:
+            kernels.conv2d_paired_fused(x8, blob8, None, O, (1, 1), (1, 1), fb, 96, 5, sc8, of8, res8, True,
+                                        ((1, 1) if res8 is None else (0, 0), 3, 5, torch.int8), res8 is not None,
+                                        cache8)
         for xs, tileds, N, kb in small:
             kernels.linear_small(xs, tileds, None, N, kb, 0, 16, 16, False, True)
     torch.cuda.synchronize()
