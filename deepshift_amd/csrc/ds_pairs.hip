@@ -1246,10 +1246,14 @@ DS_EXPORT size_t ds_conv2d_paired_fused_workspace_bytes(int Nb, int C, int Hp, i
     if (paired_args(a, nullptr, nullptr, nullptr, Nb, C, Hp, Wp, O, FH, FW, sh, sw, field_bits, x_bound)) return 0;
     if (a.M == 0 || a.K == 0) return 0;
     const long iters = (long)ceil_div(a.M, kPairPixels) * (a.N / 64) * a.comm;
-    // (room for the larger of the forms that the launch may take)
-    const size_t need = pairs_fused_workspace(iters, pairs_tile_form(a, iters / a.comm));
-    const size_t wide = pairs_fused_workspace(iters, kTileWide);
-    return need > wide ? need : wide;
+    // (room for whichever form the launch takes: the test hook may change the choice between this call and the
+    // launch)
+    size_t need = 0;
+    for (int form : {kTileWide, kTilePacked, kTileThree}) {
+        const size_t bytes = pairs_fused_workspace(iters, form);
+        if (bytes > need) need = bytes;
+    }
+    return need;
 }
 
 DS_EXPORT int ds_conv2d_paired_fused_i8(const int8_t *x, const void *paired, const int32_t *bias, float *out, void *q,
